@@ -1,0 +1,239 @@
+"""ctypes binding of libaq_mi355.so -- plumbing for tests, the smoke check and the benchmark.
+
+The product is the shared library; this module only loads it and marshals numpy
+arrays and device pointers into its C ABI (include/aq_mi355.h, include/aq_mi355_host.h).
+It raises if the library has not been built: there is no fallback path.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "libaq_mi355.so")
+
+AQ_OK = 0
+AQ_ERR_ARG = -1
+AQ_ERR_SHAPE = -2
+AQ_ERR_UNSUPPORTED = -3
+AQ_ERR_INDEX = -4
+AQ_ERR_NOMEM = -5
+AQ_ERR_NODEVICE = -6
+AQ_ERR_SIZE = -7
+AQ_OUT_F32 = 0x1
+
+OP_QMV = 0
+OP_QMM = 1
+
+_c = ctypes
+_vp, _i, _u, _sz, _f = _c.c_void_p, _c.c_int, _c.c_uint, _c.c_size_t, _c.c_float
+_cp = _c.c_char_p
+
+# name -> (restype, argtypes); every symbol include/*.h declares
+PROTOTYPES = {
+    "aq_version": (_cp, []),
+    "aq_last_error": (_cp, []),
+    "aq_create": (_i, [_i, _c.POINTER(_vp)]),
+    "aq_destroy": (None, [_vp]),
+    "aq_use_stream": (_i, [_vp, _vp]),
+    "aq_use_own_stream": (_i, [_vp]),
+    "aq_device_name": (_i, [_vp, _cp, _sz]),
+    "aq_malloc": (_i, [_vp, _sz, _c.POINTER(_vp)]),
+    "aq_free": (_i, [_vp, _vp]),
+    "aq_h2d": (_i, [_vp, _vp, _vp, _sz]),
+    "aq_d2h": (_i, [_vp, _vp, _vp, _sz]),
+    "aq_d2d": (_i, [_vp, _vp, _vp, _sz]),
+    "aq_fill_zero": (_i, [_vp, _vp, _sz]),
+    "aq_sync": (_i, [_vp]),
+    "aq_timer_start": (_i, [_vp]),
+    "aq_timer_stop": (_i, [_vp, _c.POINTER(_f)]),
+    "aq_qmv": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _u]),
+    "aq_qmm": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _u]),
+    "aq_gather_qmv": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _u]),
+    "aq_dequant_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _c.c_int64, _i, _i, _i]),
+    "aq_matvec_host": (_i, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _i, _i, _i, _i, _vp, _sz]),
+    "aq_proj_quant_matmul_host": (_i, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _i, _i, _i, _i, _i]),
+    "aq_variant_count": (_i, [_i]),
+    "aq_variant_name": (_cp, [_i, _i]),
+    "aq_force_variant": (_i, [_vp, _i, _i]),
+    "aq_last_variant": (_cp, [_vp, _i]),
+    "aqh_last_error": (_cp, []),
+    "aqh_register_rocm_backend": (None, []),
+    "aqh_backend_quant_registered": (_i, [_cp, _cp]),
+    "aqh_backend_quant_bits": (_i, [_cp, _cp]),
+    "aqh_backend_quant_matvec": (_i, [_cp, _cp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _i, _i, _i, _i, _vp, _sz,
+                                      _c.POINTER(_sz)]),
+    "aqh_proj_quant_matmul_into": (_i, [_vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _i, _i, _i, _i, _i]),
+    "aqh_concat_quant_rows": (_i, [_vp, _sz, _vp, _sz, _vp, _i, _vp, _sz, _vp, _sz, _vp, _i, _i, _i, _i, _i, _i, _i,
+                                   _vp, _vp, _vp, _c.POINTER(_i)]),
+    "aqh_affine_geometry": (None, [_i, _i, _i, _c.POINTER(_i), _c.POINTER(_i)]),
+}
+
+
+class AqError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("aq_mi355 error %d: %s" % (code, msg))
+        self.code = code
+        self.msg = msg
+
+
+_lib = None
+
+
+def load():
+    """dlopen the in-tree library; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError("libaq_mi355.so is not built (run: python go-inference_amd/build.py); "
+                           "there is no non-HIP path")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in PROTOTYPES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def _ptr(obj):
+    """Device pointer (int / DeviceBuffer) or host numpy array -> void*."""
+    if obj is None:
+        return None
+    if isinstance(obj, DeviceBuffer):
+        return obj.ptr
+    if isinstance(obj, np.ndarray):
+        return obj.ctypes.data
+    return int(obj)
+
+
+class DeviceBuffer:
+    """A hipMalloc'd span owned through aq_malloc / aq_free."""
+
+    def __init__(self, ctx, nbytes):
+        self.ctx = ctx
+        self.nbytes = int(nbytes)
+        p = _vp()
+        ctx._check(ctx.lib.aq_malloc(ctx.handle, self.nbytes, ctypes.byref(p)))
+        self.ptr = p.value or 0
+
+    def upload(self, arr):
+        arr = np.ascontiguousarray(arr)
+        assert arr.nbytes <= self.nbytes
+        self.ctx._check(self.ctx.lib.aq_h2d(self.ctx.handle, self.ptr, arr.ctypes.data, arr.nbytes))
+        return self
+
+    def download(self, dtype, count=None):
+        dtype = np.dtype(dtype)
+        if count is None:
+            count = self.nbytes // dtype.itemsize
+        out = np.empty(count, dtype=dtype)
+        self.ctx._check(self.ctx.lib.aq_d2h(self.ctx.handle, out.ctypes.data, self.ptr, out.nbytes))
+        return out
+
+    def free(self):
+        if self.ptr:
+            self.ctx.lib.aq_free(self.ctx.handle, self.ptr)
+            self.ptr = 0
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Context:
+    def __init__(self, device=0):
+        self.lib = load()
+        h = _vp()
+        rc = self.lib.aq_create(device, ctypes.byref(h))
+        if rc != AQ_OK:
+            raise AqError(rc, self.lib.aq_last_error().decode())
+        self.handle = h
+
+    def close(self):
+        if self.handle:
+            self.lib.aq_destroy(self.handle)
+            self.handle = None
+
+    def _check(self, rc):
+        if rc != AQ_OK:
+            raise AqError(rc, self.lib.aq_last_error().decode())
+
+    def device_name(self):
+        buf = ctypes.create_string_buffer(256)
+        self._check(self.lib.aq_device_name(self.handle, buf, 256))
+        return buf.value.decode()
+
+    def alloc(self, nbytes):
+        return DeviceBuffer(self, nbytes)
+
+    def to_device(self, arr):
+        arr = np.ascontiguousarray(arr)
+        return DeviceBuffer(self, max(arr.nbytes, 16)).upload(arr)
+
+    def sync(self):
+        self._check(self.lib.aq_sync(self.handle))
+
+    def fill_zero(self, buf, nbytes=None):
+        self._check(self.lib.aq_fill_zero(self.handle, _ptr(buf), buf.nbytes if nbytes is None else nbytes))
+
+    def timer_start(self):
+        self._check(self.lib.aq_timer_start(self.handle))
+
+    def timer_stop(self):
+        ms = _f()
+        self._check(self.lib.aq_timer_stop(self.handle, ctypes.byref(ms)))
+        return ms.value
+
+    def qmv(self, x, w, s, b, y, M, K, N, group_size=64, bits=4, flags=0):
+        self._check(self.lib.aq_qmv(self.handle, _ptr(x), _ptr(w), _ptr(s), _ptr(b), _ptr(y), M, K, N, group_size,
+                                    bits, flags))
+
+    def qmm(self, x, w, s, b, y, M, K, N, group_size=64, bits=4, flags=0):
+        self._check(self.lib.aq_qmm(self.handle, _ptr(x), _ptr(w), _ptr(s), _ptr(b), _ptr(y), M, K, N, group_size,
+                                    bits, flags))
+
+    def gather_qmv(self, x, w, s, b, lhs, rhs, y, routes, x_rows, K, N, num_experts, expert_rows, row_base=0,
+                   group_size=64, bits=4, flags=0):
+        self._check(self.lib.aq_gather_qmv(self.handle, _ptr(x), _ptr(w), _ptr(s), _ptr(b), _ptr(lhs), _ptr(rhs),
+                                           _ptr(y), routes, x_rows, K, N, num_experts, expert_rows, row_base,
+                                           group_size, bits, flags))
+
+    def dequant_f32(self, w, s, b, out, N, K, group_size=64, bits=4):
+        self._check(self.lib.aq_dequant_f32(self.handle, _ptr(w), _ptr(s), _ptr(b), _ptr(out), N, K, group_size,
+                                            bits))
+
+    def force_variant(self, op, variant):
+        self._check(self.lib.aq_force_variant(self.handle, op, variant))
+
+    def last_variant(self, op):
+        return self.lib.aq_last_variant(self.handle, op).decode()
+
+    # host-slice entry points -------------------------------------------------
+    def matvec_host(self, x, packed, scales, biases, out_dim, in_dim, group_size, bits):
+        """model.QuantMatVec.MatVec over host bytes; returns out_dim*2 bytes (uint8 array)."""
+        x, packed, scales, biases = (np.ascontiguousarray(a).view(np.uint8).reshape(-1)
+                                     for a in (x, packed, scales, biases))
+        out = np.zeros(max(out_dim, 0) * 2, dtype=np.uint8)
+        self._check(self.lib.aq_matvec_host(self.handle, x.ctypes.data, x.size, packed.ctypes.data, packed.size,
+                                            scales.ctypes.data, scales.size, biases.ctypes.data, biases.size,
+                                            out_dim, in_dim, group_size, bits, out.ctypes.data, out.size))
+        return out
+
+    def proj_quant_matmul_host(self, x_f32, packed, scales, biases, M, K, N, group_size, bits):
+        x_f32 = np.ascontiguousarray(x_f32, dtype=np.float32).reshape(-1)
+        packed, scales, biases = (np.ascontiguousarray(a).view(np.uint8).reshape(-1) for a in (packed, scales, biases))
+        out = np.zeros(max(M * N, 0), dtype=np.float32)
+        self._check(self.lib.aq_proj_quant_matmul_host(self.handle, out.ctypes.data, x_f32.ctypes.data, x_f32.size,
+                                                       packed.ctypes.data, packed.size, scales.ctypes.data,
+                                                       scales.size, biases.ctypes.data, biases.size, M, K, N,
+                                                       group_size, bits))
+        return out.reshape(M, N)
+
+
+def variant_names(op):
+    lib = load()
+    return [lib.aq_variant_name(op, i).decode() for i in range(lib.aq_variant_count(op))]

@@ -1,0 +1,516 @@
+// C-ABI layer of libaq_mi355.so: context, device memory, host-side argument
+// validation, kernel selection and launch.  See include/aq_mi355.h for the
+// contract of each entry point and the reference interface it replaces.
+#include "../../include/aq_mi355.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "aq_kernels.h"
+#include "aq_qmm.h"
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return code;
+}
+
+int hip_fail(hipError_t rc, const char* what) {
+    // Same wording as the reference's driver errors (go/engine/hip/hip_driver_cgo.go:1728-1730).
+    return fail((int)rc, "rocm.hip.%s: HIP returned %d (%s)", what, (int)rc, hipGetErrorString(rc));
+}
+
+#define AQ_HIP(call, what)                              \
+    do {                                                \
+        hipError_t rc__ = (call);                       \
+        if (rc__ != hipSuccess) return hip_fail(rc__, what); \
+    } while (0)
+
+bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
+int ilog2(int v) {
+    int s = 0;
+    while ((1 << s) < v) s++;
+    return s;
+}
+bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+}  // namespace
+
+struct aq_ctx {
+    int device = 0;
+    hipStream_t own_stream = nullptr;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    std::mutex mu;
+    int forced[2] = {-1, -1};
+    const char* last_variant[2] = {"", ""};
+    int cu_count = 0;
+    char name[256] = {0};
+};
+
+namespace {
+
+// Widths every path accepts (MLX affine widths the reference dispatches,
+// go/model/quant_weight.go:11-13); 1-bit packs are widened to 2-bit by the
+// loader (go/model/linear.go:66-84) and are rejected here.
+bool width_ok(int bits) { return bits == 2 || bits == 3 || bits == 4 || bits == 5 || bits == 6 || bits == 8; }
+
+// Mirrors validateHIPMLXAffineProjectionShape (go/engine/hip/hip_projection_reference.go:122-144)
+// and MatMulQuantF32NTInto's geometry checks (go/engine/metal/quant_seam_backend.go:41-49).
+int check_geometry(const char* op, int K, int group_size, int bits) {
+    if (!width_ok(bits)) return fail(AQ_ERR_UNSUPPORTED, "%s: unsupported affine width %d bits", op, bits);
+    if (group_size <= 0) return fail(AQ_ERR_SHAPE, "%s: group size must be positive", op);
+    if (K % group_size != 0) return fail(AQ_ERR_SHAPE, "%s: cols %d must be divisible by group size %d", op, K, group_size);
+    if (((int64_t)K * bits) % 32 != 0)
+        return fail(AQ_ERR_SHAPE, "%s: cols*bits must be divisible by 32 for MLX affine packing", op);
+    return AQ_OK;
+}
+
+// The dot2 kernels need 16-byte chunks of a row to sit inside one group and
+// 128-bit aligned rows.
+bool dot2_eligible(int K, int group_size, int bits, const void* x, const void* w, size_t lds_bytes) {
+    if (bits != 4 && bits != 8) return false;
+    if (group_size != 32 && group_size != 64 && group_size != 128) return false;
+    if (((int64_t)K * bits) % 128 != 0 || K % 8 != 0) return false;
+    if (!aligned(x, 16) || !aligned(w, 16)) return false;
+    return lds_bytes <= 160 * 1024;
+}
+
+// Pick a dot2 variant: largest rows-per-wavefront that still yields at least
+// ~8 wavefronts per CU, 4 wavefronts per workgroup.
+int pick_qmv_variant(const aq_ctx* ctx, int bits, int m, bool gather, int N, int K, int routes) {
+    const int cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
+    const int64_t total_rows = (int64_t)N * (gather ? routes : 1);
+    int want_rows = 1;
+    const int chunks = K * bits / 128;
+    const int slices = (chunks + 63) / 64;
+    for (int r : {8, 4, 2}) {
+        if (total_rows / r >= (int64_t)cus * 8 && r * slices >= 2) {
+            want_rows = r;
+            break;
+        }
+    }
+    if (m > 1 && want_rows > 4) want_rows = 4;
+    int best = -1;
+    for (int i = 0; i < aq::qmv_variant_count(); i++) {
+        const aq::QmvVariant* v = aq::qmv_variant(i);
+        if (v->bits != bits || v->m != m || (v->gather != 0) != gather) continue;
+        if (v->waves != 4 || v->depth != 2) continue;
+        if (v->rows == want_rows) return i;
+        if (best < 0 || (v->rows < want_rows && v->rows > aq::qmv_variant(best)->rows)) best = i;
+    }
+    return best;
+}
+
+int launch_qmv_rows(aq_ctx* ctx, aq::QmvArgs a, int group_size, int bits, bool gather) {
+    const int M = a.M;
+    const bool fast = dot2_eligible(a.K, group_size, bits, a.x, a.w, (size_t)(M < 4 ? M : 4) * a.K * 2);
+    if (!fast) {
+        ctx->last_variant[0] = "qmv_generic";
+        AQ_HIP(aq::qmv_generic_launch(a, bits, group_size, gather, ctx->stream), "hipLaunchKernel");
+        return AQ_OK;
+    }
+    a.gs_shift = ilog2(group_size);
+    const size_t esize = a.out_f32 ? 4 : 2;
+    for (int m0 = 0; m0 < M;) {
+        int m = M - m0 < 4 ? M - m0 : 4;
+        int idx = ctx->forced[0];
+        if (idx >= 0) {
+            const aq::QmvVariant* v = aq::qmv_variant(idx);
+            if (!v || v->bits != bits || (v->gather != 0) != gather || v->m > M - m0)
+                return fail(AQ_ERR_ARG, "aq_qmv: forced variant %d does not fit bits=%d gather=%d rows=%d", idx, bits,
+                            (int)gather, M - m0);
+            m = v->m;
+        } else {
+            idx = pick_qmv_variant(ctx, bits, m, gather, a.N, a.K, a.routes);
+            if (idx < 0) return fail(AQ_ERR_UNSUPPORTED, "aq_qmv: no kernel variant for bits=%d m=%d", bits, m);
+        }
+        aq::QmvArgs c = a;
+        c.M = m;
+        c.x = a.x + (size_t)m0 * a.K;
+        c.y = static_cast<char*>(a.y) + (size_t)m0 * a.N * esize;
+        ctx->last_variant[0] = aq::qmv_variant(idx)->name;
+        AQ_HIP(aq::qmv_launch(idx, c, ctx->stream), "hipLaunchKernel");
+        m0 += m;
+    }
+    return AQ_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* aq_version(void) { return "aq_mi355 0.1 (gfx950)"; }
+const char* aq_last_error(void) { return g_last_error.c_str(); }
+
+int aq_create(int device, aq_ctx** out) {
+    if (!out) return fail(AQ_ERR_ARG, "aq_create: out is null");
+    *out = nullptr;
+    int count = 0;
+    hipError_t rc = hipGetDeviceCount(&count);
+    if (rc != hipSuccess || count <= 0) return fail(AQ_ERR_NODEVICE, "aq_create: no HIP device available");
+    if (device < 0 || device >= count) return fail(AQ_ERR_ARG, "aq_create: device %d out of range (have %d)", device, count);
+    AQ_HIP(hipSetDevice(device), "hipSetDevice");
+    hipDeviceProp_t prop;
+    AQ_HIP(hipGetDeviceProperties(&prop, device), "hipGetDeviceProperties");
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(AQ_ERR_NODEVICE, "aq_create: device %d is %s; this library carries gfx950 code only", device,
+                    prop.gcnArchName);
+    aq_ctx* ctx = new (std::nothrow) aq_ctx();
+    if (!ctx) return fail(AQ_ERR_NOMEM, "aq_create: out of host memory");
+    ctx->device = device;
+    ctx->cu_count = prop.multiProcessorCount;
+    snprintf(ctx->name, sizeof ctx->name, "%s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
+    rc = hipStreamCreateWithFlags(&ctx->own_stream, hipStreamNonBlocking);
+    if (rc == hipSuccess) rc = hipEventCreate(&ctx->ev0);
+    if (rc == hipSuccess) rc = hipEventCreate(&ctx->ev1);
+    if (rc != hipSuccess) {
+        aq_destroy(ctx);
+        return hip_fail(rc, "hipStreamCreate");
+    }
+    ctx->stream = ctx->own_stream;
+    *out = ctx;
+    return AQ_OK;
+}
+
+void aq_destroy(aq_ctx* ctx) {
+    if (!ctx) return;
+    if (ctx->own_stream) {
+        (void)hipStreamSynchronize(ctx->own_stream);
+        (void)hipStreamDestroy(ctx->own_stream);
+    }
+    if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
+    if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
+    delete ctx;
+}
+
+int aq_use_stream(aq_ctx* ctx, void* hip_stream) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_use_stream: ctx is null");
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    ctx->stream = static_cast<hipStream_t>(hip_stream);
+    return AQ_OK;
+}
+
+int aq_use_own_stream(aq_ctx* ctx) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_use_own_stream: ctx is null");
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    ctx->stream = ctx->own_stream;
+    return AQ_OK;
+}
+
+int aq_device_name(aq_ctx* ctx, char* buf, size_t buf_len) {
+    if (!ctx || !buf || buf_len == 0) return fail(AQ_ERR_ARG, "aq_device_name: bad argument");
+    snprintf(buf, buf_len, "%s", ctx->name);
+    return AQ_OK;
+}
+
+int aq_malloc(aq_ctx* ctx, size_t bytes, void** dptr) {
+    if (!ctx || !dptr) return fail(AQ_ERR_ARG, "aq_malloc: bad argument");
+    *dptr = nullptr;
+    if (bytes == 0) return AQ_OK;
+    AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    AQ_HIP(hipMalloc(dptr, bytes), "hipMalloc");
+    return AQ_OK;
+}
+
+int aq_free(aq_ctx* ctx, void* dptr) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_free: ctx is null");
+    if (!dptr) return AQ_OK;
+    AQ_HIP(hipFree(dptr), "hipFree");
+    return AQ_OK;
+}
+
+int aq_h2d(aq_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes) {
+    if (!ctx || (bytes && (!dst_dev || !src_host))) return fail(AQ_ERR_ARG, "aq_h2d: bad argument");
+    if (!bytes) return AQ_OK;
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    AQ_HIP(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, ctx->stream), "hipMemcpyHtoD");
+    AQ_HIP(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+    return AQ_OK;
+}
+
+int aq_d2h(aq_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes) {
+    if (!ctx || (bytes && (!dst_host || !src_dev))) return fail(AQ_ERR_ARG, "aq_d2h: bad argument");
+    if (!bytes) return AQ_OK;
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    AQ_HIP(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream), "hipMemcpyDtoH");
+    AQ_HIP(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+    return AQ_OK;
+}
+
+int aq_d2d(aq_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes) {
+    if (!ctx || (bytes && (!dst_dev || !src_dev))) return fail(AQ_ERR_ARG, "aq_d2d: bad argument");
+    if (!bytes) return AQ_OK;
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    AQ_HIP(hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, ctx->stream), "hipMemcpyDtoD");
+    return AQ_OK;
+}
+
+int aq_fill_zero(aq_ctx* ctx, void* dptr, size_t bytes) {
+    if (!ctx || (bytes && !dptr)) return fail(AQ_ERR_ARG, "aq_fill_zero: bad argument");
+    if (!bytes) return AQ_OK;
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    AQ_HIP(aq::fill_zero_launch(dptr, bytes, ctx->stream), "hipLaunchKernel");
+    return AQ_OK;
+}
+
+int aq_sync(aq_ctx* ctx) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_sync: ctx is null");
+    AQ_HIP(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+    return AQ_OK;
+}
+
+int aq_timer_start(aq_ctx* ctx) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_timer_start: ctx is null");
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    AQ_HIP(hipEventRecord(ctx->ev0, ctx->stream), "hipEventRecord");
+    return AQ_OK;
+}
+
+int aq_timer_stop(aq_ctx* ctx, float* elapsed_ms) {
+    if (!ctx || !elapsed_ms) return fail(AQ_ERR_ARG, "aq_timer_stop: bad argument");
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    AQ_HIP(hipEventRecord(ctx->ev1, ctx->stream), "hipEventRecord");
+    AQ_HIP(hipEventSynchronize(ctx->ev1), "hipEventSynchronize");
+    AQ_HIP(hipEventElapsedTime(elapsed_ms, ctx->ev0, ctx->ev1), "hipEventElapsedTime");
+    return AQ_OK;
+}
+
+int aq_qmv(aq_ctx* ctx, const void* x, const void* packed, const void* scales, const void* biases, void* y, int M,
+           int K, int N, int group_size, int bits, unsigned flags) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_qmv: ctx is null");
+    if (M < 0 || K < 0 || N < 0) return fail(AQ_ERR_SHAPE, "aq_qmv: M, K, N must be non-negative");
+    if (M == 0 || N == 0 || K == 0) return AQ_OK;
+    if (int rc = check_geometry("aq_qmv", K, group_size, bits)) return rc;
+    if (!x || !packed || !scales || !biases || !y) return fail(AQ_ERR_ARG, "aq_qmv: null operand");
+    if (!aligned(x, 2) || !aligned(packed, 4) || !aligned(scales, 2) || !aligned(biases, 2) || !aligned(y, 2))
+        return fail(AQ_ERR_ARG, "aq_qmv: operand pointer is not element-aligned");
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    if (M > aq::kQmvMaxRows && ctx->forced[0] < 0) {
+        return aq::qmm_dispatch(ctx->stream, ctx->cu_count, ctx->forced[1], &ctx->last_variant[1], x, packed, scales,
+                                biases, y, M, K, N, group_size, bits, (flags & AQ_OUT_F32) != 0, fail);
+    }
+    aq::QmvArgs a{};
+    a.x = static_cast<const uint16_t*>(x);
+    a.w = static_cast<const uint32_t*>(packed);
+    a.s = static_cast<const uint16_t*>(scales);
+    a.b = static_cast<const uint16_t*>(biases);
+    a.y = y;
+    a.K = K;
+    a.N = N;
+    a.M = M;
+    a.out_f32 = (flags & AQ_OUT_F32) ? 1 : 0;
+    a.routes = 1;
+    return launch_qmv_rows(ctx, a, group_size, bits, false);
+}
+
+int aq_qmm(aq_ctx* ctx, const void* x, const void* packed, const void* scales, const void* biases, void* y, int M,
+           int K, int N, int group_size, int bits, unsigned flags) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_qmm: ctx is null");
+    // go/engine/metal/quant_seam_backend.go:41-43: the matmul seam rejects non-positive dims.
+    if (M <= 0 || K <= 0 || N <= 0) return fail(AQ_ERR_SHAPE, "aq_qmm: M, N, K must be positive");
+    if (int rc = check_geometry("aq_qmm", K, group_size, bits)) return rc;
+    if (!x || !packed || !scales || !biases || !y) return fail(AQ_ERR_ARG, "aq_qmm: null operand");
+    if (!aligned(x, 2) || !aligned(packed, 4) || !aligned(scales, 2) || !aligned(biases, 2) || !aligned(y, 2))
+        return fail(AQ_ERR_ARG, "aq_qmm: operand pointer is not element-aligned");
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    return aq::qmm_dispatch(ctx->stream, ctx->cu_count, ctx->forced[1], &ctx->last_variant[1], x, packed, scales,
+                            biases, y, M, K, N, group_size, bits, (flags & AQ_OUT_F32) != 0, fail);
+}
+
+int aq_gather_qmv(aq_ctx* ctx, const void* x, const void* packed, const void* scales, const void* biases,
+                  const int32_t* lhs, const int32_t* rhs, void* y, int routes, int x_rows, int K, int N,
+                  int num_experts, int expert_rows, int row_base, int group_size, int bits, unsigned flags) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_gather_qmv: ctx is null");
+    if (routes < 0 || K < 0 || N < 0) return fail(AQ_ERR_SHAPE, "aq_gather_qmv: routes, K, N must be non-negative");
+    if (routes == 0 || N == 0 || K == 0) return AQ_OK;  // qmv_gather.go:422-424
+    if (num_experts <= 0 || expert_rows <= 0 || x_rows <= 0)
+        return fail(AQ_ERR_SHAPE, "aq_gather_qmv: num_experts, expert_rows and x_rows must be positive");
+    if (row_base < 0 || (int64_t)row_base + N > expert_rows)
+        return fail(AQ_ERR_SHAPE, "aq_gather_qmv: rows [%d, %d) fall outside an expert slab of %d rows", row_base,
+                    row_base + N, expert_rows);
+    if (int rc = check_geometry("aq_gather_qmv", K, group_size, bits)) return rc;
+    if (!x || !packed || !scales || !biases || !rhs || !y) return fail(AQ_ERR_ARG, "aq_gather_qmv: null operand");
+    if (!aligned(x, 2) || !aligned(packed, 4) || !aligned(scales, 2) || !aligned(biases, 2) || !aligned(y, 2) ||
+        !aligned(rhs, 4) || (lhs && !aligned(lhs, 4)))
+        return fail(AQ_ERR_ARG, "aq_gather_qmv: operand pointer is not element-aligned");
+    if (routes > 65535) return fail(AQ_ERR_UNSUPPORTED, "aq_gather_qmv: at most 65535 routes per call");
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    aq::QmvArgs a{};
+    a.x = static_cast<const uint16_t*>(x);
+    a.w = static_cast<const uint32_t*>(packed);
+    a.s = static_cast<const uint16_t*>(scales);
+    a.b = static_cast<const uint16_t*>(biases);
+    a.y = y;
+    a.lhs = lhs;
+    a.rhs = rhs;
+    a.K = K;
+    a.N = N;
+    a.M = 1;
+    a.out_f32 = (flags & AQ_OUT_F32) ? 1 : 0;
+    a.num_experts = num_experts;
+    a.expert_rows = expert_rows;
+    a.row_base = row_base;
+    a.x_rows = x_rows;
+    a.routes = routes;
+    // every expert slab must keep 16-byte row alignment for the dot2 kernels
+    return launch_qmv_rows(ctx, a, group_size, bits, true);
+}
+
+int aq_dequant_f32(aq_ctx* ctx, const void* packed, const void* scales, const void* biases, float* out_f32, int64_t N,
+                   int K, int group_size, int bits) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_dequant_f32: ctx is null");
+    // mlxaffine.go:182-184: non-positive dims are invalid for the dequantizer.
+    if (N <= 0 || K <= 0 || group_size <= 0 || K % group_size != 0)
+        return fail(AQ_ERR_SHAPE, "aq_dequant_f32: invalid dimensions");
+    if (!(bits == 1 || width_ok(bits))) return fail(AQ_ERR_UNSUPPORTED, "aq_dequant_f32: unsupported bits %d", bits);
+    if (((int64_t)K * bits) % 32 != 0) return fail(AQ_ERR_SHAPE, "aq_dequant_f32: cols*bits must be divisible by 32");
+    if (!packed || !scales || !biases || !out_f32) return fail(AQ_ERR_ARG, "aq_dequant_f32: null operand");
+    if (N * (int64_t)K / 8 > 0x7fffffffLL * 32) return fail(AQ_ERR_UNSUPPORTED, "aq_dequant_f32: tensor too large");
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    AQ_HIP(aq::dequant_launch(static_cast<const uint32_t*>(packed), static_cast<const uint16_t*>(scales),
+                              static_cast<const uint16_t*>(biases), out_f32, N, K, group_size, bits, ctx->stream),
+           "hipLaunchKernel");
+    return AQ_OK;
+}
+
+namespace {
+// Scoped device allocations for the host-slice entry points.
+struct DevBuf {
+    void* p = nullptr;
+    ~DevBuf() {
+        if (p) (void)hipFree(p);
+    }
+    hipError_t alloc(size_t n) { return hipMalloc(&p, n ? n : 1); }
+};
+}  // namespace
+
+int aq_matvec_host(aq_ctx* ctx, const uint8_t* x, size_t x_len, const uint8_t* packed, size_t packed_len,
+                   const uint8_t* scales, size_t scales_len, const uint8_t* biases, size_t biases_len, int out_dim,
+                   int in_dim, int group_size, int bits, uint8_t* out, size_t out_len) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_matvec_host: ctx is null");
+    // Order and conditions of enginetest.ReferenceAffineMatVec (quant_reference.go:79-106).
+    if (out_dim < 0 || in_dim < 0) return fail(AQ_ERR_SHAPE, "aq_matvec_host: outDim/inDim must be non-negative");
+    if (out_dim == 0 || in_dim == 0) return AQ_OK;
+    if (bits <= 0 || bits > 8) return fail(AQ_ERR_UNSUPPORTED, "aq_matvec_host: bits must be in 1..8");
+    if (group_size <= 0 || in_dim % group_size != 0)
+        return fail(AQ_ERR_SHAPE, "aq_matvec_host: groupSize must be > 0 and divide inDim");
+    if (((int64_t)in_dim * bits) % 8 != 0) return fail(AQ_ERR_SHAPE, "aq_matvec_host: inDim*bits must be byte-aligned");
+    if (x_len != (size_t)in_dim * 2) return fail(AQ_ERR_SIZE, "aq_matvec_host: len(x) must equal inDim bf16 bytes");
+    const size_t row_packed = (size_t)in_dim * bits / 8;
+    const size_t row_sb = (size_t)(in_dim / group_size) * 2;
+    if (packed_len != (size_t)out_dim * row_packed || scales_len != (size_t)out_dim * row_sb ||
+        biases_len != (size_t)out_dim * row_sb)
+        return fail(AQ_ERR_SIZE, "aq_matvec_host: packed/scales/biases size mismatch");
+    if (out_len < (size_t)out_dim * 2) return fail(AQ_ERR_SIZE, "aq_matvec_host: out holds fewer than outDim bf16 values");
+    if (!x || !packed || !scales || !biases || !out) return fail(AQ_ERR_ARG, "aq_matvec_host: null operand");
+    if (int rc = check_geometry("aq_matvec_host", in_dim, group_size, bits)) return rc;
+    DevBuf dx, dw, ds, db, dy;
+    AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    AQ_HIP(dx.alloc(x_len), "hipMalloc");
+    AQ_HIP(dw.alloc(packed_len), "hipMalloc");
+    AQ_HIP(ds.alloc(scales_len), "hipMalloc");
+    AQ_HIP(db.alloc(biases_len), "hipMalloc");
+    AQ_HIP(dy.alloc((size_t)out_dim * 2), "hipMalloc");
+    if (int rc = aq_h2d(ctx, dx.p, x, x_len)) return rc;
+    if (int rc = aq_h2d(ctx, dw.p, packed, packed_len)) return rc;
+    if (int rc = aq_h2d(ctx, ds.p, scales, scales_len)) return rc;
+    if (int rc = aq_h2d(ctx, db.p, biases, biases_len)) return rc;
+    if (int rc = aq_qmv(ctx, dx.p, dw.p, ds.p, db.p, dy.p, 1, in_dim, out_dim, group_size, bits, 0)) return rc;
+    return aq_d2h(ctx, out, dy.p, (size_t)out_dim * 2);
+}
+
+int aq_proj_quant_matmul_host(aq_ctx* ctx, float* out, const float* x, size_t x_len, const uint8_t* packed,
+                              size_t packed_len, const uint8_t* scales, size_t scales_len, const uint8_t* biases,
+                              size_t biases_len, int M, int K, int N, int group_size, int bits) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_proj_quant_matmul_host: ctx is null");
+    // quant_seam_backend.go:41-49
+    if (M <= 0 || N <= 0 || K <= 0) return fail(AQ_ERR_SHAPE, "aq_proj_quant_matmul_host: M, N, K must be positive");
+    if (x_len != (size_t)M * K) return fail(AQ_ERR_SIZE, "aq_proj_quant_matmul_host: len(x) must equal M*K");
+    if (group_size <= 0 || bits <= 0 || K % group_size != 0)
+        return fail(AQ_ERR_SHAPE, "aq_proj_quant_matmul_host: invalid quant geometry");
+    if (int rc = check_geometry("aq_proj_quant_matmul_host", K, group_size, bits)) return rc;
+    const size_t want_packed = (size_t)N * ((size_t)K * bits / 32) * 4;
+    const size_t want_sb = (size_t)N * (K / group_size) * 2;
+    if (packed_len != want_packed || scales_len != want_sb || biases_len != want_sb)
+        return fail(AQ_ERR_SIZE, "aq_proj_quant_matmul_host: packed/scales/biases size mismatch");
+    if (!out || !x || !packed || !scales || !biases) return fail(AQ_ERR_ARG, "aq_proj_quant_matmul_host: null operand");
+    // f32 -> bf16 RNE at the seam (quant_seam_backend.go:50,66-74; codec mlxaffine.go:229-237)
+    std::vector<uint16_t> xb((size_t)M * K);
+    for (size_t i = 0; i < xb.size(); i++) {
+        uint32_t u;
+        memcpy(&u, &x[i], 4);
+        if ((u & 0x7fffffffu) > 0x7f800000u) {
+            xb[i] = (uint16_t)((u >> 16) | 0x0040u);
+        } else {
+            u += 0x7fffu + ((u >> 16) & 1u);
+            xb[i] = (uint16_t)(u >> 16);
+        }
+    }
+    DevBuf dx, dw, ds, db, dy;
+    AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    AQ_HIP(dx.alloc(xb.size() * 2), "hipMalloc");
+    AQ_HIP(dw.alloc(packed_len), "hipMalloc");
+    AQ_HIP(ds.alloc(scales_len), "hipMalloc");
+    AQ_HIP(db.alloc(biases_len), "hipMalloc");
+    AQ_HIP(dy.alloc((size_t)M * N * 2), "hipMalloc");
+    if (int rc = aq_h2d(ctx, dx.p, xb.data(), xb.size() * 2)) return rc;
+    if (int rc = aq_h2d(ctx, dw.p, packed, packed_len)) return rc;
+    if (int rc = aq_h2d(ctx, ds.p, scales, scales_len)) return rc;
+    if (int rc = aq_h2d(ctx, db.p, biases, biases_len)) return rc;
+    int rc = (M == 1) ? aq_qmv(ctx, dx.p, dw.p, ds.p, db.p, dy.p, 1, K, N, group_size, bits, 0)
+                      : aq_qmm(ctx, dx.p, dw.p, ds.p, db.p, dy.p, M, K, N, group_size, bits, 0);
+    if (rc) return rc;
+    std::vector<uint16_t> yb((size_t)M * N);
+    if (int rc2 = aq_d2h(ctx, yb.data(), dy.p, yb.size() * 2)) return rc2;
+    for (size_t i = 0; i < yb.size(); i++) {
+        uint32_t u = (uint32_t)yb[i] << 16;
+        memcpy(&out[i], &u, 4);
+    }
+    return AQ_OK;
+}
+
+int aq_variant_count(int op) {
+    if (op == 0) return aq::qmv_variant_count();
+    if (op == 1) return aq::qmm_variant_count();
+    return 0;
+}
+
+const char* aq_variant_name(int op, int variant) {
+    if (op == 0) {
+        const aq::QmvVariant* v = aq::qmv_variant(variant);
+        return v ? v->name : "";
+    }
+    if (op == 1) return aq::qmm_variant_name(variant);
+    return "";
+}
+
+int aq_force_variant(aq_ctx* ctx, int op, int variant) {
+    if (!ctx || op < 0 || op > 1) return fail(AQ_ERR_ARG, "aq_force_variant: bad argument");
+    if (variant >= aq_variant_count(op)) return fail(AQ_ERR_ARG, "aq_force_variant: variant %d out of range", variant);
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    ctx->forced[op] = variant < 0 ? -1 : variant;
+    return AQ_OK;
+}
+
+const char* aq_last_variant(aq_ctx* ctx, int op) {
+    if (!ctx || op < 0 || op > 1) return "";
+    return ctx->last_variant[op];
+}
+
+}  // extern "C"

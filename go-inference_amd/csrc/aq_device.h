@@ -1,0 +1,88 @@
+// Device-side helpers shared by the gfx950 affine kernels: bf16 codecs that
+// match the reference's integer RNE codec bit for bit, the packed-code ->
+// bf16-pair unpackers, and a 64-lane DPP sum.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace aq {
+
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+constexpr int kWave = 64;
+
+// bf16 -> f32 is a 16-bit left shift (go/model/quant/mlxaffine/mlxaffine.go:239-241).
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+
+// f32 -> bf16, round-to-nearest-even on the kept LSB, NaN forced quiet: the
+// same integer recipe as go/model/quant/mlxaffine/mlxaffine.go:229-237, so a
+// store of the same fp32 value gives the same 16 bits as the CPU path.
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+// (a & mask) | magic in one VALU op.  gfx9 VOP3 cannot carry 32-bit literals,
+// so the mask rides in an SGPR and the magic in a VGPR; written as asm because
+// the compiler otherwise picks two literal-carrying VOP2 ops.
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask_s, uint32_t magic_v) {
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(mask_s), "v"(magic_v));
+    return r;
+}
+
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float acc) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), acc,
+                                           false);
+}
+
+// One packed word of eight 4-bit codes c0..c7 -> four bf16 pairs
+//   p[i] = (128 + c_i, 128 + c_{i+4})        (low half, high half)
+// 0x4300 is bf16 128.0, whose mantissa LSB weighs exactly 1, so OR-ing a
+// nibble into the low mantissa bits gives 128 + code with no rounding.  The
+// matching activation order is (x_i, x_{i+4}); the 128 offset is removed by
+// the caller through the chunk's activation sum.
+constexpr uint32_t kNibbleMask = 0x000F000Fu;
+constexpr uint32_t kMagic128 = 0x43004300u;
+constexpr float kNibbleOffset = 128.0f;
+
+__device__ __forceinline__ void unpack4_word(uint32_t w, uint32_t mask_s, uint32_t magic_v, uint32_t p[4]) {
+    p[0] = and_or(w, mask_s, magic_v);
+    p[1] = and_or(w >> 4, mask_s, magic_v);
+    p[2] = and_or(w >> 8, mask_s, magic_v);
+    p[3] = and_or(w >> 12, mask_s, magic_v);
+}
+
+// One packed word of four 8-bit codes c0..c3 -> two bf16 pairs (c0,c1),(c2,c3).
+// Codes <= 255 have 8 significant bits, so float(code) has a zero low half
+// and taking the high halves is an exact bf16 conversion.
+__device__ __forceinline__ void unpack8_word(uint32_t w, uint32_t p[2]) {
+    uint32_t f0 = __float_as_uint((float)(w & 0xffu));
+    uint32_t f1 = __float_as_uint((float)((w >> 8) & 0xffu));
+    uint32_t f2 = __float_as_uint((float)((w >> 16) & 0xffu));
+    uint32_t f3 = __float_as_uint((float)(w >> 24));
+    p[0] = __builtin_amdgcn_perm(f1, f0, 0x07060302u);
+    p[1] = __builtin_amdgcn_perm(f3, f2, 0x07060302u);
+}
+
+// Sum over the 64 lanes of a wavefront; every lane returns the total.
+// Four DPP adds fold each 16-lane row, then the four row totals are read
+// through SGPRs.
+__device__ __forceinline__ float wave_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));
+    float a = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+    float b = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+    float c = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+    float d = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+    return (a + b) + (c + d);
+}
+
+}  // namespace aq

@@ -1,0 +1,59 @@
+// Launch-side declarations shared between the kernel translation units and the
+// C-ABI layer.  Plain structs and ints only; nothing here touches the public
+// header's types.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace aq {
+
+// Operands of one affine matvec / gathered matvec launch.  Layouts follow the
+// MLX group-affine format (go/model/quant/mlxaffine/mlxaffine.go:14-20):
+//   w [rows, K*bits/32] u32, s/b [rows, K/group] bf16, x [x_rows, K] bf16.
+struct QmvArgs {
+    const uint16_t* x;
+    const uint32_t* w;
+    const uint16_t* s;
+    const uint16_t* b;
+    void* y;             // [M, N] (plain) or [routes, N] (gather); bf16 or f32
+    const int32_t* lhs;  // gather only: route -> x row, nullptr = row 0 for all
+    const int32_t* rhs;  // gather only: route -> expert id
+    int K;
+    int N;
+    int M;            // activation rows (plain); 1 for gather
+    int gs_shift;     // log2(group size)
+    int out_f32;      // 0: bf16 stores, 1: f32 stores
+    int num_experts;  // gather only
+    int expert_rows;  // gather only: rows per expert in the slab
+    int row_base;     // gather only: first row of the slab used
+    int x_rows;       // gather only: rows in x (bounds for lhs)
+    int routes;       // gather only
+};
+
+struct QmvVariant {
+    const char* name;
+    int bits;
+    int m;       // activation rows handled per pass (1..4)
+    int rows;    // output rows per wavefront
+    int waves;   // wavefronts per workgroup
+    int depth;   // K slices in flight per wavefront
+    int gather;  // 1: reads rhs/lhs on device, grid.y = routes
+};
+
+int qmv_variant_count();
+const QmvVariant* qmv_variant(int idx);
+// Launch variant `idx` (from the table) on `stream`.  Shapes must already be
+// validated by the caller.
+hipError_t qmv_launch(int idx, const QmvArgs& a, hipStream_t stream);
+// LDS bytes variant idx needs for these args (x staging).
+size_t qmv_lds_bytes(int idx, const QmvArgs& a);
+
+// Any-width (2..8 bit, codes may straddle words), any-group fallback.
+hipError_t qmv_generic_launch(const QmvArgs& a, int bits, int group_size, bool gather, hipStream_t stream);
+
+// fp32 dequantisation of a whole tensor, bits in {1,2,4,8} (word-clean widths)
+// or {3,5,6} through the straddling path.
+hipError_t dequant_launch(const uint32_t* w, const uint16_t* s, const uint16_t* b, float* out, int64_t N, int K,
+                          int group_size, int bits, hipStream_t stream);
+
+}  // namespace aq

@@ -1,0 +1,174 @@
+// fp32 dequantisation and the any-width fallback matvec.
+//
+// dequant: mlxaffine.DequantizeTensor (go/model/quant/mlxaffine/mlxaffine.go:178-208),
+// out = scale * float(code) + bias in fp32.  scale*code is exact in fp32 (8-bit
+// significand times <= 8-bit integer), so the single rounding of the add makes
+// the result independent of whether the multiply-add is fused: the output is
+// bit-identical to the CPU path.
+//
+// generic qmv: the arithmetic of hipReferenceMLXAffineProjection
+// (go/engine/hip/hip_projection_reference.go:92-116, unpack :200-222) for
+// widths the tuned kernels do not cover (2,3,5,6 bit; groups other than
+// 32/64/128), one wavefront per output row.
+#include "aq_device.h"
+#include "aq_kernels.h"
+
+namespace aq {
+
+// Code `col` of a packed row, any width 1..8, codes may cross a word boundary.
+__device__ __forceinline__ uint32_t extract_code(const uint32_t* row, int64_t words, int64_t col, int bits) {
+    const int64_t bit = col * bits;
+    const int64_t wi = bit >> 5;
+    const unsigned sh = (unsigned)(bit & 31);
+    uint32_t v = row[wi] >> sh;
+    if (sh + (unsigned)bits > 32u && wi + 1 < words) v |= row[wi + 1] << (32u - sh);
+    return v & ((1u << bits) - 1u);
+}
+
+// Word-clean widths: one thread expands one packed word (32/bits codes).
+template <int BITS>
+__global__ __launch_bounds__(256) void dequant_words_kernel(const uint32_t* __restrict__ w,
+                                                            const uint16_t* __restrict__ s,
+                                                            const uint16_t* __restrict__ b, float* __restrict__ out,
+                                                            int64_t total_words, int words_per_row, int group_size) {
+    constexpr int PER = 32 / BITS;
+    const int64_t wi = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (wi >= total_words) return;
+    const int64_t row = wi / words_per_row;
+    const int wcol = (int)(wi - row * words_per_row);
+    const int k0 = wcol * PER;
+    const int groups_per_row = (words_per_row * PER) / group_size;
+    const uint32_t word = w[wi];
+    float* o = out + wi * PER;
+    // a word never straddles a group when group_size % PER == 0; otherwise look up per code
+    if (group_size % PER == 0) {
+        const int64_t gi = row * groups_per_row + k0 / group_size;
+        const float sc = bf16_bits_to_f32(s[gi]);
+        const float bi = bf16_bits_to_f32(b[gi]);
+#pragma unroll
+        for (int p = 0; p < PER; p++) {
+            const float code = (float)((word >> (p * BITS)) & ((1u << BITS) - 1u));
+            o[p] = __fmaf_rn(sc, code, bi);
+        }
+    } else {
+#pragma unroll
+        for (int p = 0; p < PER; p++) {
+            const int64_t gi = row * groups_per_row + (k0 + p) / group_size;
+            const float code = (float)((word >> (p * BITS)) & ((1u << BITS) - 1u));
+            o[p] = __fmaf_rn(bf16_bits_to_f32(s[gi]), code, bf16_bits_to_f32(b[gi]));
+        }
+    }
+}
+
+// Straddling widths: one thread per element.
+__global__ __launch_bounds__(256) void dequant_any_kernel(const uint32_t* __restrict__ w,
+                                                          const uint16_t* __restrict__ s,
+                                                          const uint16_t* __restrict__ b, float* __restrict__ out,
+                                                          int64_t N, int K, int group_size, int bits) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= N * K) return;
+    const int64_t row = i / K;
+    const int col = (int)(i - row * K);
+    const int64_t words = (int64_t)K * bits / 32;
+    const float code = (float)extract_code(w + row * words, words, col, bits);
+    const int64_t gi = row * (K / group_size) + col / group_size;
+    out[i] = __fmaf_rn(bf16_bits_to_f32(s[gi]), code, bf16_bits_to_f32(b[gi]));
+}
+
+hipError_t dequant_launch(const uint32_t* w, const uint16_t* s, const uint16_t* b, float* out, int64_t N, int K,
+                          int group_size, int bits, hipStream_t stream) {
+    const int words_per_row = (int)((int64_t)K * bits / 32);
+    const int64_t total_words = N * words_per_row;
+    const unsigned grid_w = (unsigned)((total_words + 255) / 256);
+    switch (bits) {
+        case 1:
+            hipLaunchKernelGGL(dequant_words_kernel<1>, dim3(grid_w), dim3(256), 0, stream, w, s, b, out,
+                               total_words, words_per_row, group_size);
+            break;
+        case 2:
+            hipLaunchKernelGGL(dequant_words_kernel<2>, dim3(grid_w), dim3(256), 0, stream, w, s, b, out,
+                               total_words, words_per_row, group_size);
+            break;
+        case 4:
+            hipLaunchKernelGGL(dequant_words_kernel<4>, dim3(grid_w), dim3(256), 0, stream, w, s, b, out,
+                               total_words, words_per_row, group_size);
+            break;
+        case 8:
+            hipLaunchKernelGGL(dequant_words_kernel<8>, dim3(grid_w), dim3(256), 0, stream, w, s, b, out,
+                               total_words, words_per_row, group_size);
+            break;
+        default: {
+            const unsigned grid_e = (unsigned)((N * K + 255) / 256);
+            hipLaunchKernelGGL(dequant_any_kernel, dim3(grid_e), dim3(256), 0, stream, w, s, b, out, N, K,
+                               group_size, bits);
+        }
+    }
+    return hipGetLastError();
+}
+
+// One wavefront per (row, activation-row block of up to 4).  fp32 weight
+// (scale*code + bias, exact product) times bf16 x widened to fp32, fp32 sums.
+__global__ __launch_bounds__(256) void qmv_generic_kernel(const QmvArgs a, int bits, int group_size, int gather) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int row = blockIdx.x * 4 + wave;
+    const int K = a.K, N = a.N;
+    if (row >= N) return;
+    const int64_t words = (int64_t)K * bits / 32;
+    const int gpr = K / group_size;
+    const uint32_t* wbase = a.w;
+    const uint16_t* sbase = a.s;
+    const uint16_t* bbase = a.b;
+    const uint16_t* xbase = a.x;
+    int64_t yoff = 0;
+    int m_count = a.M;
+    bool ok = true;
+    if (gather) {
+        const int z = blockIdx.y;
+        const int e = a.rhs[z];
+        int xr = a.lhs ? a.lhs[z] : 0;
+        ok = (unsigned)e < (unsigned)a.num_experts && (unsigned)xr < (unsigned)a.x_rows;
+        const int64_t row0 = ok ? ((int64_t)e * a.expert_rows + a.row_base) : 0;
+        if (!ok) xr = 0;
+        wbase += row0 * words;
+        sbase += row0 * gpr;
+        bbase += row0 * gpr;
+        xbase += (int64_t)xr * K;
+        yoff = (int64_t)z * N;
+        m_count = 1;
+    }
+    const uint32_t* wr = wbase + (int64_t)row * words;
+    for (int m0 = 0; m0 < m_count; m0 += 4) {
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int k = lane; k < K; k += kWave) {
+            const float code = (float)extract_code(wr, words, k, bits);
+            const int64_t gi = (int64_t)row * gpr + k / group_size;
+            const float wv = __fmaf_rn(bf16_bits_to_f32(sbase[gi]), code, bf16_bits_to_f32(bbase[gi]));
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                if (m0 + j < m_count) acc[j] = __fmaf_rn(wv, bf16_bits_to_f32(xbase[(int64_t)(m0 + j) * K + k]), acc[j]);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            float tot = wave_sum(acc[j]);
+            if (!ok) tot = 0.0f;
+            if (lane == 0 && m0 + j < m_count) {
+                const int64_t o = yoff + (int64_t)(m0 + j) * N + row;
+                if (a.out_f32) {
+                    reinterpret_cast<float*>(a.y)[o] = tot;
+                } else {
+                    reinterpret_cast<uint16_t*>(a.y)[o] = f32_to_bf16_bits(tot);
+                }
+            }
+        }
+    }
+}
+
+hipError_t qmv_generic_launch(const QmvArgs& a, int bits, int group_size, bool gather, hipStream_t stream) {
+    dim3 grid((unsigned)((a.N + 3) / 4), gather ? (unsigned)a.routes : 1u, 1u);
+    hipLaunchKernelGGL(qmv_generic_kernel, grid, dim3(256), 0, stream, a, bits, group_size, gather ? 1 : 0);
+    return hipGetLastError();
+}
+
+}  // namespace aq

@@ -1,0 +1,44 @@
+// MFMA matmul path (affine_qmm and the M > 4 rows of affine_qmv).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace aq {
+
+// Largest M the dot2 matvec kernels take in one pass; above it aq_qmv hands
+// the call to the MFMA kernels.
+constexpr int kQmvMaxRows = 4;
+
+struct QmmArgs {
+    const uint16_t* x;  // [M, K] bf16
+    const uint32_t* w;  // [N, K*bits/32]
+    const uint16_t* s;  // [N, K/group]
+    const uint16_t* b;  // [N, K/group]
+    void* y;            // [M, N] bf16 or f32
+    int M, K, N;
+    int gs_blocks;  // 64-code blocks per quantisation group (1 for group 64, 2 for 128)
+    int out_f32;
+};
+
+struct QmmVariant {
+    const char* name;
+    int bits;
+    int mb, nb;  // 32x32 MFMA blocks per wavefront along M and N
+    int wm, wn;  // wavefronts per workgroup along M and N
+};
+
+int qmm_variant_count();
+const char* qmm_variant_name(int idx);
+const QmmVariant* qmm_variant(int idx);
+hipError_t qmm_launch(int idx, const QmmArgs& a, hipStream_t stream);
+hipError_t fill_zero_launch(void* p, size_t bytes, hipStream_t stream);
+
+typedef int (*FailFn)(int code, const char* fmt, ...);
+
+// Validated-shape dispatch used by aq_qmm and by aq_qmv for M > kQmvMaxRows.
+// Returns an AQ_* / hipError_t code through `fail`.
+int qmm_dispatch(hipStream_t stream, int cu_count, int forced, const char** last_variant, const void* x,
+                 const void* packed, const void* scales, const void* biases, void* y, int M, int K, int N,
+                 int group_size, int bits, bool out_f32, FailFn fail);
+
+}  // namespace aq

@@ -1,0 +1,147 @@
+/*
+ * aq_mi355.h -- C ABI of libaq_mi355.so: MLX group-affine quantized matvec /
+ * matmul / expert-gathered matvec for AMD MI355X (gfx950).
+ *
+ * This is the boundary a go-inference backend binds (cgo or dlopen) in place
+ * of its own HIP module + launch-packet path.  Every entry point names the
+ * reference interface it stands in for (paths relative to the go-inference
+ * checkout).  Plain pointers and sizes only.
+ *
+ * Tensor layout (go/model/quant/mlxaffine/mlxaffine.go:14-20):
+ *   packed  uint32 little-endian [N, K*bits/32]; code p of a word occupies bits
+ *           [p*bits, p*bits+bits), LSB first, along K
+ *   scales  bf16 [N, K/group]     biases  bf16 [N, K/group]
+ *   w[n,k] = scale[n,k/group] * code[n,k] + bias[n,k/group]
+ * Activations and results are bf16 row-major unless AQ_OUT_F32 is given.
+ *
+ * Return value: 0 = ok; < 0 = argument rejected on the host before any launch
+ * (AQ_ERR_*), > 0 = a hipError_t from the runtime.  aq_last_error() describes
+ * the last failure of the calling thread.  The reference reports the same
+ * conditions as Go errors ("HIP returned <rc>", go/engine/hip/hip_driver_cgo.go:1728-1730;
+ * shape errors, go/engine/hip/hip_projection_reference.go:122-144).
+ *
+ * Threading: calls on one aq_ctx are serialised by an internal mutex; kernels
+ * are enqueued on the context's stream and are asynchronous with respect to
+ * the host unless the entry point says otherwise.
+ */
+#ifndef AQ_MI355_H
+#define AQ_MI355_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AQ_OK 0
+#define AQ_ERR_ARG (-1)         /* null pointer, negative size, misaligned pointer       */
+#define AQ_ERR_SHAPE (-2)       /* dims do not describe a valid affine tensor            */
+#define AQ_ERR_UNSUPPORTED (-3) /* valid, but no kernel for this width / group           */
+#define AQ_ERR_INDEX (-4)       /* expert / row index out of range (host-visible ids)    */
+#define AQ_ERR_NOMEM (-5)       /* host allocation failed                                */
+#define AQ_ERR_NODEVICE (-6)    /* no usable gfx950 device                               */
+#define AQ_ERR_SIZE (-7)        /* a host buffer length disagrees with the dims          */
+
+#define AQ_OUT_F32 0x1u /* y is float32 instead of bf16 (validation of the fp32 accumulator) */
+
+typedef struct aq_ctx aq_ctx;
+
+/* Library / error plumbing.  No reference counterpart beyond core.E strings. */
+const char *aq_version(void);
+const char *aq_last_error(void);
+
+/* Context: device selection, one stream, timing events.
+ * Replaces hipRuntime/cgoHIPDriver set-up (go/engine/hip/hip_runtime.go:21-50,
+ * go/engine/hip/hip_driver_cgo.go:1667-1726: hipSetDevice, module load, function cache). */
+int aq_create(int device, aq_ctx **out);
+void aq_destroy(aq_ctx *ctx);
+/* Enqueue on a caller-owned hipStream_t instead of the context's own stream
+ * (pass NULL for the legacy default stream the reference launches on,
+ * go/engine/hip/hip_driver_cgo.go:452-478).  aq_use_own_stream() goes back. */
+int aq_use_stream(aq_ctx *ctx, void *hip_stream);
+int aq_use_own_stream(aq_ctx *ctx);
+int aq_device_name(aq_ctx *ctx, char *buf, size_t buf_len);
+
+/* Device memory: nativeHIPDriver.Malloc / Free / CopyHostToDevice / CopyDeviceToHost
+ * (go/engine/hip/hip_runtime.go:23-30).  Pointers are ordinary HIP device
+ * pointers and may equally come from the caller's own hipMalloc. */
+int aq_malloc(aq_ctx *ctx, size_t bytes, void **dptr);
+int aq_free(aq_ctx *ctx, void *dptr);
+int aq_h2d(aq_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);  /* synchronous */
+int aq_d2h(aq_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);  /* synchronous */
+int aq_d2d(aq_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes);   /* stream-ordered */
+int aq_fill_zero(aq_ctx *ctx, void *dptr, size_t bytes);                     /* stream-ordered */
+int aq_sync(aq_ctx *ctx);                                                    /* DeviceSynchronize, hip_launch.go:393-407 */
+
+/* hipEvent pair on the context's stream: the per-kernel timing the reference
+ * takes with a device synchronise per launch (go/engine/hip/hip_decode_route_metrics.go:17-52). */
+int aq_timer_start(aq_ctx *ctx);
+int aq_timer_stop(aq_ctx *ctx, float *elapsed_ms); /* records, waits, reports */
+
+/* affine_qmv: y[M,N] = x[M,K] . dequant(w[N,K])^T, all operands device-resident.
+ * Stands in for rocm_mlx_q4_projection / _batch launches
+ * (go/engine/hip/hip_projection_launch.go:1306-1406, 2671-2720, 4907-5287) with the bf16
+ * semantics of MLX affine_qmv (go/engine/metal/qmv.go:354-421) and the M-row
+ * form (go/engine/metal/qmv_rows.go:14-60).  M >= 1; rows of x are contiguous.
+ * N == 0 or K == 0 is a no-op returning AQ_OK (qmv.go:365-371). */
+int aq_qmv(aq_ctx *ctx, const void *x, const void *packed, const void *scales, const void *biases, void *y, int M,
+           int K, int N, int group_size, int bits, unsigned flags);
+
+/* affine_qmm: same contract as aq_qmv, tuned for prefill-sized M
+ * (go/engine/metal/quant_seam_backend.go:77-109 qmmTBF16Into; reference HIP
+ * batch kernels go/engine/hip/kernels/quant/affine_projection_tuned.hipinc:166-1109).
+ * Every element of y[M,N] is written, ragged N included. */
+int aq_qmm(aq_ctx *ctx, const void *x, const void *packed, const void *scales, const void *biases, void *y, int M,
+           int K, int N, int group_size, int bits, unsigned flags);
+
+/* gather_qmv: for each route z, y[z,:N] = x[lhs[z] or 0, :K] . dequant(W_e)^T with
+ * e = rhs[z] read ON DEVICE; W_e = rows [row_base, row_base+N) of expert e's slab.
+ *   packed [num_experts, expert_rows, K*bits/32], scales/biases [num_experts, expert_rows, K/group]
+ *   lhs, rhs: device int32[routes]; lhs may be NULL (every route reads x row 0)
+ * Semantics: go/engine/metal/kernels/moe/lthn_gather_qmv.metal:54-66,
+ * go/engine/metal/qmv_gather.go:295-313; replaces the host-grouped
+ * rocm_moe_mlx_affine_routes path (go/engine/hip/hip_gemma4_moe.go:294-446).
+ * A route whose expert id or x row is out of range yields zeros (the host
+ * cannot see device ids; the by-index helper of qmv_gather.go:405-409 checks
+ * on the host instead). */
+int aq_gather_qmv(aq_ctx *ctx, const void *x, const void *packed, const void *scales, const void *biases,
+                  const int32_t *lhs, const int32_t *rhs, void *y, int routes, int x_rows, int K, int N,
+                  int num_experts, int expert_rows, int row_base, int group_size, int bits, unsigned flags);
+
+/* mlxaffine.DequantizeTensor on device (go/model/quant/mlxaffine/mlxaffine.go:178-208):
+ * out_f32[N,K] = scale*code + bias, bit-exact with the CPU path. */
+int aq_dequant_f32(aq_ctx *ctx, const void *packed, const void *scales, const void *biases, float *out_f32, int64_t N,
+                   int K, int group_size, int bits);
+
+/* model.QuantMatVec.MatVec with HOST byte slices (go/model/quant.go:35-38): uploads,
+ * runs aq_qmv with M = 1, downloads out_dim*2 bf16 bytes into out, synchronous.
+ * Lengths are checked like enginetest.ReferenceAffineMatVec checks them
+ * (go/engine/enginetest/quant_reference.go:78-106); out_dim == 0 or in_dim == 0
+ * returns AQ_OK and writes nothing. */
+int aq_matvec_host(aq_ctx *ctx, const uint8_t *x, size_t x_len, const uint8_t *packed, size_t packed_len,
+                   const uint8_t *scales, size_t scales_len, const uint8_t *biases, size_t biases_len, int out_dim,
+                   int in_dim, int group_size, int bits, uint8_t *out, size_t out_len);
+
+/* attn.ProjQuantMatMulInto with HOST slices (go/model/attn/gated_delta.go:46-58), behaviour of
+ * native.MatMulQuantF32NTInto (go/engine/metal/quant_seam_backend.go:37-75): x f32 [M,K] is
+ * rounded to bf16 (RNE), M == 1 runs qmv and M > 1 qmm, the bf16 result is widened
+ * into out f32 [M,N].  Synchronous. */
+int aq_proj_quant_matmul_host(aq_ctx *ctx, float *out, const float *x, size_t x_len, const uint8_t *packed,
+                              size_t packed_len, const uint8_t *scales, size_t scales_len, const uint8_t *biases,
+                              size_t biases_len, int M, int K, int N, int group_size, int bits);
+
+/* Kernel-variant introspection and override, for tuning sweeps and profiles.
+ * op: 0 = qmv/gather (dot2 kernels), 1 = qmm (MFMA kernels).  variant -1 restores automatic
+ * selection (the counterpart of the reference's shape->kernel selector tables,
+ * go/engine/hip/hip_projection_launch.go:4925-5064 and its GO_ROCM_* route switches :107-137). */
+int aq_variant_count(int op);
+const char *aq_variant_name(int op, int variant);
+int aq_force_variant(aq_ctx *ctx, int op, int variant);
+/* Name of the kernel variant the last launch of `op` on this context used. */
+const char *aq_last_variant(aq_ctx *ctx, int op);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

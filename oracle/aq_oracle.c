@@ -1,0 +1,429 @@
+/*
+ * aq_oracle.c -- CPU restatement of the reference's MLX group-affine path.
+ * TEST INFRASTRUCTURE ONLY (see aq_oracle.h).  Plain C, scalar loops, one
+ * function per reference function; the file:line each follows is in the header
+ * and repeated above each body.
+ */
+#include "aq_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+/* ---- bf16 codecs ------------------------------------------------------- */
+
+/* mlxaffine.go:229-237 / quant_reference.go:27-34 */
+uint16_t orc_f32_to_bf16(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) { /* NaN stays NaN: force a quiet bit */
+        return (uint16_t)((u >> 16) | 0x0040u);
+    }
+    u += 0x7fffu + ((u >> 16) & 1u); /* ties to even on the kept LSB */
+    return (uint16_t)(u >> 16);
+}
+
+/* mlxaffine.go:239-241 / quant_reference.go:22-24 */
+float orc_bf16_to_f32(uint16_t h) {
+    uint32_t u = (uint32_t)h << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+static inline uint16_t ld_u16(const uint8_t *p) { return (uint16_t)(p[0] | ((uint16_t)p[1] << 8)); }
+static inline uint32_t ld_u32(const uint8_t *p) {
+    return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
+}
+static inline void st_u16(uint8_t *p, uint16_t v) {
+    p[0] = (uint8_t)v;
+    p[1] = (uint8_t)(v >> 8);
+}
+static inline void st_u32(uint8_t *p, uint32_t v) {
+    p[0] = (uint8_t)v;
+    p[1] = (uint8_t)(v >> 8);
+    p[2] = (uint8_t)(v >> 16);
+    p[3] = (uint8_t)(v >> 24);
+}
+
+/* ---- code extraction ---------------------------------------------------- */
+
+/* quant_reference.go:36-52: gather `bits` bits starting at bit_off, LSB first,
+ * walking bytes. */
+uint32_t orc_extract_code(const uint8_t *row, int64_t bit_off, int bits) {
+    uint32_t v = 0;
+    int got = 0;
+    while (got < bits) {
+        int64_t pos = bit_off + got;
+        int in_byte = (int)(pos & 7);
+        int take = 8 - in_byte;
+        if (take > bits - got) take = bits - got;
+        uint32_t piece = ((uint32_t)row[pos >> 3] >> in_byte) & ((1u << take) - 1u);
+        v |= piece << got;
+        got += take;
+    }
+    return v;
+}
+
+/* quant_reference.go:54-68 */
+void orc_set_code(uint8_t *row, int64_t bit_off, int bits, uint32_t code) {
+    int got = 0;
+    while (got < bits) {
+        int64_t pos = bit_off + got;
+        int in_byte = (int)(pos & 7);
+        int take = 8 - in_byte;
+        if (take > bits - got) take = bits - got;
+        uint8_t mask = (uint8_t)(((1u << take) - 1u) << in_byte);
+        uint8_t val = (uint8_t)(((code >> got) << in_byte) & mask);
+        row[pos >> 3] = (uint8_t)((row[pos >> 3] & (uint8_t)~mask) | val);
+        got += take;
+    }
+}
+
+/* hip_projection_reference.go:200-222: word-granular extraction, a code whose
+ * field runs past bit 31 takes its high part from the next word. */
+int orc_unpack_word_value(const uint32_t *row_words, int64_t n_words, int col, int bits, uint32_t *code) {
+    if (bits == 0) bits = 4;
+    if (bits != 4 && bits != 6 && bits != 8) return ORC_ERR_BITS;
+    if (col < 0) return ORC_ERR_DIMS;
+    uint64_t bit = (uint64_t)col * (uint64_t)bits;
+    int64_t wi = (int64_t)(bit / 32);
+    unsigned sh = (unsigned)(bit % 32);
+    if (wi >= n_words) return ORC_ERR_SIZE;
+    uint32_t v = row_words[wi] >> sh;
+    if (sh + (unsigned)bits > 32) {
+        if (wi + 1 >= n_words) return ORC_ERR_SIZE;
+        v |= row_words[wi + 1] << (32 - sh);
+    }
+    *code = v & ((1u << bits) - 1u);
+    return ORC_OK;
+}
+
+/* ---- dequantize --------------------------------------------------------- */
+
+static int width_is_word_clean(int bits) { return bits == 1 || bits == 2 || bits == 4 || bits == 8; }
+
+/* mlxaffine.go:178-208.  fp32: out = scale * float(code) + bias, one element
+ * at a time.  Built with -ffp-contract=off: mul then add (scale*code is exact
+ * in fp32 for bf16 scales and <=8-bit codes, so a fused form agrees anyway). */
+int orc_dequantize(const uint8_t *packed, size_t packed_len, const uint8_t *scales, size_t scales_len,
+                   const uint8_t *biases, size_t biases_len, int out_dim, int in_dim, int bits, int group_size,
+                   float *out) {
+    if (!width_is_word_clean(bits)) return ORC_ERR_BITS;
+    if (out_dim <= 0 || in_dim <= 0 || group_size <= 0 || in_dim % group_size != 0) return ORC_ERR_DIMS;
+    int per_word = 32 / bits;
+    size_t words_per_row = (size_t)in_dim * (size_t)bits / 32;
+    size_t groups_per_row = (size_t)(in_dim / group_size);
+    if (packed_len != (size_t)out_dim * words_per_row * 4) return ORC_ERR_SIZE;
+    if (scales_len != (size_t)out_dim * groups_per_row * 2 || biases_len != scales_len) return ORC_ERR_SIZE;
+    uint32_t mask = (1u << bits) - 1u;
+    for (int r = 0; r < out_dim; r++) {
+        for (int j = 0; j < in_dim; j++) {
+            size_t wi = (size_t)r * words_per_row + (size_t)(j / per_word);
+            unsigned sh = (unsigned)(j % per_word) * (unsigned)bits;
+            uint32_t code = (ld_u32(packed + wi * 4) >> sh) & mask;
+            size_t gi = ((size_t)r * groups_per_row + (size_t)(j / group_size)) * 2;
+            float scale = orc_bf16_to_f32(ld_u16(scales + gi));
+            float bias = orc_bf16_to_f32(ld_u16(biases + gi));
+            float prod = scale * (float)code;
+            out[(size_t)r * (size_t)in_dim + (size_t)j] = prod + bias;
+        }
+    }
+    return ORC_OK;
+}
+
+/* ---- quantize (fixture builder) ---------------------------------------- */
+
+static float round_half_away(float v) { return (float)round((double)v); } /* mlxaffine.go:210-213 */
+
+/* mlxaffine.go:131-162 (affineGroup): anchor the larger-magnitude edge to an
+ * exact code, sign the scale by which edge dominates, re-derive scale = edge/q0. */
+static void affine_group(const float *g, int n, float n_bins, float *scale_out, float *bias_out) {
+    float lo = g[0], hi = g[0];
+    for (int i = 1; i < n; i++) {
+        if (g[i] < lo) lo = g[i];
+        if (g[i] > hi) hi = g[i];
+    }
+    float scale = (hi - lo) / n_bins;
+    if (scale < 1e-7f) scale = 1e-7f;
+    float edge = hi;
+    if (fabsf(lo) > fabsf(hi)) {
+        edge = lo;
+    } else {
+        scale = -scale;
+    }
+    float q0 = round_half_away(edge / scale);
+    if (q0 == 0.0f) {
+        *scale_out = scale;
+        *bias_out = 0.0f;
+        return;
+    }
+    *scale_out = edge / q0;
+    *bias_out = edge;
+}
+
+/* mlxaffine.go:80-129 with quantiseCode :164-174.  Codes are derived from the
+ * UNROUNDED fp32 scale/bias; the bf16 rounding only affects what is stored. */
+int orc_quantize(const float *values, size_t n_values, int out_dim, int in_dim, int bits, int group_size,
+                 uint8_t *packed, uint8_t *scales, uint8_t *biases) {
+    if (!width_is_word_clean(bits)) return ORC_ERR_BITS;
+    if (out_dim <= 0 || in_dim <= 0) return ORC_ERR_DIMS;
+    if (group_size <= 0 || in_dim % group_size != 0) return ORC_ERR_DIMS;
+    int per_word = 32 / bits;
+    if (group_size % per_word != 0) return ORC_ERR_DIMS;
+    if (n_values != (size_t)out_dim * (size_t)in_dim) return ORC_ERR_SIZE;
+    size_t words_per_row = (size_t)in_dim * (size_t)bits / 32;
+    int words_per_group = group_size / per_word;
+    int groups_per_row = in_dim / group_size;
+    float n_bins = (float)((1 << bits) - 1);
+    for (int r = 0; r < out_dim; r++) {
+        for (int g = 0; g < groups_per_row; g++) {
+            const float *grp = values + (size_t)r * (size_t)in_dim + (size_t)g * (size_t)group_size;
+            float scale, bias;
+            affine_group(grp, group_size, n_bins, &scale, &bias);
+            size_t sbi = ((size_t)r * (size_t)groups_per_row + (size_t)g) * 2;
+            st_u16(scales + sbi, orc_f32_to_bf16(scale));
+            st_u16(biases + sbi, orc_f32_to_bf16(bias));
+            for (int wg = 0; wg < words_per_group; wg++) {
+                uint32_t word = 0;
+                for (int p = 0; p < per_word; p++) {
+                    float q = round_half_away((grp[wg * per_word + p] - bias) / scale);
+                    if (q < 0.0f) {
+                        q = 0.0f;
+                    } else if (q > n_bins) {
+                        q = n_bins;
+                    }
+                    word |= (uint32_t)q << ((unsigned)p * (unsigned)bits);
+                }
+                size_t wi = (size_t)r * words_per_row + (size_t)g * (size_t)words_per_group + (size_t)wg;
+                st_u32(packed + wi * 4, word);
+            }
+        }
+    }
+    return ORC_OK;
+}
+
+/* repack.go:27-62 (codes only; scales/biases are carried through unchanged by
+ * the caller). */
+int orc_repack_b1_to_b2(const uint8_t *packed, size_t packed_len, int out_dim, int in_dim, uint8_t *packed2) {
+    if (out_dim <= 0 || in_dim <= 0) return ORC_ERR_DIMS;
+    if (in_dim % 32 != 0) return ORC_ERR_DIMS;
+    size_t w1 = (size_t)in_dim / 32, w2 = (size_t)in_dim / 16;
+    if (packed_len != (size_t)out_dim * w1 * 4) return ORC_ERR_SIZE;
+    memset(packed2, 0, (size_t)out_dim * w2 * 4);
+    for (int r = 0; r < out_dim; r++) {
+        for (int j = 0; j < in_dim; j++) {
+            uint32_t src = ld_u32(packed + ((size_t)r * w1 + (size_t)(j / 32)) * 4);
+            uint32_t code = (src >> (unsigned)(j % 32)) & 1u;
+            if (!code) continue;
+            uint8_t *dst = packed2 + ((size_t)r * w2 + (size_t)(j / 16)) * 4;
+            st_u32(dst, ld_u32(dst) | (code << ((unsigned)(j % 16) * 2)));
+        }
+    }
+    return ORC_OK;
+}
+
+/* ---- the reference's CPU qmv / qmm -------------------------------------- */
+
+/* gated_delta.go:63-89.  A row of K fp32 weights is materialised by the
+ * dequantizer above, then dotted against each activation row in float64,
+ * ascending k; the float64 sum is narrowed to float32 on store. */
+int orc_matnt_quant_host(float *out, const float *x, const uint8_t *packed, const uint8_t *scales,
+                         const uint8_t *biases, int M, int K, int N, int group_size, int bits, int threads) {
+    if (!width_is_word_clean(bits)) return ORC_ERR_BITS;
+    if (M <= 0 || K <= 0 || N <= 0 || group_size <= 0 || K % group_size != 0) return ORC_ERR_DIMS;
+    size_t row_bytes = (size_t)K * (size_t)bits / 32 * 4;
+    size_t sb_bytes = (size_t)(K / group_size) * 2;
+    int bad = 0;
+#ifdef _OPENMP
+    if (threads < 1) threads = 1;
+#pragma omp parallel num_threads(threads)
+#endif
+    {
+        float *wrow = (float *)malloc((size_t)K * sizeof(float));
+#ifdef _OPENMP
+#pragma omp for schedule(static)
+#endif
+        for (int n = 0; n < N; n++) {
+            if (!wrow || orc_dequantize(packed + (size_t)n * row_bytes, row_bytes, scales + (size_t)n * sb_bytes,
+                                        sb_bytes, biases + (size_t)n * sb_bytes, sb_bytes, 1, K, bits, group_size,
+                                        wrow) != ORC_OK) {
+#ifdef _OPENMP
+#pragma omp atomic write
+#endif
+                bad = 1;
+                continue;
+            }
+            for (int m = 0; m < M; m++) {
+                const float *xr = x + (size_t)m * (size_t)K;
+                double acc = 0.0;
+                for (int k = 0; k < K; k++) {
+                    acc += (double)xr[k] * (double)wrow[k];
+                }
+                out[(size_t)m * (size_t)N + (size_t)n] = (float)acc;
+            }
+        }
+        free(wrow);
+    }
+    (void)threads;
+    return bad ? ORC_ERR_SIZE : ORC_OK;
+}
+
+/* quant_reference.go:78-127 */
+int orc_reference_affine_matvec(const uint8_t *x, size_t x_len, const uint8_t *packed, size_t packed_len,
+                                const uint8_t *scales, size_t scales_len, const uint8_t *biases, size_t biases_len,
+                                int out_dim, int in_dim, int group_size, int bits, uint8_t *out) {
+    if (out_dim < 0 || in_dim < 0) return ORC_ERR_DIMS;
+    if (out_dim == 0 || in_dim == 0) {
+        if (out && out_dim > 0) memset(out, 0, (size_t)out_dim * 2);
+        return ORC_OK;
+    }
+    if (bits <= 0 || bits > 8) return ORC_ERR_BITS;
+    if (group_size <= 0 || in_dim % group_size != 0) return ORC_ERR_DIMS;
+    if (((int64_t)in_dim * bits) % 8 != 0) return ORC_ERR_DIMS;
+    if (x_len != (size_t)in_dim * 2) return ORC_ERR_SIZE;
+    size_t row_packed = (size_t)in_dim * (size_t)bits / 8;
+    size_t row_sb = (size_t)(in_dim / group_size) * 2;
+    if (packed_len != (size_t)out_dim * row_packed || scales_len != (size_t)out_dim * row_sb ||
+        biases_len != (size_t)out_dim * row_sb) {
+        return ORC_ERR_SIZE;
+    }
+    double *xf = (double *)malloc((size_t)in_dim * sizeof(double));
+    if (!xf) return ORC_ERR_SIZE;
+    for (int i = 0; i < in_dim; i++) xf[i] = (double)orc_bf16_to_f32(ld_u16(x + (size_t)i * 2));
+    for (int r = 0; r < out_dim; r++) {
+        const uint8_t *prow = packed + (size_t)r * row_packed;
+        const uint8_t *srow = scales + (size_t)r * row_sb;
+        const uint8_t *brow = biases + (size_t)r * row_sb;
+        double acc = 0.0;
+        for (int c = 0; c < in_dim; c++) {
+            int g = c / group_size;
+            double scale = (double)orc_bf16_to_f32(ld_u16(srow + (size_t)g * 2));
+            double bias = (double)orc_bf16_to_f32(ld_u16(brow + (size_t)g * 2));
+            double code = (double)orc_extract_code(prow, (int64_t)c * bits, bits);
+            double w = scale * code + bias;
+            acc += w * xf[c];
+        }
+        st_u16(out + (size_t)r * 2, orc_f32_to_bf16((float)acc));
+    }
+    free(xf);
+    return ORC_OK;
+}
+
+/* hip_projection_reference.go:122-144 + :161-178 */
+static int projection_shape_ok(size_t input_len, size_t weight_len, size_t scale_len, size_t bias_len, int rows,
+                               int cols, int group_size, int bits, size_t *words_per_row) {
+    if (rows <= 0 || cols <= 0 || group_size <= 0) return ORC_ERR_DIMS;
+    if (bits != 4 && bits != 6 && bits != 8) return ORC_ERR_BITS;
+    uint64_t total_bits = (uint64_t)cols * (uint64_t)bits;
+    if (total_bits % 32 != 0) return ORC_ERR_DIMS;
+    *words_per_row = (size_t)(total_bits / 32);
+    if (cols % group_size != 0) return ORC_ERR_DIMS;
+    if (input_len != (size_t)cols) return ORC_ERR_SIZE;
+    if (weight_len != (size_t)rows * *words_per_row) return ORC_ERR_SIZE;
+    size_t groups = (size_t)rows * (size_t)(cols / group_size);
+    if (scale_len != groups || bias_len != groups) return ORC_ERR_SIZE;
+    return ORC_OK;
+}
+
+/* hip_projection_reference.go:92-116: everything in float32, weight formed as
+ * float(q)*scale + bias, then sum += input*weight in ascending column order. */
+int orc_hip_reference_projection(const float *input, size_t input_len, const uint32_t *weights, size_t weight_len,
+                                 const uint16_t *scales, size_t scale_len, const uint16_t *biases, size_t bias_len,
+                                 int rows, int cols, int group_size, int bits, float *output) {
+    if (bits == 0) bits = 4;
+    size_t wpr = 0;
+    int rc = projection_shape_ok(input_len, weight_len, scale_len, bias_len, rows, cols, group_size, bits, &wpr);
+    if (rc != ORC_OK) return rc;
+    int groups_per_row = cols / group_size;
+    for (int row = 0; row < rows; row++) {
+        float sum = 0.0f;
+        for (int col = 0; col < cols; col++) {
+            uint32_t q = 0;
+            rc = orc_unpack_word_value(weights + (size_t)row * wpr, (int64_t)wpr, col, bits, &q);
+            if (rc != ORC_OK) return rc;
+            size_t g = (size_t)row * (size_t)groups_per_row + (size_t)(col / group_size);
+            float qs = (float)q * orc_bf16_to_f32(scales[g]);
+            float weight = qs + orc_bf16_to_f32(biases[g]);
+            float term = input[col] * weight;
+            sum = sum + term;
+        }
+        output[row] = sum;
+    }
+    return ORC_OK;
+}
+
+int orc_hip_reference_projection_batch(const float *input, int tokens, const uint32_t *weights,
+                                       const uint16_t *scales, const uint16_t *biases, int rows, int cols,
+                                       int group_size, int bits, float *output) {
+    if (tokens <= 0) return ORC_ERR_DIMS;
+    if (bits == 0) bits = 4;
+    if (rows <= 0 || cols <= 0 || group_size <= 0 || cols % group_size != 0) return ORC_ERR_DIMS;
+    if (((uint64_t)cols * (uint64_t)bits) % 32 != 0) return ORC_ERR_DIMS;
+    size_t wpr = (size_t)cols * (size_t)bits / 32;
+    size_t groups = (size_t)rows * (size_t)(cols / group_size);
+    for (int m = 0; m < tokens; m++) {
+        int rc = orc_hip_reference_projection(input + (size_t)m * (size_t)cols, (size_t)cols, weights,
+                                              (size_t)rows * wpr, scales, groups, biases, groups, rows, cols,
+                                              group_size, bits, output + (size_t)m * (size_t)rows);
+        if (rc != ORC_OK) return rc;
+    }
+    return ORC_OK;
+}
+
+/* ---- expert-gathered matvec -------------------------------------------- */
+
+/* lthn_gather_qmv.metal:54-66: w += rhs[z]*expert_rows*K*bits/32 words,
+ * scales/biases += rhs[z]*expert_rows*(K/group), x += lhs[z]*K (batched x),
+ * y += z*N; the row_base byte offsets of qmv_gather.go:295-313 select a
+ * sub-slab of rows.  Range check: qmv_gather.go:405-409. */
+int orc_gather_qmv(const uint16_t *x, int x_rows, const uint32_t *packed, const uint16_t *scales,
+                   const uint16_t *biases, const int32_t *lhs, const int32_t *rhs, int routes, int num_experts,
+                   int expert_rows, int row_base, int N, int K, int group_size, int bits, double *out_f64,
+                   uint16_t *out_bf16) {
+    if (routes < 0 || num_experts <= 0 || expert_rows <= 0 || N < 0 || K < 0 || x_rows <= 0) return ORC_ERR_DIMS;
+    if (routes == 0 || N == 0 || K == 0) return ORC_OK;
+    if (bits <= 0 || bits > 8) return ORC_ERR_BITS;
+    if (group_size <= 0 || K % group_size != 0) return ORC_ERR_DIMS;
+    if (((int64_t)K * bits) % 32 != 0) return ORC_ERR_DIMS;
+    if (row_base < 0 || row_base + N > expert_rows) return ORC_ERR_DIMS;
+    size_t wpr = (size_t)K * (size_t)bits / 32;
+    size_t gpr = (size_t)(K / group_size);
+    for (int z = 0; z < routes; z++) {
+        if (rhs[z] < 0 || rhs[z] >= num_experts) return ORC_ERR_INDEX;
+        if (lhs && (lhs[z] < 0 || lhs[z] >= x_rows)) return ORC_ERR_INDEX;
+    }
+    for (int z = 0; z < routes; z++) {
+        size_t e = (size_t)rhs[z];
+        const uint16_t *xr = x + (lhs ? (size_t)lhs[z] * (size_t)K : 0);
+        for (int n = 0; n < N; n++) {
+            size_t row = e * (size_t)expert_rows + (size_t)row_base + (size_t)n;
+            const uint8_t *prow = (const uint8_t *)(packed + row * wpr);
+            const uint16_t *srow = scales + row * gpr;
+            const uint16_t *brow = biases + row * gpr;
+            double acc = 0.0;
+            for (int c = 0; c < K; c++) {
+                int g = c / group_size;
+                double w = (double)orc_bf16_to_f32(srow[g]) * (double)orc_extract_code(prow, (int64_t)c * bits, bits) +
+                           (double)orc_bf16_to_f32(brow[g]);
+                acc += w * (double)orc_bf16_to_f32(xr[c]);
+            }
+            size_t o = (size_t)z * (size_t)N + (size_t)n;
+            if (out_f64) out_f64[o] = acc;
+            if (out_bf16) out_bf16[o] = orc_f32_to_bf16((float)acc);
+        }
+    }
+    return ORC_OK;
+}
+
+int orc_max_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}

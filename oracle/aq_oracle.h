@@ -1,0 +1,120 @@
+/*
+ * aq_oracle.h -- CPU restatement of go-inference's MLX group-affine quantized
+ * dequant / matvec / matmul / gather path.
+ *
+ * THIS IS TEST INFRASTRUCTURE.  It is the checker the GPU kernels are compared
+ * against and the CPU baseline the benchmark times.  Nothing the product ships
+ * may call, link or import it: only tests/, the smoke check and the benchmark's
+ * cpu_baseline leg load liborc.so.
+ *
+ * Every function names the reference file:line whose arithmetic it restates
+ * (paths relative to the go-inference checkout).  Build: `make -C oracle`
+ * (gcc, -ffp-contract=off so no multiply-add is fused behind the algorithm's
+ * back).
+ *
+ * Layout used everywhere (go/model/quant/mlxaffine/mlxaffine.go:14-20):
+ *   packed  uint32 little-endian [N, K*bits/32]; code p of a word sits at bits
+ *           [p*bits, p*bits+bits), LSB first, along K
+ *   scales  bf16 [N, K/group]      biases  bf16 [N, K/group]
+ *   w[n,k] = scale[n,k/group] * code[n,k] + bias[n,k/group]
+ *
+ * Return value of every int function: 0 = ok, negative = rejected argument
+ * (the reference returns a Go error in the same situations).
+ */
+#ifndef AQ_ORACLE_H
+#define AQ_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ORC_OK 0
+#define ORC_ERR_BITS (-1)  /* unsupported code width            */
+#define ORC_ERR_DIMS (-2)  /* non-positive / non-dividing dims  */
+#define ORC_ERR_SIZE (-3)  /* a buffer length disagrees         */
+#define ORC_ERR_INDEX (-4) /* expert / row index out of range   */
+
+/* bf16 codecs: mlxaffine.go:229-241, quant_reference.go:22-34,
+ * hip_bf16_portable.go:12-23.  Round-to-nearest-even, NaN -> quiet NaN. */
+uint16_t orc_f32_to_bf16(float f);
+float orc_bf16_to_f32(uint16_t h);
+
+/* LSB-first code extraction over a bit-contiguous byte row, any width 1..8,
+ * codes may straddle bytes: quant_reference.go:36-52 (affineExtractCode). */
+uint32_t orc_extract_code(const uint8_t *row, int64_t bit_off, int bits);
+/* inverse, used to build fixtures: quant_reference.go:54-68 (affineSetCode). */
+void orc_set_code(uint8_t *row, int64_t bit_off, int bits, uint32_t code);
+
+/* uint32-word code extraction incl. codes that cross a word boundary (6-bit):
+ * hip_projection_reference.go:200-222 (hipMLXAffineUnpackValue). */
+int orc_unpack_word_value(const uint32_t *row_words, int64_t n_words, int col, int bits, uint32_t *code);
+
+/* mlxaffine.DequantizeTensor, mlxaffine.go:178-208.  bits in {1,2,4,8}.
+ * packed_len / sb_len are byte lengths and are checked exactly as the
+ * reference checks its slices.  out holds out_dim*in_dim float32. */
+int orc_dequantize(const uint8_t *packed, size_t packed_len, const uint8_t *scales, size_t scales_len,
+                   const uint8_t *biases, size_t biases_len, int out_dim, int in_dim, int bits, int group_size,
+                   float *out);
+
+/* mlxaffine.QuantizeTensor, mlxaffine.go:80-176 (affineGroup edge anchoring,
+ * round-half-away codes).  Only used to build realistic fixtures. */
+int orc_quantize(const float *values, size_t n_values, int out_dim, int in_dim, int bits, int group_size,
+                 uint8_t *packed, uint8_t *scales, uint8_t *biases);
+
+/* mlxaffine.RepackB1ToB2, repack.go:27-62: widen 1-bit codes to 2-bit fields. */
+int orc_repack_b1_to_b2(const uint8_t *packed, size_t packed_len, int out_dim, int in_dim, uint8_t *packed2);
+
+/* attn.matNTQuantHost, gated_delta.go:63-89: the reference's CPU qmv/qmm.
+ * Per output row n: fp32 dequant of the row, then for each activation row m an
+ * ascending-k float64 dot, stored as float32 at out[m*N+n].
+ * threads <= 1: the single-threaded loop the Go original runs.
+ * threads  > 1: the same loop with output rows shared out over OpenMP threads
+ * (each row's arithmetic is unchanged, so results are bit-identical). */
+int orc_matnt_quant_host(float *out, const float *x, const uint8_t *packed, const uint8_t *scales,
+                         const uint8_t *biases, int M, int K, int N, int group_size, int bits, int threads);
+
+/* enginetest.ReferenceAffineMatVec, quant_reference.go:78-127: bf16 x, weight
+ * formed in float64 (no fp32 rounding of w), float64 accumulate, bf16 result.
+ * Any width 1..8 over bit-contiguous rows.  Zero out_dim/in_dim: ok, nothing
+ * written.  x_len etc. are byte lengths. */
+int orc_reference_affine_matvec(const uint8_t *x, size_t x_len, const uint8_t *packed, size_t packed_len,
+                                const uint8_t *scales, size_t scales_len, const uint8_t *biases, size_t biases_len,
+                                int out_dim, int in_dim, int group_size, int bits, uint8_t *out);
+
+/* hip.hipReferenceMLXAffineProjection, hip_projection_reference.go:92-116 with
+ * the shape validation of :122-144 -- fp32 weight, fp32 ascending-col
+ * accumulate ("the fp32-accumulated reference").  bits in {4,6,8}.  Lengths
+ * are element counts, as in the Go signature. */
+int orc_hip_reference_projection(const float *input, size_t input_len, const uint32_t *weights, size_t weight_len,
+                                 const uint16_t *scales, size_t scale_len, const uint16_t *biases, size_t bias_len,
+                                 int rows, int cols, int group_size, int bits, float *output);
+
+/* Batched form of the same projection as the reference batch kernels are
+ * tested with (hip_kernels_test.go:612-654): out[m*rows + r]. */
+int orc_hip_reference_projection_batch(const float *input, int tokens, const uint32_t *weights,
+                                       const uint16_t *scales, const uint16_t *biases, int rows, int cols,
+                                       int group_size, int bits, float *output);
+
+/* Expert-gathered matvec.  Addressing: lthn_gather_qmv.metal:54-66 (expert
+ * slab offsets from rhs[z], x row from lhs[z] when batched, y row z) and the
+ * range check of qmv_gather.go:401-409.  Arithmetic per route is the fp64
+ * form of orc_reference_affine_matvec; out_f64 (optional) receives the
+ * unrounded sums, out_bf16 (optional) the bf16 stores.
+ *   packed [E, expert_rows, K*bits/32] u32, scales/biases [E, expert_rows, K/group]
+ *   row_base selects rows [row_base, row_base+N) of each expert's slab
+ *   lhs == NULL -> every route reads x row 0 */
+int orc_gather_qmv(const uint16_t *x, int x_rows, const uint32_t *packed, const uint16_t *scales,
+                   const uint16_t *biases, const int32_t *lhs, const int32_t *rhs, int routes, int num_experts,
+                   int expert_rows, int row_base, int N, int K, int group_size, int bits, double *out_f64,
+                   uint16_t *out_bf16);
+
+/* Number of hardware threads OpenMP would use (for reporting). */
+int orc_max_threads(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,175 @@
+"""ctypes binding of oracle/liborc.so -- TEST INFRASTRUCTURE.
+
+Only tests/, the smoke check and the benchmark's cpu_baseline leg import this module;
+the product (go-inference_amd/) never does.  `build()` runs `make -C oracle`.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "liborc.so")
+
+ORC_OK = 0
+ORC_ERR_BITS = -1
+ORC_ERR_DIMS = -2
+ORC_ERR_SIZE = -3
+ORC_ERR_INDEX = -4
+
+_lib = None
+
+
+def build(force=False):
+    if force or not os.path.exists(LIB_PATH):
+        subprocess.run(["make", "-C", _HERE] + (["-B"] if force else []), check=True, stdout=subprocess.PIPE,
+                       stderr=subprocess.STDOUT)
+    return LIB_PATH
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        _lib = ctypes.CDLL(LIB_PATH)
+        _lib.orc_f32_to_bf16.restype = ctypes.c_uint16
+        _lib.orc_f32_to_bf16.argtypes = [ctypes.c_float]
+        _lib.orc_bf16_to_f32.restype = ctypes.c_float
+        _lib.orc_bf16_to_f32.argtypes = [ctypes.c_uint16]
+        _lib.orc_extract_code.restype = ctypes.c_uint32
+        _lib.orc_extract_code.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int]
+        _lib.orc_set_code.restype = None
+        _lib.orc_set_code.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_uint32]
+        _lib.orc_max_threads.restype = ctypes.c_int
+    return _lib
+
+
+def _u8(a):
+    return np.ascontiguousarray(a).view(np.uint8).reshape(-1)
+
+
+def _p(a):
+    return ctypes.c_void_p(a.ctypes.data) if a is not None else None
+
+
+class OracleError(ValueError):
+    def __init__(self, code):
+        super().__init__("oracle rejected the arguments (code %d)" % code)
+        self.code = code
+
+
+def _check(rc):
+    if rc != ORC_OK:
+        raise OracleError(rc)
+
+
+def f32_to_bf16(v):
+    return int(lib().orc_f32_to_bf16(ctypes.c_float(v)))
+
+
+def bf16_to_f32(h):
+    return float(lib().orc_bf16_to_f32(ctypes.c_uint16(h)))
+
+
+def extract_code(row_bytes, bit_off, bits):
+    row_bytes = _u8(row_bytes)
+    return int(lib().orc_extract_code(_p(row_bytes), bit_off, bits))
+
+
+def set_code(row_bytes, bit_off, bits, code):
+    assert row_bytes.dtype == np.uint8 and row_bytes.flags.c_contiguous
+    lib().orc_set_code(_p(row_bytes), bit_off, bits, code)
+
+
+def dequantize(packed, scales, biases, out_dim, in_dim, bits, group_size):
+    packed, scales, biases = _u8(packed), _u8(scales), _u8(biases)
+    out = np.empty(max(out_dim, 0) * max(in_dim, 0), dtype=np.float32)
+    rc = lib().orc_dequantize(_p(packed), ctypes.c_size_t(packed.size), _p(scales), ctypes.c_size_t(scales.size),
+                              _p(biases), ctypes.c_size_t(biases.size), out_dim, in_dim, bits, group_size, _p(out))
+    _check(rc)
+    return out.reshape(out_dim, in_dim)
+
+
+def quantize(values, out_dim, in_dim, bits, group_size):
+    values = np.ascontiguousarray(values, dtype=np.float32).reshape(-1)
+    packed = np.zeros(max(out_dim * in_dim * bits // 8, 1), dtype=np.uint8)
+    sb = max(out_dim * (in_dim // max(group_size, 1)) * 2, 1)
+    scales = np.zeros(sb, dtype=np.uint8)
+    biases = np.zeros(sb, dtype=np.uint8)
+    rc = lib().orc_quantize(_p(values), ctypes.c_size_t(values.size), out_dim, in_dim, bits, group_size, _p(packed),
+                            _p(scales), _p(biases))
+    _check(rc)
+    return packed, scales, biases
+
+
+def repack_b1_to_b2(packed, out_dim, in_dim):
+    packed = _u8(packed)
+    out = np.zeros(max(out_dim * in_dim // 4, 1), dtype=np.uint8)
+    _check(lib().orc_repack_b1_to_b2(_p(packed), ctypes.c_size_t(packed.size), out_dim, in_dim, _p(out)))
+    return out
+
+
+def matnt_quant_host(x_f32, packed, scales, biases, M, K, N, group_size, bits, threads=1):
+    x = np.ascontiguousarray(x_f32, dtype=np.float32).reshape(-1)
+    packed, scales, biases = _u8(packed), _u8(scales), _u8(biases)
+    out = np.zeros(M * N, dtype=np.float32)
+    _check(lib().orc_matnt_quant_host(_p(out), _p(x), _p(packed), _p(scales), _p(biases), M, K, N, group_size, bits,
+                                      threads))
+    return out.reshape(M, N)
+
+
+def reference_affine_matvec(x, packed, scales, biases, out_dim, in_dim, group_size, bits):
+    """bf16 bytes in, bf16 bytes (uint8 array, out_dim*2) out."""
+    x, packed, scales, biases = _u8(x), _u8(packed), _u8(scales), _u8(biases)
+    out = np.zeros(max(out_dim, 0) * 2, dtype=np.uint8)
+    rc = lib().orc_reference_affine_matvec(_p(x), ctypes.c_size_t(x.size), _p(packed), ctypes.c_size_t(packed.size),
+                                           _p(scales), ctypes.c_size_t(scales.size), _p(biases),
+                                           ctypes.c_size_t(biases.size), out_dim, in_dim, group_size, bits, _p(out))
+    _check(rc)
+    return out
+
+
+def hip_reference_projection(x_f32, weights_u32, scales_u16, biases_u16, rows, cols, group_size, bits):
+    x = np.ascontiguousarray(x_f32, dtype=np.float32).reshape(-1)
+    w = np.ascontiguousarray(weights_u32, dtype=np.uint32).reshape(-1)
+    s = np.ascontiguousarray(scales_u16, dtype=np.uint16).reshape(-1)
+    b = np.ascontiguousarray(biases_u16, dtype=np.uint16).reshape(-1)
+    out = np.zeros(max(rows, 0), dtype=np.float32)
+    rc = lib().orc_hip_reference_projection(_p(x), ctypes.c_size_t(x.size), _p(w), ctypes.c_size_t(w.size), _p(s),
+                                            ctypes.c_size_t(s.size), _p(b), ctypes.c_size_t(b.size), rows, cols,
+                                            group_size, bits, _p(out))
+    _check(rc)
+    return out
+
+
+def hip_reference_projection_batch(x_f32, tokens, weights_u32, scales_u16, biases_u16, rows, cols, group_size, bits):
+    x = np.ascontiguousarray(x_f32, dtype=np.float32).reshape(-1)
+    w = np.ascontiguousarray(weights_u32, dtype=np.uint32).reshape(-1)
+    s = np.ascontiguousarray(scales_u16, dtype=np.uint16).reshape(-1)
+    b = np.ascontiguousarray(biases_u16, dtype=np.uint16).reshape(-1)
+    out = np.zeros(tokens * rows, dtype=np.float32)
+    _check(lib().orc_hip_reference_projection_batch(_p(x), tokens, _p(w), _p(s), _p(b), rows, cols, group_size, bits,
+                                                    _p(out)))
+    return out.reshape(tokens, rows)
+
+
+def gather_qmv(x_u16, x_rows, packed_u32, scales_u16, biases_u16, lhs, rhs, routes, num_experts, expert_rows,
+               row_base, N, K, group_size, bits):
+    """Returns (float64 sums [routes,N], bf16 bits [routes,N])."""
+    x = np.ascontiguousarray(x_u16, dtype=np.uint16).reshape(-1)
+    w = np.ascontiguousarray(packed_u32, dtype=np.uint32).reshape(-1)
+    s = np.ascontiguousarray(scales_u16, dtype=np.uint16).reshape(-1)
+    b = np.ascontiguousarray(biases_u16, dtype=np.uint16).reshape(-1)
+    lhs_a = None if lhs is None else np.ascontiguousarray(lhs, dtype=np.int32)
+    rhs_a = np.ascontiguousarray(rhs, dtype=np.int32)
+    o64 = np.zeros(max(routes * N, 1), dtype=np.float64)
+    o16 = np.zeros(max(routes * N, 1), dtype=np.uint16)
+    rc = lib().orc_gather_qmv(_p(x), x_rows, _p(w), _p(s), _p(b), _p(lhs_a), _p(rhs_a), routes, num_experts,
+                              expert_rows, row_base, N, K, group_size, bits, _p(o64), _p(o16))
+    _check(rc)
+    return o64[:routes * N].reshape(routes, N), o16[:routes * N].reshape(routes, N)
+
+
+def max_threads():
+    return int(lib().orc_max_threads())

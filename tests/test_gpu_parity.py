@@ -1,0 +1,381 @@
+"""GPU parity: the HIP path, called through the C ABI, against the CPU oracle and the
+reference's fixtures.  Bar: dequantised weights bit-exact; fp32 accumulators within
+max-abs-err 1e-2 and rel-err 2e-3 of the fp32-weight reference; bf16 stores within one bf16
+ulp of bf16(reference)."""
+import numpy as np
+import pytest
+
+import fixtures as F
+from gpu_util import DeviceAffine, check_accumulators, check_bf16_store, run_qmv, say
+
+pytestmark = pytest.mark.gpu
+
+
+# ---- dequant: bit exact -----------------------------------------------------------------------
+
+@pytest.mark.parametrize("N,K,bits,gs", [(8, 128, 4, 64), (33, 704, 4, 64), (64, 2048, 4, 64), (7, 256, 8, 32),
+                                         (16, 512, 8, 64), (5, 640, 2, 64), (4, 128, 1, 128), (9, 512, 4, 128),
+                                         (6, 192, 6, 32), (6, 256, 3, 64), (6, 256, 5, 64), (3, 64, 4, 16)])
+def test_dequant_bit_exact(ctx, orc, N, K, bits, gs):
+    say("dequant", N, K, bits, gs)
+    rng = np.random.default_rng(N * 1000 + K + bits)
+    codes = rng.integers(0, 1 << bits, size=(N, K)).astype(np.uint32)
+    words = F.pack_codes(codes, bits)
+    s = rng.integers(0, 65536, size=(N, K // gs)).astype(np.uint16)
+    b = rng.integers(0, 65536, size=(N, K // gs)).astype(np.uint16)
+    # keep scales/biases finite: clear the top exponent bit pattern 0xFF
+    s = np.where((s & 0x7F80) == 0x7F80, s & 0xBFFF, s).astype(np.uint16)
+    b = np.where((b & 0x7F80) == 0x7F80, b & 0xBFFF, b).astype(np.uint16)
+    dw = DeviceAffine(ctx, words, s, b)
+    dout = ctx.alloc(N * K * 4)
+    ctx.dequant_f32(dw.w, dw.s, dw.b, dout, N, K, gs, bits)
+    ctx.sync()
+    got = dout.download(np.uint32, N * K).reshape(N, K)
+    if bits in (1, 2, 4, 8):
+        want = orc.dequantize(words, s, b, N, K, bits, gs).view(np.uint32)
+    else:  # straddling widths are outside DequantizeTensor: same formula over the word unpacker
+        want = F.numpy_dequant(words, s, b, bits, gs, K).view(np.uint32)
+    assert np.array_equal(got, want)
+    dw.free()
+    dout.free()
+
+
+def test_dequant_config0_bit_exact(ctx, orc):
+    say("dequant cfg0 8192x2048")
+    words, s, b = F.synthetic_affine(8192, 2048, 4, 64, seed=F.BASE_SEED)
+    dw = DeviceAffine(ctx, words, s, b)
+    dout = ctx.alloc(8192 * 2048 * 4)
+    ctx.dequant_f32(dw.w, dw.s, dw.b, dout, 8192, 2048, 64, 4)
+    ctx.sync()
+    got = dout.download(np.uint32, 8192 * 2048)
+    want = orc.dequantize(words, s, b, 8192, 2048, 4, 64).view(np.uint32).reshape(-1)
+    assert np.array_equal(got, want)
+    dw.free()
+    dout.free()
+
+
+# ---- qmv --------------------------------------------------------------------------------------
+
+def _qmv_case(ctx, orc, M, K, N, bits, gs, seed, fn="qmv"):
+    words, s, b = F.synthetic_affine(N, K, bits, gs, seed=seed)
+    x = F.synthetic_x(M, K, seed=seed + 1)
+    ref = F.reference_f64(x, words, s, b, bits, gs, K)
+    dw = DeviceAffine(ctx, words, s, b)
+    acc = run_qmv(ctx, x, dw, M, K, N, gs, bits, True, fn)
+    check_accumulators(acc, ref, "%s M=%d K=%d N=%d b=%d g=%d" % (fn, M, K, N, bits, gs))
+    out = run_qmv(ctx, x, dw, M, K, N, gs, bits, False, fn)
+    check_bf16_store(out, ref, "bf16 store")
+    # the bf16 store is the RNE of the same accumulator
+    assert np.array_equal(out, F.f32_to_bf16_bits(acc).reshape(M, N))
+    dw.free()
+    return acc, ref, (words, s, b, x)
+
+
+def test_qmv_config0_vs_oracle(ctx, orc):
+    """cfg 0: M=1, K=2048, N=8192, 4-bit g64 -- also against the reference's own CPU paths."""
+    say("qmv cfg0")
+    acc, ref, (words, s, b, x) = _qmv_case(ctx, orc, 1, 2048, 8192, 4, 64, F.BASE_SEED)
+    xf = F.bf16_bits_to_f32(x).reshape(-1)
+    fp32_ref = orc.hip_reference_projection(xf, words, s, b, 8192, 2048, 64, 4)       # fp32-accumulated
+    host_ref = orc.matnt_quant_host(xf, words, s, b, 1, 2048, 8192, 64, 4).reshape(-1)  # matNTQuantHost
+    check_accumulators(acc, fp32_ref, "vs hipReferenceMLXAffineProjection")
+    check_accumulators(acc, host_ref, "vs matNTQuantHost")
+    bf = orc.reference_affine_matvec(x, words, s, b, 8192, 2048, 64, 4).view(np.uint16)
+    check_bf16_store(F.f32_to_bf16_bits(acc), F.bf16_bits_to_f32(bf).astype(np.float64), "vs ReferenceAffineMatVec")
+
+
+@pytest.mark.parametrize("name,K,N", [("q", 4096, 4096), ("kv", 4096, 1024), ("gate_up", 4096, 14336), ("down", 14336, 4096)])
+def test_qmv_config1_layer_shapes(ctx, orc, name, K, N):
+    say("qmv cfg1", name)
+    _qmv_case(ctx, orc, 1, K, N, 4, 64, F.BASE_SEED + 1)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("M", [2, 3, 4, 8, 16, 32])
+def test_qmv_config2_batched_rows(ctx, orc, bits, M):
+    say("qmv cfg2", bits, M)
+    _qmv_case(ctx, orc, M, 4096, 14336, bits, 64, F.BASE_SEED + 2)
+
+
+@pytest.mark.parametrize("bits,gs,K,N,M", [(4, 64, 2816, 1408, 1), (4, 64, 1408, 2816, 1), (4, 64, 704, 17, 1), (4, 32, 256, 40, 1),
+                                           (4, 128, 512, 24, 1), (8, 64, 512, 40, 1), (8, 32, 3072, 5, 1), (8, 128, 1024, 9, 2),
+                                           (4, 64, 64, 3, 1), (4, 64, 512, 1, 4), (4, 64, 2048 + 64, 70, 3), (8, 64, 64, 2, 1)])
+def test_qmv_ragged_and_thin_shapes(ctx, orc, bits, gs, K, N, M):
+    say("qmv ragged", bits, gs, K, N, M)
+    _qmv_case(ctx, orc, M, K, N, bits, gs, 77 + K + N)
+
+
+@pytest.mark.parametrize("bits,gs,K,N,M", [(2, 64, 640, 9, 1), (3, 64, 256, 9, 1), (5, 64, 256, 9, 2), (6, 32, 192, 11, 1),
+                                           (6, 16, 64, 5, 3), (4, 16, 64, 5, 1), (2, 128, 256, 24, 5)])
+def test_qmv_other_widths_generic_kernel(ctx, orc, bits, gs, K, N, M):
+    say("qmv generic", bits, gs, K, N, M)
+    rng = np.random.default_rng(bits * 100 + K)
+    codes = rng.integers(0, 1 << bits, size=(N, K)).astype(np.uint32)
+    words = F.pack_codes(codes, bits)
+    _, s, b = F.synthetic_affine(N, K, 4, gs, seed=bits)
+    x = F.synthetic_x(M, K, seed=bits + 5)
+    ref = F.reference_f64(x, words, s, b, bits, gs, K)
+    dw = DeviceAffine(ctx, words, s, b)
+    acc = run_qmv(ctx, x, dw, M, K, N, gs, bits, True)
+    check_accumulators(acc, ref, "generic")
+    assert ctx.last_variant(0) == "qmv_generic"
+    dw.free()
+
+
+def test_qmv_every_variant(ctx, orc):
+    """Each tuned dot2 kernel variant, forced, on a shape with a masked K tail and ragged N."""
+    import aq_mi355
+    K, N = 2816, 150
+    names = aq_mi355.variant_names(0)
+    data = {}
+    try:
+        for idx, name in enumerate(names):
+            say("variant", idx, name)
+            parts = dict((p[0], p[1:]) for p in name.split("_")[1:])
+            bits, m, gather = int(parts["b"]), int(parts["m"]), int(parts["g"])
+            if gather:
+                continue
+            if bits not in data:
+                words, s, b = F.synthetic_affine(N, K, bits, 64, seed=500 + bits)
+                x = F.synthetic_x(4, K, seed=600 + bits)
+                data[bits] = (DeviceAffine(ctx, words, s, b), x, F.reference_f64(x, words, s, b, bits, 64, K))
+            dw, x, ref = data[bits]
+            ctx.force_variant(0, idx)
+            acc = run_qmv(ctx, x[:m], dw, m, K, N, 64, bits, True)
+            assert ctx.last_variant(0) == name
+            check_accumulators(acc, ref[:m], name)
+    finally:
+        ctx.force_variant(0, -1)
+    for dw, _, _ in data.values():
+        dw.free()
+
+
+def test_qmv_rows_match_single_row_bytes(ctx, orc):
+    """M-row qmv is byte-identical, row by row, to M single-row calls
+    (the contract of go/engine/metal/qmv_rows_test.go:31-100)."""
+    say("qmv rows == per-row")
+    K, N = 2048, 520
+    words, s, b = F.synthetic_affine(N, K, 4, 64, seed=91)
+    x = F.synthetic_x(4, K, seed=92)
+    dw = DeviceAffine(ctx, words, s, b)
+    for M in (2, 3, 4):
+        both = run_qmv(ctx, x[:M], dw, M, K, N, 64, 4, False)
+        for m in range(M):
+            one = run_qmv(ctx, x[m:m + 1], dw, 1, K, N, 64, 4, False)
+            assert np.array_equal(both[m], one[0]), (M, m)
+    dw.free()
+
+
+def test_concat_rows_is_byte_identical(ctx, orc):
+    """gate||up as one matvec equals the two matvecs (go/model/quant_weight.go:32-44)."""
+    say("concat rows")
+    K = 1024
+    wa, sa, ba = F.synthetic_affine(96, K, 4, 64, seed=31)
+    wb, sb_, bb = F.synthetic_affine(160, K, 4, 64, seed=32)
+    x = F.synthetic_x(1, K, seed=33)
+    da, db = DeviceAffine(ctx, wa, sa, ba), DeviceAffine(ctx, wb, sb_, bb)
+    dc = DeviceAffine(ctx, np.concatenate([wa, wb]), np.concatenate([sa, sb_]), np.concatenate([ba, bb]))
+    ya = run_qmv(ctx, x, da, 1, K, 96, 64, 4, False)
+    yb = run_qmv(ctx, x, db, 1, K, 160, 64, 4, False)
+    yc = run_qmv(ctx, x, dc, 1, K, 256, 64, 4, False)
+    assert np.array_equal(yc[0, :96], ya[0]) and np.array_equal(yc[0, 96:], yb[0])
+    for d in (da, db, dc):
+        d.free()
+
+
+def test_qmv_zero_sized_and_errors(ctx):
+    import aq_mi355
+    say("qmv zero/err")
+    ctx.qmv(None, None, None, None, None, 1, 0, 8, 64, 4)   # K == 0: no-op
+    ctx.qmv(None, None, None, None, None, 1, 64, 0, 64, 4)  # N == 0: no-op
+    buf = ctx.alloc(4096)
+    for kw, code in [(dict(K=64, gs=3), aq_mi355.AQ_ERR_SHAPE), (dict(K=64, bits=0), aq_mi355.AQ_ERR_UNSUPPORTED),
+                     (dict(K=64, bits=9), aq_mi355.AQ_ERR_UNSUPPORTED), (dict(K=7, gs=7), aq_mi355.AQ_ERR_SHAPE),
+                     (dict(K=-1), aq_mi355.AQ_ERR_SHAPE)]:
+        with pytest.raises(aq_mi355.AqError) as e:
+            ctx.qmv(buf, buf, buf, buf, buf, 1, kw.get("K", 64), 4, kw.get("gs", 64), kw.get("bits", 4))
+        assert e.value.code == code, kw
+    with pytest.raises(aq_mi355.AqError) as e:
+        ctx.qmv(None, buf, buf, buf, buf, 1, 64, 4, 64, 4)
+    assert e.value.code == aq_mi355.AQ_ERR_ARG
+    buf.free()
+
+
+# ---- gather_qmv -------------------------------------------------------------------------------
+
+def _gather_run(ctx, fx, routes, E, expert_rows, row_base, N, K, gs, bits, f32):
+    import aq_mi355
+    dx = ctx.to_device(fx["x"])
+    dw = DeviceAffine(ctx, fx["packed"], fx["scales"], fx["biases"])
+    dl = ctx.to_device(fx["lhs"]) if fx["lhs"] is not None else None
+    dr = ctx.to_device(fx["rhs"])
+    dy = ctx.alloc(routes * N * (4 if f32 else 2))
+    ctx.fill_zero(dy)
+    ctx.gather_qmv(dx, dw.w, dw.s, dw.b, dl, dr, dy, routes, fx["x_rows"], K, N, E, expert_rows, row_base, gs, bits,
+                   aq_mi355.AQ_OUT_F32 if f32 else 0)
+    ctx.sync()
+    out = dy.download(np.float32 if f32 else np.uint16, routes * N).reshape(routes, N)
+    for t in (dx, dl, dr, dy):
+        if t is not None:
+            t.free()
+    return out, dw
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4, 5, 6, 8])
+@pytest.mark.parametrize("name,out_dim,in_dim,gs,expert_rows,row_base,batched", [
+    ("fast shared-x", 32, 512, 64, 32, 0, False), ("fast batched-x", 32, 512, 64, 32, 0, True),
+    ("plain shared-x", 24, 256, 32, 24, 0, False), ("fast gate_up rowBase", 32, 512, 64, 64, 32, False)])
+def test_gather_reference_cases(ctx, orc, bits, name, out_dim, in_dim, gs, expert_rows, row_base, batched):
+    """The sweep of go/engine/metal/qmv_gather_test.go:87-129, device vs oracle, and byte-identity with the
+    plain qmv on the expert slice (go/engine/metal/moe_quant_test.go:1143-1185)."""
+    if in_dim * bits % 32:
+        pytest.skip("packed-row alignment")
+    say("gather", bits, name)
+    E, routes = 4, 3
+    fx = F.gather_fixture(out_dim, in_dim, gs, bits, E, expert_rows, batched, routes)
+    ref64, _ = orc.gather_qmv(fx["x"], fx["x_rows"], fx["packed"], fx["scales"], fx["biases"], fx["lhs"], fx["rhs"], routes, E,
+                              expert_rows, row_base, out_dim, in_dim, gs, bits)
+    acc, dw = _gather_run(ctx, fx, routes, E, expert_rows, row_base, out_dim, in_dim, gs, bits, True)
+    # these fixtures have |w| up to ~400 and outputs up to ~1e4: the stated bounds are relative to that scale
+    scale = max(1.0, np.abs(ref64).max())
+    check_accumulators(acc / scale, ref64 / scale, "gather f32")
+    out, dw2 = _gather_run(ctx, fx, routes, E, expert_rows, row_base, out_dim, in_dim, gs, bits, False)
+    assert np.array_equal(out, F.f32_to_bf16_bits(acc).reshape(routes, out_dim))
+    # sliced plain qmv gives the same bytes
+    wpr, gpr = in_dim * bits // 32, in_dim // gs
+    W = fx["packed"].reshape(E, expert_rows, wpr)
+    S = fx["scales"].reshape(E, expert_rows, gpr)
+    B = fx["biases"].reshape(E, expert_rows, gpr)
+    X = fx["x"].reshape(fx["x_rows"], in_dim)
+    for z in range(routes):
+        e = fx["rhs"][z]
+        sl = slice(row_base, row_base + out_dim)
+        ds = DeviceAffine(ctx, W[e, sl], S[e, sl], B[e, sl])
+        xr = X[fx["lhs"][z]] if batched else X[0]
+        one = run_qmv(ctx, xr.reshape(1, -1), ds, 1, in_dim, out_dim, gs, bits, False)
+        assert np.array_equal(one[0], out[z]), (name, z)
+        ds.free()
+    dw.free()
+    dw2.free()
+
+
+def test_gather_config4_shape(ctx, orc):
+    """cfg 4 geometry at a reduced expert count: 8 tokens x top-8 of 16 experts, in-proj [1408 x 2816]
+    with lhs = route -> token, then down [2816 x 1408] with lhs = iota."""
+    rng = np.random.default_rng(F.BASE_SEED + 4)
+    E, tokens, topk = 16, 8, 8
+    routes = tokens * topk
+    ids = np.concatenate([rng.permutation(E)[:topk] for _ in range(tokens)]).astype(np.int32)
+    for (N, K, lhs, x_rows) in [(1408, 2816, np.repeat(np.arange(tokens), topk).astype(np.int32), tokens),
+                                (2816, 1408, np.arange(routes, dtype=np.int32), routes)]:
+        say("gather cfg4", N, K)
+        words, s, b = F.synthetic_affine(E * N, K, 4, 64, seed=F.BASE_SEED + 40 + N)
+        x = F.synthetic_x(x_rows, K, seed=F.BASE_SEED + 41 + N)
+        fx = dict(x=x, x_rows=x_rows, packed=words, scales=s, biases=b, lhs=lhs, rhs=ids)
+        acc, dw = _gather_run(ctx, fx, routes, E, N, 0, N, K, 64, 4, True)
+        wq = F.numpy_dequant(words, s, b, 4, 64, K).astype(np.float64).reshape(E, N, K)
+        xf = F.bf16_bits_to_f32(x).astype(np.float64).reshape(x_rows, K)
+        ref = np.stack([wq[ids[z]] @ xf[lhs[z]] for z in range(routes)])
+        check_accumulators(acc, ref, "gather cfg4")
+        # a subset of routes against the oracle itself
+        sub = [0, 17, 63]
+        r64, _ = orc.gather_qmv(x, x_rows, words, s, b, lhs[sub], ids[sub], len(sub), E, N, 0, N, K, 64, 4)
+        check_accumulators(acc[sub], r64, "gather cfg4 vs oracle")
+        dw.free()
+
+
+def test_gather_out_of_range_ids_give_zeros(ctx):
+    say("gather bad ids")
+    fx = F.gather_fixture(32, 512, 64, 4, 4, 32, False, 3)
+    fx["rhs"] = np.array([1, 9, -2], dtype=np.int32)
+    out, dw = _gather_run(ctx, fx, 3, 4, 32, 0, 32, 512, 64, 4, True)
+    assert np.all(out[1] == 0) and np.all(out[2] == 0) and np.any(out[0] != 0)
+    dw.free()
+
+
+def test_gather_errors(ctx):
+    import aq_mi355
+    buf = ctx.alloc(4096)
+    with pytest.raises(aq_mi355.AqError) as e:
+        ctx.gather_qmv(buf, buf, buf, buf, None, buf, buf, 3, 1, 64, 8, 4, 8, 4, 64, 4)  # row_base+N > expert_rows
+    assert e.value.code == aq_mi355.AQ_ERR_SHAPE
+    ctx.gather_qmv(buf, buf, buf, buf, None, buf, buf, 0, 1, 64, 8, 4, 8, 0, 64, 4)      # zero routes: no-op
+    buf.free()
+
+
+# ---- qmm --------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("M,K,N,bits,gs", [(3, 512, 64, 4, 64), (5, 256, 40, 4, 64), (2, 128, 8, 8, 64), (33, 1024, 130, 4, 64),
+                                           (64, 512, 256, 8, 64), (100, 2816, 96, 4, 64), (17, 704, 17, 4, 64), (40, 1408, 70, 4, 128),
+                                           (130, 320, 33, 8, 128), (256, 1024, 512, 4, 64)])
+def test_qmm_small_cases(ctx, orc, M, K, N, bits, gs):
+    say("qmm", M, K, N, bits, gs)
+    _qmv_case(ctx, orc, M, K, N, bits, gs, 900 + M + N, fn="qmm")
+
+
+def test_qmm_every_variant(ctx, orc):
+    import aq_mi355
+    names = aq_mi355.variant_names(1)
+    M, K, N = 150, 704, 200
+    data = {}
+    try:
+        for idx, name in enumerate(names):
+            say("qmm variant", idx, name)
+            bits = int(name.split("_")[1][1:])
+            if bits not in data:
+                words, s, b = F.synthetic_affine(N, K, bits, 64, seed=700 + bits)
+                x = F.synthetic_x(M, K, seed=800 + bits)
+                data[bits] = (DeviceAffine(ctx, words, s, b), x, F.reference_f64(x, words, s, b, bits, 64, K))
+            dw, x, ref = data[bits]
+            ctx.force_variant(1, idx)
+            acc = run_qmv(ctx, x, dw, M, K, N, 64, bits, True, "qmm")
+            assert ctx.last_variant(1) == name
+            check_accumulators(acc, ref, name)
+    finally:
+        ctx.force_variant(1, -1)
+    for dw, _, _ in data.values():
+        dw.free()
+
+
+def test_qmm_hardware_fixture_q4_g64_tokens16(ctx, orc):
+    """17 x 704 x 16 batch fixture of go/engine/hip/hip_hardware_test.go:7822-7878 (reference tolerance 1e-3)."""
+    say("qmm hw fixture")
+    fx = F.hw_fixture_q4_g64_tokens16()
+    want = orc.hip_reference_projection_batch(fx["x"], fx["tokens"], fx["packed"], fx["scales"], fx["biases"], fx["rows"], fx["cols"], 64, 4)
+    dw = DeviceAffine(ctx, fx["packed"], fx["scales"], fx["biases"])
+    # x = (integer/8) * (t+1)/16 has at most 6 significant bits: exact in bf16
+    xb = F.f32_to_bf16_bits(fx["x"])
+    assert np.array_equal(F.bf16_bits_to_f32(xb).reshape(fx["x"].shape), fx["x"])
+    got = run_qmv(ctx, xb, dw, fx["tokens"], fx["cols"], fx["rows"], 64, 4, True, "qmm")
+    assert np.abs(got - want).max() <= fx["tol"]
+    dw.free()
+
+
+def test_qmm_config3_full_size_sampled_columns(ctx, orc):
+    """cfg 3 at full size (M=2048, K=4096, N=14336): every output of 192 sampled weight rows against the
+    float64 reference, plus linearity in x over the whole output (size-independent)."""
+    say("qmm cfg3 full")
+    M, K, N = 2048, 4096, 14336
+    words, s, b = F.synthetic_affine(N, K, 4, 64, seed=F.BASE_SEED + 3)
+    x = F.synthetic_x(M, K, seed=F.BASE_SEED + 1003)
+    dw = DeviceAffine(ctx, words, s, b)
+    acc = run_qmv(ctx, x, dw, M, K, N, 64, 4, True, "qmm")
+    rng = np.random.default_rng(3)
+    cols = np.sort(rng.choice(N, 192, replace=False))
+    ref = F.reference_f64(x, words[cols], s[cols], b[cols], 4, 64, K)
+    check_accumulators(acc[:, cols], ref, "cfg3 sampled")
+    # y(2x) == 2 y(x) exactly: doubling bf16 inputs doubles every exact product and every fp32 partial sum
+    x2 = F.f32_to_bf16_bits(F.bf16_bits_to_f32(x) * np.float32(2))
+    acc2 = run_qmv(ctx, x2, dw, M, K, N, 64, 4, True, "qmm")
+    assert np.array_equal(acc2, acc * np.float32(2))
+    dw.free()
+
+
+def test_qmm_errors(ctx):
+    import aq_mi355
+    buf = ctx.alloc(4096)
+    for args in [(0, 64, 4, 64, 4), (1, 64, 0, 64, 4), (1, 0, 4, 64, 4)]:
+        with pytest.raises(aq_mi355.AqError) as e:
+            ctx.qmm(buf, buf, buf, buf, buf, *args)
+        assert e.value.code == aq_mi355.AQ_ERR_SHAPE
+    buf.free()

@@ -1,0 +1,365 @@
+"""Pins the CPU oracle (oracle/aq_oracle.c) against the known-answer vectors and fixtures the
+reference's own tests hold, and against what the mathematics fixes.  No GPU."""
+import math
+
+import numpy as np
+import pytest
+
+import fixtures as F
+
+
+# ---- bf16 codecs ---------------------------------------------------------------------------
+
+def test_bf16_round_trip_list(orc):
+    # go/engine/enginetest/quant_reference_test.go:98-110
+    for v in [0, 1, -1, 12.5, 0.25, -3.75, 100, -0.03125]:
+        assert orc.bf16_to_f32(orc.f32_to_bf16(v)) == v
+
+
+def test_bf16_constants(orc):
+    # go/engine/hip/hip_projection_reference_test.go:201-210
+    assert orc.bf16_to_f32(0x3F80) == 1.0
+    assert orc.bf16_to_f32(0xC000) == -2.0
+    assert orc.bf16_to_f32(0x7F80) == math.inf
+    assert math.isnan(orc.bf16_to_f32(0x7FC0))
+    assert orc.f32_to_bf16(12.5) == 0x4148
+
+
+def test_bf16_widen_exhaustive(orc):
+    for h in range(0, 65536, 1):
+        want = np.array([h], dtype=np.uint32) << 16
+        got = np.array([orc.bf16_to_f32(h)], dtype=np.float32).view(np.uint32)
+        if not (math.isnan(orc.bf16_to_f32(h))):
+            assert got[0] == want[0]
+
+
+def test_bf16_rne_ties_and_nan(orc):
+    # 1 + 2^-8 is exactly half way between bf16 1.0 (even) and 1.0078125 (odd): stays 1.0
+    assert orc.f32_to_bf16(1.0 + 2.0 ** -8) == 0x3F80
+    # 1.0078125 + 2^-8 is half way between odd 0x3F81 and even 0x3F82: goes up
+    assert orc.f32_to_bf16(1.0078125 + 2.0 ** -8) == 0x3F82
+    assert orc.f32_to_bf16(1.0 + 2.0 ** -8 + 2.0 ** -20) == 0x3F81
+    assert orc.f32_to_bf16(-(1.0 + 2.0 ** -8)) == 0xBF80
+    assert orc.f32_to_bf16(3.4e38) == 0x7F80  # rounds up into +inf
+    h = orc.f32_to_bf16(float("nan"))
+    assert (h & 0x7F80) == 0x7F80 and (h & 0x007F) != 0
+
+
+def test_bf16_rne_matches_torch(orc):
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(7)
+    vals = np.concatenate([rng.normal(0, 1, 4000), rng.normal(0, 1e-3, 2000), rng.normal(0, 1e4, 2000)]).astype(np.float32)
+    want = torch.from_numpy(vals).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    got = np.array([orc.f32_to_bf16(float(v)) for v in vals], dtype=np.uint16)
+    assert np.array_equal(got, want)
+    assert np.array_equal(F.f32_to_bf16_bits(vals), want)  # the numpy helper the other tests lean on
+
+
+# ---- code packing ---------------------------------------------------------------------------
+
+def test_set_extract_packing_order(orc):
+    # codes [3,5] at 4 bit pack to 0x53 (go/engine/enginetest/quant_reference_test.go:13-21)
+    row = np.zeros(1, dtype=np.uint8)
+    orc.set_code(row, 0, 4, 3)
+    orc.set_code(row, 4, 4, 5)
+    assert row[0] == 0x53
+    # 0x76543210 holds codes 0..7 in column order (go/engine/hip/hip_projection_reference_test.go:71-85)
+    word = np.array([0x76543210], dtype=np.uint32)
+    assert [orc.extract_code(word, 4 * c, 4) for c in range(8)] == list(range(8))
+
+
+@pytest.mark.parametrize("bits", [1, 2, 3, 4, 5, 6, 7, 8])
+def test_set_extract_round_trip_all_widths(orc, bits):
+    rng = np.random.default_rng(bits)
+    k = 64
+    codes = rng.integers(0, 1 << bits, size=k)
+    row = np.zeros(k * bits // 8, dtype=np.uint8)
+    for c, v in enumerate(codes):
+        orc.set_code(row, c * bits, bits, int(v))
+    assert [orc.extract_code(row, c * bits, bits) for c in range(k)] == [int(v) for v in codes]
+    # the byte-walking packer and the word packer used by the fixtures describe the same layout
+    assert np.array_equal(F.pack_codes(codes.reshape(1, -1), bits).view(np.uint8).reshape(-1), row)
+
+
+def test_quant_affine_fixture_round_trips(orc):
+    # go/engine/enginetest/quant_reference_test.go:80-92
+    fx = F.quant_affine_fixture()
+    rows = fx["packed"].view(np.uint8).reshape(fx["out_dim"], -1)
+    for r in range(fx["out_dim"]):
+        for c in range(fx["in_dim"]):
+            assert orc.extract_code(rows[r], c * 4, 4) == (c * 5 + r * 3 + 1) % 16
+
+
+# ---- ReferenceAffineMatVec -------------------------------------------------------------------
+
+def test_reference_affine_matvec_good(orc):
+    # 1x2, scale 2, bias 1, codes [3,5] -> w [7,11]; x [1, 0.5] -> 12.5 exactly (quant_reference_test.go:13-38)
+    packed = np.array([0x53], dtype=np.uint8)
+    s = np.array([orc.f32_to_bf16(2.0)], dtype=np.uint16)
+    b = np.array([orc.f32_to_bf16(1.0)], dtype=np.uint16)
+    x = np.array([orc.f32_to_bf16(1.0), orc.f32_to_bf16(0.5)], dtype=np.uint16)
+    out = orc.reference_affine_matvec(x, packed, s, b, 1, 2, 2, 4)
+    assert out.view(np.uint16)[0] == orc.f32_to_bf16(12.5)
+
+
+def test_reference_affine_matvec_bad(orc):
+    # quant_reference_test.go:42-61
+    fx = F.quant_affine_fixture()
+    x, p, s, b = fx["x"].view(np.uint8), fx["packed"].view(np.uint8), fx["scales"].view(np.uint8), fx["biases"].view(np.uint8)
+    od, idim, gs, bits = fx["out_dim"], fx["in_dim"], fx["group_size"], fx["bits"]
+    with pytest.raises(orc.OracleError):
+        orc.reference_affine_matvec(x[:-1], p, s, b, od, idim, gs, bits)
+    with pytest.raises(orc.OracleError):
+        orc.reference_affine_matvec(x, p.reshape(-1)[:-1], s, b, od, idim, gs, bits)
+    with pytest.raises(orc.OracleError):
+        orc.reference_affine_matvec(x, p, s, b, od, idim, 3, bits)
+    with pytest.raises(orc.OracleError):
+        orc.reference_affine_matvec(x, p, s, b, od, idim, gs, 0)
+    with pytest.raises(orc.OracleError):
+        orc.reference_affine_matvec(x, p, s, b, od, idim, gs, 9)
+
+
+def test_reference_affine_matvec_ugly_zero_sized(orc):
+    # quant_reference_test.go:66-74
+    e = np.zeros(0, dtype=np.uint8)
+    assert orc.reference_affine_matvec(e, e, e, e, 0, 0, 64, 4).size == 0
+
+
+# ---- hipReferenceMLXAffineProjection ---------------------------------------------------------
+
+def test_hip_reference_q4_known_answer(orc):
+    # go/engine/hip/hip_projection_reference_test.go:71-85 -> [28, 38]
+    out = orc.hip_reference_projection(np.ones(8), [0x76543210, 0xFEDCBA98], [0x3F80, 0x3F00], [0x0000, 0xBF80], 2, 8, 8, 4)
+    assert out.tolist() == [28.0, 38.0]
+
+
+def test_hip_reference_q6_q8_known_answers(orc):
+    # go/engine/hip/hip_projection_reference_test.go:87-106 -> [120, 136] and [10, 26]
+    v6 = np.array([list(range(16)), [16, 15, 14, 13, 12, 11, 10, 9, 8, 7, 6, 5, 4, 3, 2, 1]])
+    out6 = orc.hip_reference_projection(np.ones(16), F.pack_codes(v6, 6), [0x3F80, 0x3F80], [0, 0], 2, 16, 16, 6)
+    assert out6.tolist() == [120.0, 136.0]
+    v8 = np.array([[1, 2, 3, 4], [5, 6, 7, 8]])
+    out8 = orc.hip_reference_projection(np.ones(4), F.pack_codes(v8, 8), [0x3F80, 0x3F80], [0, 0], 2, 4, 4, 8)
+    assert out8.tolist() == [10.0, 26.0]
+
+
+def test_hip_reference_batch_known_answer(orc):
+    # go/engine/hip/hip_kernels_test.go:612-654 -> [28, 38, 56, 76], laid out [token][row]
+    x = np.concatenate([np.ones(8), 2 * np.ones(8)])
+    out = orc.hip_reference_projection_batch(x, 2, [0x76543210, 0xFEDCBA98], [0x3F80, 0x3F00], [0x0000, 0xBF80], 2, 8, 8, 4)
+    assert out.reshape(-1).tolist() == [28.0, 38.0, 56.0, 76.0]
+
+
+def test_hip_reference_bad_shapes(orc):
+    # go/engine/hip/hip_projection_reference_test.go:139-145: cols*bits not a word multiple; group not dividing
+    with pytest.raises(orc.OracleError):
+        orc.hip_reference_projection([1.0], [0], [0x3F80], [0], 1, 7, 7, 4)
+    with pytest.raises(orc.OracleError):
+        orc.hip_reference_projection(np.ones(8), [0], [0x3F80], [0], 1, 8, 3, 4)
+    with pytest.raises(orc.OracleError):
+        orc.hip_reference_projection(np.ones(8), [0], [0x3F80], [0], 1, 8, 8, 5)
+
+
+# ---- DequantizeTensor / QuantizeTensor -------------------------------------------------------
+
+def test_example_quantize_tensor(orc):
+    # go/model/quant/mlxaffine/mlxaffine_example_test.go:14-35
+    w = np.array([np.float32(0.01) * np.float32(i - 32) for i in range(64)], dtype=np.float32)
+    p, s, b = orc.quantize(w, 1, 64, 4, 64)
+    assert (p.size, s.size, b.size) == (32, 2, 2)
+    got = orc.dequantize(p, s, b, 1, 64, 4, 64)
+    assert "%.3f" % w[0] == "-0.320" and "%.3f" % got[0, 0] == "-0.320"
+
+
+@pytest.mark.parametrize("bits,gs,out_dim,in_dim", [(4, 64, 8, 3840), (4, 32, 4, 256), (8, 64, 6, 512), (8, 32, 3, 128),
+                                                     (2, 64, 5, 640), (4, 64, 3, 64)])
+def test_quantize_round_trip_within_group_bound(orc, bits, gs, out_dim, in_dim):
+    # go/model/quant/mlxaffine/mlxaffine_test.go:32-78
+    w = F.synth_weight(out_dim, in_dim)
+    p, s, b = orc.quantize(w, out_dim, in_dim, bits, gs)
+    got = orc.dequantize(p, s, b, out_dim, in_dim, bits, gs)
+    assert np.isfinite(got).all()
+    wg = w.reshape(out_dim, in_dim // gs, gs)
+    step = (wg.max(axis=2) - wg.min(axis=2)) / np.float32((1 << bits) - 1)
+    bound = 1.5 * step + 0.02 * np.abs(wg).max(axis=2) + 1e-6
+    err = np.abs(got.reshape(wg.shape) - wg)
+    assert (err <= bound[..., None]).all()
+
+
+def test_quantize_codes_are_a_fixed_point(orc):
+    # go/model/quant/mlxaffine/mlxaffine_test.go:87-112
+    w = F.synth_weight(6, 512)
+    p1, s1, b1 = orc.quantize(w, 6, 512, 4, 64)
+    d1 = orc.dequantize(p1, s1, b1, 6, 512, 4, 64)
+    p2, s2, b2 = orc.quantize(d1, 6, 512, 4, 64)
+    assert np.array_equal(p1, p2)
+    d2 = orc.dequantize(p2, s2, b2, 6, 512, 4, 64)
+    assert np.abs(d2 - d1).max() <= 5e-3
+
+
+def test_quantize_constant_group(orc):
+    # go/model/quant/mlxaffine/mlxaffine_test.go:117-139
+    w = np.full(2 * 64, 0.25, dtype=np.float32)
+    p, s, b = orc.quantize(w, 2, 64, 4, 64)
+    got = orc.dequantize(p, s, b, 2, 64, 4, 64)
+    assert np.isfinite(got).all() and np.abs(got - 0.25).max() <= 0.01
+
+
+@pytest.mark.parametrize("out_dim,in_dim,gs", [(4, 128, 128), (8, 256, 128), (3, 64, 64), (5, 96, 32)])
+def test_repack_b1_to_b2_exact(orc, out_dim, in_dim, gs):
+    # go/model/quant/mlxaffine/repack_test.go:26-65: exact float32 equality
+    w = F.synth_weight(out_dim, in_dim)
+    p, s, b = orc.quantize(w, out_dim, in_dim, 1, gs)
+    ref = orc.dequantize(p, s, b, out_dim, in_dim, 1, gs)
+    p2 = orc.repack_b1_to_b2(p, out_dim, in_dim)
+    assert p2.size == out_dim * (in_dim // 16) * 4
+    got = orc.dequantize(p2, s, b, out_dim, in_dim, 2, gs)
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+
+
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+def test_dequantize_brute_force_all_codes(orc, bits):
+    """Every code value against sampled bf16 (scale, bias) pairs: the C loop must equal a float32
+    multiply-then-add done one scalar at a time in numpy, and also the fused form (the product is
+    exact, so both must agree)."""
+    rng = np.random.default_rng(100 + bits)
+    ncodes = 1 << bits
+    per = 32 // bits
+    k = max(per, ncodes)  # one group holding every code at least once
+    k = (k + per - 1) // per * per
+    for _ in range(200):
+        sb = rng.integers(0, 65536, size=2).astype(np.uint16)
+        sf, bf = F.bf16_bits_to_f32(sb)
+        if not (np.isfinite(sf) and np.isfinite(bf)):
+            continue
+        codes = (np.arange(k) % ncodes).astype(np.uint32).reshape(1, k)
+        got = orc.dequantize(F.pack_codes_fast(codes, bits), sb[:1], sb[1:], 1, k, bits, k)
+        with np.errstate(all="ignore"):
+            want = (np.float32(sf) * codes.astype(np.float32)).astype(np.float32) + np.float32(bf)
+            fused = (np.float64(sf) * codes.astype(np.float64) + np.float64(bf)).astype(np.float32)
+        assert np.array_equal(got.view(np.uint32), want.astype(np.float32).view(np.uint32))
+        ok = np.isfinite(fused)
+        assert np.array_equal(got[ok].view(np.uint32), fused[ok].view(np.uint32))
+
+
+def test_dequantize_matches_numpy_formula_and_rejects_bad_sizes(orc):
+    """Same tensor through the broadcast-shift numpy formula of tools/mlxaffine_dequant.py:52-69."""
+    words, s, b = F.synthetic_affine(24, 512, 4, 64, seed=11)
+    got = orc.dequantize(words, s, b, 24, 512, 4, 64)
+    assert np.array_equal(got.view(np.uint32), F.numpy_dequant(words, s, b, 4, 64, 512).view(np.uint32))
+    words8, s8, b8 = F.synthetic_affine(7, 256, 8, 32, seed=12)
+    got8 = orc.dequantize(words8, s8, b8, 7, 256, 8, 32)
+    assert np.array_equal(got8.view(np.uint32), F.numpy_dequant(words8, s8, b8, 8, 32, 256).view(np.uint32))
+    with pytest.raises(orc.OracleError):
+        orc.dequantize(words.reshape(-1)[:-1], s, b, 24, 512, 4, 64)
+    with pytest.raises(orc.OracleError):
+        orc.dequantize(words, s.reshape(-1)[:-1], b, 24, 512, 4, 64)
+    with pytest.raises(orc.OracleError):
+        orc.dequantize(words, s, b, 24, 512, 3, 64)
+    with pytest.raises(orc.OracleError):
+        orc.dequantize(words, s, b, 24, 512, 4, 60)
+
+
+# ---- matNTQuantHost and cross-agreement ------------------------------------------------------
+
+def test_matnt_quant_host_is_sequential_f64(orc):
+    """Tiny case recomputed with a python float (= float64) ascending-k loop over numpy's fp32 dequant."""
+    words, s, b = F.synthetic_affine(5, 128, 4, 64, seed=21)
+    x = F.bf16_bits_to_f32(F.synthetic_x(3, 128, seed=22)).reshape(3, 128)
+    got = orc.matnt_quant_host(x, words, s, b, 3, 128, 5, 64, 4)
+    w = F.numpy_dequant(words, s, b, 4, 64, 128)
+    for m in range(3):
+        for n in range(5):
+            acc = 0.0
+            for k in range(128):
+                acc += float(x[m, k]) * float(w[n, k])
+            assert got[m, n] == np.float32(acc)
+
+
+def test_matnt_quant_host_threads_bit_identical(orc):
+    words, s, b = F.synthetic_affine(64, 256, 4, 64, seed=23)
+    x = F.bf16_bits_to_f32(F.synthetic_x(4, 256, seed=24)).reshape(4, 256)
+    a = orc.matnt_quant_host(x, words, s, b, 4, 256, 64, 64, 4, threads=1)
+    c = orc.matnt_quant_host(x, words, s, b, 4, 256, 64, 64, 4, threads=4)
+    assert np.array_equal(a.view(np.uint32), c.view(np.uint32))
+
+
+def test_all_ones_closed_form(orc):
+    """x = 1: y[n] = sum_g (scale_g * sum(codes in g) + group * bias_g), exact in float64.
+    A dropped bias term, a wrong group index or a transposed scale table fails here."""
+    rng = np.random.default_rng(5)
+    n, k, gs = 6, 256, 64
+    codes = rng.integers(0, 16, size=(n, k)).astype(np.uint32)
+    s = F.f32_to_bf16_bits(rng.uniform(0.01, 0.2, size=(n, k // gs)).astype(np.float32))
+    b = F.f32_to_bf16_bits(rng.uniform(-1, 1, size=(n, k // gs)).astype(np.float32))
+    sf, bf = F.bf16_bits_to_f32(s).astype(np.float64), F.bf16_bits_to_f32(b).astype(np.float64)
+    want = (sf * codes.reshape(n, k // gs, gs).sum(axis=2) + gs * bf).sum(axis=1)
+    ones = np.full(k, 0x3F80, dtype=np.uint16)
+    words = F.pack_codes_fast(codes, 4)
+    got_bf16 = F.bf16_bits_to_f32(orc.reference_affine_matvec(ones, words, s, b, n, k, gs, 4).view(np.uint16))
+    assert np.array_equal(got_bf16, F.bf16_bits_to_f32(F.f32_to_bf16_bits(want.astype(np.float32))))
+    got_host = orc.matnt_quant_host(np.ones(k, dtype=np.float32), words, s, b, 1, k, n, gs, 4)
+    assert np.allclose(got_host.reshape(-1), want, rtol=1e-6, atol=1e-6)
+    got_hip = orc.hip_reference_projection(np.ones(k), words, s, b, n, k, gs, 4)
+    assert np.allclose(got_hip, want, rtol=1e-5, atol=1e-5)
+
+
+def test_references_agree_on_the_parity_fixture(orc):
+    """a3 (fp32 w, f64 acc), a4 (f64 w, f64 acc, bf16 out) and a5 (fp32 acc) on quantAffineFixture,
+    against an independent numpy float64 matmul."""
+    fx = F.quant_affine_fixture()
+    xf = F.bf16_bits_to_f32(fx["x"])
+    want = F.reference_f64(fx["x"], fx["packed"], fx["scales"], fx["biases"], 4, 64, 128).reshape(-1)
+    a4 = F.bf16_bits_to_f32(orc.reference_affine_matvec(fx["x"], fx["packed"], fx["scales"], fx["biases"], 8, 128, 64, 4).view(np.uint16))
+    assert np.array_equal(a4, F.bf16_bits_to_f32(F.f32_to_bf16_bits(want.astype(np.float32))))
+    a3 = orc.matnt_quant_host(xf, fx["packed"], fx["scales"], fx["biases"], 1, 128, 8, 64, 4).reshape(-1)
+    assert np.allclose(a3, want, rtol=0, atol=1e-5)
+    a5 = orc.hip_reference_projection(xf, fx["packed"], fx["scales"], fx["biases"], 8, 128, 64, 4)
+    assert np.allclose(a5, want, rtol=0, atol=1e-4)
+
+
+@pytest.mark.parametrize("fixture", ["hw_fixture_q8_cols256", "hw_fixture_q8_cols3072"])
+def test_hardware_fixtures_against_numpy(orc, fixture):
+    fx = getattr(F, fixture)()
+    want = F.numpy_dequant(fx["packed"], fx["scales"], fx["biases"], 8, fx["group_size"], fx["cols"]).astype(np.float64) @ fx["x"].astype(np.float64)
+    got = orc.hip_reference_projection(fx["x"], fx["packed"], fx["scales"], fx["biases"], fx["rows"], fx["cols"], fx["group_size"], 8)
+    assert np.abs(got - want).max() <= 1e-3
+
+
+# ---- gather ---------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("bits", [2, 3, 4, 5, 6, 8])
+@pytest.mark.parametrize("name,out_dim,in_dim,gs,expert_rows,row_base,batched", [
+    ("fast shared-x", 32, 512, 64, 32, 0, False), ("fast batched-x", 32, 512, 64, 32, 0, True),
+    ("plain shared-x", 24, 256, 32, 24, 0, False), ("fast gate_up rowBase", 32, 512, 64, 64, 32, False)])
+def test_gather_equals_sliced_matvec(orc, bits, name, out_dim, in_dim, gs, expert_rows, row_base, batched):
+    """Route z == the plain matvec on expert rhs[z]'s row slice with x row lhs[z]
+    (the cases of go/engine/metal/qmv_gather_test.go:87-129; invariant of moe_quant_test.go:1143-1185)."""
+    if in_dim * bits % 32:
+        pytest.skip("packed-row alignment")
+    E, routes = 4, 3
+    fx = F.gather_fixture(out_dim, in_dim, gs, bits, E, expert_rows, batched, routes)
+    _, got = orc.gather_qmv(fx["x"], fx["x_rows"], fx["packed"], fx["scales"], fx["biases"], fx["lhs"], fx["rhs"], routes, E,
+                            expert_rows, row_base, out_dim, in_dim, gs, bits)
+    wpr, gpr = in_dim * bits // 32, in_dim // gs
+    W = fx["packed"].reshape(E, expert_rows, wpr)
+    S = fx["scales"].reshape(E, expert_rows, gpr)
+    B = fx["biases"].reshape(E, expert_rows, gpr)
+    X = fx["x"].reshape(fx["x_rows"], in_dim)
+    for z in range(routes):
+        e = fx["rhs"][z]
+        xr = X[fx["lhs"][z]] if batched else X[0]
+        want = orc.reference_affine_matvec(xr, W[e, row_base:row_base + out_dim], S[e, row_base:row_base + out_dim],
+                                           B[e, row_base:row_base + out_dim], out_dim, in_dim, gs, bits)
+        assert np.array_equal(got[z], want.view(np.uint16))
+
+
+def test_gather_rejects_bad_indices(orc):
+    fx = F.gather_fixture(8, 64, 64, 4, 4, 8, False, 3)
+    bad = fx["rhs"].copy()
+    bad[1] = 4
+    with pytest.raises(orc.OracleError):
+        orc.gather_qmv(fx["x"], 1, fx["packed"], fx["scales"], fx["biases"], None, bad, 3, 4, 8, 0, 8, 64, 64, 4)
+    bad[1] = -1
+    with pytest.raises(orc.OracleError):
+        orc.gather_qmv(fx["x"], 1, fx["packed"], fx["scales"], fx["biases"], None, bad, 3, 4, 8, 0, 8, 64, 64, 4)
