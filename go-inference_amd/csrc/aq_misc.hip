@@ -1,10 +1,12 @@
 // fp32 dequantisation and the any-width fallback matvec.
 //
 // dequant: mlxaffine.DequantizeTensor (go/model/quant/mlxaffine/mlxaffine.go:178-208),
-// out = scale * float(code) + bias in fp32.  scale*code is exact in fp32 (8-bit
-// significand times <= 8-bit integer), so the single rounding of the add makes
-// the result independent of whether the multiply-add is fused: the output is
-// bit-identical to the CPU path.
+// out = scale * float(code) + bias in fp32, as a multiply followed by an add
+// (contraction switched off for that expression), the two roundings the
+// reference's amd64 build performs.  For finite products scale*code is exact
+// (8-bit significand times <= 8-bit integer), so a fused form would agree;
+// it differs only when the product overflows, and the unfused form keeps the
+// result bit-identical to the CPU path there too.
 //
 // generic qmv: the arithmetic of hipReferenceMLXAffineProjection
 // (go/engine/hip/hip_projection_reference.go:92-116, unpack :200-222) for
@@ -14,6 +16,12 @@
 #include "aq_kernels.h"
 
 namespace aq {
+
+__device__ __forceinline__ float affine_weight(float scale, float code, float bias) {
+#pragma clang fp contract(off)
+    const float prod = scale * code;
+    return prod + bias;
+}
 
 // Code `col` of a packed row, any width 1..8, codes may cross a word boundary.
 __device__ __forceinline__ uint32_t extract_code(const uint32_t* row, int64_t words, int64_t col, int bits) {
@@ -48,14 +56,14 @@ __global__ __launch_bounds__(256) void dequant_words_kernel(const uint32_t* __re
 #pragma unroll
         for (int p = 0; p < PER; p++) {
             const float code = (float)((word >> (p * BITS)) & ((1u << BITS) - 1u));
-            o[p] = __fmaf_rn(sc, code, bi);
+            o[p] = affine_weight(sc, code, bi);
         }
     } else {
 #pragma unroll
         for (int p = 0; p < PER; p++) {
             const int64_t gi = row * groups_per_row + (k0 + p) / group_size;
             const float code = (float)((word >> (p * BITS)) & ((1u << BITS) - 1u));
-            o[p] = __fmaf_rn(bf16_bits_to_f32(s[gi]), code, bf16_bits_to_f32(b[gi]));
+            o[p] = affine_weight(bf16_bits_to_f32(s[gi]), code, bf16_bits_to_f32(b[gi]));
         }
     }
 }
@@ -72,7 +80,7 @@ __global__ __launch_bounds__(256) void dequant_any_kernel(const uint32_t* __rest
     const int64_t words = (int64_t)K * bits / 32;
     const float code = (float)extract_code(w + row * words, words, col, bits);
     const int64_t gi = row * (K / group_size) + col / group_size;
-    out[i] = __fmaf_rn(bf16_bits_to_f32(s[gi]), code, bf16_bits_to_f32(b[gi]));
+    out[i] = affine_weight(bf16_bits_to_f32(s[gi]), code, bf16_bits_to_f32(b[gi]));
 }
 
 hipError_t dequant_launch(const uint32_t* w, const uint16_t* s, const uint16_t* b, float* out, int64_t N, int K,
@@ -143,7 +151,7 @@ __global__ __launch_bounds__(256) void qmv_generic_kernel(const QmvArgs a, int b
         for (int k = lane; k < K; k += kWave) {
             const float code = (float)extract_code(wr, words, k, bits);
             const int64_t gi = (int64_t)row * gpr + k / group_size;
-            const float wv = __fmaf_rn(bf16_bits_to_f32(sbase[gi]), code, bf16_bits_to_f32(bbase[gi]));
+            const float wv = affine_weight(bf16_bits_to_f32(sbase[gi]), code, bf16_bits_to_f32(bbase[gi]));
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 if (m0 + j < m_count) acc[j] = __fmaf_rn(wv, bf16_bits_to_f32(xbase[(int64_t)(m0 + j) * K + k]), acc[j]);

@@ -7,6 +7,7 @@ import fixtures as F
 
 MAX_ABS = 1e-2   # max-abs-err bound on the fp32 accumulator vs the fp32-weight reference
 REL = 2e-3       # rel-err bound (elementwise where |ref| >= 1, and as an L2 ratio overall)
+BF16_ABS = 2e-3  # absolute escape of the one-ulp bf16 store check, for outputs near zero
 
 
 def say(*a):
@@ -32,7 +33,9 @@ def check_accumulators(got_f32, ref_f64, what):
 
 
 def check_bf16_store(got_bits, ref_f64, what):
-    """bf16 outputs must sit within one bf16 ulp of bf16(reference)."""
+    """bf16 outputs must sit within one bf16 ulp of bf16(reference).  Near zero a bf16 ulp is finer
+    than any fp32 summation-order difference, so a store also passes when it is within BF16_ABS of
+    the reference in absolute terms (a fifth of the stated max-abs-err bound)."""
     got_bits = np.asarray(got_bits, dtype=np.uint16).reshape(-1)
     ref_bits = F.f32_to_bf16_bits(np.asarray(ref_f64, dtype=np.float64).reshape(-1).astype(np.float32))
     # monotone integer key of a bf16 pattern, so adjacent values differ by 1
@@ -40,7 +43,9 @@ def check_bf16_store(got_bits, ref_f64, what):
         b = b.astype(np.int32)
         return np.where(b & 0x8000, -(b & 0x7FFF), b & 0x7FFF)
     d = np.abs(key(got_bits) - key(ref_bits))
-    assert d.max() <= 1, "%s: bf16 store is %d ulp from bf16(reference)" % (what, d.max())
+    absd = np.abs(F.bf16_bits_to_f32(got_bits).astype(np.float64) - F.bf16_bits_to_f32(ref_bits).astype(np.float64))
+    bad = (d > 1) & (absd > BF16_ABS)
+    assert not bad.any(), "%s: bf16 store is %d ulp from bf16(reference)" % (what, d[bad].max())
 
 
 class DeviceAffine:

@@ -23,7 +23,8 @@ def test_dequant_bit_exact(ctx, orc, N, K, bits, gs):
     words = F.pack_codes(codes, bits)
     s = rng.integers(0, 65536, size=(N, K // gs)).astype(np.uint16)
     b = rng.integers(0, 65536, size=(N, K // gs)).astype(np.uint16)
-    # keep scales/biases finite: clear the top exponent bit pattern 0xFF
+    # any finite bf16 pattern, denormals and values whose product with a code overflows included;
+    # inf/NaN inputs are left out (a NaN's payload is not part of the contract)
     s = np.where((s & 0x7F80) == 0x7F80, s & 0xBFFF, s).astype(np.uint16)
     b = np.where((b & 0x7F80) == 0x7F80, b & 0xBFFF, b).astype(np.uint16)
     dw = DeviceAffine(ctx, words, s, b)
@@ -35,7 +36,9 @@ def test_dequant_bit_exact(ctx, orc, N, K, bits, gs):
         want = orc.dequantize(words, s, b, N, K, bits, gs).view(np.uint32)
     else:  # straddling widths are outside DequantizeTensor: same formula over the word unpacker
         want = F.numpy_dequant(words, s, b, bits, gs, K).view(np.uint32)
-    assert np.array_equal(got, want)
+    nan = np.isnan(want.view(np.float32))  # inf - inf: both sides must agree it is NaN
+    assert np.array_equal(np.isnan(got.view(np.float32)), nan)
+    assert np.array_equal(got[~nan], want[~nan])
     dw.free()
     dout.free()
 
@@ -307,7 +310,7 @@ def test_gather_errors(ctx):
 
 @pytest.mark.parametrize("M,K,N,bits,gs", [(3, 512, 64, 4, 64), (5, 256, 40, 4, 64), (2, 128, 8, 8, 64), (33, 1024, 130, 4, 64),
                                            (64, 512, 256, 8, 64), (100, 2816, 96, 4, 64), (17, 704, 17, 4, 64), (40, 1408, 70, 4, 128),
-                                           (130, 320, 33, 8, 128), (256, 1024, 512, 4, 64)])
+                                           (130, 384, 33, 8, 128), (256, 1024, 512, 4, 64)])
 def test_qmm_small_cases(ctx, orc, M, K, N, bits, gs):
     say("qmm", M, K, N, bits, gs)
     _qmv_case(ctx, orc, M, K, N, bits, gs, 900 + M + N, fn="qmm")
