@@ -47,6 +47,10 @@ PROTOTYPES = {
     "aq_sync": (_i, [_vp]),
     "aq_timer_start": (_i, [_vp]),
     "aq_timer_stop": (_i, [_vp, _c.POINTER(_f)]),
+    "aq_capture_begin": (_i, [_vp]),
+    "aq_capture_end": (_i, [_vp, _c.POINTER(_vp)]),
+    "aq_graph_launch": (_i, [_vp, _vp]),
+    "aq_graph_destroy": (None, [_vp]),
     "aq_qmv": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _u]),
     "aq_qmm": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _u]),
     "aq_gather_qmv": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _u]),
@@ -187,6 +191,20 @@ class Context:
         ms = _f()
         self._check(self.lib.aq_timer_stop(self.handle, ctypes.byref(ms)))
         return ms.value
+
+    def capture_begin(self):
+        self._check(self.lib.aq_capture_begin(self.handle))
+
+    def capture_end(self):
+        g = _vp()
+        self._check(self.lib.aq_capture_end(self.handle, ctypes.byref(g)))
+        return g
+
+    def graph_launch(self, graph):
+        self._check(self.lib.aq_graph_launch(self.handle, graph))
+
+    def graph_destroy(self, graph):
+        self.lib.aq_graph_destroy(graph)
 
     def qmv(self, x, w, s, b, y, M, K, N, group_size=64, bits=4, flags=0):
         self._check(self.lib.aq_qmv(self.handle, _ptr(x), _ptr(w), _ptr(s), _ptr(b), _ptr(y), M, K, N, group_size,

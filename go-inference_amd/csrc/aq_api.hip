@@ -110,26 +110,63 @@ int pick_qmv_variant(const aq_ctx* ctx, int bits, int m, bool gather, int N, int
     for (int i = 0; i < aq::qmv_variant_count(); i++) {
         const aq::QmvVariant* v = aq::qmv_variant(i);
         if (v->bits != bits || v->m != m || (v->gather != 0) != gather) continue;
-        if (v->waves != 4 || v->depth != 2) continue;
+        if (v->waves != 4 || v->depth != 2 || v->xmode != 0) continue;
         if (v->rows == want_rows) return i;
         if (best < 0 || (v->rows < want_rows && v->rows > aq::qmv_variant(best)->rows)) best = i;
     }
     return best;
 }
 
+// One index space over both matvec kernel families: dot2 variants first, MFMA variants after.
+int qmv_total_variants() { return aq::qmv_variant_count() + aq::qmvx_variant_count(); }
+const aq::QmvVariant* qmv_any_variant(int idx) {
+    const int nd = aq::qmv_variant_count();
+    return idx < nd ? aq::qmv_variant(idx) : aq::qmvx_variant(idx - nd);
+}
+
+constexpr size_t kMaxLds = 160 * 1024;
+
+bool mfma_eligible(const aq::QmvArgs& a, int group_size, int bits) {
+    if (bits != 4 && bits != 8) return false;
+    // scales are staged as pairs of consecutive groups: group size 64 and an even group count
+    if (group_size != 64 || a.K % 128 != 0 || a.M > 32) return false;
+    return aligned(a.x, 16) && aligned(a.w, 16) && aligned(a.s, 4) && aligned(a.b, 4);
+}
+
+int find_qmvx(int bits, int mr_max_m, int ks, bool gather) {
+    for (int i = 0; i < aq::qmvx_variant_count(); i++) {
+        const aq::QmvVariant* v = aq::qmvx_variant(i);
+        if (v->bits == bits && v->m == mr_max_m && v->waves == ks && (v->gather != 0) == gather) return i;
+    }
+    return -1;
+}
+
 int launch_qmv_rows(aq_ctx* ctx, aq::QmvArgs a, int group_size, int bits, bool gather) {
     const int M = a.M;
+    a.gs_shift = is_pow2(group_size) ? ilog2(group_size) : 0;
+    const int nd = aq::qmv_variant_count();
+    int forced = ctx->forced[0];
+    if (forced >= nd) {
+        // a forced MFMA variant: the whole call in one launch
+        const aq::QmvVariant* v = aq::qmvx_variant(forced - nd);
+        if (!v || v->bits != bits || (v->gather != 0) != gather || M > v->m || !mfma_eligible(a, group_size, bits) ||
+            aq::qmvx_lds_bytes(forced - nd, a) > kMaxLds)
+            return fail(AQ_ERR_ARG, "aq_qmv: forced variant %d does not fit bits=%d gather=%d rows=%d K=%d", forced, bits,
+                        (int)gather, M, a.K);
+        ctx->last_variant[0] = v->name;
+        AQ_HIP(aq::qmvx_launch(forced - nd, a, ctx->stream), "hipLaunchKernel");
+        return AQ_OK;
+    }
     const bool fast = dot2_eligible(a.K, group_size, bits, a.x, a.w, (size_t)(M < 4 ? M : 4) * a.K * 2);
     if (!fast) {
         ctx->last_variant[0] = "qmv_generic";
         AQ_HIP(aq::qmv_generic_launch(a, bits, group_size, gather, ctx->stream), "hipLaunchKernel");
         return AQ_OK;
     }
-    a.gs_shift = ilog2(group_size);
     const size_t esize = a.out_f32 ? 4 : 2;
     for (int m0 = 0; m0 < M;) {
         int m = M - m0 < 4 ? M - m0 : 4;
-        int idx = ctx->forced[0];
+        int idx = forced;
         if (idx >= 0) {
             const aq::QmvVariant* v = aq::qmv_variant(idx);
             if (!v || v->bits != bits || (v->gather != 0) != gather || v->m > M - m0)
@@ -289,6 +326,54 @@ int aq_timer_stop(aq_ctx* ctx, float* elapsed_ms) {
     AQ_HIP(hipEventSynchronize(ctx->ev1), "hipEventSynchronize");
     AQ_HIP(hipEventElapsedTime(elapsed_ms, ctx->ev0, ctx->ev1), "hipEventElapsedTime");
     return AQ_OK;
+}
+
+struct aq_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+};
+
+int aq_capture_begin(aq_ctx* ctx) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_capture_begin: ctx is null");
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    if (ctx->stream == nullptr) return fail(AQ_ERR_UNSUPPORTED, "aq_capture_begin: the legacy default stream cannot be captured");
+    AQ_HIP(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
+    return AQ_OK;
+}
+
+int aq_capture_end(aq_ctx* ctx, aq_graph** out) {
+    if (!ctx || !out) return fail(AQ_ERR_ARG, "aq_capture_end: bad argument");
+    *out = nullptr;
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    hipGraph_t g = nullptr;
+    AQ_HIP(hipStreamEndCapture(ctx->stream, &g), "hipStreamEndCapture");
+    aq_graph* ag = new (std::nothrow) aq_graph();
+    if (!ag) {
+        (void)hipGraphDestroy(g);
+        return fail(AQ_ERR_NOMEM, "aq_capture_end: out of host memory");
+    }
+    ag->graph = g;
+    hipError_t rc = hipGraphInstantiate(&ag->exec, g, nullptr, nullptr, 0);
+    if (rc != hipSuccess) {
+        aq_graph_destroy(ag);
+        return hip_fail(rc, "hipGraphInstantiate");
+    }
+    *out = ag;
+    return AQ_OK;
+}
+
+int aq_graph_launch(aq_ctx* ctx, aq_graph* graph) {
+    if (!ctx || !graph || !graph->exec) return fail(AQ_ERR_ARG, "aq_graph_launch: bad argument");
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    AQ_HIP(hipGraphLaunch(graph->exec, ctx->stream), "hipGraphLaunch");
+    return AQ_OK;
+}
+
+void aq_graph_destroy(aq_graph* graph) {
+    if (!graph) return;
+    if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
+    if (graph->graph) (void)hipGraphDestroy(graph->graph);
+    delete graph;
 }
 
 int aq_qmv(aq_ctx* ctx, const void* x, const void* packed, const void* scales, const void* biases, void* y, int M,
@@ -486,14 +571,14 @@ int aq_proj_quant_matmul_host(aq_ctx* ctx, float* out, const float* x, size_t x_
 }
 
 int aq_variant_count(int op) {
-    if (op == 0) return aq::qmv_variant_count();
+    if (op == 0) return qmv_total_variants();
     if (op == 1) return aq::qmm_variant_count();
     return 0;
 }
 
 const char* aq_variant_name(int op, int variant) {
     if (op == 0) {
-        const aq::QmvVariant* v = aq::qmv_variant(variant);
+        const aq::QmvVariant* v = (variant >= 0 && variant < qmv_total_variants()) ? qmv_any_variant(variant) : nullptr;
         return v ? v->name : "";
     }
     if (op == 1) return aq::qmm_variant_name(variant);

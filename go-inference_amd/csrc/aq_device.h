@@ -27,13 +27,21 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
     return (uint16_t)(u >> 16);
 }
 
-// (a & mask) | magic in one VALU op.  gfx9 VOP3 cannot carry 32-bit literals,
-// so the mask rides in an SGPR and the magic in a VGPR; written as asm because
-// the compiler otherwise picks two literal-carrying VOP2 ops.
-__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask_s, uint32_t magic_v) {
-    uint32_t r;
-    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(mask_s), "v"(magic_v));
-    return r;
+// (a & mask) | magic, meant to become one v_and_or_b32.  gfx9 VOP3 cannot carry 32-bit literals,
+// so with literal constants the compiler emits two VOP2 ops; callers therefore pass the mask and
+// the magic through opaque_s / opaque_v, which hides their values and leaves them in registers.
+// Plain C on purpose: an inline-asm VALU instruction is invisible to the compiler's hazard
+// recogniser, and next to MFMAs (operands or results in VGPRs) that produced wrong sums.
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t magic) { return (a & mask) | magic; }
+
+// Launder a constant through an empty asm so that it stays in an SGPR / VGPR.
+__device__ __forceinline__ uint32_t opaque_s(uint32_t v) {
+    asm volatile("" : "+s"(v));
+    return v;
+}
+__device__ __forceinline__ uint32_t opaque_v(uint32_t v) {
+    asm volatile("" : "+v"(v));
+    return v;
 }
 
 __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float acc) {

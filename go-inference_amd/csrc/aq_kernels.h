@@ -38,6 +38,8 @@ struct QmvVariant {
     int waves;   // wavefronts per workgroup
     int depth;   // K slices in flight per wavefront
     int gather;  // 1: reads rhs/lhs on device, grid.y = routes
+    int xmode;   // 0: x staged through LDS, 1: every lane reads its x chunk from global
+    int kind;    // 0: VALU dot2 kernel (aq_qmv.hip), 1: MFMA kernel (aq_qmv_mfma.hip; m = most rows it takes)
 };
 
 int qmv_variant_count();
@@ -47,6 +49,12 @@ const QmvVariant* qmv_variant(int idx);
 hipError_t qmv_launch(int idx, const QmvArgs& a, hipStream_t stream);
 // LDS bytes variant idx needs for these args (x staging).
 size_t qmv_lds_bytes(int idx, const QmvArgs& a);
+
+// MFMA matvec kernels (M <= 32), same argument block.
+int qmvx_variant_count();
+const QmvVariant* qmvx_variant(int idx);
+hipError_t qmvx_launch(int idx, const QmvArgs& a, hipStream_t stream);
+size_t qmvx_lds_bytes(int idx, const QmvArgs& a);
 
 // Any-width (2..8 bit, codes may straddle words), any-group fallback.
 hipError_t qmv_generic_launch(const QmvArgs& a, int bits, int group_size, bool gather, hipStream_t stream);

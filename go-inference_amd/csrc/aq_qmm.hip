@@ -193,9 +193,8 @@ __global__ __launch_bounds__(WM* WN* kWave) void qmm_kernel(const QmmArgs a) {
 #pragma unroll
         for (int q = 0; q < 4; q++) sq[nb][q] = bq[nb][q] = 0u;
 
-    const uint32_t mask_s = kMask16;
-    uint32_t magic_v = kMagic16;
-    asm volatile("" : "+v"(magic_v));
+    const uint32_t mask_s = opaque_s(kMask16);   // both stay in registers so that
+    const uint32_t magic_v = opaque_v(kMagic16);  // (w & mask) | magic is a single v_and_or_b32
 
     load_x(0);
     load_w(0, raw, sbits, bbits);

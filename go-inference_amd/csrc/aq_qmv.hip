@@ -39,33 +39,39 @@ struct Codec<8> {
     static constexpr float kOffset = 0.0f;
 };
 
-// One slice of R rows held in registers.
-template <int R>
+// One slice of R rows held in registers (plus, in direct-x mode, the lane's x chunk).
+template <int R, int XREGS>
 struct Slice {
     uint4 w[R];
     uint16_t s[R];
     uint16_t b[R];
+    uint4 x[XREGS > 0 ? XREGS : 1];
 };
 
-template <int BITS, int M, int R, int NW, int DEPTH, bool GATHER>
+// XMODE 0: x staged once per workgroup into LDS (x loads are issued before any weight load so the
+//          barrier never waits for HBM); XMODE 1 (M == 1 only): every lane pulls its own 64-byte
+//          x chunk straight from global/L2 with the slice, no LDS and no barrier.
+template <int BITS, int M, int R, int NW, int DEPTH, bool GATHER, int XMODE>
 __global__ __launch_bounds__(NW* kWave) void qmv_dot2_kernel(const QmvArgs a) {
     using C = Codec<BITS>;
     constexpr int CPC = C::kCodesPerChunk;
     constexpr int PAIRS = C::kPairs;
-    extern __shared__ uint32_t xs[];  // [M][K/2] bf16 pairs, unpack order
+    constexpr int XREGS = XMODE == 1 ? PAIRS / 4 : 0;
+    static_assert(XMODE == 0 || M == 1, "direct x mode is single-row only");
+    extern __shared__ uint32_t xs[];  // [M][K/2] bf16 pairs, unpack order (XMODE 0)
 
     const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int K = a.K;
     const int N = a.N;
     const int chunks_per_row = K / CPC;  // 16-byte chunks in a packed row
-    const int64_t words_per_row = (int64_t)chunks_per_row * 4;
+    const uint32_t row_bytes = (uint32_t)chunks_per_row * 16u;
     const int groups_per_row = K >> a.gs_shift;
     const int nslices = (chunks_per_row + kWave - 1) / kWave;
 
-    const uint32_t* wbase = a.w;
-    const uint16_t* sbase = a.s;
-    const uint16_t* bbase = a.b;
+    const char* wbase = reinterpret_cast<const char*>(a.w);
+    const char* sbase = reinterpret_cast<const char*>(a.s);
+    const char* bbase = reinterpret_cast<const char*>(a.b);
     const uint16_t* xrow = a.x;
     int64_t yoff = 0;
     bool route_ok = true;
@@ -76,42 +82,62 @@ __global__ __launch_bounds__(NW* kWave) void qmv_dot2_kernel(const QmvArgs a) {
         route_ok = (unsigned)e < (unsigned)a.num_experts && (unsigned)xr < (unsigned)a.x_rows;
         const int64_t row0 = route_ok ? ((int64_t)e * a.expert_rows + a.row_base) : 0;
         if (!route_ok) xr = 0;
-        wbase += row0 * words_per_row;
-        sbase += row0 * groups_per_row;
-        bbase += row0 * groups_per_row;
+        wbase += row0 * row_bytes;
+        sbase += row0 * groups_per_row * 2;
+        bbase += row0 * groups_per_row * 2;
         xrow += (int64_t)xr * K;
         yoff = (int64_t)z * N;
     }
 
+    // wave-uniform 64-bit bases + 32-bit lane offsets: rows past N are clamped onto the last row
     const int row_first = (blockIdx.x * NW + wave) * R;
-    int rows[R];
+    const int row_base_clamped = min(row_first, N - 1);
+    wbase += (int64_t)row_base_clamped * row_bytes;
+    sbase += (int64_t)row_base_clamped * groups_per_row * 2;
+    bbase += (int64_t)row_base_clamped * groups_per_row * 2;
+    uint32_t rel[R];
 #pragma unroll
-    for (int r = 0; r < R; r++) rows[r] = min(row_first + r, N - 1);  // clamp: loads stay in range
+    for (int r = 0; r < R; r++) rel[r] = (uint32_t)min(r, N - 1 - row_base_clamped);
 
-    auto load_slice = [&](Slice<R>& t, int sl) {
+    // Stage x (XMODE 0): global loads first, so that nothing below queues ahead of them.
+    constexpr int XPT = 4;  // 16-byte x pieces held per thread between load and LDS write
+    uint4 xstage[XPT];
+    const int pieces = M * (K / 8);
+    if constexpr (XMODE == 0) {
+        const uint4* src = reinterpret_cast<const uint4*>(xrow);
+#pragma unroll
+        for (int q = 0; q < XPT; q++) {
+            const int p = threadIdx.x + q * NW * kWave;
+            if (p < pieces) xstage[q] = src[p];
+        }
+    }
+
+    auto load_slice = [&](Slice<R, XREGS>& t, int sl) {
         const int c = sl * kWave + lane;
         if (sl < nslices && c < chunks_per_row) {
-            const int g = (c * CPC) >> a.gs_shift;
+            const uint32_t g2 = (uint32_t)((c * CPC) >> a.gs_shift) * 2u;
+            if constexpr (XMODE == 1) {
+                const uint4* xp = reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(xrow) + (uint32_t)c * (PAIRS * 4u));
+#pragma unroll
+                for (int q = 0; q < XREGS; q++) t.x[q] = xp[q];
+            }
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                t.w[r] = reinterpret_cast<const uint4*>(wbase + (int64_t)rows[r] * words_per_row)[c];
-                t.s[r] = sbase[(int64_t)rows[r] * groups_per_row + g];
-                t.b[r] = bbase[(int64_t)rows[r] * groups_per_row + g];
+                t.s[r] = *reinterpret_cast<const uint16_t*>(sbase + (rel[r] * (uint32_t)groups_per_row * 2u + g2));
+                t.b[r] = *reinterpret_cast<const uint16_t*>(bbase + (rel[r] * (uint32_t)groups_per_row * 2u + g2));
             }
+#pragma unroll
+            for (int r = 0; r < R; r++)
+                t.w[r] = *reinterpret_cast<const uint4*>(wbase + (rel[r] * row_bytes + (uint32_t)c * 16u));
         }
     };
 
-    Slice<R> ring[DEPTH];
+    Slice<R, XREGS> ring[DEPTH];
 #pragma unroll
     for (int d = 0; d < DEPTH; d++) load_slice(ring[d], d);
 
-    // Stage x: every thread moves 16-byte pieces (8 bf16) from global to LDS.
-    {
-        const int pieces = M * (K / 8);
-        const uint4* src = reinterpret_cast<const uint4*>(xrow);
-        uint4* dst = reinterpret_cast<uint4*>(xs);
-        for (int p = threadIdx.x; p < pieces; p += NW * kWave) {
-            uint4 v = src[p];
+    if constexpr (XMODE == 0) {
+        auto permute = [](uint4 v) {
             if constexpr (BITS == 4) {
                 // (x0,x1)(x2,x3)(x4,x5)(x6,x7) -> (x0,x4)(x1,x5)(x2,x6)(x3,x7)
                 uint4 o;
@@ -119,12 +145,22 @@ __global__ __launch_bounds__(NW* kWave) void qmv_dot2_kernel(const QmvArgs a) {
                 o.y = (v.x >> 16) | (v.z & 0xffff0000u);
                 o.z = (v.y & 0xffffu) | (v.w << 16);
                 o.w = (v.y >> 16) | (v.w & 0xffff0000u);
-                v = o;
+                return o;
+            } else {
+                return v;
             }
-            dst[p] = v;
+        };
+        uint4* dst = reinterpret_cast<uint4*>(xs);
+#pragma unroll
+        for (int q = 0; q < XPT; q++) {
+            const int p = threadIdx.x + q * NW * kWave;
+            if (p < pieces) dst[p] = permute(xstage[q]);
         }
+        // long activations: the rest goes through without the early issue
+        const uint4* src = reinterpret_cast<const uint4*>(xrow);
+        for (int p = threadIdx.x + XPT * NW * kWave; p < pieces; p += NW * kWave) dst[p] = permute(src[p]);
+        __syncthreads();
     }
-    __syncthreads();
 
     float acc[R][M];
 #pragma unroll
@@ -132,25 +168,42 @@ __global__ __launch_bounds__(NW* kWave) void qmv_dot2_kernel(const QmvArgs a) {
 #pragma unroll
         for (int m = 0; m < M; m++) acc[r][m] = 0.0f;
 
-    const uint32_t mask_s = kNibbleMask;
-    uint32_t magic_v = kMagic128;
-    asm volatile("" : "+v"(magic_v));  // keep the constant in a VGPR across the loop
+    const uint32_t mask_s = opaque_s(kNibbleMask);   // both stay in registers so that
+    const uint32_t magic_v = opaque_v(kMagic128);  // (w & mask) | magic is a single v_and_or_b32
 
-    auto compute_slice = [&](const Slice<R>& t, int sl) {
+    auto compute_slice = [&](const Slice<R, XREGS>& t, int sl) {
         const int c = sl * kWave + lane;
         if (sl < nslices && c < chunks_per_row) {
             uint32_t xq[M][PAIRS];
             float xsum[M];
 #pragma unroll
             for (int m = 0; m < M; m++) {
-                const uint4* xp = reinterpret_cast<const uint4*>(xs + (size_t)m * (K / 2) + (size_t)c * PAIRS);
+                if constexpr (XMODE == 1) {
 #pragma unroll
-                for (int q = 0; q < PAIRS / 4; q++) {
-                    uint4 v = xp[q];
-                    xq[m][4 * q + 0] = v.x;
-                    xq[m][4 * q + 1] = v.y;
-                    xq[m][4 * q + 2] = v.z;
-                    xq[m][4 * q + 3] = v.w;
+                    for (int q = 0; q < PAIRS / 4; q++) {
+                        const uint4 v = t.x[q];
+                        if constexpr (BITS == 4) {
+                            xq[m][4 * q + 0] = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);
+                            xq[m][4 * q + 1] = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);
+                            xq[m][4 * q + 2] = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);
+                            xq[m][4 * q + 3] = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
+                        } else {
+                            xq[m][4 * q + 0] = v.x;
+                            xq[m][4 * q + 1] = v.y;
+                            xq[m][4 * q + 2] = v.z;
+                            xq[m][4 * q + 3] = v.w;
+                        }
+                    }
+                } else {
+                    const uint4* xp = reinterpret_cast<const uint4*>(xs + (size_t)m * (K / 2) + (size_t)c * PAIRS);
+#pragma unroll
+                    for (int q = 0; q < PAIRS / 4; q++) {
+                        const uint4 v = xp[q];
+                        xq[m][4 * q + 0] = v.x;
+                        xq[m][4 * q + 1] = v.y;
+                        xq[m][4 * q + 2] = v.z;
+                        xq[m][4 * q + 3] = v.w;
+                    }
                 }
                 float sx = 0.0f;
 #pragma unroll
@@ -231,18 +284,23 @@ struct QmvEntry {
     QmvKernel fn;
 };
 
-#define AQ_QMV(BITS, M, R, NW, DEPTH, G)                                                           \
-    {                                                                                              \
-        {"qmv_b" #BITS "_m" #M "_r" #R "_w" #NW "_d" #DEPTH "_g" #G, BITS, M, R, NW, DEPTH, G},    \
-            qmv_dot2_kernel<BITS, M, R, NW, DEPTH, (G != 0)>                                       \
+#define AQ_QMV_X(BITS, M, R, NW, DEPTH, G, X)                                                           \
+    {                                                                                                   \
+        {"qmv_b" #BITS "_m" #M "_r" #R "_w" #NW "_d" #DEPTH "_g" #G "_x" #X, BITS, M, R, NW, DEPTH, G, X}, \
+            qmv_dot2_kernel<BITS, M, R, NW, DEPTH, (G != 0), X>                                         \
     }
+#define AQ_QMV(BITS, M, R, NW, DEPTH, G) AQ_QMV_X(BITS, M, R, NW, DEPTH, G, 0)
 
 #define AQ_QMV_M1_SET(BITS, G)                                                                     \
     AQ_QMV(BITS, 1, 1, 4, 2, G), AQ_QMV(BITS, 1, 1, 4, 4, G), AQ_QMV(BITS, 1, 1, 8, 2, G),         \
         AQ_QMV(BITS, 1, 2, 2, 2, G), AQ_QMV(BITS, 1, 2, 4, 2, G), AQ_QMV(BITS, 1, 2, 4, 4, G),     \
         AQ_QMV(BITS, 1, 2, 8, 2, G), AQ_QMV(BITS, 1, 4, 2, 2, G), AQ_QMV(BITS, 1, 4, 4, 2, G),     \
         AQ_QMV(BITS, 1, 4, 4, 4, G), AQ_QMV(BITS, 1, 4, 8, 2, G), AQ_QMV(BITS, 1, 8, 2, 2, G),     \
-        AQ_QMV(BITS, 1, 8, 4, 2, G), AQ_QMV(BITS, 1, 7, 4, 2, G), AQ_QMV(BITS, 1, 7, 8, 2, G)
+        AQ_QMV(BITS, 1, 8, 4, 2, G), AQ_QMV(BITS, 1, 7, 4, 2, G), AQ_QMV(BITS, 1, 7, 8, 2, G),       \
+        AQ_QMV_X(BITS, 1, 1, 4, 2, G, 1), AQ_QMV_X(BITS, 1, 2, 4, 2, G, 1), AQ_QMV_X(BITS, 1, 4, 4, 2, G, 1), \
+        AQ_QMV_X(BITS, 1, 2, 8, 2, G, 1), AQ_QMV_X(BITS, 1, 4, 8, 2, G, 1), AQ_QMV_X(BITS, 1, 4, 2, 2, G, 1), \
+        AQ_QMV_X(BITS, 1, 2, 4, 4, G, 1), AQ_QMV_X(BITS, 1, 8, 4, 2, G, 1), AQ_QMV_X(BITS, 1, 4, 1, 2, G, 1), \
+        AQ_QMV_X(BITS, 1, 2, 1, 2, G, 1), AQ_QMV_X(BITS, 1, 8, 1, 2, G, 1), AQ_QMV_X(BITS, 1, 4, 4, 1, G, 1)
 
 #define AQ_QMV_MN_SET(BITS, M)                                                                     \
     AQ_QMV(BITS, M, 1, 4, 2, 0), AQ_QMV(BITS, M, 2, 4, 2, 0), AQ_QMV(BITS, M, 4, 4, 2, 0),         \
@@ -263,7 +321,7 @@ const QmvVariant* qmv_variant(int idx) {
 
 size_t qmv_lds_bytes(int idx, const QmvArgs& a) {
     const QmvVariant* v = qmv_variant(idx);
-    if (!v) return 0;
+    if (!v || v->xmode == 1) return 0;
     return (size_t)v->m * (size_t)a.K * 2;
 }
 

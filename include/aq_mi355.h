@@ -79,6 +79,19 @@ int aq_sync(aq_ctx *ctx);                                                    /* 
 int aq_timer_start(aq_ctx *ctx);
 int aq_timer_stop(aq_ctx *ctx, float *elapsed_ms); /* records, waits, reports */
 
+/* Launch batching: everything enqueued on the context between aq_capture_begin and
+ * aq_capture_end is recorded into a HIP graph instead of being executed; aq_graph_launch
+ * replays the whole batch with one submission.  Counterpart of the reference's per-step
+ * launch batch (hipLaunchKernelContext batching, go/engine/hip/hip_launch.go:240-273,
+ * cgoHIPDriver.LaunchKernelBatch go/engine/hip/hip_driver_cgo.go:1137-1190).  Only the
+ * kernel entry points (aq_qmv, aq_qmm, aq_gather_qmv, aq_dequant_f32, aq_fill_zero, aq_d2d)
+ * may be called while capturing; the pointers they were given must stay valid for replays. */
+typedef struct aq_graph aq_graph;
+int aq_capture_begin(aq_ctx *ctx);
+int aq_capture_end(aq_ctx *ctx, aq_graph **out);
+int aq_graph_launch(aq_ctx *ctx, aq_graph *graph);
+void aq_graph_destroy(aq_graph *graph);
+
 /* affine_qmv: y[M,N] = x[M,K] . dequant(w[N,K])^T, all operands device-resident.
  * Stands in for rocm_mlx_q4_projection / _batch launches
  * (go/engine/hip/hip_projection_launch.go:1306-1406, 2671-2720, 4907-5287) with the bf16

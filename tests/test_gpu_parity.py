@@ -125,32 +125,83 @@ def test_qmv_other_widths_generic_kernel(ctx, orc, bits, gs, K, N, M):
     dw.free()
 
 
+def _parse_variant(name):
+    """-> (family, bits, rows it runs in one launch, gather)"""
+    parts = dict((p.rstrip("0123456789"), int(p[len(p.rstrip("0123456789")):])) for p in name.split("_")[1:])
+    if name.startswith("qmvx_"):
+        return "mfma", parts["b"], {1: 1, 4: 8, 8: 16, 16: 32}[parts["mr"]], parts["g"]
+    return "dot2", parts["b"], parts["m"], parts["g"]
+
+
 def test_qmv_every_variant(ctx, orc):
-    """Each tuned dot2 kernel variant, forced, on a shape with a masked K tail and ragged N."""
+    """Each tuned matvec kernel variant (dot2 and MFMA), forced, on a shape with a masked K tail
+    (K = 44 group blocks) and ragged N."""
     import aq_mi355
     K, N = 2816, 150
     names = aq_mi355.variant_names(0)
     data = {}
     try:
         for idx, name in enumerate(names):
-            say("variant", idx, name)
-            parts = dict((p[0], p[1:]) for p in name.split("_")[1:])
-            bits, m, gather = int(parts["b"]), int(parts["m"]), int(parts["g"])
+            fam, bits, m, gather = _parse_variant(name)
             if gather:
-                continue
+                continue  # covered by test_gather_every_variant
+            say("variant", idx, name)
             if bits not in data:
                 words, s, b = F.synthetic_affine(N, K, bits, 64, seed=500 + bits)
-                x = F.synthetic_x(4, K, seed=600 + bits)
+                x = F.synthetic_x(32, K, seed=600 + bits)
                 data[bits] = (DeviceAffine(ctx, words, s, b), x, F.reference_f64(x, words, s, b, bits, 64, K))
             dw, x, ref = data[bits]
             ctx.force_variant(0, idx)
-            acc = run_qmv(ctx, x[:m], dw, m, K, N, 64, bits, True)
-            assert ctx.last_variant(0) == name
-            check_accumulators(acc, ref[:m], name)
+            if fam == "dot2":
+                acc = run_qmv(ctx, x[:m], dw, m, K, N, 64, bits, True)
+                assert ctx.last_variant(0) == name
+                check_accumulators(acc, ref[:m], name)
+                continue
+            # the MFMA kernels keep all of x in LDS next to their weight tiles: a row count that
+            # does not fit is refused with AQ_ERR_ARG, so walk down until one fits
+            rows, done = m, 0
+            while rows >= 1 and done < 2:
+                try:
+                    acc = run_qmv(ctx, x[:rows], dw, rows, K, N, 64, bits, True)
+                except aq_mi355.AqError as e:
+                    assert e.code == aq_mi355.AQ_ERR_ARG
+                    rows -= 3
+                    continue
+                assert ctx.last_variant(0) == name
+                check_accumulators(acc, ref[:rows], "%s rows=%d" % (name, rows))
+                done += 1
+                rows -= 3
+            assert done >= 1, name
     finally:
         ctx.force_variant(0, -1)
     for dw, _, _ in data.values():
         dw.free()
+
+
+def test_gather_every_variant(ctx, orc):
+    """Each gather-capable kernel variant, forced, against the oracle (batched x, row_base slab offset)."""
+    import aq_mi355
+    names = aq_mi355.variant_names(0)
+    E, routes, out_dim, in_dim, expert_rows, row_base = 4, 5, 40, 1408, 96, 32
+    try:
+        for idx, name in enumerate(names):
+            fam, bits, m, gather = _parse_variant(name)
+            if not gather:
+                continue
+            say("gather variant", idx, name)
+            fx = F.gather_fixture(out_dim, in_dim, 64, bits, E, expert_rows, True, routes)
+            # tame magnitudes: keep the fixture's codes, use benchmark-like scales
+            _, s, b = F.synthetic_affine(E * expert_rows, in_dim, bits, 64, seed=40 + bits)
+            fx["scales"], fx["biases"] = s, b
+            ref64, _ = orc.gather_qmv(fx["x"], fx["x_rows"], fx["packed"], s, b, fx["lhs"], fx["rhs"], routes, E, expert_rows,
+                                      row_base, out_dim, in_dim, 64, bits)
+            ctx.force_variant(0, idx)
+            acc, dw = _gather_run(ctx, fx, routes, E, expert_rows, row_base, out_dim, in_dim, 64, bits, True)
+            assert ctx.last_variant(0) == name
+            check_accumulators(acc, ref64, name)
+            dw.free()
+    finally:
+        ctx.force_variant(0, -1)
 
 
 def test_qmv_rows_match_single_row_bytes(ctx, orc):
