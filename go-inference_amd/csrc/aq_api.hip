@@ -117,11 +117,15 @@ int pick_qmv_variant(const aq_ctx* ctx, int bits, int m, bool gather, int N, int
     return best;
 }
 
-// One index space over both matvec kernel families: dot2 variants first, MFMA variants after.
-int qmv_total_variants() { return aq::qmv_variant_count() + aq::qmvx_variant_count(); }
+// One index space over the matvec kernel families: dot2 variants first, then the 32x32 MFMA
+// variants, then the block-MFMA variants.
+int qmv_total_variants() { return aq::qmv_variant_count() + aq::qmvx_variant_count() + aq::qmvb_variant_count(); }
 const aq::QmvVariant* qmv_any_variant(int idx) {
     const int nd = aq::qmv_variant_count();
-    return idx < nd ? aq::qmv_variant(idx) : aq::qmvx_variant(idx - nd);
+    const int nx = aq::qmvx_variant_count();
+    if (idx < nd) return aq::qmv_variant(idx);
+    if (idx < nd + nx) return aq::qmvx_variant(idx - nd);
+    return aq::qmvb_variant(idx - nd - nx);
 }
 
 constexpr size_t kMaxLds = 160 * 1024;
@@ -145,7 +149,43 @@ int launch_qmv_rows(aq_ctx* ctx, aq::QmvArgs a, int group_size, int bits, bool g
     const int M = a.M;
     a.gs_shift = is_pow2(group_size) ? ilog2(group_size) : 0;
     const int nd = aq::qmv_variant_count();
+    const int nx = aq::qmvx_variant_count();
     int forced = ctx->forced[0];
+    if (forced >= nd + nx || (forced < 0 && M >= 2)) {
+        // block-MFMA family: forced, or the default for 2 and more activation rows wherever the shape
+        // fits it (a single row is faster on the dot2 kernels).  Rows beyond what one launch of the
+        // family takes for this K go in further launches.
+        const size_t esize = a.out_f32 ? 4 : 2;
+        const int blk_forced = forced < 0 ? -1 : forced - nd - nx;
+        // rows the family takes in one launch for this shape: all that are left, else 16, else 4
+        auto plan_rows = [&](aq::QmvArgs& c, int rows_left, aq::BlkPlan* plan) {
+            for (int rows : {rows_left, 16, 4}) {
+                if (rows > rows_left || (rows != rows_left && forced >= 0)) continue;  // forced: whole or not at all
+                c.M = rows;
+                if (aq::qmvb_plan(c, bits, group_size, gather, ctx->cu_count, blk_forced, plan)) return rows;
+            }
+            return 0;
+        };
+        bool ok = true;
+        for (int m0 = 0; m0 < M;) {
+            aq::QmvArgs c = a;
+            c.x = a.x + (size_t)m0 * a.K;
+            c.y = static_cast<char*>(a.y) + (size_t)m0 * a.N * esize;
+            aq::BlkPlan plan;
+            const int rows = plan_rows(c, M - m0, &plan);
+            if (rows == 0) {
+                ok = false;
+                break;
+            }
+            ctx->last_variant[0] = aq::qmvb_variant(plan.idx)->name;
+            AQ_HIP(aq::qmvb_launch(plan, c, ctx->stream), "hipLaunchKernel");
+            m0 += rows;
+        }
+        if (ok) return AQ_OK;
+        if (forced >= 0)
+            return fail(AQ_ERR_ARG, "aq_qmv: forced variant %d does not fit bits=%d gather=%d rows=%d K=%d N=%d", forced,
+                        bits, (int)gather, M, a.K, a.N);
+    }
     if (forced >= nd) {
         // a forced MFMA variant: the whole call in one launch
         const aq::QmvVariant* v = aq::qmvx_variant(forced - nd);
@@ -386,10 +426,6 @@ int aq_qmv(aq_ctx* ctx, const void* x, const void* packed, const void* scales, c
     if (!aligned(x, 2) || !aligned(packed, 4) || !aligned(scales, 2) || !aligned(biases, 2) || !aligned(y, 2))
         return fail(AQ_ERR_ARG, "aq_qmv: operand pointer is not element-aligned");
     std::lock_guard<std::mutex> lk(ctx->mu);
-    if (M > aq::kQmvMaxRows && ctx->forced[0] < 0) {
-        return aq::qmm_dispatch(ctx->stream, ctx->cu_count, ctx->forced[1], &ctx->last_variant[1], x, packed, scales,
-                                biases, y, M, K, N, group_size, bits, (flags & AQ_OUT_F32) != 0, fail);
-    }
     aq::QmvArgs a{};
     a.x = static_cast<const uint16_t*>(x);
     a.w = static_cast<const uint32_t*>(packed);
@@ -401,6 +437,16 @@ int aq_qmv(aq_ctx* ctx, const void* x, const void* packed, const void* scales, c
     a.M = M;
     a.out_f32 = (flags & AQ_OUT_F32) ? 1 : 0;
     a.routes = 1;
+    if (M > aq::kQmvMaxRows && ctx->forced[0] < 0) {
+        // more rows than the dot2 kernels take: the block-MFMA family where the shape fits (it takes 4
+        // rows a launch whenever it takes any), else the matmul tiles
+        aq::BlkPlan plan;
+        aq::QmvArgs probe = a;
+        probe.M = 4;
+        if (M > 64 || !aq::qmvb_plan(probe, bits, group_size, false, ctx->cu_count, -1, &plan))
+            return aq::qmm_dispatch(ctx->stream, ctx->cu_count, ctx->forced[1], &ctx->last_variant[1], x, packed,
+                                    scales, biases, y, M, K, N, group_size, bits, (flags & AQ_OUT_F32) != 0, fail);
+    }
     return launch_qmv_rows(ctx, a, group_size, bits, false);
 }
 

@@ -39,7 +39,8 @@ struct QmvVariant {
     int depth;   // K slices in flight per wavefront
     int gather;  // 1: reads rhs/lhs on device, grid.y = routes
     int xmode;   // 0: x staged through LDS, 1: every lane reads its x chunk from global
-    int kind;    // 0: VALU dot2 kernel (aq_qmv.hip), 1: MFMA kernel (aq_qmv_mfma.hip; m = most rows it takes)
+    int kind;    // 0: VALU dot2 kernel (aq_qmv.hip), 1: MFMA kernel (aq_qmv_mfma.hip; m = most rows it takes),
+                 // 2: block-MFMA kernel (aq_qmv_blk.hip; m = most rows, depth = K pieces per wavefront)
 };
 
 int qmv_variant_count();
@@ -55,6 +56,33 @@ int qmvx_variant_count();
 const QmvVariant* qmvx_variant(int idx);
 hipError_t qmvx_launch(int idx, const QmvArgs& a, hipStream_t stream);
 size_t qmvx_lds_bytes(int idx, const QmvArgs& a);
+
+// Block-MFMA matvec kernels (aq_qmv_blk.hip; M <= 16, persistent workgroups that split K among their
+// wavefronts).  A launch needs a plan: which kernel, how many wavefronts and workgroups, LDS bytes.
+struct BlkGeom {
+    uint32_t row_bytes;     // packed bytes per weight row
+    uint32_t sb_row_bytes;  // bytes per row of scales (= biases)
+    uint32_t wstep;         // bytes between a wavefront's consecutive K pieces
+    int gpw;                // groups in one wavefront K piece
+    int hh_shift;           // log2(gpw / 4): 8-byte scale pieces per K piece
+    int rpp;                // row groups one 64-lane staging pass covers
+    int stage_bufs;         // 1, or 2 when a workgroup walks more than one batch
+    int total_rg;           // row groups (4 rows each)
+    int batch;              // row groups whose scales are staged and whose partial sums meet in LDS at once
+};
+struct BlkPlan {
+    int idx;  // variant
+    int nw;   // wavefronts per workgroup
+    int nwg;  // workgroups along x
+    size_t lds;
+    BlkGeom geom;
+};
+int qmvb_variant_count();
+const QmvVariant* qmvb_variant(int idx);
+// False when the shape does not fit these kernels (the caller then uses another family).
+// forced_idx < 0: choose the variant; otherwise plan for exactly that one.
+bool qmvb_plan(const QmvArgs& a, int bits, int group_size, bool gather, int cu_count, int forced_idx, BlkPlan* out);
+hipError_t qmvb_launch(const BlkPlan& p, const QmvArgs& a, hipStream_t stream);
 
 // Any-width (2..8 bit, codes may straddle words), any-group fallback.
 hipError_t qmv_generic_launch(const QmvArgs& a, int bits, int group_size, bool gather, hipStream_t stream);

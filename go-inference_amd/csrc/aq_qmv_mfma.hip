@@ -78,10 +78,6 @@ __global__ __launch_bounds__(KS* kWave) void qmv_mfma_kernel(const QmvArgs a) {
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
-#ifdef AQ_PHASE_TIMING
-    unsigned long long tphase[6];
-    tphase[0] = __builtin_readcyclecounter();
-#endif
     const int j = lane & 31;
     const int h = lane >> 5;
     const int K = a.K, N = a.N, M = a.M;
@@ -173,9 +169,6 @@ __global__ __launch_bounds__(KS* kWave) void qmv_mfma_kernel(const QmvArgs a) {
     uint4 ra[4], rb[4];
     load_step(ra, 0);
     load_step(rb, 1);
-#ifdef AQ_PHASE_TIMING
-    tphase[1] = __builtin_readcyclecounter();
-#endif
 
     // ---- 3. stage x into fragment order with per-(row, group block) sums; scales/biases as [pair][row] ----
     auto stage_piece = [&](int p, uint4 v) {
@@ -234,9 +227,6 @@ __global__ __launch_bounds__(KS* kWave) void qmv_mfma_kernel(const QmvArgs a) {
         }
     }
     __syncthreads();
-#ifdef AQ_PHASE_TIMING
-    tphase[2] = __builtin_readcyclecounter();
-#endif
 
     float acc[MR];
 #pragma unroll
@@ -323,20 +313,10 @@ __global__ __launch_bounds__(KS* kWave) void qmv_mfma_kernel(const QmvArgs a) {
         load_step(rb, st + 3);
     }
 
-#ifdef AQ_PHASE_TIMING
-    tphase[3] = __builtin_readcyclecounter();
-#endif
     // ---- combine the KS partial sums, store 32 consecutive outputs per row ----
 #pragma unroll
     for (int r = 0; r < MR; r++) red[(wave * MR + r) * kWave + lane] = acc[r];
     __syncthreads();
-#ifdef AQ_PHASE_TIMING
-    tphase[4] = __builtin_readcyclecounter();
-    if (blockIdx.x == 0 && blockIdx.y == 0 && lane == 0) {
-        unsigned long long* dbg = reinterpret_cast<unsigned long long*>(static_cast<char*>(a.y) + (((size_t)M * N * 4 + 255) & ~(size_t)255));
-        for (int i = 0; i < 5; i++) dbg[wave * 8 + i] = tphase[i];
-    }
-#endif
     for (int e = tid; e < MR * kWave; e += NT) {
         const int r = e / kWave, l = e & (kWave - 1);
         float tot = 0.0f;

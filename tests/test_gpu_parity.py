@@ -130,7 +130,14 @@ def _parse_variant(name):
     parts = dict((p.rstrip("0123456789"), int(p[len(p.rstrip("0123456789")):])) for p in name.split("_")[1:])
     if name.startswith("qmvx_"):
         return "mfma", parts["b"], {1: 1, 4: 8, 8: 16, 16: 32}[parts["mr"]], parts["g"]
+    if name.startswith("qmvb_"):
+        return "blk", parts["b"], parts["m"], parts["g"]
     return "dot2", parts["b"], parts["m"], parts["g"]
+
+
+def _blk_pieces(name):
+    """K pieces per wavefront of a block-MFMA variant"""
+    return int(name.split("_ki")[1].split("_")[0])
 
 
 def test_qmv_every_variant(ctx, orc):
@@ -143,8 +150,8 @@ def test_qmv_every_variant(ctx, orc):
     try:
         for idx, name in enumerate(names):
             fam, bits, m, gather = _parse_variant(name)
-            if gather:
-                continue  # covered by test_gather_every_variant
+            if gather or fam == "blk":
+                continue  # covered by test_gather_every_variant / test_qmvb_every_variant
             say("variant", idx, name)
             if bits not in data:
                 words, s, b = F.synthetic_affine(N, K, bits, 64, seed=500 + bits)
@@ -186,11 +193,109 @@ def test_gather_every_variant(ctx, orc):
     try:
         for idx, name in enumerate(names):
             fam, bits, m, gather = _parse_variant(name)
-            if not gather:
+            if not gather or fam == "blk":
                 continue
             say("gather variant", idx, name)
             fx = F.gather_fixture(out_dim, in_dim, 64, bits, E, expert_rows, True, routes)
             # tame magnitudes: keep the fixture's codes, use benchmark-like scales
+            _, s, b = F.synthetic_affine(E * expert_rows, in_dim, bits, 64, seed=40 + bits)
+            fx["scales"], fx["biases"] = s, b
+            ref64, _ = orc.gather_qmv(fx["x"], fx["x_rows"], fx["packed"], s, b, fx["lhs"], fx["rhs"], routes, E, expert_rows,
+                                      row_base, out_dim, in_dim, 64, bits)
+            ctx.force_variant(0, idx)
+            acc, dw = _gather_run(ctx, fx, routes, E, expert_rows, row_base, out_dim, in_dim, 64, bits, True)
+            assert ctx.last_variant(0) == name
+            check_accumulators(acc, ref64, name)
+            dw.free()
+    finally:
+        ctx.force_variant(0, -1)
+
+
+def test_qmvb_every_variant(ctx, orc):
+    """Each block-MFMA matvec variant, forced: K = 3 (4 bit) or 4 (8 bit) wavefronts x its pieces per wavefront, a row count
+    that leaves the last round of workgroups ragged, the most activation rows it takes and one fewer."""
+    import aq_mi355
+    names = aq_mi355.variant_names(0)
+    N = 4 * 523
+    data = {}
+    try:
+        for idx, name in enumerate(names):
+            fam, bits, m, gather = _parse_variant(name)
+            if fam != "blk" or gather:
+                continue
+            ki = _blk_pieces(name)
+            K = 1536 * ki if bits == 4 else 1024 * ki
+            say("variant", idx, name, "K", K)
+            if (bits, K) not in data:
+                words, s, b = F.synthetic_affine(N, K, bits, 64, seed=510 + bits + ki)
+                x = F.synthetic_x(16, K, seed=610 + bits + ki)
+                data[(bits, K)] = (DeviceAffine(ctx, words, s, b), x, F.reference_f64(x, words, s, b, bits, 64, K))
+            dw, x, ref = data[(bits, K)]
+            ctx.force_variant(0, idx)
+            for rows in sorted({m, max(1, m - 1)}):
+                acc = run_qmv(ctx, x[:rows], dw, rows, K, N, 64, bits, True)
+                assert ctx.last_variant(0) == name
+                check_accumulators(acc, ref[:rows], "%s rows=%d" % (name, rows))
+            # a shape outside the family is refused, not silently rerouted
+            with pytest.raises(aq_mi355.AqError) as ei:
+                run_qmv(ctx, x[:1, :K - 64], dw, 1, K - 64, N, 64, bits, True)
+            assert ei.value.code == aq_mi355.AQ_ERR_ARG
+    finally:
+        ctx.force_variant(0, -1)
+    for dw, _, _ in data.values():
+        dw.free()
+
+
+@pytest.mark.parametrize("M,K,N,gs,bits", [
+    (2, 4096, 1024, 64, 4), (5, 4096, 1024, 64, 4), (16, 2048, 516, 64, 4), (24, 1024, 256, 64, 4),
+    (3, 2048, 512, 32, 4), (4, 2048, 512, 128, 4), (7, 1024, 512, 64, 8), (2, 2048, 256, 32, 8),
+    (4, 14336, 256, 64, 4), (9, 14336, 64, 64, 4)])
+def test_qmv_small_m_default_path(ctx, orc, M, K, N, gs, bits):
+    """2..24 activation rows through aq_qmv with nothing forced: fp32 outputs against the float64
+    reference, bf16 stores against its rounding, over the group sizes and widths the block-MFMA
+    family takes (and shapes that need several launches, or fall through to another family)."""
+    say("small-M default", M, K, N, gs, bits)
+    words, s, b = F.synthetic_affine(N, K, bits, gs, seed=77 + M)
+    x = F.synthetic_x(M, K, seed=78 + M)
+    ref = F.reference_f64(x, words, s, b, bits, gs, K)
+    dw = DeviceAffine(ctx, words, s, b)
+    acc = run_qmv(ctx, x, dw, M, K, N, gs, bits, True)
+    say("  ran on", ctx.last_variant(0), ctx.last_variant(1))
+    check_accumulators(acc, ref, "small-M f32")
+    out = run_qmv(ctx, x, dw, M, K, N, gs, bits, False)
+    check_bf16_store(out, ref, "small-M bf16")
+    dw.free()
+
+
+def test_qmv_block_family_many_batches(ctx, orc):
+    """A matrix tall enough that every workgroup of the block-MFMA kernel walks more row groups than one
+    batch of staged scales holds (K = 512: one wavefront per workgroup, 4096 workgroups)."""
+    M, K, N = 3, 512, 4 * 4096 * 19 + 8
+    say("many batches", M, K, N)
+    words, s, b = F.synthetic_affine(N, K, 4, 64, seed=5)
+    x = F.synthetic_x(M, K, seed=6)
+    ref = F.reference_f64(x, words, s, b, 4, 64, K)
+    dw = DeviceAffine(ctx, words, s, b)
+    acc = run_qmv(ctx, x, dw, M, K, N, 64, 4, True)
+    assert ctx.last_variant(0).startswith("qmvb_"), ctx.last_variant(0)
+    check_accumulators(acc, ref, "many batches")
+    dw.free()
+
+
+def test_qmvb_gather_every_variant(ctx, orc):
+    """Each gather-capable block-MFMA variant, forced, against the oracle (batched x, row_base slab
+    offset)."""
+    import aq_mi355
+    names = aq_mi355.variant_names(0)
+    E, routes, out_dim, expert_rows, row_base = 4, 6, 40, 96, 32
+    try:
+        for idx, name in enumerate(names):
+            fam, bits, m, gather = _parse_variant(name)
+            if fam != "blk" or not gather:
+                continue
+            in_dim = (512 if bits == 4 else 256) * _blk_pieces(name) * 2
+            say("gather variant", idx, name, "K", in_dim)
+            fx = F.gather_fixture(out_dim, in_dim, 64, bits, E, expert_rows, True, routes)
             _, s, b = F.synthetic_affine(E * expert_rows, in_dim, bits, 64, seed=40 + bits)
             fx["scales"], fx["biases"] = s, b
             ref64, _ = orc.gather_qmv(fx["x"], fx["x_rows"], fx["packed"], s, b, fx["lhs"], fx["rhs"], routes, E, expert_rows,
