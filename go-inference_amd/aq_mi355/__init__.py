@@ -53,6 +53,7 @@ PROTOTYPES = {
     "aq_graph_destroy": (None, [_vp]),
     "aq_qmv": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _u]),
     "aq_qmm": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _u]),
+    "aq_reserve_workspace": (_i, [_vp, _i, _i]),
     "aq_gather_qmv": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _u]),
     "aq_dequant_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _c.c_int64, _i, _i, _i]),
     "aq_matvec_host": (_i, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _i, _i, _i, _i, _vp, _sz]),
@@ -213,6 +214,9 @@ class Context:
     def qmm(self, x, w, s, b, y, M, K, N, group_size=64, bits=4, flags=0):
         self._check(self.lib.aq_qmm(self.handle, _ptr(x), _ptr(w), _ptr(s), _ptr(b), _ptr(y), M, K, N, group_size,
                                     bits, flags))
+
+    def reserve_workspace(self, M, K):
+        self._check(self.lib.aq_reserve_workspace(self.handle, M, K))
 
     def gather_qmv(self, x, w, s, b, lhs, rhs, y, routes, x_rows, K, N, num_experts, expert_rows, row_base=0,
                    group_size=64, bits=4, flags=0):

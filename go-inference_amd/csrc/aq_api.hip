@@ -60,6 +60,7 @@ struct aq_ctx {
     int forced[2] = {-1, -1};
     const char* last_variant[2] = {"", ""};
     int cu_count = 0;
+    aq::Workspace ws;  // scratch of the matmul path (aq_qmm.h)
     char name[256] = {0};
 };
 
@@ -271,6 +272,7 @@ void aq_destroy(aq_ctx* ctx) {
         (void)hipStreamSynchronize(ctx->own_stream);
         (void)hipStreamDestroy(ctx->own_stream);
     }
+    if (ctx->ws.ptr) (void)hipFree(ctx->ws.ptr);
     if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
     if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
     delete ctx;
@@ -444,7 +446,7 @@ int aq_qmv(aq_ctx* ctx, const void* x, const void* packed, const void* scales, c
         aq::QmvArgs probe = a;
         probe.M = 4;
         if (M > 64 || !aq::qmvb_plan(probe, bits, group_size, false, ctx->cu_count, -1, &plan))
-            return aq::qmm_dispatch(ctx->stream, ctx->cu_count, ctx->forced[1], &ctx->last_variant[1], x, packed,
+            return aq::qmm_dispatch(ctx->stream, &ctx->ws, ctx->cu_count, ctx->forced[1], &ctx->last_variant[1], x, packed,
                                     scales, biases, y, M, K, N, group_size, bits, (flags & AQ_OUT_F32) != 0, fail);
     }
     return launch_qmv_rows(ctx, a, group_size, bits, false);
@@ -460,8 +462,17 @@ int aq_qmm(aq_ctx* ctx, const void* x, const void* packed, const void* scales, c
     if (!aligned(x, 2) || !aligned(packed, 4) || !aligned(scales, 2) || !aligned(biases, 2) || !aligned(y, 2))
         return fail(AQ_ERR_ARG, "aq_qmm: operand pointer is not element-aligned");
     std::lock_guard<std::mutex> lk(ctx->mu);
-    return aq::qmm_dispatch(ctx->stream, ctx->cu_count, ctx->forced[1], &ctx->last_variant[1], x, packed, scales,
+    return aq::qmm_dispatch(ctx->stream, &ctx->ws, ctx->cu_count, ctx->forced[1], &ctx->last_variant[1], x, packed, scales,
                             biases, y, M, K, N, group_size, bits, (flags & AQ_OUT_F32) != 0, fail);
+}
+
+int aq_reserve_workspace(aq_ctx* ctx, int M, int K) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_reserve_workspace: ctx is null");
+    if (M < 0 || K < 0) return fail(AQ_ERR_SHAPE, "aq_reserve_workspace: M and K must be non-negative");
+    if (M == 0 || K == 0) return AQ_OK;
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    return aq::qmm_reserve(ctx->stream, &ctx->ws, M, K, fail);
 }
 
 int aq_gather_qmv(aq_ctx* ctx, const void* x, const void* packed, const void* scales, const void* biases,
@@ -618,7 +629,7 @@ int aq_proj_quant_matmul_host(aq_ctx* ctx, float* out, const float* x, size_t x_
 
 int aq_variant_count(int op) {
     if (op == 0) return qmv_total_variants();
-    if (op == 1) return aq::qmm_variant_count();
+    if (op == 1) return aq::qmm_variant_count() + aq::qmmt_variant_count();
     return 0;
 }
 
@@ -627,7 +638,12 @@ const char* aq_variant_name(int op, int variant) {
         const aq::QmvVariant* v = (variant >= 0 && variant < qmv_total_variants()) ? qmv_any_variant(variant) : nullptr;
         return v ? v->name : "";
     }
-    if (op == 1) return aq::qmm_variant_name(variant);
+    if (op == 1) {
+        const int nd = aq::qmm_variant_count();
+        if (variant < nd) return aq::qmm_variant_name(variant);
+        const aq::QmmVariant* v = aq::qmmt_variant(variant - nd);
+        return v ? v->name : "";
+    }
     return "";
 }
 

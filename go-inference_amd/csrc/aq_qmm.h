@@ -27,6 +27,34 @@ struct QmmVariant {
     int wm, wn;  // wavefronts per workgroup along M and N
 };
 
+// Operands of the LDS-staged tile kernels (aq_qmm_tile.hip): x has been rewritten by their pass over x.
+struct QmmTileArgs {
+    const uint16_t* xf;  // activations in A-fragment order, rows padded to a multiple of 32
+    const uint16_t* xs;  // per 64-code block sums of x as (hi, lo) bf16, four blocks per 16 bytes
+    const uint32_t* w;
+    const uint16_t* s;
+    const uint16_t* b;
+    void* y;
+    int M, K, N;
+    int gs_blocks;
+    int out_f32;
+    int mblks;             // ceil(M / 32)
+    int tiles_m, tiles_n;  // workgroup tiles along M and N
+};
+
+int qmmt_variant_count();
+const QmmVariant* qmmt_variant(int idx);
+// Device bytes the tile kernels need beside their operands for an M x K activation matrix.
+size_t qmmt_workspace_bytes(int M, int K);
+// Pass over x + tile kernel `idx`; `workspace` holds at least qmmt_workspace_bytes(M, K).
+hipError_t qmmt_launch(int idx, const QmmArgs& a, void* workspace, hipStream_t stream);
+
+// Scratch memory a context lends to the matmul path; grown on demand, never while a capture is open.
+struct Workspace {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+};
+
 int qmm_variant_count();
 const char* qmm_variant_name(int idx);
 const QmmVariant* qmm_variant(int idx);
@@ -35,9 +63,13 @@ hipError_t fill_zero_launch(void* p, size_t bytes, hipStream_t stream);
 
 typedef int (*FailFn)(int code, const char* fmt, ...);
 
+// Sizes ws for activations of M x K ahead of time (not during capture).
+int qmm_reserve(hipStream_t stream, Workspace* ws, int M, int K, FailFn fail);
+
 // Validated-shape dispatch used by aq_qmm and by aq_qmv for M > kQmvMaxRows.
 // Returns an AQ_* / hipError_t code through `fail`.
-int qmm_dispatch(hipStream_t stream, int cu_count, int forced, const char** last_variant, const void* x,
+// `forced` indexes the direct-load variants first, then the tile variants.
+int qmm_dispatch(hipStream_t stream, Workspace* ws, int cu_count, int forced, const char** last_variant, const void* x,
                  const void* packed, const void* scales, const void* biases, void* y, int M, int K, int N,
                  int group_size, int bits, bool out_f32, FailFn fail);
 

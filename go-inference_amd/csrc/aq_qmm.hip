@@ -386,7 +386,40 @@ static int find_qmm(int bits, int mb, int nb, int wm, int wn) {
     return -1;
 }
 
-int qmm_dispatch(hipStream_t stream, int cu_count, int forced, const char** last_variant, const void* x,
+// Makes ws hold at least `need` bytes.  Growing frees the old block, so everything queued on the stream
+// is drained first; a stream that is being captured cannot be drained.
+static int grow_workspace(Workspace* ws, size_t need, hipStream_t stream, FailFn fail) {
+    if (ws->bytes >= need) return AQ_OK;
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (stream != nullptr && hipStreamIsCapturing(stream, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone)
+        return fail(AQ_ERR_UNSUPPORTED,
+                    "aq_qmm: the matmul workspace must grow to %zu bytes, which cannot happen during stream capture; "
+                    "call aq_reserve_workspace before capturing", need);
+    hipError_t rc = hipStreamSynchronize(stream);
+    if (rc != hipSuccess) return fail((int)rc, "rocm.hip.hipStreamSynchronize: HIP returned %d", (int)rc);
+    if (ws->ptr) (void)hipFree(ws->ptr);
+    ws->ptr = nullptr;
+    ws->bytes = 0;
+    const size_t want = need + need / 4;  // headroom: prompts grow a little from call to call
+    rc = hipMalloc(&ws->ptr, want);
+    if (rc != hipSuccess) return fail(AQ_ERR_NOMEM, "aq_qmm: cannot allocate a %zu-byte workspace (HIP %d)", want, (int)rc);
+    ws->bytes = want;
+    return AQ_OK;
+}
+
+int qmm_reserve(hipStream_t stream, Workspace* ws, int M, int K, FailFn fail) {
+    return grow_workspace(ws, qmmt_workspace_bytes(M, K), stream, fail);
+}
+
+static int find_qmmt(int bits, int mb, int nb, int wm, int wn) {
+    for (int i = 0; i < qmmt_variant_count(); i++) {
+        const QmmVariant* v = qmmt_variant(i);
+        if (v->bits == bits && v->mb == mb && v->nb == nb && v->wm == wm && v->wn == wn) return i;
+    }
+    return -1;
+}
+
+int qmm_dispatch(hipStream_t stream, Workspace* ws, int cu_count, int forced, const char** last_variant, const void* x,
                  const void* packed, const void* scales, const void* biases, void* y, int M, int K, int N,
                  int group_size, int bits, bool out_f32, FailFn fail) {
     (void)cu_count;
@@ -422,6 +455,24 @@ int qmm_dispatch(hipStream_t stream, int cu_count, int forced, const char** last
     a.gs_blocks = group_size / 64;
     a.out_f32 = out_f32 ? 1 : 0;
     int idx = forced;
+    const int n_direct = qmm_variant_count();
+    int tile_idx = -1;
+    if (idx >= n_direct) {
+        tile_idx = idx - n_direct;
+        const QmmVariant* v = qmmt_variant(tile_idx);
+        if (!v || v->bits != bits) return fail(AQ_ERR_ARG, "aq_qmm: forced variant %d does not fit bits=%d", idx, bits);
+    } else if (idx < 0 && M >= 64) {
+        // prefill sizes: the LDS-staged 128 x 128 tiles (four 64 x 64 wavefront tiles, two workgroups a CU);
+        // the 128 x 64 wavefront tiles need more registers than two wavefronts a SIMD leave and measure slower
+        tile_idx = find_qmmt(bits, 2, 2, 2, 2);
+    }
+    if (tile_idx >= 0) {
+        if (int rc = grow_workspace(ws, qmmt_workspace_bytes(M, K), stream, fail)) return rc;
+        *last_variant = qmmt_variant(tile_idx)->name;
+        hipError_t rc = qmmt_launch(tile_idx, a, ws->ptr, stream);
+        if (rc != hipSuccess) return fail((int)rc, "rocm.hip.hipLaunchKernel: HIP returned %d (%s)", (int)rc, hipGetErrorString(rc));
+        return AQ_OK;
+    }
     if (idx >= 0) {
         const QmmVariant* v = qmm_variant(idx);
         if (!v || v->bits != bits) return fail(AQ_ERR_ARG, "aq_qmm: forced variant %d does not fit bits=%d", idx, bits);

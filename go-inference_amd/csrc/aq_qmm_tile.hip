@@ -1,0 +1,493 @@
+// affine_qmm for gfx950, prefill sizes: both operands staged through LDS in MFMA-fragment order.
+//
+// Replaces rocm_mlx_q4_projection_batch* (go/engine/hip/kernels/quant/affine_projection_tuned.hipinc:166-1109)
+// with the semantics of MLX affine_qmm_t (go/engine/metal/quant_seam_backend.go:77-109).  The
+// arithmetic is that of aq_qmm.hip: the matrix cores multiply the activations with the exact codes
+// (4 bit: 16 + c, 8 bit: c, as bf16), every 64-code block of K ends with out += scale * P in fp32,
+// and one extra MFMA per four blocks adds (bias - off*scale) * sum(x) with the sums split into two
+// bf16 values.  What changes is how the operands reach the matrix cores:
+//   * a small pass over x (qmm_prep_kernel) writes the activations once in A-fragment order
+//     (1 KiB per 32 rows x 16 K, lane-major, K already in the order the unpacker emits codes) and
+//     the per-block sums as (hi, lo) bf16 pairs.  The main kernel then copies A tiles global -> LDS
+//     with global_load_lds_dwordx4: no registers, no VALU work, no LDS write instructions;
+//   * the packed weights of a tile are fetched once per workgroup (not once per wavefront), unpacked
+//     cooperatively into B fragments in LDS, and read back by every wavefront with ds_read_b128;
+//   * wavefront tiles are 128 x 64 (or 64 x 64): LDS read bandwidth (128 B/clk/CU), not the matrix
+//     pipe, bounds smaller ones;
+//   * every global load has the MFMAs of one 64-code block to arrive: three LDS stages of A (the copy
+//     of block g+2 starts while block g+1 is still to be read), two of B fed from packed words that
+//     wait in registers; one barrier per block;
+//   * tiles are numbered so that the workgroups of one XCD (every 8th workgroup) walk one band of
+//     rows of x across N: the band's A tile stays in that XCD's L2 while the weights stream by.
+#include "aq_device.h"
+#include "aq_kernels.h"
+#include "aq_qmm.h"
+
+#include "../../include/aq_mi355.h"
+
+#include <type_traits>
+
+namespace aq {
+
+namespace {
+
+constexpr uint32_t kMask16 = 0x00780078u;   // a nibble moved to mantissa bits [6:3]
+constexpr uint32_t kMagic16 = 0x41804180u;  // bf16 16.0 in both halves: 16 + code, exact
+
+// 8 codes of one packed word -> 8 bf16 (16 + c) in slot order (c0,c4)(c1,c5)(c2,c6)(c3,c7)
+__device__ __forceinline__ uint4 unpack_word4(uint32_t w, uint32_t mask_s, uint32_t magic_v) {
+    uint4 v;
+    v.x = and_or(w << 3, mask_s, magic_v);
+    v.y = and_or(w >> 1, mask_s, magic_v);
+    v.z = and_or(w >> 5, mask_s, magic_v);
+    v.w = and_or(w >> 9, mask_s, magic_v);
+    return v;
+}
+
+__device__ __forceinline__ uint4 unpack_words8(uint32_t w0, uint32_t w1) {
+    uint32_t p[4];
+    unpack8_word(w0, p);
+    unpack8_word(w1, p + 2);
+    return make_uint4(p[0], p[1], p[2], p[3]);
+}
+
+__device__ __forceinline__ uint32_t dup16(uint32_t h) { return (h & 0xffffu) | (h << 16); }
+
+typedef const __attribute__((address_space(1))) void* gvoid_t;
+typedef __attribute__((address_space(3))) void* lvoid_t;
+
+}  // namespace
+
+// ---- pass over x ----------------------------------------------------------------------------
+// xf: [mblks][K/16][64 lanes][8] bf16.  Lane (j, h) of fragment (mblk, 4g + t) holds
+//     x[32 mblk + j][64 g + 16 t + 8 h + order(0..7)], order = 0,4,1,5,2,6,3,7 at 4 bit, natural at 8 bit.
+// xs: [mblks * 32][ceil(G/4)][4 blocks][hi, lo] bf16: sum of x over each 64-code block, hi + lo.
+// Rows past M are written as zeros.
+template <int BITS>
+__global__ __launch_bounds__(256) void qmm_prep_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ xf,
+                                                        uint16_t* __restrict__ xs, int M, int K, int mblks) {
+    const int G = K / 64;
+    const int G4 = (G + 3) / 4;
+    const int64_t p = (int64_t)blockIdx.x * 256 + threadIdx.x;  // ((row * G) + g) * 8 + c8
+    const int64_t total = (int64_t)mblks * 32 * G * 8;
+    if (p >= total) return;  // whole groups of 8 lanes leave together
+    const int c8 = (int)(p & 7);
+    const int64_t rg = p >> 3;
+    const int g = (int)(rg % G);
+    const int row = (int)(rg / G);
+    uint4 v = {0u, 0u, 0u, 0u};
+    if (row < M) v = *reinterpret_cast<const uint4*>(x + (int64_t)row * K + g * 64 + c8 * 8);
+    float sx = 0.0f;
+    sx = dot2_bf16(v.x, 0x3F803F80u, sx);
+    sx = dot2_bf16(v.y, 0x3F803F80u, sx);
+    sx = dot2_bf16(v.z, 0x3F803F80u, sx);
+    sx = dot2_bf16(v.w, 0x3F803F80u, sx);
+    // the 8 lanes that hold one row's block: xor 1, xor 2, mirror within 8
+    sx += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sx), 0xB1, 0xF, 0xF, true));
+    sx += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sx), 0x4E, 0xF, 0xF, true));
+    sx += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sx), 0x141, 0xF, 0xF, true));
+    if (c8 == 0) {
+        const uint32_t hi = f32_to_bf16_bits(sx);
+        const uint32_t lo = f32_to_bf16_bits(sx - bf16_bits_to_f32(hi));
+        uint32_t* dst = reinterpret_cast<uint32_t*>(xs) + ((int64_t)row * G4 + (g >> 2)) * 4;
+        dst[g & 3] = hi | (lo << 16);
+        if (g == G - 1)
+            for (int q = (g & 3) + 1; q < 4; q++) dst[q] = 0u;
+    }
+    if constexpr (BITS == 4) {
+        uint4 o;
+        o.x = (v.x & 0xffffu) | (v.z << 16);
+        o.y = (v.x >> 16) | (v.z & 0xffff0000u);
+        o.z = (v.y & 0xffffu) | (v.w << 16);
+        o.w = (v.y >> 16) | (v.w & 0xffff0000u);
+        v = o;
+    }
+    const int t = c8 >> 1, h = c8 & 1;
+    const int64_t frag = (int64_t)(row >> 5) * (K / 16) + g * 4 + t;
+    *reinterpret_cast<uint4*>(xf + (frag * 64 + h * 32 + (row & 31)) * 8) = v;
+}
+
+// ---- main kernel ----------------------------------------------------------------------------
+// Wavefront tiles of at most 64 x 64 keep under 256 registers, so two wavefronts share a SIMD.
+template <int BITS, int MB, int NB, int WM, int WN>
+__global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTileArgs a) {
+    constexpr int BM = WM * MB * 32;
+    constexpr int BN = WN * NB * 32;
+    constexpr int NWAVE = WM * WN;
+    constexpr int NT = NWAVE * kWave;
+    constexpr int A_STAGE = (BM / 32) * 4096;
+    constexpr int B_STAGE = (BN / 32) * 4096;
+    constexpr int A_BLOCKS = (BM / 32) * 4;        // 1 KiB fragments of A per stage
+    constexpr int WPB = BITS == 4 ? 8 : 16;        // packed words per row and 64-code block
+    constexpr int W_PIECES = BN * WPB / 4;         // 16-byte pieces of packed weights per stage
+    constexpr int WPT = W_PIECES / NT;             // per thread
+    constexpr float OFFSET = BITS == 4 ? 16.0f : 0.0f;
+    static_assert(A_BLOCKS % NWAVE == 0, "A fragments must divide among the wavefronts");
+    static_assert(W_PIECES % NT == 0 && WPT >= 1, "weight pieces must divide among the threads");
+
+
+    extern __shared__ __align__(16) uint8_t lds[];
+    uint8_t* const abuf = lds;                // [3][A_STAGE]
+    uint8_t* const bbuf = lds + 3 * A_STAGE;  // [2][B_STAGE]
+
+    // tile of this workgroup: workgroups are dealt to the 8 XCDs round-robin, so every 8th one
+    // shares an L2; give each XCD a contiguous run of tiles in row-band-major order
+    const int T = a.tiles_m * a.tiles_n;
+    const int per_xcd = (T + 7) / 8;
+    const int id = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    if (id >= T) return;
+    const int tm = id / a.tiles_n;
+    const int tn = id - tm * a.tiles_n;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int wave_m = wave / WN;
+    const int wave_n = wave % WN;
+    const int j = lane & 31;
+    const int h = lane >> 5;
+
+    const int K = a.K, M = a.M, N = a.N;
+    const int G = K / 64;
+    const int G4 = (G + 3) / 4;
+    const int ksteps = K / 16;
+    const int sb_per_row = G / a.gs_blocks;
+    const int64_t words_per_row = (int64_t)K * BITS / 32;
+    const int m0 = tm * BM;
+    const int n0 = tn * BN;
+
+    // A: this wavefront copies fragments wave, wave + NWAVE, ... of every stage
+    auto issue_a = [&](int g, int stage) {
+        uint8_t* dst = abuf + stage * A_STAGE;
+#pragma unroll
+        for (int q = 0; q < A_BLOCKS / NWAVE; q++) {
+            const int blk = wave + q * NWAVE;
+            int mblk = m0 / 32 + (blk >> 2);
+            mblk = mblk < a.mblks ? mblk : a.mblks - 1;  // past the end: any valid rows, never stored
+            const uint16_t* src = a.xf + ((int64_t)mblk * ksteps + g * 4 + (blk & 3)) * 512 + lane * 8;
+            __builtin_amdgcn_global_load_lds((gvoid_t)src, (lvoid_t)(dst + blk * 1024), 16, 0, 0);
+        }
+    };
+
+    // B: packed pieces of the tile's rows, WPT per thread
+    const uint32_t* wsrc[WPT];
+    uint32_t bdst[WPT];  // LDS byte offset of the first fragment piece this thread writes
+#pragma unroll
+    for (int i = 0; i < WPT; i++) {
+        const int p = tid + i * NT;
+        if constexpr (BITS == 4) {
+            const int r = p >> 1, half = p & 1;  // words 4*half .. 4*half+3 = k steps 2*half, 2*half+1
+            const int n = min(n0 + r, N - 1);
+            wsrc[i] = a.w + (int64_t)n * words_per_row + half * 4;
+            bdst[i] = (uint32_t)(((r >> 5) * 4 + 2 * half) * 1024 + (r & 31) * 16);
+        } else {
+            const int r = p >> 2, q = p & 3;  // words 4q .. 4q+3 = k step q
+            const int n = min(n0 + r, N - 1);
+            wsrc[i] = a.w + (int64_t)n * words_per_row + q * 4;
+            bdst[i] = (uint32_t)(((r >> 5) * 4 + q) * 1024 + (r & 31) * 16);
+        }
+    }
+    uint4 w_even[WPT], w_odd[WPT];  // packed words in flight: block b waits in w_even when b is even
+    auto load_w = [&](int g, uint4 (&dst)[WPT]) {
+#pragma unroll
+        for (int i = 0; i < WPT; i++) dst[i] = *reinterpret_cast<const uint4*>(wsrc[i] + (int64_t)g * WPB);
+    };
+    const uint32_t mask_s = opaque_s(kMask16);
+    const uint32_t magic_v = opaque_v(kMagic16);
+    auto store_b = [&](int g, const uint4 (&wreg)[WPT]) {
+        uint8_t* dst = bbuf + (g & 1) * B_STAGE;
+#pragma unroll
+        for (int i = 0; i < WPT; i++) {
+            if constexpr (BITS == 4) {
+                // word w of the piece -> k step 2*half + w/2, lane half w & 1
+                *reinterpret_cast<uint4*>(dst + bdst[i]) = unpack_word4(wreg[i].x, mask_s, magic_v);
+                *reinterpret_cast<uint4*>(dst + bdst[i] + 512) = unpack_word4(wreg[i].y, mask_s, magic_v);
+                *reinterpret_cast<uint4*>(dst + bdst[i] + 1024) = unpack_word4(wreg[i].z, mask_s, magic_v);
+                *reinterpret_cast<uint4*>(dst + bdst[i] + 1536) = unpack_word4(wreg[i].w, mask_s, magic_v);
+            } else {
+                *reinterpret_cast<uint4*>(dst + bdst[i]) = unpack_words8(wreg[i].x, wreg[i].y);
+                *reinterpret_cast<uint4*>(dst + bdst[i] + 512) = unpack_words8(wreg[i].z, wreg[i].w);
+            }
+        }
+    };
+
+    // Scales, biases and block sums are fetched per QUAD of four 64-code blocks, one quad ahead: the bf16
+    // bits of the quad's four blocks in two words per array and column tile (8-byte loads where the
+    // rows allow it), and 16 bytes of (hi, lo) sums per row tile.
+    const uint16_t* srow[NB];
+    const uint16_t* brow[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) {
+        const int n = min(n0 + (wave_n * NB + nb) * 32 + j, N - 1);
+        srow[nb] = a.s + (int64_t)n * sb_per_row;
+        brow[nb] = a.b + (int64_t)n * sb_per_row;
+    }
+    const bool quad_loads = a.gs_blocks == 1 && (G & 3) == 0 && (((uintptr_t)a.s | (uintptr_t)a.b) & 7) == 0;
+    uint2 s_cur[NB], b_cur[NB], s_nxt[NB], b_nxt[NB];
+    auto load_quad = [&](int quad, uint2 (&sd)[NB], uint2 (&bd)[NB]) {
+        if (quad_loads) {
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) {
+                sd[nb] = *reinterpret_cast<const uint2*>(srow[nb] + quad * 4);
+                bd[nb] = *reinterpret_cast<const uint2*>(brow[nb] + quad * 4);
+            }
+        } else {
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) {
+                uint32_t sv[4], bv[4];
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    int idx = (quad * 4 + k) / a.gs_blocks;
+                    idx = idx < sb_per_row ? idx : sb_per_row - 1;  // blocks past K: never used
+                    sv[k] = srow[nb][idx];
+                    bv[k] = brow[nb][idx];
+                }
+                sd[nb] = make_uint2(sv[0] | (sv[1] << 16), sv[2] | (sv[3] << 16));
+                bd[nb] = make_uint2(bv[0] | (bv[1] << 16), bv[2] | (bv[3] << 16));
+            }
+        }
+    };
+    // bf16 bits of block q (0..3) of a quad, as the high half of a word (= the fp32 value)
+    auto quad_hi = [](const uint2& v, int q) {
+        const uint32_t w = q < 2 ? v.x : v.y;
+        return (q & 1) ? (w & 0xffff0000u) : (w << 16);
+    };
+    const uint4* xsrow[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) {
+        int row = m0 + (wave_m * MB + mb) * 32 + j;
+        row = row < a.mblks * 32 ? row : a.mblks * 32 - 1;
+        xsrow[mb] = reinterpret_cast<const uint4*>(a.xs) + (int64_t)row * G4;
+    }
+    uint4 xs_cur[MB], xs_nxt[MB];
+    auto load_xs = [&](int quad, uint4 (&dst)[MB]) {
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) dst[mb] = xsrow[mb][quad];
+    };
+
+    f32x16_t out[MB][NB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) out[mb][nb][r] = 0.0f;
+
+    // One 64-code block; Q = g & 3 is static so that everything indexed by it stays in fixed
+    // registers.  The packed words alternate between two register sets, and nothing that is still in
+    // flight is ever copied (a copy would wait for the newest load).  Iteration g requests the packed
+    // words of block g+2 before its MFMAs (at Q = 1 also the next quad's scales, biases and sums), and
+    // the A copies of block g+2 after its LDS writes: the compiler drains every outstanding copy into
+    // LDS before an LDS write it cannot tell apart from the copy's target, so a copy issued earlier
+    // would be waited for in the same iteration.  Each request has one block of MFMAs to arrive.  Past
+    // the end of K the last block is requested again.
+    const int glast = G - 1;
+    int sa = 0;  // LDS stage of A that holds block g
+    auto iteration = [&](auto q_tag, int g, uint4 (&w_load)[WPT], const uint4 (&w_use)[WPT]) {
+        constexpr int Q = decltype(q_tag)::value;
+        const bool more = g + 1 < G;
+        load_w(g + 2 < G ? g + 2 : glast, w_load);
+        if constexpr (Q == 1) {
+            const int nq = (g >> 2) + 1 < G4 ? (g >> 2) + 1 : G4 - 1;
+            load_quad(nq, s_nxt, b_nxt);
+            load_xs(nq, xs_nxt);
+        }
+
+        const uint8_t* ab = abuf + sa * A_STAGE + (wave_m * MB) * 4096 + lane * 16;
+        const uint8_t* bb = bbuf + (g & 1) * B_STAGE + (wave_n * NB) * 4096 + lane * 16;
+        bf16x8_t bfrag[NB][4];
+        float sc[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+#pragma unroll
+            for (int t = 0; t < 4; t++) bfrag[nb][t] = *reinterpret_cast<const bf16x8_t*>(bb + (nb * 4 + t) * 1024);
+            sc[nb] = __uint_as_float(quad_hi(s_cur[nb], Q));
+        }
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) {
+            bf16x8_t afrag[4];
+#pragma unroll
+            for (int t = 0; t < 4; t++) afrag[t] = *reinterpret_cast<const bf16x8_t*>(ab + (mb * 4 + t) * 1024);
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) {
+                f32x16_t p = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int t = 0; t < 4; t++) p = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag[t], bfrag[nb][t], p, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 16; r++) out[mb][nb][r] = __fmaf_rn(sc[nb], p[r], out[mb][nb][r]);
+            }
+        }
+
+        if (Q == 3 || !more) {
+            // affine terms of the quad's blocks 0..Q in one MFMA: k-slots (2q, 2q+1) carry
+            // (Sx_hi, Sx_lo) of block q on the A side; lanes h=0 pair them with bias, lanes h=1 with
+            // -off*scale; blocks past Q (only at the end of K) contribute zeros
+            bf16x8_t bbf[NB];
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) {
+                uint32_t v[4];
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    if (q <= Q) {
+                        const uint32_t neg = __float_as_uint(__uint_as_float(quad_hi(s_cur[nb], q)) * -OFFSET) >> 16;
+                        const uint32_t bia = quad_hi(b_cur[nb], q) >> 16;
+                        v[q] = dup16(h ? neg : bia);
+                    } else {
+                        v[q] = 0u;
+                    }
+                }
+                const uint4 u = {v[0], v[1], v[2], v[3]};
+                bbf[nb] = __builtin_bit_cast(bf16x8_t, u);
+            }
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++) {
+                const bf16x8_t aa = __builtin_bit_cast(bf16x8_t, xs_cur[mb]);
+#pragma unroll
+                for (int nb = 0; nb < NB; nb++)
+                    out[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aa, bbf[nb], out[mb][nb], 0, 0, 0);
+            }
+        }
+
+        // block g+1: its packed words have waited in registers; expand them into the other B stage
+        store_b(g + 1, w_use);
+        // the A copies of block g+1 (requested at the end of the last iteration) have landed, and so
+        // has everything requested above
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        issue_a(g + 2 < G ? g + 2 : glast, sa == 0 ? 2 : sa - 1);  // stage (sa + 2) % 3: read last in iteration g-1
+        sa = sa == 2 ? 0 : sa + 1;
+        if constexpr (Q == 3) {
+            // the next quad's values arrived two blocks ago
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) {
+                s_cur[nb] = s_nxt[nb];
+                b_cur[nb] = b_nxt[nb];
+            }
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++) xs_cur[mb] = xs_nxt[mb];
+        }
+        __syncthreads();
+    };
+
+    // blocks 0 and 1 and the first quad are requested up front
+    issue_a(0, 0);
+    load_w(0, w_even);
+    load_quad(0, s_cur, b_cur);
+    load_xs(0, xs_cur);
+    load_w(1 < G ? 1 : glast, w_odd);
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) {
+        s_nxt[nb] = s_cur[nb];
+        b_nxt[nb] = b_cur[nb];
+    }
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) xs_nxt[mb] = xs_cur[mb];
+    store_b(0, w_even);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    issue_a(1 < G ? 1 : glast, 1);
+    __syncthreads();
+
+    for (int g = 0; g < G; g += 4) {
+        iteration(std::integral_constant<int, 0>{}, g, w_even, w_odd);
+        if (g + 1 < G) iteration(std::integral_constant<int, 1>{}, g + 1, w_odd, w_even);
+        if (g + 2 < G) iteration(std::integral_constant<int, 2>{}, g + 2, w_even, w_odd);
+        if (g + 3 < G) iteration(std::integral_constant<int, 3>{}, g + 3, w_odd, w_even);
+    }
+
+    // D layout of v_mfma_f32_32x32x*: lane (j, h), register r -> row 8*(r/4) + 4*h + r%4, column j
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) {
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+            const int n = n0 + (wave_n * NB + nb) * 32 + j;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int m = m0 + (wave_m * MB + mb) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+                if (m < M && n < N) {
+                    const int64_t o = (int64_t)m * N + n;
+                    if (a.out_f32) {
+                        reinterpret_cast<float*>(a.y)[o] = out[mb][nb][r];
+                    } else {
+                        reinterpret_cast<uint16_t*>(a.y)[o] = f32_to_bf16_bits(out[mb][nb][r]);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ---- variant table ----------------------------------------------------------------------------
+
+typedef void (*QmmTileKernel)(const QmmTileArgs);
+struct QmmTileEntry {
+    QmmVariant v;
+    QmmTileKernel fn;
+    int lds_bytes;
+};
+
+#define AQ_QMMT(BITS, MB, NB, WM, WN)                                                    \
+    {                                                                                    \
+        {"qmmt_b" #BITS "_mb" #MB "_nb" #NB "_wm" #WM "_wn" #WN, BITS, MB, NB, WM, WN},  \
+            qmm_tile_kernel<BITS, MB, NB, WM, WN>, (3 * WM * MB + 2 * WN * NB) * 4096        \
+    }
+#define AQ_QMMT_SET(BITS)                                                                        \
+    AQ_QMMT(BITS, 4, 2, 2, 2), AQ_QMMT(BITS, 4, 2, 1, 2), AQ_QMMT(BITS, 2, 2, 2, 2),             \
+        AQ_QMMT(BITS, 2, 2, 1, 2), AQ_QMMT(BITS, 4, 2, 1, 4),         \
+        AQ_QMMT(BITS, 2, 2, 2, 4), AQ_QMMT(BITS, 1, 2, 1, 4)
+
+static const QmmTileEntry kQmmTileTable[] = {AQ_QMMT_SET(4), AQ_QMMT_SET(8)};
+
+int qmmt_variant_count() { return (int)(sizeof(kQmmTileTable) / sizeof(kQmmTileTable[0])); }
+const QmmVariant* qmmt_variant(int idx) {
+    if (idx < 0 || idx >= qmmt_variant_count()) return nullptr;
+    return &kQmmTileTable[idx].v;
+}
+
+size_t qmmt_workspace_bytes(int M, int K) {
+    const size_t mblks = ((size_t)M + 31) / 32;
+    const size_t g4 = ((size_t)K / 64 + 3) / 4;
+    return mblks * 32 * (size_t)K * 2 + mblks * 32 * g4 * 16;
+}
+
+hipError_t qmmt_launch(int idx, const QmmArgs& q, void* workspace, hipStream_t stream) {
+    if (idx < 0 || idx >= qmmt_variant_count()) return hipErrorInvalidValue;
+    const QmmTileEntry& e = kQmmTileTable[idx];
+    const int mblks = (q.M + 31) / 32;
+    uint16_t* xf = static_cast<uint16_t*>(workspace);
+    uint16_t* xs = xf + (size_t)mblks * 32 * q.K;
+    const int64_t pieces = (int64_t)mblks * 32 * (q.K / 64) * 8;
+    const unsigned prep_blocks = (unsigned)((pieces + 255) / 256);
+    if (e.v.bits == 4)
+        hipLaunchKernelGGL(qmm_prep_kernel<4>, dim3(prep_blocks), dim3(256), 0, stream, q.x, xf, xs, q.M, q.K, mblks);
+    else
+        hipLaunchKernelGGL(qmm_prep_kernel<8>, dim3(prep_blocks), dim3(256), 0, stream, q.x, xf, xs, q.M, q.K, mblks);
+    hipError_t rc = hipGetLastError();
+    if (rc != hipSuccess) return rc;
+
+    QmmTileArgs a{};
+    a.xf = xf;
+    a.xs = xs;
+    a.w = q.w;
+    a.s = q.s;
+    a.b = q.b;
+    a.y = q.y;
+    a.M = q.M;
+    a.K = q.K;
+    a.N = q.N;
+    a.gs_blocks = q.gs_blocks;
+    a.out_f32 = q.out_f32;
+    a.mblks = mblks;
+    const int bm = e.v.wm * e.v.mb * 32, bn = e.v.wn * e.v.nb * 32;
+    a.tiles_m = (q.M + bm - 1) / bm;
+    a.tiles_n = (q.N + bn - 1) / bn;
+    const int T = a.tiles_m * a.tiles_n;
+    const unsigned grid = (unsigned)(((T + 7) / 8) * 8);
+    if (e.lds_bytes > 48 * 1024) {
+        rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e.fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                 e.lds_bytes);
+        if (rc != hipSuccess) return rc;
+    }
+    hipLaunchKernelGGL(e.fn, dim3(grid), dim3((unsigned)(e.v.wm * e.v.wn * kWave)), (size_t)e.lds_bytes, stream, a);
+    return hipGetLastError();
+}
+
+}  // namespace aq

@@ -108,6 +108,14 @@ int aq_qmv(aq_ctx *ctx, const void *x, const void *packed, const void *scales, c
 int aq_qmm(aq_ctx *ctx, const void *x, const void *packed, const void *scales, const void *biases, void *y, int M,
            int K, int N, int group_size, int bits, unsigned flags);
 
+/* Prefill-sized aq_qmm / aq_qmv calls (M >= 64) rewrite x into MFMA operand order first and keep that
+ * copy (about M*K*2 bytes) in a workspace the context owns.  The workspace grows on demand, which
+ * drains the stream and allocates: not allowed while a capture is open and unwelcome in a serving
+ * loop.  This call sizes it ahead of time for activations of up to M x K.  The reference sizes its
+ * own scratch the same way at model load (hipMLXQ4DeviceWeightConfig and the batch scratch of
+ * go/engine/hip/hip_projection_launch.go:2671-2720). */
+int aq_reserve_workspace(aq_ctx *ctx, int M, int K);
+
 /* gather_qmv: for each route z, y[z,:N] = x[lhs[z] or 0, :K] . dequant(W_e)^T with
  * e = rhs[z] read ON DEVICE; W_e = rows [row_base, row_base+N) of expert e's slab.
  *   packed [num_experts, expert_rows, K*bits/32], scales/biases [num_experts, expert_rows, K/group]
