@@ -5,8 +5,9 @@ A "step" is one pass of the decode hot path over one Gemma-style decoder layer: 
 group-64 quantized GEMVs at batch 1 (q, k, v, o, gate, up, down).  Weights are synthetic (seeded),
 resident in HBM before the timed region, and the steps rotate over enough distinct layer copies that
 no launch finds its weights in the 256 MB Infinity Cache.  The printed JSON line carries the
-whole-layer GB/s (`value`), the roofline of the dominant kernel (the 4096 -> 14336 qmv), the prefill
-qmm at M = 2048 as an extra, and the reference CPU path timed on this box's host cores.
+whole-layer GB/s (`value`), the roofline of the dominant kernel (the 4096 -> 14336 qmv), and as extras
+the prefill qmm at M = 2048, the M = 1..32 sweep at 4 and 8 bit, the MoE gather block, and the
+reference CPU path timed on this box's host cores.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W]
 """
@@ -42,6 +43,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-qmm", action="store_true", help="skip the prefill qmm extra")
+    ap.add_argument("--no-extras", action="store_true", help="skip the small-M and MoE gather extras")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the path has no collectives); --gpus %d is not supported" % args.gpus,
@@ -81,11 +83,28 @@ def main():
     ys = {name: ctx.alloc(N * 2) for name, K, N in LAYER}
     ctx.sync()
 
-    def step(i):
+    def step_separate(i):
         t = layers[i % copies]
         for name, K, N in LAYER:
             w, s, b = t[name]
             ctx.qmv(x14336 if K == 14336 else x4096, w, s, b, ys[name], 1, K, N, GROUP, BITS)
+
+    dims = {name: (K, N) for name, K, N in LAYER}
+
+    def multi(t, names):
+        ctx.qmv_multi(x4096, [t[n][0] for n in names], [t[n][1] for n in names], [t[n][2] for n in names],
+                      [ys[n] for n in names], [dims[n][1] for n in names], 1, 4096, GROUP, BITS)
+
+    def step(i):
+        # the same seven GEMVs in four launches: projections that share their input go out as one grid
+        # (aq_qmv_multi, byte-identical outputs)
+        t = layers[i % copies]
+        multi(t, ("q", "k", "v"))
+        w, s, b = t["o"]
+        ctx.qmv(x4096, w, s, b, ys["o"], 1, 4096, 4096, GROUP, BITS)
+        multi(t, ("gate", "up"))
+        w, s, b = t["down"]
+        ctx.qmv(x14336, w, s, b, ys["down"], 1, 14336, 4096, GROUP, BITS)
 
     # ---- timed region: W warm-up steps, then exactly K steps between syncs ----------------------
     for i in range(args.warmup):
@@ -100,6 +119,14 @@ def main():
     t_host = time.perf_counter() - t_host0
     ms_per_step = ms / args.steps
     value = layer_bytes / (ms_per_step * 1e-3) / 1e9
+    # the same layer as seven separate launches
+    for i in range(args.warmup):
+        step_separate(i)
+    ctx.sync()
+    ctx.timer_start()
+    for i in range(args.steps):
+        step_separate(args.warmup + i)
+    ms_separate = ctx.timer_stop() / args.steps
     variants = {}
     for name, K, N in LAYER:
         w, s, b = layers[0][name]
@@ -163,6 +190,7 @@ def main():
         M, K, N = 2048, 4096, 14336
         xm = ctx.to_device(F.synthetic_x(M, K, seed=F.BASE_SEED + 1003))
         ym = ctx.alloc(M * N * 2)
+        ctx.reserve_workspace(M, K)
         pool = [layers[c]["gate"] for c in range(copies)]
         for i in range(3):
             w, s, b = pool[i % copies]
@@ -181,6 +209,92 @@ def main():
                             "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None}}
         xm.free()
         ym.free()
+
+    # ---- extra: batched / speculative-verify decode (cfg 2): M rows against the gate projection ------
+    small_m = None
+    gather = None
+    if not args.no_extras:
+        small_m = {}
+        K, N = 4096, 14336
+        pools = {4: [layers[c]["gate"] for c in range(copies)]}
+        w8, s8, b8 = F.synthetic_affine(N, K, 8, GROUP, seed=F.BASE_SEED + 30)
+        n8 = max(2, int(640e6 // (w8.nbytes + s8.nbytes + b8.nbytes)) + 1)
+        first8 = (ctx.to_device(w8), ctx.to_device(s8), ctx.to_device(b8))
+        pools[8] = [first8]
+        for c in range(1, n8):
+            dst = tuple(ctx.alloc(t.nbytes) for t in first8)
+            for d, t in zip(dst, first8):
+                ctx._check(ctx.lib.aq_d2d(ctx.handle, d.ptr, t.ptr, t.nbytes))
+            pools[8].append(dst)
+        ctx.reserve_workspace(64, K)
+        for bits in (4, 8):
+            pool = pools[bits]
+            for M in (1, 2, 4, 8, 16, 32):
+                xm = ctx.to_device(F.synthetic_x(M, K, seed=F.BASE_SEED + 1100 + M))
+                ym = ctx.alloc(M * N * 2)
+                n = 60
+                for i in range(6):
+                    w, s, b = pool[i % len(pool)]
+                    ctx.qmv(xm, w, s, b, ym, M, K, N, GROUP, bits)
+                ctx.sync()
+                ctx.timer_start()
+                for i in range(n):
+                    w, s, b = pool[i % len(pool)]
+                    ctx.qmv(xm, w, s, b, ym, M, K, N, GROUP, bits)
+                us = ctx.timer_stop() * 1e3 / n
+                by = qmv_bytes(K, N, M, bits)
+                small_m["b%d_m%d" % (bits, M)] = {"us": round(us, 3), "GBps": round(by / us / 1e3, 1),
+                                                  "pct_of_hbm_peak": round(by / us / 1e3 / HBM_PEAK_GBPS * 100, 2),
+                                                  "kernel": ctx.last_variant(0) or ctx.last_variant(1)}
+                xm.free()
+                ym.free()
+        for t in pools[8]:
+            for d in t:
+                d.free()
+
+        # ---- extra: MoE gather_qmv decode (cfg 4): 128 experts, 8 tokens x top-8, ids read on device --
+        E, TOK, TOPK, DM, DFF = 128, 8, 8, 2816, 1408
+        routes = TOK * TOPK
+        rng = np.random.Generator(np.random.PCG64(F.BASE_SEED + 77))
+        rhs = np.concatenate([rng.permutation(E)[:TOPK] for _ in range(TOK)]).astype(np.int32)
+        lhs_tok = np.repeat(np.arange(TOK, dtype=np.int32), TOPK)
+        lhs_route = np.arange(routes, dtype=np.int32)
+        gate = F.synthetic_affine(E * DFF, DM, BITS, GROUP, seed=F.BASE_SEED + 40)   # [E, DFF, DM]: K = 2816 -> N = 1408
+        down = F.synthetic_affine(E * DM, DFF, BITS, GROUP, seed=F.BASE_SEED + 41)   # [E, DM, DFF]: K = 1408 -> N = 2816
+        dg = tuple(ctx.to_device(t) for t in gate)
+        du = tuple(ctx.alloc(t.nbytes) for t in dg)
+        for d, t in zip(du, dg):
+            ctx._check(ctx.lib.aq_d2d(ctx.handle, d.ptr, t.ptr, t.nbytes))
+        dd = tuple(ctx.to_device(t) for t in down)
+        xt = ctx.to_device(F.synthetic_x(TOK, DM, seed=F.BASE_SEED + 1200))
+        xr = ctx.to_device(F.synthetic_x(routes, DFF, seed=F.BASE_SEED + 1201))
+        d_rhs, d_tok, d_route = ctx.to_device(rhs), ctx.to_device(lhs_tok), ctx.to_device(lhs_route)
+        yg, yu, yd = ctx.alloc(routes * DFF * 2), ctx.alloc(routes * DFF * 2), ctx.alloc(routes * DM * 2)
+
+        def moe_step():
+            ctx.gather_qmv(xt, dg[0], dg[1], dg[2], d_tok, d_rhs, yg, routes, TOK, DM, DFF, E, DFF, 0, GROUP, BITS)
+            ctx.gather_qmv(xt, du[0], du[1], du[2], d_tok, d_rhs, yu, routes, TOK, DM, DFF, E, DFF, 0, GROUP, BITS)
+            ctx.gather_qmv(xr, dd[0], dd[1], dd[2], d_route, d_rhs, yd, routes, routes, DFF, DM, E, DM, 0, GROUP, BITS)
+
+        for _ in range(5):
+            moe_step()
+        ctx.sync()
+        n = 50
+        ctx.timer_start()
+        for _ in range(n):
+            moe_step()
+        us = ctx.timer_stop() * 1e3 / n
+        per_route = 2 * qmv_bytes(DM, DFF) + qmv_bytes(DFF, DM)
+        distinct = len(set(rhs.tolist()))
+        gather = {"experts": E, "tokens": TOK, "top_k": TOPK, "routes": routes, "distinct_experts": distinct,
+                  "us_per_moe_block": round(us, 3), "launches": 3,
+                  "GBps_route_bytes": round(routes * per_route / us / 1e3, 1),
+                  "pct_of_hbm_peak": round(routes * per_route / us / 1e3 / HBM_PEAK_GBPS * 100, 2),
+                  "note": "gate, up (K=2816,N=1408) and down (K=1408,N=2816) gathers; bytes = routes x one expert's "
+                          "codes+scales+biases+x+y; the same expert ids every step, so repeated experts may hit cache",
+                  "kernel": ctx.last_variant(0)}
+        for t in dg + du + dd + (xt, xr, d_rhs, d_tok, d_route, yg, yu, yd):
+            t.free()
 
     # ---- CPU baseline: the reference's CPU path (oracle port of matNTQuantHost), bounded sample ----
     cpu = None
@@ -221,9 +335,12 @@ def main():
                 "weights resident in HBM, %d layer copies rotated (%.0f MB)" % (copies, copies * weight_bytes / 1e6),
         "config": {"workload": "cfg1: Gemma-style decoder layer at batch 1, 4-bit group-64: q/o 4096x4096, k/v 4096->1024, "
                                "gate/up 4096->14336, down 14336->4096; %d algorithmic bytes per step" % layer_bytes,
-                   "device": dev_name, "launches_per_step": len(LAYER)},
+                   "device": dev_name, "launches_per_step": 4,
+                   "launches": "q|k|v fused, o, gate|up fused, down (aq_qmv_multi: one grid over projections that share x)"},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "ms_per_step_graph_replay": round(ms_graph, 5),
+        "ms_per_step_seven_launches": round(ms_separate, 5),
+        "GBps_seven_launches": round(layer_bytes / (ms_separate * 1e-3) / 1e9, 1),
         "host_wall_ms_per_step": round(t_host * 1e3 / args.steps, 5),
         "roofline": {"bound": "hbm", "kernel": variants["gate"], "shape": "qmv M=1 K=4096 N=14336 4-bit g64",
                      "achieved": round(dom_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
@@ -233,6 +350,8 @@ def main():
         "cpu_baseline": cpu,
         "per_shape": per_shape,
         "qmm": qmm,
+        "small_m": small_m,
+        "gather": gather,
     }
     print(json.dumps(out))
     ctx.close()

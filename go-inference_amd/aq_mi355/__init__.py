@@ -53,6 +53,7 @@ PROTOTYPES = {
     "aq_graph_destroy": (None, [_vp]),
     "aq_qmv": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _u]),
     "aq_qmm": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _u]),
+    "aq_qmv_multi": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _u]),
     "aq_reserve_workspace": (_i, [_vp, _i, _i]),
     "aq_gather_qmv": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _u]),
     "aq_dequant_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _c.c_int64, _i, _i, _i]),
@@ -214,6 +215,13 @@ class Context:
     def qmm(self, x, w, s, b, y, M, K, N, group_size=64, bits=4, flags=0):
         self._check(self.lib.aq_qmm(self.handle, _ptr(x), _ptr(w), _ptr(s), _ptr(b), _ptr(y), M, K, N, group_size,
                                     bits, flags))
+
+    def qmv_multi(self, x, ws, ss, bs, ys, Ns, M, K, group_size=64, bits=4, flags=0):
+        """ws, ss, bs, ys: sequences of device buffers (one per weight matrix); Ns: their row counts."""
+        n = len(ws)
+        arr = lambda seq: (_c.c_void_p * n)(*[_ptr(t) for t in seq])
+        self._check(self.lib.aq_qmv_multi(self.handle, _ptr(x), n, arr(ws), arr(ss), arr(bs), arr(ys),
+                                          (_c.c_int * n)(*Ns), M, K, group_size, bits, flags))
 
     def reserve_workspace(self, M, K):
         self._check(self.lib.aq_reserve_workspace(self.handle, M, K))

@@ -92,16 +92,17 @@ bool dot2_eligible(int K, int group_size, int bits, const void* x, const void* w
     return lds_bytes <= 160 * 1024;
 }
 
-// Pick a dot2 variant: largest rows-per-wavefront that still yields at least
-// ~8 wavefronts per CU, 4 wavefronts per workgroup.
+// Pick a dot2 variant: rows per wavefront by how many wavefronts the matrix yields, 4 wavefronts per workgroup.
 int pick_qmv_variant(const aq_ctx* ctx, int bits, int m, bool gather, int N, int K, int routes) {
     const int cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
     const int64_t total_rows = (int64_t)N * (gather ? routes : 1);
     int want_rows = 1;
     const int chunks = K * bits / 128;
     const int slices = (chunks + 63) / 64;
-    for (int r : {8, 4, 2}) {
-        if (total_rows / r >= (int64_t)cus * 8 && r * slices >= 2) {
+    // measured on the 256-CU part: two rows per wavefront once that still gives 8 wavefronts a CU, four
+    // only for much taller matrices, one below
+    for (int r : {4, 2}) {
+        if (total_rows / r >= (int64_t)cus * (r == 4 ? 16 : 8) && r * slices >= 2) {
             want_rows = r;
             break;
         }
@@ -152,9 +153,9 @@ int launch_qmv_rows(aq_ctx* ctx, aq::QmvArgs a, int group_size, int bits, bool g
     const int nd = aq::qmv_variant_count();
     const int nx = aq::qmvx_variant_count();
     int forced = ctx->forced[0];
-    if (forced >= nd + nx || (forced < 0 && M >= 2)) {
-        // block-MFMA family: forced, or the default for 2 and more activation rows wherever the shape
-        // fits it (a single row is faster on the dot2 kernels).  Rows beyond what one launch of the
+    if (forced >= nd + nx || (forced < 0 && (M >= 2 || (bits == 8 && !gather)))) {
+        // block-MFMA family: forced, or the default for 2 and more activation rows (and for a single row
+        // of 8-bit codes) wherever the shape fits it; a single row of 4-bit codes is faster on the dot2 kernels.  Rows beyond what one launch of the
         // family takes for this K go in further launches.
         const size_t esize = a.out_f32 ? 4 : 2;
         const int blk_forced = forced < 0 ? -1 : forced - nd - nx;
@@ -450,6 +451,62 @@ int aq_qmv(aq_ctx* ctx, const void* x, const void* packed, const void* scales, c
                                     scales, biases, y, M, K, N, group_size, bits, (flags & AQ_OUT_F32) != 0, fail);
     }
     return launch_qmv_rows(ctx, a, group_size, bits, false);
+}
+
+int aq_qmv_multi(aq_ctx* ctx, const void* x, int count, const void* const* packed, const void* const* scales,
+                 const void* const* biases, void* const* y, const int* N, int M, int K, int group_size, int bits,
+                 unsigned flags) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_qmv_multi: ctx is null");
+    if (count < 0 || count > aq::kQmvMultiMax) return fail(AQ_ERR_ARG, "aq_qmv_multi: count must be 0..%d", aq::kQmvMultiMax);
+    if (count == 0) return AQ_OK;
+    if (!packed || !scales || !biases || !y || !N) return fail(AQ_ERR_ARG, "aq_qmv_multi: null array");
+    if (M < 0 || K < 0) return fail(AQ_ERR_SHAPE, "aq_qmv_multi: M, K must be non-negative");
+    bool fused = M == 1 && K > 0 && bits == 4 && ctx->forced[0] < 0;
+    for (int i = 0; i < count; i++) {
+        if (N[i] < 0) return fail(AQ_ERR_SHAPE, "aq_qmv_multi: N[%d] must be non-negative", i);
+        if (N[i] == 0) fused = false;  // an empty member: leave the bookkeeping to aq_qmv
+        if (N[i] > 0 && K > 0 && M > 0 && (!packed[i] || !scales[i] || !biases[i] || !y[i]))
+            return fail(AQ_ERR_ARG, "aq_qmv_multi: null operand in member %d", i);
+    }
+    if (fused) {
+        if (int rc = check_geometry("aq_qmv_multi", K, group_size, bits)) return rc;
+        if (!x) return fail(AQ_ERR_ARG, "aq_qmv_multi: null operand");
+        int64_t total = 0;
+        for (int i = 0; i < count; i++) {
+            total += N[i];
+            fused = fused && dot2_eligible(K, group_size, bits, x, packed[i], (size_t)K * 2) && aligned(scales[i], 2) &&
+                    aligned(biases[i], 2) && aligned(y[i], 2);
+        }
+        fused = fused && total < (int64_t)1 << 30;
+        if (fused) {
+            std::lock_guard<std::mutex> lk(ctx->mu);
+            const int idx = pick_qmv_variant(ctx, bits, 1, false, (int)total, K, 1);
+            const int rows = idx >= 0 ? aq::qmv_variant(idx)->rows : 0;
+            if (rows > 0 && aq::qmv_multi_supported(bits, 1, rows)) {
+                aq::QmvMultiArgs ma{};
+                ma.common.x = static_cast<const uint16_t*>(x);
+                ma.common.K = K;
+                ma.common.M = 1;
+                ma.common.gs_shift = ilog2(group_size);
+                ma.common.out_f32 = (flags & AQ_OUT_F32) ? 1 : 0;
+                ma.common.routes = 1;
+                ma.count = count;
+                for (int i = 0; i < count; i++) {
+                    ma.w[i] = static_cast<const uint32_t*>(packed[i]);
+                    ma.s[i] = static_cast<const uint16_t*>(scales[i]);
+                    ma.b[i] = static_cast<const uint16_t*>(biases[i]);
+                    ma.y[i] = y[i];
+                    ma.N[i] = N[i];
+                }
+                ctx->last_variant[0] = "qmv_multi_dot2";
+                AQ_HIP(aq::qmv_multi_launch(bits, 1, rows, ma, ctx->stream), "hipLaunchKernel");
+                return AQ_OK;
+            }
+        }
+    }
+    for (int i = 0; i < count; i++)
+        if (int rc = aq_qmv(ctx, x, packed[i], scales[i], biases[i], y[i], M, K, N[i], group_size, bits, flags)) return rc;
+    return AQ_OK;
 }
 
 int aq_qmm(aq_ctx* ctx, const void* x, const void* packed, const void* scales, const void* biases, void* y, int M,

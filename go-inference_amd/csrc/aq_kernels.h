@@ -30,6 +30,22 @@ struct QmvArgs {
     int routes;       // gather only
 };
 
+// Up to kQmvMultiMax weight matrices that share x, K, group size and width: one launch.
+constexpr int kQmvMultiMax = 4;
+struct QmvMultiArgs {
+    QmvArgs common;  // x, K, M, gs_shift, out_f32 (w, s, b, y, N are taken from the arrays below)
+    int count;
+    const uint32_t* w[kQmvMultiMax];
+    const uint16_t* s[kQmvMultiMax];
+    const uint16_t* b[kQmvMultiMax];
+    void* y[kQmvMultiMax];
+    int N[kQmvMultiMax];
+    int block_end[kQmvMultiMax];  // filled by the launcher: first workgroup past matrix i
+};
+// dot2 kernels only: 4 wavefronts a workgroup, `rows` output rows per wavefront, m = 1..4 activation rows.
+bool qmv_multi_supported(int bits, int m, int rows);
+hipError_t qmv_multi_launch(int bits, int m, int rows, QmvMultiArgs ma, hipStream_t stream);
+
 struct QmvVariant {
     const char* name;
     int bits;

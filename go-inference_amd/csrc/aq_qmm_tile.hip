@@ -175,13 +175,15 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
 #pragma unroll
     for (int i = 0; i < WPT; i++) {
         const int p = tid + i * NT;
+        // consecutive threads take consecutive rows: their fragment pieces are then consecutive 16-byte
+        // slots of LDS (threads that alternate between the halves of a row would hit the same banks)
         if constexpr (BITS == 4) {
-            const int r = p >> 1, half = p & 1;  // words 4*half .. 4*half+3 = k steps 2*half, 2*half+1
+            const int r = p % BN, half = p / BN;  // words 4*half .. 4*half+3 = k steps 2*half, 2*half+1
             const int n = min(n0 + r, N - 1);
             wsrc[i] = a.w + (int64_t)n * words_per_row + half * 4;
             bdst[i] = (uint32_t)(((r >> 5) * 4 + 2 * half) * 1024 + (r & 31) * 16);
         } else {
-            const int r = p >> 2, q = p & 3;  // words 4q .. 4q+3 = k step q
+            const int r = p % BN, q = p / BN;  // words 4q .. 4q+3 = k step q
             const int n = min(n0 + r, N - 1);
             wsrc[i] = a.w + (int64_t)n * words_per_row + q * 4;
             bdst[i] = (uint32_t)(((r >> 5) * 4 + q) * 1024 + (r & 31) * 16);

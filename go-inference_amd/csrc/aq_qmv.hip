@@ -51,8 +51,9 @@ struct Slice {
 // XMODE 0: x staged once per workgroup into LDS (x loads are issued before any weight load so the
 //          barrier never waits for HBM); XMODE 1 (M == 1 only): every lane pulls its own 64-byte
 //          x chunk straight from global/L2 with the slice, no LDS and no barrier.
+// bx: this workgroup's position among those of one weight matrix (blockIdx.x for a plain launch).
 template <int BITS, int M, int R, int NW, int DEPTH, bool GATHER, int XMODE>
-__global__ __launch_bounds__(NW* kWave) void qmv_dot2_kernel(const QmvArgs a) {
+__device__ __forceinline__ void qmv_dot2_body(const QmvArgs& a, const int bx) {
     using C = Codec<BITS>;
     constexpr int CPC = C::kCodesPerChunk;
     constexpr int PAIRS = C::kPairs;
@@ -90,7 +91,7 @@ __global__ __launch_bounds__(NW* kWave) void qmv_dot2_kernel(const QmvArgs a) {
     }
 
     // wave-uniform 64-bit bases + 32-bit lane offsets: rows past N are clamped onto the last row
-    const int row_first = (blockIdx.x * NW + wave) * R;
+    const int row_first = (bx * NW + wave) * R;
     const int row_base_clamped = min(row_first, N - 1);
     wbase += (int64_t)row_base_clamped * row_bytes;
     sbase += (int64_t)row_base_clamped * groups_per_row * 2;
@@ -275,6 +276,28 @@ __global__ __launch_bounds__(NW* kWave) void qmv_dot2_kernel(const QmvArgs a) {
     }
 }
 
+template <int BITS, int M, int R, int NW, int DEPTH, bool GATHER, int XMODE>
+__global__ __launch_bounds__(NW* kWave) void qmv_dot2_kernel(const QmvArgs a) {
+    qmv_dot2_body<BITS, M, R, NW, DEPTH, GATHER, XMODE>(a, blockIdx.x);
+}
+
+// Several weight matrices against the same activations in one launch (q|k|v, gate|up): the
+// workgroups of all matrices form one grid, and each looks up which matrix it belongs to.
+template <int BITS, int M, int R, int NW, int DEPTH>
+__global__ __launch_bounds__(NW* kWave) void qmv_dot2_multi_kernel(const QmvMultiArgs ma) {
+    int set = 0;
+#pragma unroll
+    for (int i = 1; i < kQmvMultiMax; i++)
+        if (i < ma.count && (int)blockIdx.x >= ma.block_end[i - 1]) set = i;
+    QmvArgs a = ma.common;
+    a.w = ma.w[set];
+    a.s = ma.s[set];
+    a.b = ma.b[set];
+    a.y = ma.y[set];
+    a.N = ma.N[set];
+    qmv_dot2_body<BITS, M, R, NW, DEPTH, false, 0>(a, (int)blockIdx.x - (set ? ma.block_end[set - 1] : 0));
+}
+
 // ---- variant table --------------------------------------------------------
 
 typedef void (*QmvKernel)(const QmvArgs);
@@ -338,6 +361,45 @@ hipError_t qmv_launch(int idx, const QmvArgs& a, hipStream_t stream) {
         if (rc != hipSuccess) return rc;
     }
     hipLaunchKernelGGL(e.fn, grid, block, lds, stream, a);
+    return hipGetLastError();
+}
+
+typedef void (*QmvMultiKernel)(const QmvMultiArgs);
+struct QmvMultiEntry {
+    int bits, m, rows;
+    QmvMultiKernel fn;
+};
+#define AQ_QMV_MULTI(BITS, M, R) {BITS, M, R, qmv_dot2_multi_kernel<BITS, M, R, 4, 2>}
+static const QmvMultiEntry kQmvMultiTable[] = {
+    AQ_QMV_MULTI(4, 1, 1), AQ_QMV_MULTI(4, 1, 2), AQ_QMV_MULTI(4, 1, 4), AQ_QMV_MULTI(8, 1, 1), AQ_QMV_MULTI(8, 1, 2),
+    AQ_QMV_MULTI(8, 1, 4), AQ_QMV_MULTI(4, 2, 2), AQ_QMV_MULTI(4, 3, 2), AQ_QMV_MULTI(4, 4, 2), AQ_QMV_MULTI(8, 2, 2),
+    AQ_QMV_MULTI(8, 3, 2), AQ_QMV_MULTI(8, 4, 2),
+};
+
+bool qmv_multi_supported(int bits, int m, int rows) {
+    for (const QmvMultiEntry& e : kQmvMultiTable)
+        if (e.bits == bits && e.m == m && e.rows == rows) return true;
+    return false;
+}
+
+hipError_t qmv_multi_launch(int bits, int m, int rows, QmvMultiArgs ma, hipStream_t stream) {
+    const QmvMultiEntry* e = nullptr;
+    for (const QmvMultiEntry& c : kQmvMultiTable)
+        if (c.bits == bits && c.m == m && c.rows == rows) e = &c;
+    if (!e || ma.count < 1 || ma.count > kQmvMultiMax) return hipErrorInvalidValue;
+    const int rows_per_wg = rows * 4;
+    int blocks = 0;
+    for (int i = 0; i < ma.count; i++) {
+        blocks += (ma.N[i] + rows_per_wg - 1) / rows_per_wg;
+        ma.block_end[i] = blocks;
+    }
+    const size_t lds = (size_t)m * (size_t)ma.common.K * 2;
+    if (lds > 48 * 1024) {
+        hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e->fn),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (rc != hipSuccess) return rc;
+    }
+    hipLaunchKernelGGL(e->fn, dim3((unsigned)blocks), dim3(4 * kWave), lds, stream, ma);
     return hipGetLastError();
 }
 

@@ -101,6 +101,16 @@ void aq_graph_destroy(aq_graph *graph);
 int aq_qmv(aq_ctx *ctx, const void *x, const void *packed, const void *scales, const void *biases, void *y, int M,
            int K, int N, int group_size, int bits, unsigned flags);
 
+/* `count` (1..4) independent aq_qmv calls that share x, M, K, group size and width, in ONE launch:
+ * y[i][M, N[i]] = x . dequant(packed[i], scales[i], biases[i])^T.  The arrays are host arrays of device
+ * pointers.  Results are byte-identical to `count` separate aq_qmv calls.  This is the no-copy form of
+ * running q|k|v or gate|up over model.ConcatQuantRows (go/model/quant_weight.go:32-62): at batch 1 the
+ * narrow projections are bound by launch latency, not bandwidth, and one grid over all of them fills
+ * the machine.  Shapes the fused kernels do not take are run as separate launches. */
+int aq_qmv_multi(aq_ctx *ctx, const void *x, int count, const void *const *packed, const void *const *scales,
+                 const void *const *biases, void *const *y, const int *N, int M, int K, int group_size, int bits,
+                 unsigned flags);
+
 /* affine_qmm: same contract as aq_qmv, tuned for prefill-sized M
  * (go/engine/metal/quant_seam_backend.go:77-109 qmmTBF16Into; reference HIP
  * batch kernels go/engine/hip/kernels/quant/affine_projection_tuned.hipinc:166-1109).

@@ -342,6 +342,49 @@ def test_concat_rows_is_byte_identical(ctx, orc):
         d.free()
 
 
+@pytest.mark.parametrize("M,bits,Ns", [(1, 4, (96, 160, 40)), (1, 4, (4096, 1024, 1024)), (1, 4, (50,)), (1, 4, (7, 9, 300, 64)),
+                                        (2, 4, (96, 160)), (1, 8, (64, 200)), (1, 4, (96, 0, 32))])
+def test_qmv_multi_matches_separate_calls(ctx, orc, M, bits, Ns):
+    """aq_qmv_multi (q|k|v, gate|up in one launch) is byte-identical to one aq_qmv per matrix, the
+    contract ConcatQuantRows states (go/model/quant_weight.go:32-44); members that the fused kernels
+    do not take (more rows, 8 bit, empty) run as separate launches behind the same call."""
+    import aq_mi355
+    say("qmv multi", M, bits, Ns)
+    K = 1024
+    x = F.synthetic_x(M, K, seed=333)
+    dx = ctx.to_device(x)
+    mats = [F.synthetic_affine(max(n, 1), K, bits, 64, seed=340 + i) for i, n in enumerate(Ns)]
+    dws = [DeviceAffine(ctx, *m) for m in mats]
+    for f32 in (False, True):
+        esz = 4 if f32 else 2
+        ys = [ctx.alloc(max(M * n, 1) * esz) for n in Ns]
+        for t in ys:
+            ctx.fill_zero(t)
+        ctx.qmv_multi(dx, [d.w for d in dws], [d.s for d in dws], [d.b for d in dws], ys, list(Ns), M, K, 64, bits,
+                      aq_mi355.AQ_OUT_F32 if f32 else 0)
+        ctx.sync()
+        fused_name = ctx.last_variant(0)
+        for i, n in enumerate(Ns):
+            if n == 0:
+                continue
+            got = ys[i].download(np.float32 if f32 else np.uint16, M * n).reshape(M, n)
+            want = run_qmv(ctx, x, dws[i], M, K, n, 64, bits, f32)
+            assert np.array_equal(got.view(np.uint32 if f32 else np.uint16), want.view(np.uint32 if f32 else np.uint16)), (i, n, f32)
+            ref = F.reference_f64(x, mats[i][0][:n], mats[i][1][:n], mats[i][2][:n], bits, 64, K)
+            if f32:
+                check_accumulators(got, ref, "multi member %d" % i)
+        if M == 1 and bits == 4 and all(n > 0 for n in Ns):
+            assert fused_name == "qmv_multi_dot2", fused_name
+        for t in ys:
+            t.free()
+    with pytest.raises(aq_mi355.AqError):
+        ctx.qmv_multi(dx, [d.w for d in dws] * 5, [d.s for d in dws] * 5, [d.b for d in dws] * 5, [dx] * (5 * len(Ns)),
+                      list(Ns) * 5, M, K, 64, bits, 0)
+    dx.free()
+    for d in dws:
+        d.free()
+
+
 def test_qmv_zero_sized_and_errors(ctx):
     import aq_mi355
     say("qmv zero/err")
