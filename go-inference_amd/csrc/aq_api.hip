@@ -120,17 +120,22 @@ int pick_qmv_variant(const aq_ctx* ctx, int bits, int m, bool gather, int N, int
 }
 
 // One index space over the matvec kernel families: dot2 variants first, then the 32x32 MFMA
-// variants, then the block-MFMA variants.
-int qmv_total_variants() { return aq::qmv_variant_count() + aq::qmvx_variant_count() + aq::qmvb_variant_count(); }
+// variants, then the block-MFMA variants, then the streaming dot2 variants.
+int qmv_total_variants() {
+    return aq::qmv_variant_count() + aq::qmvx_variant_count() + aq::qmvb_variant_count() + aq::qmvs_variant_count();
+}
 const aq::QmvVariant* qmv_any_variant(int idx) {
     const int nd = aq::qmv_variant_count();
     const int nx = aq::qmvx_variant_count();
     if (idx < nd) return aq::qmv_variant(idx);
     if (idx < nd + nx) return aq::qmvx_variant(idx - nd);
-    return aq::qmvb_variant(idx - nd - nx);
+    const int nb = aq::qmvb_variant_count();
+    if (idx < nd + nx + nb) return aq::qmvb_variant(idx - nd - nx);
+    return aq::qmvs_variant(idx - nd - nx - nb);
 }
 
 constexpr size_t kMaxLds = 160 * 1024;
+constexpr bool kStreamDefault = false;
 
 bool mfma_eligible(const aq::QmvArgs& a, int group_size, int bits) {
     if (bits != 4 && bits != 8) return false;
@@ -153,7 +158,20 @@ int launch_qmv_rows(aq_ctx* ctx, aq::QmvArgs a, int group_size, int bits, bool g
     const int nd = aq::qmv_variant_count();
     const int nx = aq::qmvx_variant_count();
     int forced = ctx->forced[0];
-    if (forced >= nd + nx || (forced < 0 && (M >= 2 || (bits == 8 && !gather)))) {
+    const int nbk = aq::qmvb_variant_count();
+    if (forced >= nd + nx + nbk || (forced < 0 && M == 1 && kStreamDefault)) {
+        // streaming dot2 family: forced, or the default for one activation row wherever K fits it
+        aq::StreamPlan plan;
+        if (aq::qmvs_plan(a, bits, group_size, gather, ctx->cu_count, forced < 0 ? -1 : forced - nd - nx - nbk, &plan)) {
+            ctx->last_variant[0] = aq::qmvs_variant(plan.idx)->name;
+            AQ_HIP(aq::qmvs_launch(plan, a, ctx->stream), "hipLaunchKernel");
+            return AQ_OK;
+        }
+        if (forced >= 0)
+            return fail(AQ_ERR_ARG, "aq_qmv: forced variant %d does not fit bits=%d gather=%d rows=%d K=%d N=%d", forced,
+                        bits, (int)gather, M, a.K, a.N);
+    }
+    if ((forced >= nd + nx && forced < nd + nx + nbk) || (forced < 0 && (M >= 2 || (bits == 8 && !gather)))) {
         // block-MFMA family: forced, or the default for 2 and more activation rows (and for a single row
         // of 8-bit codes) wherever the shape fits it; a single row of 4-bit codes is faster on the dot2 kernels.  Rows beyond what one launch of the
         // family takes for this K go in further launches.

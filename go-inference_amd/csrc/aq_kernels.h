@@ -56,7 +56,8 @@ struct QmvVariant {
     int gather;  // 1: reads rhs/lhs on device, grid.y = routes
     int xmode;   // 0: x staged through LDS, 1: every lane reads its x chunk from global
     int kind;    // 0: VALU dot2 kernel (aq_qmv.hip), 1: MFMA kernel (aq_qmv_mfma.hip; m = most rows it takes),
-                 // 2: block-MFMA kernel (aq_qmv_blk.hip; m = most rows, depth = K pieces per wavefront)
+                 // 2: block-MFMA kernel (aq_qmv_blk.hip; m = most rows, depth = K pieces per wavefront),
+                 // 3: streaming dot2 kernel (aq_qmv_stream.hip; depth = rows in flight, xmode = slices per row)
 };
 
 int qmv_variant_count();
@@ -99,6 +100,18 @@ const QmvVariant* qmvb_variant(int idx);
 // forced_idx < 0: choose the variant; otherwise plan for exactly that one.
 bool qmvb_plan(const QmvArgs& a, int bits, int group_size, bool gather, int cu_count, int forced_idx, BlkPlan* out);
 hipError_t qmvb_launch(const BlkPlan& p, const QmvArgs& a, hipStream_t stream);
+
+// Streaming dot2 kernels (aq_qmv_stream.hip; one activation row, K = 1, 2, 4 or 7 slices of 64 chunks,
+// long-lived wavefronts with the activations in registers).
+struct StreamPlan {
+    int idx;   // variant
+    int nwg;   // workgroups (4 wavefronts each) along x
+    bool sbw;  // scales and biases of a row fit one dword load
+};
+int qmvs_variant_count();
+const QmvVariant* qmvs_variant(int idx);
+bool qmvs_plan(const QmvArgs& a, int bits, int group_size, bool gather, int cu_count, int forced_idx, StreamPlan* out);
+hipError_t qmvs_launch(const StreamPlan& p, const QmvArgs& a, hipStream_t stream);
 
 // Any-width (2..8 bit, codes may straddle words), any-group fallback.
 hipError_t qmv_generic_launch(const QmvArgs& a, int bits, int group_size, bool gather, hipStream_t stream);
