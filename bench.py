@@ -36,6 +36,75 @@ def qmv_bytes(K, N, M=1, bits=BITS):
     return N * K * bits // 8 + 2 * N * (K // GROUP) * 2 + M * K * 2 + M * N * 2
 
 
+def pmc_summary(root):
+    """Per kernel and counter: dispatches, mean value per dispatch."""
+    import collections
+    import csv
+    acc = collections.defaultdict(list)
+    for dirpath, _, files in os.walk(root):
+        for f in files:
+            if f.endswith("counter_collection.csv"):
+                for r in csv.DictReader(open(os.path.join(dirpath, f))):
+                    acc[(r["Kernel_Name"], r["Counter_Name"])].append(float(r["Counter_Value"]))
+    for (k, c), v in sorted(acc.items()):
+        print("%-90s %-12s n=%-4d mean=%.6g" % (k[:90], c, len(v), sum(v) / len(v)))
+
+
+def traffic_from_profiles():
+    """HBM bytes per launch of the dominant kernel as recorded in profiles/ (from rocprofv3 --pmc
+    FETCH_SIZE and WRITE_SIZE passes, scaled by the kernels of known traffic in the same passes)."""
+    import re
+    path = os.path.join(ROOT, "profiles", "qmv_dominant_traffic.md")
+    try:
+        m = re.search(r"traffic_bytes_per_launch:\s*([0-9]+)", open(path).read())
+        return int(m.group(1)) if m else None
+    except OSError:
+        return None
+
+
+def run_probe(which):
+    import numpy as np
+    import aq_mi355
+    import fixtures as F
+    ctx = aq_mi355.Context(0)
+    K, N = 4096, 14336
+    w, s, b = F.synthetic_affine(N, K, BITS, GROUP, seed=F.BASE_SEED + 14)
+    ncopy = 14
+    first = (ctx.to_device(w), ctx.to_device(s), ctx.to_device(b))
+    pool = [first]
+    for _ in range(1, ncopy):
+        dst = tuple(ctx.alloc(t.nbytes) for t in first)
+        for d, t in zip(dst, first):
+            ctx._check(ctx.lib.aq_d2d(ctx.handle, d.ptr, t.ptr, t.nbytes))
+        pool.append(dst)
+    # known traffic: 256 MiB written, nothing read
+    z = ctx.alloc(256 << 20)
+    ctx.fill_zero(z)
+    # known traffic: packed codes + scales + biases read once, N*K fp32 written
+    deq = ctx.alloc(N * K * 4)
+    ctx.dequant_f32(first[0], first[1], first[2], deq, N, K, GROUP, BITS)
+    ctx.sync()
+    if which == "dominant":
+        x = ctx.to_device(F.synthetic_x(1, K, seed=F.BASE_SEED + 1000))
+        y = ctx.alloc(N * 2)
+        for i in range(20 * ncopy):
+            ww, ss, bb = pool[i % ncopy]
+            ctx.qmv(x, ww, ss, bb, y, 1, K, N, GROUP, BITS)
+    else:
+        M = 2048
+        x = ctx.to_device(F.synthetic_x(M, K, seed=F.BASE_SEED + 1003))
+        y = ctx.alloc(M * N * 2)
+        ctx.reserve_workspace(M, K)
+        for i in range(6):
+            ww, ss, bb = pool[i % ncopy]
+            ctx.qmm(x, ww, ss, bb, y, M, K, N, GROUP, BITS)
+    ctx.sync()
+    print(json.dumps({"probe": which, "fill_zero_bytes_written": 256 << 20,
+                      "dequant_bytes_read": w.nbytes + s.nbytes + b.nbytes, "dequant_bytes_written": N * K * 4,
+                      "kernel": ctx.last_variant(0 if which == "dominant" else 1)}))
+    ctx.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -44,11 +113,23 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-qmm", action="store_true", help="skip the prefill qmm extra")
     ap.add_argument("--no-extras", action="store_true", help="skip the small-M and MoE gather extras")
+    ap.add_argument("--probe", choices=["dominant", "qmm"], help="run only the named kernel a few times, preceded by two "
+                    "kernels of known traffic (a 256 MiB zero fill, a dequantisation of the gate tensor): the workload "
+                    "of the rocprofv3 --pmc passes behind roofline.traffic")
+    ap.add_argument("--pmc-summary", metavar="DIR", help="print per-kernel averages of the counters a rocprofv3 --pmc "
+                    "--output-format csv run left under DIR, and exit")
     args = ap.parse_args()
+    if args.pmc_summary:
+        pmc_summary(args.pmc_summary)
+        return
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the path has no collectives); --gpus %d is not supported" % args.gpus,
               file=sys.stderr)
         sys.exit(2)
+
+    if args.probe:
+        run_probe(args.probe)
+        return
 
     import numpy as np
     import aq_mi355
@@ -344,7 +425,7 @@ def main():
         "host_wall_ms_per_step": round(t_host * 1e3 / args.steps, 5),
         "roofline": {"bound": "hbm", "kernel": variants["gate"], "shape": "qmv M=1 K=4096 N=14336 4-bit g64",
                      "achieved": round(dom_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(dom_gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(dom_gbps / HBM_PEAK_GBPS, 4), "traffic": traffic_from_profiles(),
                      "bytes_per_launch": dom_bytes, "us_per_launch": round(dom_us, 3),
                      "us_per_launch_cached": round(dom_cached_us, 3)},
         "cpu_baseline": cpu,
