@@ -10,13 +10,16 @@
 //     (1 KiB per 32 rows x 16 K, lane-major, K already in the order the unpacker emits codes) and
 //     the per-block sums as (hi, lo) bf16 pairs.  The main kernel then copies A tiles global -> LDS
 //     with global_load_lds_dwordx4: no registers, no VALU work, no LDS write instructions;
-//   * the packed weights of a tile are fetched once per workgroup (not once per wavefront), unpacked
-//     cooperatively into B fragments in LDS, and read back by every wavefront with ds_read_b128;
+//   * the packed weights of a tile are fetched once per workgroup (not once per wavefront) the same way
+//     and stay PACKED in LDS (a quarter of the bytes of bf16 fragments: LDS read bandwidth, 128 B/clk/CU,
+//     is what bounds 64 x 64 wavefront tiles); a lane reads the 16 bytes that hold its four MFMA steps
+//     with one ds_read_b128 and expands them in registers;
+//   * no LDS write instruction and no register staging in the main loop, so the only waits on global
+//     memory are the explicit "at most this iteration's copies outstanding" before each barrier;
 //   * wavefront tiles are 128 x 64 (or 64 x 64): LDS read bandwidth (128 B/clk/CU), not the matrix
 //     pipe, bounds smaller ones;
-//   * every global load has the MFMAs of one 64-code block to arrive: three LDS stages of A (the copy
-//     of block g+2 starts while block g+1 is still to be read), two of B fed from packed words that
-//     wait in registers; one barrier per block;
+//   * three LDS stages: the copies of block g+2 are issued at the top of iteration g and have two
+//     blocks of MFMAs to arrive; one barrier per block;
 //   * tiles are numbered so that the workgroups of one XCD (every 8th workgroup) walk one band of
 //     rows of x across N: the band's A tile stays in that XCD's L2 while the weights stream by.
 #include "aq_device.h"
@@ -53,14 +56,28 @@ __device__ __forceinline__ uint4 unpack_words8(uint32_t w0, uint32_t w1) {
 
 __device__ __forceinline__ uint32_t dup16(uint32_t h) { return (h & 0xffffu) | (h << 16); }
 
-typedef const __attribute__((address_space(1))) void* gvoid_t;
-typedef __attribute__((address_space(3))) void* lvoid_t;
+// One global -> LDS copy of 16 bytes per lane (64 lanes fill 1 KiB at lds_base + 16 * lane), written as
+// inline asm on purpose.  The compiler knows that the builtin form writes LDS and, unable to tell the
+// target from the stages being read, drains EVERY outstanding copy (s_waitcnt vmcnt(0)) before the
+// next LDS access; the loop below needs the copies of block g+2 in flight while block g is read and
+// orders them itself with counted waits.  Hidden from the compiler, a copy can only make the
+// compiler's own waits for ordinary loads stricter, never weaker (completion is in order).
+// m0 is reserved by the compiler (it sets it before each of its own uses), so writing it here is safe.
+__device__ __forceinline__ void copy16_to_lds(const void* src_lane, uint32_t lds_base_uniform) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src_lane), "s"(lds_base_uniform)
+                 : "memory");
+}
+__device__ __forceinline__ uint32_t lds_offset(const void* p) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t*)p;
+}
 
 }  // namespace
 
 // ---- pass over x ----------------------------------------------------------------------------
 // xf: [mblks][K/16][64 lanes][8] bf16.  Lane (j, h) of fragment (mblk, 4g + t) holds
-//     x[32 mblk + j][64 g + 16 t + 8 h + order(0..7)], order = 0,4,1,5,2,6,3,7 at 4 bit, natural at 8 bit.
+//     x[32 mblk + j][64 g + 32 h + 8 t + order(0..7)], order = 0,4,1,5,2,6,3,7 at 4 bit, natural at 8 bit:
+//     MFMA step t pairs lane half h with the 8 codes number 4h + t of the block, so that the codes a
+//     lane needs for its four steps are contiguous in the packed row.
 // xs: [mblks * 32][ceil(G/4)][4 blocks][hi, lo] bf16: sum of x over each 64-code block, hi + lo.
 // Rows past M are written as zeros.
 template <int BITS>
@@ -102,7 +119,7 @@ __global__ __launch_bounds__(256) void qmm_prep_kernel(const uint16_t* __restric
         o.w = (v.y >> 16) | (v.w & 0xffff0000u);
         v = o;
     }
-    const int t = c8 >> 1, h = c8 & 1;
+    const int t = c8 & 3, h = c8 >> 2;
     const int64_t frag = (int64_t)(row >> 5) * (K / 16) + g * 4 + t;
     *reinterpret_cast<uint4*>(xf + (frag * 64 + h * 32 + (row & 31)) * 8) = v;
 }
@@ -116,7 +133,7 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
     constexpr int NWAVE = WM * WN;
     constexpr int NT = NWAVE * kWave;
     constexpr int A_STAGE = (BM / 32) * 4096;
-    constexpr int B_STAGE = (BN / 32) * 4096;
+    constexpr int B_STAGE = BN * (BITS == 4 ? 32 : 64);  // packed codes of one 64-code block
     constexpr int A_BLOCKS = (BM / 32) * 4;        // 1 KiB fragments of A per stage
     constexpr int WPB = BITS == 4 ? 8 : 16;        // packed words per row and 64-code block
     constexpr int W_PIECES = BN * WPB / 4;         // 16-byte pieces of packed weights per stage
@@ -126,9 +143,13 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
     static_assert(W_PIECES % NT == 0 && WPT >= 1, "weight pieces must divide among the threads");
 
 
+    constexpr int NA = A_BLOCKS / NWAVE;  // A copies a wavefront issues per block
+    constexpr int GROUP_OPS = NA + WPT;   // LDS copies a wavefront issues per block
+    static_assert(W_PIECES % kWave == 0, "a copy instruction moves 64 pieces");
+
     extern __shared__ __align__(16) uint8_t lds[];
     uint8_t* const abuf = lds;                // [3][A_STAGE]
-    uint8_t* const bbuf = lds + 3 * A_STAGE;  // [2][B_STAGE]
+    uint8_t* const bbuf = lds + 3 * A_STAGE;  // [3][B_STAGE]
 
     // tile of this workgroup: workgroups are dealt to the 8 XCDs round-robin, so every 8th one
     // shares an L2; give each XCD a contiguous run of tiles in row-band-major order
@@ -165,53 +186,29 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
             int mblk = m0 / 32 + (blk >> 2);
             mblk = mblk < a.mblks ? mblk : a.mblks - 1;  // past the end: any valid rows, never stored
             const uint16_t* src = a.xf + ((int64_t)mblk * ksteps + g * 4 + (blk & 3)) * 512 + lane * 8;
-            __builtin_amdgcn_global_load_lds((gvoid_t)src, (lvoid_t)(dst + blk * 1024), 16, 0, 0);
+            copy16_to_lds(src, __builtin_amdgcn_readfirstlane(lds_offset(dst + blk * 1024)));
         }
     };
 
-    // B: packed pieces of the tile's rows, WPT per thread
+    // B: the tile's packed rows, 16-byte pieces; copy instruction i of this wavefront moves pieces
+    // (i * NWAVE + wave) * 64 + lane to consecutive LDS slots, which leaves row r at r * (WPB * 4) bytes
     const uint32_t* wsrc[WPT];
-    uint32_t bdst[WPT];  // LDS byte offset of the first fragment piece this thread writes
 #pragma unroll
     for (int i = 0; i < WPT; i++) {
-        const int p = tid + i * NT;
-        // consecutive threads take consecutive rows: their fragment pieces are then consecutive 16-byte
-        // slots of LDS (threads that alternate between the halves of a row would hit the same banks)
-        if constexpr (BITS == 4) {
-            const int r = p % BN, half = p / BN;  // words 4*half .. 4*half+3 = k steps 2*half, 2*half+1
-            const int n = min(n0 + r, N - 1);
-            wsrc[i] = a.w + (int64_t)n * words_per_row + half * 4;
-            bdst[i] = (uint32_t)(((r >> 5) * 4 + 2 * half) * 1024 + (r & 31) * 16);
-        } else {
-            const int r = p % BN, q = p / BN;  // words 4q .. 4q+3 = k step q
-            const int n = min(n0 + r, N - 1);
-            wsrc[i] = a.w + (int64_t)n * words_per_row + q * 4;
-            bdst[i] = (uint32_t)(((r >> 5) * 4 + q) * 1024 + (r & 31) * 16);
-        }
+        const int p = (i * NWAVE + wave) * kWave + lane;
+        constexpr int PPR = WPB / 4;  // pieces per row
+        const int r = p / PPR, q = p % PPR;
+        const int n = min(n0 + r, N - 1);
+        wsrc[i] = a.w + (int64_t)n * words_per_row + q * 4;
     }
-    uint4 w_even[WPT], w_odd[WPT];  // packed words in flight: block b waits in w_even when b is even
-    auto load_w = [&](int g, uint4 (&dst)[WPT]) {
+    auto issue_b = [&](int g, int stage) {
+        uint8_t* dst = bbuf + stage * B_STAGE;
 #pragma unroll
-        for (int i = 0; i < WPT; i++) dst[i] = *reinterpret_cast<const uint4*>(wsrc[i] + (int64_t)g * WPB);
+        for (int i = 0; i < WPT; i++)
+            copy16_to_lds(wsrc[i] + (int64_t)g * WPB, __builtin_amdgcn_readfirstlane(lds_offset(dst + (i * NWAVE + wave) * 1024)));
     };
     const uint32_t mask_s = opaque_s(kMask16);
     const uint32_t magic_v = opaque_v(kMagic16);
-    auto store_b = [&](int g, const uint4 (&wreg)[WPT]) {
-        uint8_t* dst = bbuf + (g & 1) * B_STAGE;
-#pragma unroll
-        for (int i = 0; i < WPT; i++) {
-            if constexpr (BITS == 4) {
-                // word w of the piece -> k step 2*half + w/2, lane half w & 1
-                *reinterpret_cast<uint4*>(dst + bdst[i]) = unpack_word4(wreg[i].x, mask_s, magic_v);
-                *reinterpret_cast<uint4*>(dst + bdst[i] + 512) = unpack_word4(wreg[i].y, mask_s, magic_v);
-                *reinterpret_cast<uint4*>(dst + bdst[i] + 1024) = unpack_word4(wreg[i].z, mask_s, magic_v);
-                *reinterpret_cast<uint4*>(dst + bdst[i] + 1536) = unpack_word4(wreg[i].w, mask_s, magic_v);
-            } else {
-                *reinterpret_cast<uint4*>(dst + bdst[i]) = unpack_words8(wreg[i].x, wreg[i].y);
-                *reinterpret_cast<uint4*>(dst + bdst[i] + 512) = unpack_words8(wreg[i].z, wreg[i].w);
-            }
-        }
-    };
 
     // Scales, biases and block sums are fetched per QUAD of four 64-code blocks, one quad ahead: the bf16
     // bits of the quad's four blocks in two words per array and column tile (8-byte loads where the
@@ -285,24 +282,55 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
     // the end of K the last block is requested again.
     const int glast = G - 1;
     int sa = 0;  // LDS stage of A that holds block g
-    auto iteration = [&](auto q_tag, int g, uint4 (&w_load)[WPT], const uint4 (&w_use)[WPT]) {
+    auto iteration = [&](auto q_tag, int g) {
         constexpr int Q = decltype(q_tag)::value;
         const bool more = g + 1 < G;
-        load_w(g + 2 < G ? g + 2 : glast, w_load);
+        if constexpr (Q == 0) {
+            // the quad's scales, biases and sums were requested three blocks ago (the first quad: before
+            // the loop).  Taken over here, before this iteration's copies are issued: the compiler waits
+            // for every request it cannot count before the first use of a loaded register.
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) {
+                s_cur[nb] = s_nxt[nb];
+                b_cur[nb] = b_nxt[nb];
+            }
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++) xs_cur[mb] = xs_nxt[mb];
+        }
         if constexpr (Q == 1) {
+            // ordinary loads first: the wait at the end of the iteration counts the copies behind them
             const int nq = (g >> 2) + 1 < G4 ? (g >> 2) + 1 : G4 - 1;
             load_quad(nq, s_nxt, b_nxt);
             load_xs(nq, xs_nxt);
         }
+        {
+            const int g2 = g + 2 < G ? g + 2 : glast;
+            const int s2 = sa == 0 ? 2 : sa - 1;  // stage (sa + 2) % 3: read last in iteration g-1
+            issue_a(g2, s2);
+            issue_b(g2, s2);
+        }
 
         const uint8_t* ab = abuf + sa * A_STAGE + (wave_m * MB) * 4096 + lane * 16;
-        const uint8_t* bb = bbuf + (g & 1) * B_STAGE + (wave_n * NB) * 4096 + lane * 16;
+        // this lane's codes: row (wave_n * NB + nb) * 32 + j, words 4h .. 4h+3 (8 bit: 8h .. 8h+7)
+        const uint8_t* bb = bbuf + sa * B_STAGE + ((wave_n * NB) * 32 + j) * (WPB * 4) + h * (WPB * 2);
         bf16x8_t bfrag[NB][4];
         float sc[NB];
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) {
-#pragma unroll
-            for (int t = 0; t < 4; t++) bfrag[nb][t] = *reinterpret_cast<const bf16x8_t*>(bb + (nb * 4 + t) * 1024);
+            if constexpr (BITS == 4) {
+                const uint4 cw = *reinterpret_cast<const uint4*>(bb + nb * 32 * 32);
+                bfrag[nb][0] = __builtin_bit_cast(bf16x8_t, unpack_word4(cw.x, mask_s, magic_v));
+                bfrag[nb][1] = __builtin_bit_cast(bf16x8_t, unpack_word4(cw.y, mask_s, magic_v));
+                bfrag[nb][2] = __builtin_bit_cast(bf16x8_t, unpack_word4(cw.z, mask_s, magic_v));
+                bfrag[nb][3] = __builtin_bit_cast(bf16x8_t, unpack_word4(cw.w, mask_s, magic_v));
+            } else {
+                const uint4 c0 = *reinterpret_cast<const uint4*>(bb + nb * 32 * 64);
+                const uint4 c1 = *reinterpret_cast<const uint4*>(bb + nb * 32 * 64 + 16);
+                bfrag[nb][0] = __builtin_bit_cast(bf16x8_t, unpack_words8(c0.x, c0.y));
+                bfrag[nb][1] = __builtin_bit_cast(bf16x8_t, unpack_words8(c0.z, c0.w));
+                bfrag[nb][2] = __builtin_bit_cast(bf16x8_t, unpack_words8(c1.x, c1.y));
+                bfrag[nb][3] = __builtin_bit_cast(bf16x8_t, unpack_words8(c1.z, c1.w));
+            }
             sc[nb] = __uint_as_float(quad_hi(s_cur[nb], Q));
         }
 #pragma unroll
@@ -350,49 +378,31 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
             }
         }
 
-        // block g+1: its packed words have waited in registers; expand them into the other B stage
-        store_b(g + 1, w_use);
-        // the A copies of block g+1 (requested at the end of the last iteration) have landed, and so
-        // has everything requested above
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        issue_a(g + 2 < G ? g + 2 : glast, sa == 0 ? 2 : sa - 1);  // stage (sa + 2) % 3: read last in iteration g-1
         sa = sa == 2 ? 0 : sa + 1;
-        if constexpr (Q == 3) {
-            // the next quad's values arrived two blocks ago
-#pragma unroll
-            for (int nb = 0; nb < NB; nb++) {
-                s_cur[nb] = s_nxt[nb];
-                b_cur[nb] = b_nxt[nb];
-            }
-#pragma unroll
-            for (int mb = 0; mb < MB; mb++) xs_cur[mb] = xs_nxt[mb];
-        }
-        __syncthreads();
+        // Block g+1 has landed once at most this iteration's own copies (of block g+2) are outstanding;
+        // this iteration's LDS reads have returned.  A bare s_barrier on purpose: __syncthreads() carries
+        // a workgroup fence, for which the compiler drains ALL outstanding copies into LDS.
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(GROUP_OPS) : "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
     };
 
-    // blocks 0 and 1 and the first quad are requested up front
+    // the first quad and blocks 0 and 1 are requested up front
+    load_quad(0, s_nxt, b_nxt);
+    load_xs(0, xs_nxt);
     issue_a(0, 0);
-    load_w(0, w_even);
-    load_quad(0, s_cur, b_cur);
-    load_xs(0, xs_cur);
-    load_w(1 < G ? 1 : glast, w_odd);
-#pragma unroll
-    for (int nb = 0; nb < NB; nb++) {
-        s_nxt[nb] = s_cur[nb];
-        b_nxt[nb] = b_cur[nb];
-    }
-#pragma unroll
-    for (int mb = 0; mb < MB; mb++) xs_nxt[mb] = xs_cur[mb];
-    store_b(0, w_even);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    issue_b(0, 0);
     issue_a(1 < G ? 1 : glast, 1);
-    __syncthreads();
+    issue_b(1 < G ? 1 : glast, 1);
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(GROUP_OPS) : "memory");  // block 0 has landed
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
 
     for (int g = 0; g < G; g += 4) {
-        iteration(std::integral_constant<int, 0>{}, g, w_even, w_odd);
-        if (g + 1 < G) iteration(std::integral_constant<int, 1>{}, g + 1, w_odd, w_even);
-        if (g + 2 < G) iteration(std::integral_constant<int, 2>{}, g + 2, w_even, w_odd);
-        if (g + 3 < G) iteration(std::integral_constant<int, 3>{}, g + 3, w_odd, w_even);
+        iteration(std::integral_constant<int, 0>{}, g);
+        if (g + 1 < G) iteration(std::integral_constant<int, 1>{}, g + 1);
+        if (g + 2 < G) iteration(std::integral_constant<int, 2>{}, g + 2);
+        if (g + 3 < G) iteration(std::integral_constant<int, 3>{}, g + 3);
     }
 
     // D layout of v_mfma_f32_32x32x*: lane (j, h), register r -> row 8*(r/4) + 4*h + r%4, column j
@@ -429,7 +439,7 @@ struct QmmTileEntry {
 #define AQ_QMMT(BITS, MB, NB, WM, WN)                                                    \
     {                                                                                    \
         {"qmmt_b" #BITS "_mb" #MB "_nb" #NB "_wm" #WM "_wn" #WN, BITS, MB, NB, WM, WN},  \
-            qmm_tile_kernel<BITS, MB, NB, WM, WN>, (3 * WM * MB + 2 * WN * NB) * 4096        \
+            qmm_tile_kernel<BITS, MB, NB, WM, WN>, 3 * (WM * MB * 4096 + WN * NB * 32 * (BITS == 4 ? 32 : 64))        \
     }
 #define AQ_QMMT_SET(BITS)                                                                        \
     AQ_QMMT(BITS, 4, 2, 2, 2), AQ_QMMT(BITS, 4, 2, 1, 2), AQ_QMMT(BITS, 2, 2, 2, 2),             \
