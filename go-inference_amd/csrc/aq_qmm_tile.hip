@@ -405,6 +405,9 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
         if (g + 3 < G) iteration(std::integral_constant<int, 3>{}, g + 3);
     }
 
+    // the copies requested past the end of K must not outlive the wavefront's use of LDS
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
     // D layout of v_mfma_f32_32x32x*: lane (j, h), register r -> row 8*(r/4) + 4*h + r%4, column j
 #pragma unroll
     for (int mb = 0; mb < MB; mb++) {
