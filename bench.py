@@ -294,6 +294,7 @@ def main():
     # ---- extra: batched / speculative-verify decode (cfg 2): M rows against the gate projection ------
     small_m = None
     gather = None
+    mlp = None
     if not args.no_extras:
         small_m = {}
         K, N = 4096, 14336
@@ -340,41 +341,88 @@ def main():
         rhs = np.concatenate([rng.permutation(E)[:TOPK] for _ in range(TOK)]).astype(np.int32)
         lhs_tok = np.repeat(np.arange(TOK, dtype=np.int32), TOPK)
         lhs_route = np.arange(routes, dtype=np.int32)
-        gate = F.synthetic_affine(E * DFF, DM, BITS, GROUP, seed=F.BASE_SEED + 40)   # [E, DFF, DM]: K = 2816 -> N = 1408
-        down = F.synthetic_affine(E * DM, DFF, BITS, GROUP, seed=F.BASE_SEED + 41)   # [E, DM, DFF]: K = 1408 -> N = 2816
-        dg = tuple(ctx.to_device(t) for t in gate)
-        du = tuple(ctx.alloc(t.nbytes) for t in dg)
-        for d, t in zip(du, dg):
-            ctx._check(ctx.lib.aq_d2d(ctx.handle, d.ptr, t.ptr, t.nbytes))
+        gu = F.synthetic_affine(E * 2 * DFF, DM, BITS, GROUP, seed=F.BASE_SEED + 40)  # [E, gate|up = 2*DFF, DM]
+        down = F.synthetic_affine(E * DM, DFF, BITS, GROUP, seed=F.BASE_SEED + 41)    # [E, DM, DFF]: K = 1408 -> N = 2816
+        dgu = tuple(ctx.to_device(t) for t in gu)
         dd = tuple(ctx.to_device(t) for t in down)
         xt = ctx.to_device(F.synthetic_x(TOK, DM, seed=F.BASE_SEED + 1200))
-        xr = ctx.to_device(F.synthetic_x(routes, DFF, seed=F.BASE_SEED + 1201))
         d_rhs, d_tok, d_route = ctx.to_device(rhs), ctx.to_device(lhs_tok), ctx.to_device(lhs_route)
-        yg, yu, yd = ctx.alloc(routes * DFF * 2), ctx.alloc(routes * DFF * 2), ctx.alloc(routes * DM * 2)
+        yg, yu, yh = ctx.alloc(routes * DFF * 2), ctx.alloc(routes * DFF * 2), ctx.alloc(routes * DFF * 2)
+        yd = ctx.alloc(routes * DM * 2)
 
-        def moe_step():
-            ctx.gather_qmv(xt, dg[0], dg[1], dg[2], d_tok, d_rhs, yg, routes, TOK, DM, DFF, E, DFF, 0, GROUP, BITS)
-            ctx.gather_qmv(xt, du[0], du[1], du[2], d_tok, d_rhs, yu, routes, TOK, DM, DFF, E, DFF, 0, GROUP, BITS)
-            ctx.gather_qmv(xr, dd[0], dd[1], dd[2], d_route, d_rhs, yd, routes, routes, DFF, DM, E, DM, 0, GROUP, BITS)
+        def moe_unfused():
+            ctx.gather_qmv(xt, dgu[0], dgu[1], dgu[2], d_tok, d_rhs, yg, routes, TOK, DM, DFF, E, 2 * DFF, 0, GROUP, BITS)
+            ctx.gather_qmv(xt, dgu[0], dgu[1], dgu[2], d_tok, d_rhs, yu, routes, TOK, DM, DFF, E, 2 * DFF, DFF, GROUP, BITS)
+            ctx.act_mul(yg, yu, yh, routes * DFF, aq_mi355.AQ_ACT_GELU_TANH)
+            ctx.gather_qmv(yh, dd[0], dd[1], dd[2], d_route, d_rhs, yd, routes, routes, DFF, DM, E, DM, 0, GROUP, BITS)
 
-        for _ in range(5):
-            moe_step()
-        ctx.sync()
-        n = 50
-        ctx.timer_start()
-        for _ in range(n):
-            moe_step()
-        us = ctx.timer_stop() * 1e3 / n
+        def moe_fused():
+            ctx.gather_qmv_gate_up(xt, dgu[0], dgu[1], dgu[2], d_tok, d_rhs, yh, routes, TOK, DM, DFF, E, 2 * DFF, 0, DFF,
+                                   GROUP, BITS, aq_mi355.AQ_ACT_GELU_TANH)
+            ctx.gather_qmv(yh, dd[0], dd[1], dd[2], d_route, d_rhs, yd, routes, routes, DFF, DM, E, DM, 0, GROUP, BITS)
+
+        def time_us(fn, n=50):
+            for _ in range(5):
+                fn()
+            ctx.sync()
+            ctx.timer_start()
+            for _ in range(n):
+                fn()
+            return ctx.timer_stop() * 1e3 / n
+
+        us_unfused = time_us(moe_unfused)
+        us = time_us(moe_fused)
+        moe_kernel = ctx.last_variant(0)
         per_route = 2 * qmv_bytes(DM, DFF) + qmv_bytes(DFF, DM)
         distinct = len(set(rhs.tolist()))
+        # bytes of the distinct experts touched, each expert's three matrices counted once
+        expert_bytes = 3 * (DFF * DM * BITS // 8 + 2 * DFF * (DM // GROUP) * 2)
         gather = {"experts": E, "tokens": TOK, "top_k": TOPK, "routes": routes, "distinct_experts": distinct,
-                  "us_per_moe_block": round(us, 3), "launches": 3,
+                  "us_per_moe_block": round(us, 3), "launches": 2,
+                  "us_per_moe_block_unfused": round(us_unfused, 3), "launches_unfused": 4,
                   "GBps_route_bytes": round(routes * per_route / us / 1e3, 1),
                   "pct_of_hbm_peak": round(routes * per_route / us / 1e3 / HBM_PEAK_GBPS * 100, 2),
-                  "note": "gate, up (K=2816,N=1408) and down (K=1408,N=2816) gathers; bytes = routes x one expert's "
-                          "codes+scales+biases+x+y; the same expert ids every step, so repeated experts may hit cache",
-                  "kernel": ctx.last_variant(0)}
-        for t in dg + du + dd + (xt, xr, d_rhs, d_tok, d_route, yg, yu, yd):
+                  "GBps_distinct_expert_bytes": round(distinct * expert_bytes / us / 1e3, 1),
+                  "note": "experts hold a fused gate|up slab [2*1408, 2816] and a down matrix [2816, 1408]; fused = "
+                          "aq_gather_qmv_gate_up (GELU-tanh epilogue) + down gather; unfused = gate gather, up gather, "
+                          "aq_act_mul, down gather; route bytes = routes x one expert's codes+scales+biases+x+y; the "
+                          "same expert ids every step, so repeated experts may hit cache",
+                  "kernel": moe_kernel}
+        for t in dgu + dd + (xt, d_rhs, d_tok, d_route, yg, yu, yh, yd):
+            t.free()
+
+        # ---- extra: the dense MLP of the layer with the activation fused (GELU-tanh) ----------------
+        hg, hu, hh = ctx.alloc(14336 * 2), ctx.alloc(14336 * 2), ctx.alloc(14336 * 2)
+        mlp_bytes = 2 * qmv_bytes(4096, 14336) + qmv_bytes(14336, 4096)
+
+        def mlp_three(i):
+            L = layers[i % copies]
+            ctx.qmv_multi(x4096, [L["gate"][0], L["up"][0]], [L["gate"][1], L["up"][1]], [L["gate"][2], L["up"][2]],
+                          [hg, hu], [14336, 14336], 1, 4096, GROUP, BITS)
+            ctx.act_mul(hg, hu, hh, 14336, aq_mi355.AQ_ACT_GELU_TANH)
+            ctx.qmv(hh, L["down"][0], L["down"][1], L["down"][2], ys["down"], 1, 14336, 4096, GROUP, BITS)
+
+        def mlp_pair(i):
+            L = layers[i % copies]
+            ctx.qmv_gate_up(x4096, L["gate"], L["up"], hh, 1, 4096, 14336, GROUP, BITS, aq_mi355.AQ_ACT_GELU_TANH)
+            ctx.qmv(hh, L["down"][0], L["down"][1], L["down"][2], ys["down"], 1, 14336, 4096, GROUP, BITS)
+
+        def mlp_xload(i):
+            L = layers[i % copies]
+            ctx.qmv_multi(x4096, [L["gate"][0], L["up"][0]], [L["gate"][1], L["up"][1]], [L["gate"][2], L["up"][2]],
+                          [hg, hu], [14336, 14336], 1, 4096, GROUP, BITS)
+            ctx.qmv_act(hg, hu, L["down"][0], L["down"][1], L["down"][2], ys["down"], 1, 14336, 4096, GROUP, BITS,
+                        aq_mi355.AQ_ACT_GELU_TANH)
+
+        mlp = {"bytes": mlp_bytes}
+        for key, fn, launches in (("three_launches", mlp_three, 3), ("gate_up_fused", mlp_pair, 2), ("x_load_fused", mlp_xload, 2)):
+            counter = iter(range(10 ** 9))
+            t_us = time_us(lambda: fn(next(counter)), n=120)
+            mlp[key] = {"us": round(t_us, 3), "launches": launches, "GBps": round(mlp_bytes / t_us / 1e3, 1),
+                        "pct_of_hbm_peak": round(mlp_bytes / t_us / 1e3 / HBM_PEAK_GBPS * 100, 2)}
+        mlp["note"] = ("gate, up 4096->14336 and down 14336->4096 of the cfg1 layer with GELU-tanh: multi-matrix launch + "
+                       "aq_act_mul + down; aq_qmv_gate_up + down; multi-matrix launch + aq_qmv_act")
+        for t in (hg, hu, hh):
             t.free()
 
     # ---- CPU baseline: the reference's CPU path (oracle port of matNTQuantHost), bounded sample ----
@@ -433,6 +481,7 @@ def main():
         "qmm": qmm,
         "small_m": small_m,
         "gather": gather,
+        "mlp_fused": mlp,
     }
     print(json.dumps(out))
     ctx.close()

@@ -22,6 +22,8 @@ AQ_ERR_NODEVICE = -6
 AQ_ERR_SIZE = -7
 AQ_OUT_F32 = 0x1
 
+AQ_ACT_GELU_TANH = 1
+AQ_ACT_SILU = 2
 OP_QMV = 0
 OP_QMM = 1
 
@@ -56,6 +58,13 @@ PROTOTYPES = {
     "aq_qmv_multi": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _u]),
     "aq_reserve_workspace": (_i, [_vp, _i, _i]),
     "aq_gather_qmv": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _u]),
+    "aq_qmv_gate_up": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _u]),
+    "aq_gather_qmv_gate_up": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i,
+                                   _u]),
+    "aq_qmv_act": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _u]),
+    "aq_gather_qmv_act": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i,
+                               _u]),
+    "aq_act_mul": (_i, [_vp, _vp, _vp, _vp, _c.c_int64, _i]),
     "aq_dequant_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _c.c_int64, _i, _i, _i]),
     "aq_matvec_host": (_i, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _i, _i, _i, _i, _vp, _sz]),
     "aq_proj_quant_matmul_host": (_i, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _i, _i, _i, _i, _i]),
@@ -231,6 +240,31 @@ class Context:
         self._check(self.lib.aq_gather_qmv(self.handle, _ptr(x), _ptr(w), _ptr(s), _ptr(b), _ptr(lhs), _ptr(rhs),
                                            _ptr(y), routes, x_rows, K, N, num_experts, expert_rows, row_base,
                                            group_size, bits, flags))
+
+    def qmv_gate_up(self, x, gate, up, y, M, K, N, group_size=64, bits=4, act=AQ_ACT_GELU_TANH, flags=0):
+        """gate, up: (packed, scales, biases) device buffers of the two projections."""
+        self._check(self.lib.aq_qmv_gate_up(self.handle, _ptr(x), _ptr(gate[0]), _ptr(gate[1]), _ptr(gate[2]),
+                                            _ptr(up[0]), _ptr(up[1]), _ptr(up[2]), _ptr(y), M, K, N, group_size, bits,
+                                            act, flags))
+
+    def gather_qmv_gate_up(self, x, w, s, b, lhs, rhs, y, routes, x_rows, K, N, num_experts, expert_rows,
+                           gate_row_base, up_row_base, group_size=64, bits=4, act=AQ_ACT_GELU_TANH, flags=0):
+        self._check(self.lib.aq_gather_qmv_gate_up(self.handle, _ptr(x), _ptr(w), _ptr(s), _ptr(b), _ptr(lhs),
+                                                   _ptr(rhs), _ptr(y), routes, x_rows, K, N, num_experts, expert_rows,
+                                                   gate_row_base, up_row_base, group_size, bits, act, flags))
+
+    def qmv_act(self, gate_x, up_x, w, s, b, y, M, K, N, group_size=64, bits=4, act=AQ_ACT_GELU_TANH, flags=0):
+        self._check(self.lib.aq_qmv_act(self.handle, _ptr(gate_x), _ptr(up_x), _ptr(w), _ptr(s), _ptr(b), _ptr(y), M,
+                                        K, N, group_size, bits, act, flags))
+
+    def gather_qmv_act(self, gate_x, up_x, w, s, b, lhs, rhs, y, routes, x_rows, K, N, num_experts, expert_rows,
+                       row_base=0, group_size=64, bits=4, act=AQ_ACT_GELU_TANH, flags=0):
+        self._check(self.lib.aq_gather_qmv_act(self.handle, _ptr(gate_x), _ptr(up_x), _ptr(w), _ptr(s), _ptr(b),
+                                               _ptr(lhs), _ptr(rhs), _ptr(y), routes, x_rows, K, N, num_experts,
+                                               expert_rows, row_base, group_size, bits, act, flags))
+
+    def act_mul(self, gate, up, y, n, act=AQ_ACT_GELU_TANH):
+        self._check(self.lib.aq_act_mul(self.handle, _ptr(gate), _ptr(up), _ptr(y), n, act))
 
     def dequant_f32(self, w, s, b, out, N, K, group_size=64, bits=4):
         self._check(self.lib.aq_dequant_f32(self.handle, _ptr(w), _ptr(s), _ptr(b), _ptr(out), N, K, group_size,

@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <climits>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -587,6 +588,275 @@ int aq_gather_qmv(aq_ctx* ctx, const void* x, const void* packed, const void* sc
     a.routes = routes;
     // every expert slab must keep 16-byte row alignment for the dot2 kernels
     return launch_qmv_rows(ctx, a, group_size, bits, true);
+}
+
+namespace {
+
+bool act_ok(int act) { return act == AQ_ACT_GELU_TANH || act == AQ_ACT_SILU; }
+
+// Bytes of the workspace the matmul path may claim for an M x K activation matrix, rounded so that
+// whatever follows it stays 256-byte aligned.
+size_t qmm_region(int M, int K) { return (aq::qmmt_workspace_bytes(M, K) + 255) & ~(size_t)255; }
+
+// Rows per wavefront for the activation-fused dot2 kernels: `slots` row streams a wavefront of the
+// plain kernel would take for this much work, shared between the two matrices of a pair.
+int act_rows(const aq_ctx* ctx, int bits, int fuse, bool gather, int64_t N, int K, int routes) {
+    const int64_t streams = fuse == 1 ? 2 * N : N;
+    const int idx = pick_qmv_variant(ctx, bits, 1, gather, (int)(streams < INT32_MAX ? streams : INT32_MAX), K, routes);
+    int rows = idx >= 0 ? aq::qmv_variant(idx)->rows : 1;
+    if (fuse == 1) rows = rows >= 4 ? 2 : 1;
+    while (rows > 1 && !aq::qmv_act_supported(bits, fuse, rows, gather)) rows >>= 1;
+    return rows;
+}
+
+}  // namespace
+
+int aq_act_mul(aq_ctx* ctx, const void* gate, const void* up, void* y, int64_t n, int act) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_act_mul: ctx is null");
+    if (n < 0) return fail(AQ_ERR_SHAPE, "aq_act_mul: n must be non-negative");
+    if (!act_ok(act)) return fail(AQ_ERR_UNSUPPORTED, "aq_act_mul: unknown activation %d", act);
+    if (n == 0) return AQ_OK;
+    if (!gate || !up || !y) return fail(AQ_ERR_ARG, "aq_act_mul: null operand");
+    if (!aligned(gate, 2) || !aligned(up, 2) || !aligned(y, 2))
+        return fail(AQ_ERR_ARG, "aq_act_mul: operand pointer is not element-aligned");
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    AQ_HIP(aq::act_mul_launch(static_cast<const uint16_t*>(gate), static_cast<const uint16_t*>(up),
+                              static_cast<uint16_t*>(y), n, act, ctx->stream),
+           "hipLaunchKernel");
+    return AQ_OK;
+}
+
+int aq_qmv_gate_up(aq_ctx* ctx, const void* x, const void* gate_packed, const void* gate_scales, const void* gate_biases,
+                   const void* up_packed, const void* up_scales, const void* up_biases, void* y, int M, int K, int N,
+                   int group_size, int bits, int act, unsigned flags) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_qmv_gate_up: ctx is null");
+    if (M < 0 || K < 0 || N < 0) return fail(AQ_ERR_SHAPE, "aq_qmv_gate_up: M, K, N must be non-negative");
+    if (!act_ok(act)) return fail(AQ_ERR_UNSUPPORTED, "aq_qmv_gate_up: unknown activation %d", act);
+    if (M == 0 || N == 0) return AQ_OK;
+    if (K == 0) return fail(AQ_ERR_SHAPE, "aq_qmv_gate_up: K must be positive when there is output to write");
+    if (int rc = check_geometry("aq_qmv_gate_up", K, group_size, bits)) return rc;
+    if (!x || !gate_packed || !gate_scales || !gate_biases || !up_packed || !up_scales || !up_biases || !y)
+        return fail(AQ_ERR_ARG, "aq_qmv_gate_up: null operand");
+    if (!aligned(x, 2) || !aligned(gate_packed, 4) || !aligned(up_packed, 4) || !aligned(gate_scales, 2) ||
+        !aligned(gate_biases, 2) || !aligned(up_scales, 2) || !aligned(up_biases, 2) || !aligned(y, 2))
+        return fail(AQ_ERR_ARG, "aq_qmv_gate_up: operand pointer is not element-aligned");
+    const bool out_f32 = (flags & AQ_OUT_F32) != 0;
+    if (M == 1 && ctx->forced[0] < 0 && dot2_eligible(K, group_size, bits, x, gate_packed, (size_t)K * 2) &&
+        aligned(up_packed, 16)) {
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        const int rows = act_rows(ctx, bits, 1, false, N, K, 1);
+        if (aq::qmv_act_supported(bits, 1, rows, false)) {
+            aq::QmvArgs a{};
+            a.x = static_cast<const uint16_t*>(x);
+            a.w = static_cast<const uint32_t*>(gate_packed);
+            a.s = static_cast<const uint16_t*>(gate_scales);
+            a.b = static_cast<const uint16_t*>(gate_biases);
+            a.w2 = static_cast<const uint32_t*>(up_packed);
+            a.s2 = static_cast<const uint16_t*>(up_scales);
+            a.b2 = static_cast<const uint16_t*>(up_biases);
+            a.y = y;
+            a.K = K;
+            a.N = N;
+            a.M = 1;
+            a.gs_shift = ilog2(group_size);
+            a.out_f32 = out_f32 ? 1 : 0;
+            a.routes = 1;
+            a.act = act;
+            ctx->last_variant[0] = "qmv_gate_up_dot2";
+            AQ_HIP(aq::qmv_act_launch(bits, 1, rows, false, a, ctx->stream), "hipLaunchKernel");
+            return AQ_OK;
+        }
+    }
+    // two projections into fp32 scratch, then the element-wise step
+    const size_t region = qmm_region(M, K);
+    const size_t each = (((size_t)M * N * 4) + 255) & ~(size_t)255;
+    {
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+        if (int rc = aq::workspace_reserve(ctx->stream, &ctx->ws, region + 2 * each, fail)) return rc;
+    }
+    float* g = reinterpret_cast<float*>(static_cast<char*>(ctx->ws.ptr) + region);
+    float* u = reinterpret_cast<float*>(static_cast<char*>(ctx->ws.ptr) + region + each);
+    if (int rc = aq_qmv(ctx, x, gate_packed, gate_scales, gate_biases, g, M, K, N, group_size, bits, AQ_OUT_F32)) return rc;
+    if (int rc = aq_qmv(ctx, x, up_packed, up_scales, up_biases, u, M, K, N, group_size, bits, AQ_OUT_F32)) return rc;
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    AQ_HIP(aq::act_mul_f32_launch(g, u, y, (int64_t)M * N, act, out_f32 ? 1 : 0, ctx->stream), "hipLaunchKernel");
+    return AQ_OK;
+}
+
+int aq_gather_qmv_gate_up(aq_ctx* ctx, const void* x, const void* packed, const void* scales, const void* biases,
+                          const int32_t* lhs, const int32_t* rhs, void* y, int routes, int x_rows, int K, int N,
+                          int num_experts, int expert_rows, int gate_row_base, int up_row_base, int group_size,
+                          int bits, int act, unsigned flags) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_gather_qmv_gate_up: ctx is null");
+    if (routes < 0 || K < 0 || N < 0) return fail(AQ_ERR_SHAPE, "aq_gather_qmv_gate_up: routes, K, N must be non-negative");
+    if (!act_ok(act)) return fail(AQ_ERR_UNSUPPORTED, "aq_gather_qmv_gate_up: unknown activation %d", act);
+    if (routes == 0 || N == 0) return AQ_OK;
+    if (K == 0) return fail(AQ_ERR_SHAPE, "aq_gather_qmv_gate_up: K must be positive when there is output to write");
+    if (num_experts <= 0 || expert_rows <= 0 || x_rows <= 0)
+        return fail(AQ_ERR_SHAPE, "aq_gather_qmv_gate_up: num_experts, expert_rows and x_rows must be positive");
+    for (int base : {gate_row_base, up_row_base})
+        if (base < 0 || (int64_t)base + N > expert_rows)
+            return fail(AQ_ERR_SHAPE, "aq_gather_qmv_gate_up: rows [%d, %d) fall outside an expert slab of %d rows", base,
+                        base + N, expert_rows);
+    if (int rc = check_geometry("aq_gather_qmv_gate_up", K, group_size, bits)) return rc;
+    if (!x || !packed || !scales || !biases || !rhs || !y) return fail(AQ_ERR_ARG, "aq_gather_qmv_gate_up: null operand");
+    if (!aligned(x, 2) || !aligned(packed, 4) || !aligned(scales, 2) || !aligned(biases, 2) || !aligned(y, 2) ||
+        !aligned(rhs, 4) || (lhs && !aligned(lhs, 4)))
+        return fail(AQ_ERR_ARG, "aq_gather_qmv_gate_up: operand pointer is not element-aligned");
+    if (routes > 65535) return fail(AQ_ERR_UNSUPPORTED, "aq_gather_qmv_gate_up: at most 65535 routes per call");
+    const bool out_f32 = (flags & AQ_OUT_F32) != 0;
+    if (ctx->forced[0] < 0 && dot2_eligible(K, group_size, bits, x, packed, (size_t)K * 2)) {
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        const int rows = act_rows(ctx, bits, 1, true, N, K, routes);
+        if (aq::qmv_act_supported(bits, 1, rows, true)) {
+            aq::QmvArgs a{};
+            a.x = static_cast<const uint16_t*>(x);
+            a.w = a.w2 = static_cast<const uint32_t*>(packed);
+            a.s = a.s2 = static_cast<const uint16_t*>(scales);
+            a.b = a.b2 = static_cast<const uint16_t*>(biases);
+            a.y = y;
+            a.lhs = lhs;
+            a.rhs = rhs;
+            a.K = K;
+            a.N = N;
+            a.M = 1;
+            a.gs_shift = ilog2(group_size);
+            a.out_f32 = out_f32 ? 1 : 0;
+            a.num_experts = num_experts;
+            a.expert_rows = expert_rows;
+            a.row_base = gate_row_base;
+            a.row_base2 = up_row_base;
+            a.x_rows = x_rows;
+            a.routes = routes;
+            a.act = act;
+            ctx->last_variant[0] = "gather_gate_up_dot2";
+            AQ_HIP(aq::qmv_act_launch(bits, 1, rows, true, a, ctx->stream), "hipLaunchKernel");
+            return AQ_OK;
+        }
+    }
+    const size_t each = (((size_t)routes * N * 4) + 255) & ~(size_t)255;
+    {
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+        if (int rc = aq::workspace_reserve(ctx->stream, &ctx->ws, 2 * each, fail)) return rc;
+    }
+    float* g = static_cast<float*>(ctx->ws.ptr);
+    float* u = reinterpret_cast<float*>(static_cast<char*>(ctx->ws.ptr) + each);
+    if (int rc = aq_gather_qmv(ctx, x, packed, scales, biases, lhs, rhs, g, routes, x_rows, K, N, num_experts, expert_rows,
+                               gate_row_base, group_size, bits, AQ_OUT_F32))
+        return rc;
+    if (int rc = aq_gather_qmv(ctx, x, packed, scales, biases, lhs, rhs, u, routes, x_rows, K, N, num_experts, expert_rows,
+                               up_row_base, group_size, bits, AQ_OUT_F32))
+        return rc;
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    AQ_HIP(aq::act_mul_f32_launch(g, u, y, (int64_t)routes * N, act, out_f32 ? 1 : 0, ctx->stream), "hipLaunchKernel");
+    return AQ_OK;
+}
+
+int aq_qmv_act(aq_ctx* ctx, const void* gate_x, const void* up_x, const void* packed, const void* scales,
+               const void* biases, void* y, int M, int K, int N, int group_size, int bits, int act, unsigned flags) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_qmv_act: ctx is null");
+    if (M < 0 || K < 0 || N < 0) return fail(AQ_ERR_SHAPE, "aq_qmv_act: M, K, N must be non-negative");
+    if (!act_ok(act)) return fail(AQ_ERR_UNSUPPORTED, "aq_qmv_act: unknown activation %d", act);
+    if (M == 0 || N == 0 || K == 0) return AQ_OK;
+    if (int rc = check_geometry("aq_qmv_act", K, group_size, bits)) return rc;
+    if (!gate_x || !up_x || !packed || !scales || !biases || !y) return fail(AQ_ERR_ARG, "aq_qmv_act: null operand");
+    if (!aligned(gate_x, 2) || !aligned(up_x, 2) || !aligned(packed, 4) || !aligned(scales, 2) || !aligned(biases, 2) ||
+        !aligned(y, 2))
+        return fail(AQ_ERR_ARG, "aq_qmv_act: operand pointer is not element-aligned");
+    if (M == 1 && ctx->forced[0] < 0 && dot2_eligible(K, group_size, bits, gate_x, packed, (size_t)K * 2) &&
+        aligned(up_x, 16)) {
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        const int rows = act_rows(ctx, bits, 2, false, N, K, 1);
+        if (aq::qmv_act_supported(bits, 2, rows, false)) {
+            aq::QmvArgs a{};
+            a.x = static_cast<const uint16_t*>(gate_x);
+            a.x2 = static_cast<const uint16_t*>(up_x);
+            a.w = static_cast<const uint32_t*>(packed);
+            a.s = static_cast<const uint16_t*>(scales);
+            a.b = static_cast<const uint16_t*>(biases);
+            a.y = y;
+            a.K = K;
+            a.N = N;
+            a.M = 1;
+            a.gs_shift = ilog2(group_size);
+            a.out_f32 = (flags & AQ_OUT_F32) ? 1 : 0;
+            a.routes = 1;
+            a.act = act;
+            ctx->last_variant[0] = "qmv_act_dot2";
+            AQ_HIP(aq::qmv_act_launch(bits, 2, rows, false, a, ctx->stream), "hipLaunchKernel");
+            return AQ_OK;
+        }
+    }
+    const size_t region = qmm_region(M, K);
+    {
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+        if (int rc = aq::workspace_reserve(ctx->stream, &ctx->ws, region + (size_t)M * K * 2, fail)) return rc;
+    }
+    void* gated = static_cast<char*>(ctx->ws.ptr) + region;
+    if (int rc = aq_act_mul(ctx, gate_x, up_x, gated, (int64_t)M * K, act)) return rc;
+    return aq_qmv(ctx, gated, packed, scales, biases, y, M, K, N, group_size, bits, flags);
+}
+
+int aq_gather_qmv_act(aq_ctx* ctx, const void* gate_x, const void* up_x, const void* packed, const void* scales,
+                      const void* biases, const int32_t* lhs, const int32_t* rhs, void* y, int routes, int x_rows, int K,
+                      int N, int num_experts, int expert_rows, int row_base, int group_size, int bits, int act,
+                      unsigned flags) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_gather_qmv_act: ctx is null");
+    if (routes < 0 || K < 0 || N < 0) return fail(AQ_ERR_SHAPE, "aq_gather_qmv_act: routes, K, N must be non-negative");
+    if (!act_ok(act)) return fail(AQ_ERR_UNSUPPORTED, "aq_gather_qmv_act: unknown activation %d", act);
+    if (routes == 0 || N == 0 || K == 0) return AQ_OK;
+    if (num_experts <= 0 || expert_rows <= 0 || x_rows <= 0)
+        return fail(AQ_ERR_SHAPE, "aq_gather_qmv_act: num_experts, expert_rows and x_rows must be positive");
+    if (row_base < 0 || (int64_t)row_base + N > expert_rows)
+        return fail(AQ_ERR_SHAPE, "aq_gather_qmv_act: rows [%d, %d) fall outside an expert slab of %d rows", row_base,
+                    row_base + N, expert_rows);
+    if (int rc = check_geometry("aq_gather_qmv_act", K, group_size, bits)) return rc;
+    if (!gate_x || !up_x || !packed || !scales || !biases || !rhs || !y)
+        return fail(AQ_ERR_ARG, "aq_gather_qmv_act: null operand");
+    if (!aligned(gate_x, 2) || !aligned(up_x, 2) || !aligned(packed, 4) || !aligned(scales, 2) || !aligned(biases, 2) ||
+        !aligned(y, 2) || !aligned(rhs, 4) || (lhs && !aligned(lhs, 4)))
+        return fail(AQ_ERR_ARG, "aq_gather_qmv_act: operand pointer is not element-aligned");
+    if (routes > 65535) return fail(AQ_ERR_UNSUPPORTED, "aq_gather_qmv_act: at most 65535 routes per call");
+    if (ctx->forced[0] < 0 && dot2_eligible(K, group_size, bits, gate_x, packed, (size_t)K * 2) && aligned(up_x, 16)) {
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        const int rows = act_rows(ctx, bits, 2, true, N, K, routes);
+        if (aq::qmv_act_supported(bits, 2, rows, true)) {
+            aq::QmvArgs a{};
+            a.x = static_cast<const uint16_t*>(gate_x);
+            a.x2 = static_cast<const uint16_t*>(up_x);
+            a.w = static_cast<const uint32_t*>(packed);
+            a.s = static_cast<const uint16_t*>(scales);
+            a.b = static_cast<const uint16_t*>(biases);
+            a.y = y;
+            a.lhs = lhs;
+            a.rhs = rhs;
+            a.K = K;
+            a.N = N;
+            a.M = 1;
+            a.gs_shift = ilog2(group_size);
+            a.out_f32 = (flags & AQ_OUT_F32) ? 1 : 0;
+            a.num_experts = num_experts;
+            a.expert_rows = expert_rows;
+            a.row_base = row_base;
+            a.x_rows = x_rows;
+            a.routes = routes;
+            a.act = act;
+            ctx->last_variant[0] = "gather_act_dot2";
+            AQ_HIP(aq::qmv_act_launch(bits, 2, rows, true, a, ctx->stream), "hipLaunchKernel");
+            return AQ_OK;
+        }
+    }
+    {
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+        if (int rc = aq::workspace_reserve(ctx->stream, &ctx->ws, (size_t)x_rows * K * 2, fail)) return rc;
+    }
+    if (int rc = aq_act_mul(ctx, gate_x, up_x, ctx->ws.ptr, (int64_t)x_rows * K, act)) return rc;
+    return aq_gather_qmv(ctx, ctx->ws.ptr, packed, scales, biases, lhs, rhs, y, routes, x_rows, K, N, num_experts,
+                         expert_rows, row_base, group_size, bits, flags);
 }
 
 int aq_dequant_f32(aq_ctx* ctx, const void* packed, const void* scales, const void* biases, float* out_f32, int64_t N,

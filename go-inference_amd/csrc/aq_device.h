@@ -78,6 +78,33 @@ __device__ __forceinline__ void unpack8_word(uint32_t w, uint32_t p[2]) {
     p[1] = __builtin_amdgcn_perm(f3, f2, 0x07060302u);
 }
 
+// Activations of the fused kernels.  1: tanh-approximated GELU with the operation order of
+// rocm_gelu_tanh_value (go/engine/hip/kernels/common/math.hipinc:3-9); 2: SiLU, v / (1 + exp(-v))
+// (go/model/attn/gated_delta.go:228).  Every step is an explicit fp32 operation, so that each kernel
+// that inlines this computes the same bits for the same input.
+__device__ __forceinline__ float act_value(int act, float v) {
+    if (act == 2) return __fdiv_rn(v, __fadd_rn(1.0f, expf(-v)));
+    const float v3 = __fmul_rn(__fmul_rn(v, v), v);
+    const float arg = __fmul_rn(0.7978845608028654f, __fmaf_rn(0.044715f, v3, v));
+    return __fmul_rn(__fmul_rn(0.5f, v), __fadd_rn(1.0f, tanhf(arg)));
+}
+
+// bf16(act(gate) * up): fp32 inside, one rounding at the end, as lthn_gelu_gate_mul_one
+// (go/engine/metal/kernels/moe/lthn_gelu_qmv_impl.h:24-33).
+__device__ __forceinline__ uint32_t act_mul_bf16x2(uint32_t g, uint32_t u, int act) {
+    const float lo = __fmul_rn(act_value(act, bf16_bits_to_f32(g & 0xffffu)), bf16_bits_to_f32(u & 0xffffu));
+    const float hi = __fmul_rn(act_value(act, bf16_bits_to_f32(g >> 16)), bf16_bits_to_f32(u >> 16));
+    return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+}
+__device__ __forceinline__ uint4 act_mul_bf16x8(uint4 g, uint4 u, int act) {
+    uint4 o;
+    o.x = act_mul_bf16x2(g.x, u.x, act);
+    o.y = act_mul_bf16x2(g.y, u.y, act);
+    o.z = act_mul_bf16x2(g.z, u.z, act);
+    o.w = act_mul_bf16x2(g.w, u.w, act);
+    return o;
+}
+
 // Sum over the 64 lanes of a wavefront; every lane returns the total.
 // Four DPP adds fold each 16-lane row, then the four row totals are read
 // through SGPRs.

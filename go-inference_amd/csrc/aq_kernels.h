@@ -28,7 +28,29 @@ struct QmvArgs {
     int row_base;     // gather only: first row of the slab used
     int x_rows;       // gather only: rows in x (bounds for lhs)
     int routes;       // gather only
+    // activation-fused kernels only (aq_qmv_act.hip)
+    const uint16_t* x2;  // x-load fusion: the `up` activations, same shape and row indexing as x (the `gate` ones)
+    const uint32_t* w2;  // pair fusion: the `up` matrix (w, s, b are the `gate` one)
+    const uint16_t* s2;
+    const uint16_t* b2;
+    int row_base2;       // pair fusion + gather: first `up` row inside an expert's slab
+    int act;             // kActGeluTanh or kActSilu
 };
+
+constexpr int kActGeluTanh = 1;
+constexpr int kActSilu = 2;
+
+// Activation-fused dot2 kernels (aq_qmv_act.hip), one activation row.
+//   fuse 1: y[n] = act(gate[n,:] . x) * (up[n,:] . x)          (two matrices, one output)
+//   fuse 2: y[n] = w[n,:] . bf16(act(x[k]) * x2[k])            (activation applied while x is staged)
+// rows: output rows per wavefront (fuse 1: of each matrix).  False / error when no kernel fits.
+bool qmv_act_supported(int bits, int fuse, int rows, bool gather);
+hipError_t qmv_act_launch(int bits, int fuse, int rows, bool gather, const QmvArgs& a, hipStream_t stream);
+// y[i] = bf16(act(gate[i]) * up[i]) over n bf16 values.
+hipError_t act_mul_launch(const uint16_t* gate, const uint16_t* up, uint16_t* y, int64_t n, int act, hipStream_t stream);
+// y[i] = act(gate[i]) * up[i] over n fp32 values, stored as bf16 or fp32.
+hipError_t act_mul_f32_launch(const float* gate, const float* up, void* y, int64_t n, int act, int out_f32,
+                              hipStream_t stream);
 
 // Up to kQmvMultiMax weight matrices that share x, K, group size and width: one launch.
 constexpr int kQmvMultiMax = 4;

@@ -63,6 +63,10 @@ hipError_t fill_zero_launch(void* p, size_t bytes, hipStream_t stream);
 
 typedef int (*FailFn)(int code, const char* fmt, ...);
 
+// Makes ws hold at least `need` bytes (drains the stream and reallocates when it must grow; refused
+// while the stream is being captured).
+int workspace_reserve(hipStream_t stream, Workspace* ws, size_t need, FailFn fail);
+
 // Sizes ws for activations of M x K ahead of time (not during capture).
 int qmm_reserve(hipStream_t stream, Workspace* ws, int M, int K, FailFn fail);
 

@@ -393,7 +393,7 @@ static int grow_workspace(Workspace* ws, size_t need, hipStream_t stream, FailFn
     hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
     if (stream != nullptr && hipStreamIsCapturing(stream, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone)
         return fail(AQ_ERR_UNSUPPORTED,
-                    "aq_qmm: the matmul workspace must grow to %zu bytes, which cannot happen during stream capture; "
+                    "the context's workspace must grow to %zu bytes, which cannot happen during stream capture; "
                     "call aq_reserve_workspace before capturing", need);
     hipError_t rc = hipStreamSynchronize(stream);
     if (rc != hipSuccess) return fail((int)rc, "rocm.hip.hipStreamSynchronize: HIP returned %d", (int)rc);
@@ -405,6 +405,10 @@ static int grow_workspace(Workspace* ws, size_t need, hipStream_t stream, FailFn
     if (rc != hipSuccess) return fail(AQ_ERR_NOMEM, "aq_qmm: cannot allocate a %zu-byte workspace (HIP %d)", want, (int)rc);
     ws->bytes = want;
     return AQ_OK;
+}
+
+int workspace_reserve(hipStream_t stream, Workspace* ws, size_t need, FailFn fail) {
+    return grow_workspace(ws, need, stream, fail);
 }
 
 int qmm_reserve(hipStream_t stream, Workspace* ws, int M, int K, FailFn fail) {

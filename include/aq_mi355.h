@@ -84,7 +84,7 @@ int aq_timer_stop(aq_ctx *ctx, float *elapsed_ms); /* records, waits, reports */
  * replays the whole batch with one submission.  Counterpart of the reference's per-step
  * launch batch (hipLaunchKernelContext batching, go/engine/hip/hip_launch.go:240-273,
  * cgoHIPDriver.LaunchKernelBatch go/engine/hip/hip_driver_cgo.go:1137-1190).  Only the
- * kernel entry points (aq_qmv, aq_qmm, aq_gather_qmv, aq_dequant_f32, aq_fill_zero, aq_d2d)
+ * kernel entry points (aq_qmv*, aq_qmm, aq_gather_qmv*, aq_act_mul, aq_dequant_f32, aq_fill_zero, aq_d2d)
  * may be called while capturing; the pointers they were given must stay valid for replays. */
 typedef struct aq_graph aq_graph;
 int aq_capture_begin(aq_ctx *ctx);
@@ -139,6 +139,60 @@ int aq_reserve_workspace(aq_ctx *ctx, int M, int K);
 int aq_gather_qmv(aq_ctx *ctx, const void *x, const void *packed, const void *scales, const void *biases,
                   const int32_t *lhs, const int32_t *rhs, void *y, int routes, int x_rows, int K, int N,
                   int num_experts, int expert_rows, int row_base, int group_size, int bits, unsigned flags);
+
+/* Activation kinds of the fused MLP entry points below.  GELU is the tanh approximation
+ * 0.5*v*(1 + tanh(0.7978845608028654*(v + 0.044715*v^3))) of rocm_gelu_tanh_value
+ * (go/engine/hip/kernels/common/math.hipinc:3-9); SiLU is v / (1 + exp(-v))
+ * (go/model/attn/gated_delta.go:228). */
+#define AQ_ACT_GELU_TANH 1
+#define AQ_ACT_SILU 2
+
+/* Fused gate|up projection with the activation as epilogue:
+ *   y[m,n] = act(x[m,:] . dequant(gate)[n,:]) * (x[m,:] . dequant(up)[n,:])
+ * both sums in fp32, the activation and the product in fp32, one rounding at the store.  Replaces
+ * rocm_mlx_q4_gelu_tanh_multiply and its batch form (go/engine/hip/kernels/quant/affine_gelu_tanh.hipinc:3-182,
+ * launch go/engine/hip/hip_projection_launch.go:3086-3160, packet contract/launch_abi.hipinc:634-657).
+ * gate and up are [N, K*bits/32] with their own scales/biases; for a row-concatenated gate|up slab
+ * (model.ConcatQuantRows, go/model/quant_weight.go:32-62) pass the slab for gate and slab + N rows for up.
+ * M == 1 with 4/8-bit codes runs as ONE launch that reads every weight once; other shapes run the two
+ * projections and the element-wise step as separate launches through the context's workspace (which grows
+ * on demand like aq_qmm's; not while a capture is open). */
+int aq_qmv_gate_up(aq_ctx *ctx, const void *x, const void *gate_packed, const void *gate_scales,
+                   const void *gate_biases, const void *up_packed, const void *up_scales, const void *up_biases,
+                   void *y, int M, int K, int N, int group_size, int bits, int act, unsigned flags);
+
+/* The same fusion with expert ids read on the device: for each route z, with e = rhs[z],
+ *   y[z,:N] = act(x_z . gate_e^T) * (x_z . up_e^T)
+ * where gate_e / up_e are rows [gate_row_base, +N) / [up_row_base, +N) of expert e's slab (a fused
+ * gate|up slab has expert_rows = 2N, gate_row_base = 0, up_row_base = N).  Stands in for the gate|up
+ * half of rocm_moe_mlx_affine_routes (go/engine/hip/kernels/moe/routing.hipinc:160-399, store :312) and for
+ * the two emitGatherQMVAllRoutes + gelu dispatches of go/engine/metal/moe_block.go:2344-2358.
+ * Index rules as aq_gather_qmv. */
+int aq_gather_qmv_gate_up(aq_ctx *ctx, const void *x, const void *packed, const void *scales, const void *biases,
+                          const int32_t *lhs, const int32_t *rhs, void *y, int routes, int x_rows, int K, int N,
+                          int num_experts, int expert_rows, int gate_row_base, int up_row_base, int group_size,
+                          int bits, int act, unsigned flags);
+
+/* Projection whose input is formed on the fly: y[m,:N] = bf16(act(g[m,:]) * u[m,:]) . dequant(w)^T, where g and
+ * u are the bf16 gate and up activations [M, K].  The gated value is rounded to bf16 once, exactly as the
+ * stand-alone aq_act_mul stores it, so the result is byte-identical to aq_act_mul followed by aq_qmv.
+ * Replaces lthn_gelu_qmv (emitGeluQMV, go/engine/metal/dispatch_sink.go:533-552; x-load
+ * go/engine/metal/kernels/moe/lthn_gelu_qmv_impl.h:24-33). */
+int aq_qmv_act(aq_ctx *ctx, const void *gate_x, const void *up_x, const void *packed, const void *scales,
+               const void *biases, void *y, int M, int K, int N, int group_size, int bits, int act, unsigned flags);
+
+/* The gathered form, lthn_gather_qmv_gelu (go/engine/metal/kernels/moe/lthn_gather_qmv.metal:98-132,
+ * emitLthnGatherQMVGeluRoutes go/engine/metal/qmv_gather.go:319-345): gate_x and up_x are [x_rows, K] and
+ * ride the same lhs indexing. */
+int aq_gather_qmv_act(aq_ctx *ctx, const void *gate_x, const void *up_x, const void *packed, const void *scales,
+                      const void *biases, const int32_t *lhs, const int32_t *rhs, void *y, int routes, int x_rows,
+                      int K, int N, int num_experts, int expert_rows, int row_base, int group_size, int bits,
+                      int act, unsigned flags);
+
+/* y[i] = bf16(act(gate[i]) * up[i]) over n bf16 values: rocm_gelu_tanh_multiply
+ * (go/engine/hip/hip_transformer_launch.go:3765) / lthn_gelu_gate_mul_bf16, host mirror
+ * hostGeluMul (go/engine/metal/ffn_megakernel_test.go:17-31). */
+int aq_act_mul(aq_ctx *ctx, const void *gate, const void *up, void *y, int64_t n, int act);
 
 /* mlxaffine.DequantizeTensor on device (go/model/quant/mlxaffine/mlxaffine.go:178-208):
  * out_f32[N,K] = scale*code + bias, bit-exact with the CPU path. */

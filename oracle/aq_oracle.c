@@ -420,6 +420,46 @@ int orc_gather_qmv(const uint16_t *x, int x_rows, const uint32_t *packed, const 
     return ORC_OK;
 }
 
+/* hip_kernels_test.go:8127-8137 (expectedGELUTanhMultiply); SiLU per gated_delta.go:228. */
+int orc_act_multiply(int act, const float *gate, const float *up, int64_t n, float *out) {
+    if (act != ORC_ACT_GELU_TANH && act != ORC_ACT_SILU) return ORC_ERR_BITS;
+    if (n < 0) return ORC_ERR_DIMS;
+    const double sqrt2_over_pi = 0.7978845608028654;
+    const double coeff = 0.044715;
+    for (int64_t i = 0; i < n; i++) {
+        const double value = (double)gate[i];
+        double a;
+        if (act == ORC_ACT_GELU_TANH) {
+            a = 0.5 * value * (1 + tanh(sqrt2_over_pi * (value + coeff * value * value * value)));
+        } else {
+            a = value / (1 + exp(-value));
+        }
+        out[i] = (float)a * up[i];
+    }
+    return ORC_OK;
+}
+
+/* ffn_megakernel_test.go:17-31 (hostGeluMul). */
+int orc_act_gate_mul_bf16(int act, const uint16_t *gate, const uint16_t *up, int64_t n, uint16_t *out) {
+    if (act != ORC_ACT_GELU_TANH && act != ORC_ACT_SILU) return ORC_ERR_BITS;
+    if (n < 0) return ORC_ERR_DIMS;
+    for (int64_t i = 0; i < n; i++) {
+        const float g = orc_bf16_to_f32(gate[i]);
+        const float u = orc_bf16_to_f32(up[i]);
+        float a;
+        if (act == ORC_ACT_GELU_TANH) {
+            const float inner = g + 0.044715f * (g * g * g);
+            const float t = (float)tanh((double)(0.7978845608028654f * inner));
+            a = 0.5f * g * (1.0f + t);
+        } else {
+            const float e = (float)exp((double)(-g));
+            a = g / (1.0f + e);
+        }
+        out[i] = orc_f32_to_bf16(a * u);
+    }
+    return ORC_OK;
+}
+
 int orc_max_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

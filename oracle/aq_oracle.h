@@ -111,6 +111,22 @@ int orc_gather_qmv(const uint16_t *x, int x_rows, const uint32_t *packed, const 
                    int expert_rows, int row_base, int N, int K, int group_size, int bits, double *out_f64,
                    uint16_t *out_bf16);
 
+/* Activations of the fused MLP kernels. */
+#define ORC_ACT_GELU_TANH 1
+#define ORC_ACT_SILU 2
+
+/* act(gate) * up over fp32 vectors, the expectation the reference's fused gate|up kernels are tested
+ * against.  GELU: expectedGELUTanhMultiply, hip_kernels_test.go:8127-8137 -- the tanh-approximated GELU
+ * evaluated in float64 from the fp32 gate, rounded to float32, then one float32 multiply by up.
+ * SiLU: the same composition with gdSilu, gated_delta.go:228 (v / (1 + exp(-v)) in float64). */
+int orc_act_multiply(int act, const float *gate, const float *up, int64_t n, float *out);
+
+/* bf16(act(gate) * up) over bf16 vectors with fp32 internals and one rounding at the store: hostGeluMul,
+ * go/engine/metal/ffn_megakernel_test.go:17-31 (mirror of lthn_gelu_gate_mul_bf16 and of the x-load of
+ * lthn_gelu_qmv_impl.h:24-33); tanh is taken in float64 and rounded to float32 as there.  SiLU keeps the
+ * structure with expf's role played by float64 exp rounded to float32. */
+int orc_act_gate_mul_bf16(int act, const uint16_t *gate, const uint16_t *up, int64_t n, uint16_t *out);
+
 /* Number of hardware threads OpenMP would use (for reporting). */
 int orc_max_threads(void);
 

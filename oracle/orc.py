@@ -171,5 +171,27 @@ def gather_qmv(x_u16, x_rows, packed_u32, scales_u16, biases_u16, lhs, rhs, rout
     return o64[:routes * N].reshape(routes, N), o16[:routes * N].reshape(routes, N)
 
 
+ACT_GELU_TANH = 1
+ACT_SILU = 2
+
+
+def act_multiply(act, gate_f32, up_f32):
+    g = np.ascontiguousarray(gate_f32, dtype=np.float32)
+    u = np.ascontiguousarray(up_f32, dtype=np.float32)
+    assert g.shape == u.shape
+    out = np.zeros(g.shape, dtype=np.float32)
+    _check(lib().orc_act_multiply(act, _p(g), _p(u), ctypes.c_int64(g.size), _p(out)))
+    return out
+
+
+def act_gate_mul_bf16(act, gate_u16, up_u16):
+    g = np.ascontiguousarray(gate_u16, dtype=np.uint16)
+    u = np.ascontiguousarray(up_u16, dtype=np.uint16)
+    assert g.shape == u.shape
+    out = np.zeros(g.shape, dtype=np.uint16)
+    _check(lib().orc_act_gate_mul_bf16(act, _p(g), _p(u), ctypes.c_int64(g.size), _p(out)))
+    return out
+
+
 def max_threads():
     return int(lib().orc_max_threads())

@@ -141,6 +141,27 @@ def hw_fixture_q4_g64_tokens16():
                 codes=codes, rows=rows, cols=cols, group_size=gs, bits=4, tokens=batch, tol=0.001)
 
 
+def hw_fixture_q4_gelu_cols2560(group_size):
+    """testHIPHardwareMLXAffineQ4GELUTanhCols2560 (go/engine/hip/hip_hardware_test.go:2318-2407): rows=32,
+    cols=2560, 4 bit, gate built with (valueStride 5, scaleBase 2^-9), up with (7, 0.00146484375); the
+    reference accepts the device result within 0.03 of gelu_tanh(gate)*up."""
+    rows, cols, bits = 32, 2560, 4
+    groups = cols // group_size
+    x = np.array([np.float32((c % 23) - 11) / np.float32(128) for c in range(cols)], dtype=np.float32)
+
+    def make(stride, base):
+        r = np.arange(rows).reshape(-1, 1)
+        c = np.arange(cols).reshape(1, -1)
+        codes = ((r * stride + c * (stride + 2)) & 0x0F).astype(np.uint32)
+        g = np.arange(groups).reshape(1, -1)
+        s = (np.float32(base) * ((r + g) % 7 + 1).astype(np.float32)).astype(np.float32)
+        b = (-np.float32(base) * ((r + g) % 3 + 1).astype(np.float32)).astype(np.float32)
+        return dict(packed=pack_codes_fast(codes, bits), scales=f32_to_bf16_bits(s), biases=f32_to_bf16_bits(b), codes=codes)
+
+    return dict(x=x, gate=make(5, 0.001953125), up=make(7, 0.00146484375), rows=rows, cols=cols, group_size=group_size,
+                bits=bits, tol=0.03)
+
+
 def synthetic_float32(n, salt):
     """metal test helper syntheticFloat32 (go/engine/metal/test_helpers_test.go:54-60)."""
     i = np.arange(n, dtype=np.int64)
