@@ -373,6 +373,23 @@ def main():
         us_unfused = time_us(moe_unfused)
         us = time_us(moe_fused)
         moe_kernel = ctx.last_variant(0)
+
+        # the whole routed block on the device: scores -> router -> gathers -> combine, no host visit
+        rng_l = np.random.Generator(np.random.PCG64(F.BASE_SEED + 78))
+        d_logits = ctx.to_device(rng_l.normal(0.0, 1.0, size=(TOK, E)).astype(np.float32))
+        d_ids, d_wts, d_tor = ctx.alloc(routes * 4), ctx.alloc(routes * 4), ctx.alloc(routes * 4)
+        y_out = ctx.alloc(TOK * DM * 2)
+
+        def moe_block():
+            ctx.moe_route(d_logits, TOK, E, TOPK, d_ids, d_wts, d_tor)
+            ctx.gather_qmv_gate_up(xt, dgu[0], dgu[1], dgu[2], d_tor, d_ids, yh, routes, TOK, DM, DFF, E, 2 * DFF, 0, DFF,
+                                   GROUP, BITS, aq_mi355.AQ_ACT_GELU_TANH)
+            ctx.gather_qmv(yh, dd[0], dd[1], dd[2], d_route, d_ids, yd, routes, routes, DFF, DM, E, DM, 0, GROUP, BITS)
+            ctx.moe_combine(yd, d_wts, y_out, TOK, TOPK, DM)
+
+        us_block = time_us(moe_block)
+        for t in (d_logits, d_ids, d_wts, d_tor, y_out):
+            t.free()
         per_route = 2 * qmv_bytes(DM, DFF) + qmv_bytes(DFF, DM)
         distinct = len(set(rhs.tolist()))
         # bytes of the distinct experts touched, each expert's three matrices counted once
@@ -380,6 +397,7 @@ def main():
         gather = {"experts": E, "tokens": TOK, "top_k": TOPK, "routes": routes, "distinct_experts": distinct,
                   "us_per_moe_block": round(us, 3), "launches": 2,
                   "us_per_moe_block_unfused": round(us_unfused, 3), "launches_unfused": 4,
+                  "us_per_moe_block_with_router_and_combine": round(us_block, 3), "launches_with_router_and_combine": 4,
                   "GBps_route_bytes": round(routes * per_route / us / 1e3, 1),
                   "pct_of_hbm_peak": round(routes * per_route / us / 1e3 / HBM_PEAK_GBPS * 100, 2),
                   "GBps_distinct_expert_bytes": round(distinct * expert_bytes / us / 1e3, 1),

@@ -22,6 +22,9 @@ AQ_ERR_NODEVICE = -6
 AQ_ERR_SIZE = -7
 AQ_OUT_F32 = 0x1
 
+AQ_IN_F32 = 2
+AQ_LOGITS_BF16 = 4
+AQ_BF16_STEPS = 8
 AQ_ACT_GELU_TANH = 1
 AQ_ACT_SILU = 2
 OP_QMV = 0
@@ -65,6 +68,8 @@ PROTOTYPES = {
     "aq_gather_qmv_act": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i,
                                _u]),
     "aq_act_mul": (_i, [_vp, _vp, _vp, _vp, _c.c_int64, _i]),
+    "aq_moe_route": (_i, [_vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _u]),
+    "aq_moe_combine": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _u]),
     "aq_dequant_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _c.c_int64, _i, _i, _i]),
     "aq_matvec_host": (_i, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _i, _i, _i, _i, _vp, _sz]),
     "aq_proj_quant_matmul_host": (_i, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _i, _i, _i, _i, _i]),
@@ -265,6 +270,15 @@ class Context:
 
     def act_mul(self, gate, up, y, n, act=AQ_ACT_GELU_TANH):
         self._check(self.lib.aq_act_mul(self.handle, _ptr(gate), _ptr(up), _ptr(y), n, act))
+
+    def moe_route(self, logits, rows, num_experts, top_k, ids, weights, token_of_route=None, expert_scales=None,
+                  normalise=True, flags=0):
+        self._check(self.lib.aq_moe_route(self.handle, _ptr(logits), rows, num_experts, top_k, _ptr(expert_scales),
+                                          1 if normalise else 0, _ptr(ids), _ptr(weights), _ptr(token_of_route), flags))
+
+    def moe_combine(self, route_rows, weights, out, rows, top_k, n, flags=0):
+        self._check(self.lib.aq_moe_combine(self.handle, _ptr(route_rows), _ptr(weights), _ptr(out), rows, top_k, n,
+                                            flags))
 
     def dequant_f32(self, w, s, b, out, N, K, group_size=64, bits=4):
         self._check(self.lib.aq_dequant_f32(self.handle, _ptr(w), _ptr(s), _ptr(b), _ptr(out), N, K, group_size,

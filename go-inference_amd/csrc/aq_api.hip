@@ -859,6 +859,62 @@ int aq_gather_qmv_act(aq_ctx* ctx, const void* gate_x, const void* up_x, const v
                          expert_rows, row_base, group_size, bits, flags);
 }
 
+int aq_moe_route(aq_ctx* ctx, const void* logits, int rows, int num_experts, int top_k, const float* expert_scales,
+                 int normalise_top_k, int32_t* ids, float* weights, int32_t* token_of_route, unsigned flags) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_moe_route: ctx is null");
+    if (rows < 0) return fail(AQ_ERR_SHAPE, "aq_moe_route: rows must be non-negative");
+    // rocmReferenceRouteExperts (moe_quant_reference.go:28-33): logits required, 0 < top-k <= experts
+    if (num_experts <= 0) return fail(AQ_ERR_SHAPE, "aq_moe_route: router logits are required");
+    if (top_k <= 0 || top_k > num_experts) return fail(AQ_ERR_SHAPE, "aq_moe_route: top-k must be within the expert count");
+    if (num_experts > aq::kMoeMaxExperts || top_k > aq::kMoeMaxTopK)
+        return fail(AQ_ERR_UNSUPPORTED, "aq_moe_route: at most %d experts and top-%d", aq::kMoeMaxExperts, aq::kMoeMaxTopK);
+    if (rows == 0) return AQ_OK;
+    if (!logits || !ids || !weights) return fail(AQ_ERR_ARG, "aq_moe_route: null operand");
+    const bool lb = (flags & AQ_LOGITS_BF16) != 0;
+    if (!aligned(logits, lb ? 2 : 4) || !aligned(ids, 4) || !aligned(weights, 4) ||
+        (expert_scales && !aligned(expert_scales, 4)) || (token_of_route && !aligned(token_of_route, 4)))
+        return fail(AQ_ERR_ARG, "aq_moe_route: operand pointer is not element-aligned");
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    aq::MoeRouteArgs a{};
+    a.logits = logits;
+    a.expert_scales = expert_scales;
+    a.ids = ids;
+    a.weights = weights;
+    a.token_of_route = token_of_route;
+    a.rows = rows;
+    a.num_experts = num_experts;
+    a.top_k = top_k;
+    a.normalise = normalise_top_k ? 1 : 0;
+    a.logits_bf16 = lb ? 1 : 0;
+    AQ_HIP(aq::moe_route_launch(a, ctx->stream), "hipLaunchKernel");
+    return AQ_OK;
+}
+
+int aq_moe_combine(aq_ctx* ctx, const void* route_rows, const float* weights, void* out, int rows, int top_k, int n,
+                   unsigned flags) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_moe_combine: ctx is null");
+    if (rows < 0 || n < 0) return fail(AQ_ERR_SHAPE, "aq_moe_combine: rows and n must be non-negative");
+    if (top_k <= 0) return fail(AQ_ERR_SHAPE, "aq_moe_combine: top-k must be positive");
+    if (rows == 0 || n == 0) return AQ_OK;
+    if (!route_rows || !weights || !out) return fail(AQ_ERR_ARG, "aq_moe_combine: null operand");
+    const bool in_f32 = (flags & AQ_IN_F32) != 0, out_f32 = (flags & AQ_OUT_F32) != 0;
+    if (!aligned(route_rows, in_f32 ? 4 : 2) || !aligned(weights, 4) || !aligned(out, out_f32 ? 4 : 2))
+        return fail(AQ_ERR_ARG, "aq_moe_combine: operand pointer is not element-aligned");
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    aq::MoeCombineArgs a{};
+    a.route_rows = route_rows;
+    a.weights = weights;
+    a.out = out;
+    a.rows = rows;
+    a.top_k = top_k;
+    a.n = n;
+    a.in_f32 = in_f32 ? 1 : 0;
+    a.out_f32 = out_f32 ? 1 : 0;
+    a.bf16_steps = (flags & AQ_BF16_STEPS) ? 1 : 0;
+    AQ_HIP(aq::moe_combine_launch(a, ctx->stream), "hipLaunchKernel");
+    return AQ_OK;
+}
+
 int aq_dequant_f32(aq_ctx* ctx, const void* packed, const void* scales, const void* biases, float* out_f32, int64_t N,
                    int K, int group_size, int bits) {
     if (!ctx) return fail(AQ_ERR_ARG, "aq_dequant_f32: ctx is null");

@@ -80,20 +80,27 @@ __device__ __forceinline__ void unpack8_word(uint32_t w, uint32_t p[2]) {
 
 // Activations of the fused kernels.  1: tanh-approximated GELU with the operation order of
 // rocm_gelu_tanh_value (go/engine/hip/kernels/common/math.hipinc:3-9); 2: SiLU, v / (1 + exp(-v))
-// (go/model/attn/gated_delta.go:228).  Every step is an explicit fp32 operation, so that each kernel
-// that inlines this computes the same bits for the same input.
+// (go/model/attn/gated_delta.go:228).  Contraction is off, so every step is one fp32 operation and each
+// kernel that inlines this computes the same bits for the same input.
 __device__ __forceinline__ float act_value(int act, float v) {
-    if (act == 2) return __fdiv_rn(v, __fadd_rn(1.0f, expf(-v)));
-    const float v3 = __fmul_rn(__fmul_rn(v, v), v);
-    const float arg = __fmul_rn(0.7978845608028654f, __fmaf_rn(0.044715f, v3, v));
-    return __fmul_rn(__fmul_rn(0.5f, v), __fadd_rn(1.0f, tanhf(arg)));
+#pragma clang fp contract(off)
+    if (act == 2) return v / (1.0f + expf(-v));
+    const float v3 = (v * v) * v;
+    const float arg = 0.7978845608028654f * __builtin_fmaf(0.044715f, v3, v);
+    return (0.5f * v) * (1.0f + tanhf(arg));
+}
+
+__device__ __forceinline__ float fmul_unfused(float a, float b) {
+#pragma clang fp contract(off)
+    return a * b;
 }
 
 // bf16(act(gate) * up): fp32 inside, one rounding at the end, as lthn_gelu_gate_mul_one
 // (go/engine/metal/kernels/moe/lthn_gelu_qmv_impl.h:24-33).
 __device__ __forceinline__ uint32_t act_mul_bf16x2(uint32_t g, uint32_t u, int act) {
-    const float lo = __fmul_rn(act_value(act, bf16_bits_to_f32(g & 0xffffu)), bf16_bits_to_f32(u & 0xffffu));
-    const float hi = __fmul_rn(act_value(act, bf16_bits_to_f32(g >> 16)), bf16_bits_to_f32(u >> 16));
+#pragma clang fp contract(off)
+    const float lo = act_value(act, bf16_bits_to_f32(g & 0xffffu)) * bf16_bits_to_f32(u & 0xffffu);
+    const float hi = act_value(act, bf16_bits_to_f32(g >> 16)) * bf16_bits_to_f32(u >> 16);
     return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
 }
 __device__ __forceinline__ uint4 act_mul_bf16x8(uint4 g, uint4 u, int act) {

@@ -135,6 +135,29 @@ const QmvVariant* qmvs_variant(int idx);
 bool qmvs_plan(const QmvArgs& a, int bits, int group_size, bool gather, int cu_count, int forced_idx, StreamPlan* out);
 hipError_t qmvs_launch(const StreamPlan& p, const QmvArgs& a, hipStream_t stream);
 
+// MoE router and combine (aq_moe.hip).
+constexpr int kMoeMaxExperts = 1024;
+constexpr int kMoeMaxTopK = 64;
+struct MoeRouteArgs {
+    const void* logits;           // [rows, num_experts] f32 or bf16
+    const float* expert_scales;   // [num_experts] or nullptr
+    int32_t* ids;                 // [rows, top_k]
+    float* weights;               // [rows, top_k]
+    int32_t* token_of_route;      // [rows, top_k] or nullptr
+    int rows, num_experts, top_k;
+    int normalise;                // 1: softmax over the selected scores; 0: softmax over all, gathered
+    int logits_bf16;
+};
+struct MoeCombineArgs {
+    const void* route_rows;  // [rows * top_k, n] bf16 or f32
+    const float* weights;    // [rows * top_k]
+    void* out;               // [rows, n] bf16 or f32
+    int rows, top_k, n;
+    int in_f32, out_f32, bf16_steps;
+};
+hipError_t moe_route_launch(const MoeRouteArgs& a, hipStream_t stream);
+hipError_t moe_combine_launch(const MoeCombineArgs& a, hipStream_t stream);
+
 // Any-width (2..8 bit, codes may straddle words), any-group fallback.
 hipError_t qmv_generic_launch(const QmvArgs& a, int bits, int group_size, bool gather, hipStream_t stream);
 

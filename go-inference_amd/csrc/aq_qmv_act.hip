@@ -76,9 +76,10 @@ __global__ __launch_bounds__(256) void act_mul_bf16_kernel(const uint16_t* __res
 
 __global__ __launch_bounds__(256) void act_mul_f32_kernel(const float* __restrict__ g, const float* __restrict__ u,
                                                           void* __restrict__ y, int64_t n, int act, int out_f32) {
+#pragma clang fp contract(off)
     const int64_t stride = (int64_t)gridDim.x * 256;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
-        const float v = __fmul_rn(act_value(act, g[i]), u[i]);
+        const float v = act_value(act, g[i]) * u[i];
         if (out_f32) {
             static_cast<float*>(y)[i] = v;
         } else {

@@ -292,7 +292,7 @@ __device__ __forceinline__ void qmv_dot2_body(const QmvArgs& a, const int bx) {
 #pragma unroll
         for (int m = 0; m < M; m++) {
             float tot = wave_sum(acc[r][m]);
-            if constexpr (FUSE == 1) tot = act_value(a.act, tot) * wave_sum(acc[r + R][m]);
+            if constexpr (FUSE == 1) tot = fmul_unfused(act_value(a.act, tot), wave_sum(acc[r + R][m]));
             if (!route_ok) tot = 0.0f;
             const int row = row_first + r;
             if (lane == 0 && row < N) {

@@ -43,7 +43,10 @@ extern "C" {
 #define AQ_ERR_NODEVICE (-6)    /* no usable gfx950 device                               */
 #define AQ_ERR_SIZE (-7)        /* a host buffer length disagrees with the dims          */
 
-#define AQ_OUT_F32 0x1u /* y is float32 instead of bf16 (validation of the fp32 accumulator) */
+#define AQ_OUT_F32 0x1u     /* y is float32 instead of bf16 (validation of the fp32 accumulator) */
+#define AQ_IN_F32 0x2u      /* aq_moe_combine: the route rows are float32 instead of bf16           */
+#define AQ_LOGITS_BF16 0x4u /* aq_moe_route: the router scores are bf16 instead of float32          */
+#define AQ_BF16_STEPS 0x8u  /* aq_moe_combine: round every product and partial sum to bf16          */
 
 typedef struct aq_ctx aq_ctx;
 
@@ -84,7 +87,7 @@ int aq_timer_stop(aq_ctx *ctx, float *elapsed_ms); /* records, waits, reports */
  * replays the whole batch with one submission.  Counterpart of the reference's per-step
  * launch batch (hipLaunchKernelContext batching, go/engine/hip/hip_launch.go:240-273,
  * cgoHIPDriver.LaunchKernelBatch go/engine/hip/hip_driver_cgo.go:1137-1190).  Only the
- * kernel entry points (aq_qmv*, aq_qmm, aq_gather_qmv*, aq_act_mul, aq_dequant_f32, aq_fill_zero, aq_d2d)
+ * kernel entry points (aq_qmv*, aq_qmm, aq_gather_qmv*, aq_act_mul, aq_moe_*, aq_dequant_f32, aq_fill_zero, aq_d2d)
  * may be called while capturing; the pointers they were given must stay valid for replays. */
 typedef struct aq_graph aq_graph;
 int aq_capture_begin(aq_ctx *ctx);
@@ -193,6 +196,33 @@ int aq_gather_qmv_act(aq_ctx *ctx, const void *gate_x, const void *up_x, const v
  * (go/engine/hip/hip_transformer_launch.go:3765) / lthn_gelu_gate_mul_bf16, host mirror
  * hostGeluMul (go/engine/metal/ffn_megakernel_test.go:17-31). */
 int aq_act_mul(aq_ctx *ctx, const void *gate, const void *up, void *y, int64_t n, int act);
+
+/* Device MoE router: for each of `rows` tokens, the top_k experts by (score descending, expert id
+ * ascending on ties) and their weights, written where aq_gather_qmv* read them, so no score ever visits the
+ * host.  logits [rows, num_experts] float32 (bf16 with AQ_LOGITS_BF16), device-resident.
+ *   ids            int32 [rows, top_k]   -> the `rhs` of the gathers
+ *   weights        float [rows, top_k]   -> aq_moe_combine
+ *   token_of_route int32 [rows, top_k]   (may be NULL) = the row, i.e. the `lhs` of the gate|up gather
+ * normalise_top_k != 0: weights = softmax over the selected scores (rocm_moe_router,
+ * go/engine/hip/kernels/moe/routing.hipinc:3-77; CPU form rocmReferenceRouteExperts,
+ * go/engine/hip/moe_quant_reference.go:27-78); == 0: softmax over all experts, gathered, not renormalised
+ * (hipQwen3MoERouterSelect, go/engine/hip/hip_qwen3_moe_router.go:25-88).  expert_scales (device float
+ * [num_experts], may be NULL) multiplies each weight by its expert's scale, as
+ * hipGemma4MoEBatchRouteGroups does on the host (go/engine/hip/hip_gemma4_moe.go:294-366) - the D2H copy,
+ * host grouping and chunk upload of that path are what this call removes.  num_experts <= 1024,
+ * top_k <= 64.  A NaN score ranks last; the reference rejects non-finite scores on the host, which a
+ * device-resident router cannot do. */
+int aq_moe_route(aq_ctx *ctx, const void *logits, int rows, int num_experts, int top_k, const float *expert_scales,
+                 int normalise_top_k, int32_t *ids, float *weights, int32_t *token_of_route, unsigned flags);
+
+/* MoE combine: out[row, :n] = sum over rank of route_rows[row*top_k + rank, :n] * weights[row*top_k + rank],
+ * ranks ascending, fp32 (rocm_moe_batch_scatter_routes + rocm_moe_batch_reduce_routes,
+ * go/engine/hip/kernels/moe/routing.hipinc:100-158).  route_rows is the down gather's output: bf16, or
+ * float32 with AQ_IN_F32; out is bf16, or float32 with AQ_OUT_F32.  AQ_BF16_STEPS rounds the weight, every
+ * product and every partial sum to bf16, which reproduces lthn_moe_weighted_sum_bf16 byte for byte
+ * (go/engine/metal/kernels/moe/lthn_moe_weighted_sum.metal:17-38). */
+int aq_moe_combine(aq_ctx *ctx, const void *route_rows, const float *weights, void *out, int rows, int top_k, int n,
+                   unsigned flags);
 
 /* mlxaffine.DequantizeTensor on device (go/model/quant/mlxaffine/mlxaffine.go:178-208):
  * out_f32[N,K] = scale*code + bias, bit-exact with the CPU path. */

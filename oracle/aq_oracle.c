@@ -460,6 +460,90 @@ int orc_act_gate_mul_bf16(int act, const uint16_t *gate, const uint16_t *up, int
     return ORC_OK;
 }
 
+/* moe_quant_reference.go:27-55,268-286; hip_gemma4_moe.go:318-360; hip_qwen3_moe_router.go:33-45,78-85. */
+int orc_moe_route(const float *logits, int rows, int num_experts, int top_k, const float *expert_scales, int normalise,
+                  int32_t *ids, float *weights) {
+    if (rows < 0 || num_experts <= 0 || top_k <= 0 || top_k > num_experts) return ORC_ERR_DIMS;
+    int *sel = (int *)malloc((size_t)top_k * sizeof(int));
+    if (!sel) return ORC_ERR_SIZE;
+    for (int row = 0; row < rows; row++) {
+        const float *sc = logits + (size_t)row * num_experts;
+        for (int e = 0; e < num_experts; e++)
+            if (isnan(sc[e]) || isinf(sc[e])) {
+                free(sel);
+                return ORC_ERR_INDEX;
+            }
+        /* insertion into a list kept in (score desc, id asc) order */
+        int count = 0;
+        for (int e = 0; e < num_experts; e++) {
+            int insert = top_k;
+            for (int r = 0; r < top_k; r++) {
+                if (r >= count || sc[e] > sc[sel[r]] || (sc[e] == sc[sel[r]] && e < sel[r])) {
+                    insert = r;
+                    break;
+                }
+            }
+            if (insert == top_k) continue;
+            for (int r = top_k - 1; r > insert; r--) sel[r] = sel[r - 1];
+            sel[insert] = e;
+            if (count < top_k) count++;
+        }
+        if (normalise) {
+            float max_value = sc[sel[0]];
+            for (int r = 1; r < top_k; r++)
+                if (sc[sel[r]] > max_value) max_value = sc[sel[r]];
+            double sum = 0;
+            for (int r = 0; r < top_k; r++) {
+                const double ex = exp((double)(sc[sel[r]] - max_value));
+                weights[(size_t)row * top_k + r] = (float)ex;
+                sum += ex;
+            }
+            for (int r = 0; r < top_k; r++)
+                weights[(size_t)row * top_k + r] = (float)((double)weights[(size_t)row * top_k + r] / sum);
+        } else {
+            float max_logit = -INFINITY;
+            for (int e = 0; e < num_experts; e++)
+                if (sc[e] > max_logit) max_logit = sc[e];
+            double total = 0;
+            for (int e = 0; e < num_experts; e++) total += exp((double)(sc[e] - max_logit));
+            if (total == 0) total = 1;
+            for (int r = 0; r < top_k; r++)
+                weights[(size_t)row * top_k + r] = (float)(exp((double)(sc[sel[r]] - max_logit)) / total);
+        }
+        for (int r = 0; r < top_k; r++) {
+            ids[(size_t)row * top_k + r] = sel[r];
+            if (expert_scales) weights[(size_t)row * top_k + r] *= expert_scales[sel[r]];
+        }
+    }
+    free(sel);
+    return ORC_OK;
+}
+
+/* routing.hipinc:100-158; lthn_moe_weighted_sum.metal:17-38. */
+int orc_moe_combine(const float *route_rows, const float *weights, int rows, int top_k, int n, int bf16_steps,
+                    float *out) {
+    if (rows < 0 || top_k <= 0 || n < 0) return ORC_ERR_DIMS;
+    for (int row = 0; row < rows; row++) {
+        for (int c = 0; c < n; c++) {
+            float acc = 0.0f;
+            for (int r = 0; r < top_k; r++) {
+                const size_t pair = (size_t)row * top_k + r;
+                const float y = route_rows[pair * n + c];
+                if (bf16_steps) {
+                    const float w = orc_bf16_to_f32(orc_f32_to_bf16(weights[pair]));
+                    const float scaled = orc_bf16_to_f32(orc_f32_to_bf16(y * w));
+                    acc = r == 0 ? scaled : orc_bf16_to_f32(orc_f32_to_bf16(acc + scaled));
+                } else {
+                    const float scaled = y * weights[pair];
+                    acc = acc + scaled;
+                }
+            }
+            out[(size_t)row * n + c] = acc;
+        }
+    }
+    return ORC_OK;
+}
+
 int orc_max_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

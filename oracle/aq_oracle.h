@@ -127,6 +127,25 @@ int orc_act_multiply(int act, const float *gate, const float *up, int64_t n, flo
  * structure with expf's role played by float64 exp rounded to float32. */
 int orc_act_gate_mul_bf16(int act, const uint16_t *gate, const uint16_t *up, int64_t n, uint16_t *out);
 
+/* MoE router, one call over `rows` token rows.  Selection: the top_k experts by (score descending, expert
+ * id ascending) -- rocmReferenceRouteExperts' stable sort, go/engine/hip/moe_quant_reference.go:27-55, the
+ * same order hipGemma4MoEBatchRouteGroups' insertion keeps (hip_gemma4_moe.go:318-342).
+ * normalise != 0: softmaxFloat32 over the selected scores (moe_quant_reference.go:268-286: float64 exp of
+ * the float32 difference, stored as float32, divided by the float64 sum); == 0: hipQwen3MoERouterSelect
+ * with normalise=false (hip_qwen3_moe_router.go:33-45,78-85): float64 softmax over all experts, gathered.
+ * expert_scales (may be NULL): weight = prob * scale in float32, hip_gemma4_moe.go:356-360.
+ * Rejects non-finite scores (ORC_ERR_INDEX) as both Go routers do. */
+int orc_moe_route(const float *logits, int rows, int num_experts, int top_k, const float *expert_scales, int normalise,
+                  int32_t *ids, float *weights);
+
+/* MoE combine.  bf16_steps == 0: out[row,c] = sum over rank (ascending) of float32(in * weight), float32
+ * adds: rocm_moe_batch_scatter_routes + rocm_moe_batch_reduce_routes, kernels/moe/routing.hipinc:100-158.
+ * bf16_steps != 0: lthn_moe_weighted_sum_bf16, go/engine/metal/kernels/moe/lthn_moe_weighted_sum.metal:17-38
+ * (weight, each product and each partial sum rounded to bf16).  in/out are float32 here; the caller
+ * widens / narrows bf16 storage. */
+int orc_moe_combine(const float *route_rows, const float *weights, int rows, int top_k, int n, int bf16_steps,
+                    float *out);
+
 /* Number of hardware threads OpenMP would use (for reporting). */
 int orc_max_threads(void);
 

@@ -193,5 +193,24 @@ def act_gate_mul_bf16(act, gate_u16, up_u16):
     return out
 
 
+def moe_route(logits_f32, top_k, expert_scales=None, normalise=True):
+    """logits [rows, experts] -> (ids int32 [rows, top_k], weights float32 [rows, top_k])."""
+    lg = np.ascontiguousarray(logits_f32, dtype=np.float32)
+    rows, experts = lg.shape
+    sc = None if expert_scales is None else np.ascontiguousarray(expert_scales, dtype=np.float32)
+    ids = np.zeros((rows, max(top_k, 1)), dtype=np.int32)
+    w = np.zeros((rows, max(top_k, 1)), dtype=np.float32)
+    _check(lib().orc_moe_route(_p(lg), rows, experts, top_k, _p(sc), 1 if normalise else 0, _p(ids), _p(w)))
+    return ids, w
+
+
+def moe_combine(route_rows_f32, weights_f32, rows, top_k, n, bf16_steps=False):
+    y = np.ascontiguousarray(route_rows_f32, dtype=np.float32).reshape(rows * top_k, n)
+    w = np.ascontiguousarray(weights_f32, dtype=np.float32).reshape(-1)
+    out = np.zeros((rows, n), dtype=np.float32)
+    _check(lib().orc_moe_combine(_p(y), _p(w), rows, top_k, n, 1 if bf16_steps else 0, _p(out)))
+    return out
+
+
 def max_threads():
     return int(lib().orc_max_threads())

@@ -448,3 +448,111 @@ def test_gelu_hardware_fixture_oracle_vs_independent_float64(orc, gs):
     ref = torch.nn.functional.gelu(torch.from_numpy(g64), approximate="tanh").numpy() * u64
     assert np.abs(want - ref).max() <= 1e-5     # far inside the reference's own 0.03
     assert np.abs(ref).max() > 1e-3             # the fixture's outputs are small but not trivial
+
+
+# ---- MoE router and combine ---------------------------------------------------------------------------
+
+def _independent_route(logits, top_k, scales=None, normalise=True):
+    """numpy restatement by another route: lexsort for the order, scipy for the softmax."""
+    from scipy.special import softmax
+    lg = np.asarray(logits, dtype=np.float32)
+    ids = np.stack([np.lexsort((np.arange(lg.shape[1]), -r.astype(np.float64)))[:top_k] for r in lg]).astype(np.int32)
+    sel = np.take_along_axis(lg.astype(np.float64), ids, axis=1)
+    w = softmax(sel, axis=1) if normalise else np.take_along_axis(softmax(lg.astype(np.float64), axis=1), ids, axis=1)
+    if scales is not None:
+        w = w * np.asarray(scales, dtype=np.float64)[ids]
+    return ids, w
+
+
+def test_moe_route_reference_known_answers(orc):
+    # go/engine/hip/hip_qwen3_moe_router_test.go:19-58: a two-way softmax is a sigmoid
+    ids, w = orc.moe_route(np.array([[1, 3, 2, 0]], np.float32), 2, normalise=True)
+    assert ids.tolist() == [[1, 2]]
+    s1 = 1 / (1 + math.exp(-1))
+    assert abs(w[0, 0] - s1) < 1e-7 and abs(w[0, 1] - (1 - s1)) < 1e-7
+    assert abs(w.sum() - 1) < 1e-6
+    ids, w = orc.moe_route(np.array([[1, 3, 2, 0]], np.float32), 2, normalise=False)
+    total = math.exp(1) + math.exp(3) + math.exp(2) + math.exp(0)
+    assert ids.tolist() == [[1, 2]]
+    assert abs(w[0, 0] - math.exp(3) / total) < 1e-7 and abs(w[0, 1] - math.exp(2) / total) < 1e-7
+    assert w.sum() < 1.0
+    # :64-73 both orders select the same experts
+    lg = np.array([[-2, 5, 0.5, 3, -1, 1.2]], np.float32)
+    assert orc.moe_route(lg, 3, normalise=True)[0].tolist() == orc.moe_route(lg, 3, normalise=False)[0].tolist() == [[1, 3, 5]]
+    # go/engine/hip/hip_moe_launch_test.go:1861-1882
+    assert orc.moe_route(np.array([[0.1, 2, 1, -1]], np.float32), 2)[0].tolist() == [[1, 2]]
+
+
+def test_moe_route_gemma_batch_fixture_with_expert_scales(orc):
+    """TestHIPGemma4MoEBatchRouteGroups_Good_MatchesReference (go/engine/hip/hip_moe_launch_test.go:1369-1400):
+    weight = prob * expert scale; row 1 holds a tie (5, 5) that the lower expert id wins."""
+    scores = np.array([[1, 4, 2, 3], [5, 5, -1, 0], [-2, 1, 7, 3]], np.float32)
+    scales = np.array([1, 0.5, 2, 1.5], np.float32)
+    ids, w = orc.moe_route(scores, 2, expert_scales=scales)
+    assert ids.tolist() == [[1, 3], [0, 1], [2, 3]]
+    wi, ww = _independent_route(scores, 2, scales)
+    assert np.array_equal(ids, wi) and np.abs(w - ww).max() < 1e-7
+    assert abs(w[1, 0] - 0.5 * 1.0) < 1e-7 and abs(w[1, 1] - 0.5 * 0.5) < 1e-7   # equal scores: 1/2 each, scaled
+
+
+def test_moe_route_hardware_fixture_128_experts_with_ties(orc):
+    """TestHIPHardwareMoERouterParallel_Good (go/engine/hip/hip_hardware_test.go:1197-1220): logits
+    (e*37 % 23)/8 over 128 experts, top 8 -- every score value repeats five or six times."""
+    lg = np.array([[np.float32((e * 37) % 23) / np.float32(8) for e in range(128)]], np.float32)
+    for norm in (True, False):
+        ids, w = orc.moe_route(lg, 8, normalise=norm)
+        wi, ww = _independent_route(lg, 8, normalise=norm)
+        assert np.array_equal(ids, wi)
+        assert np.abs(w - ww).max() < 1e-7
+    ids, _ = orc.moe_route(lg, 8)
+    sel = lg[0, ids[0]]
+    assert np.all(np.diff(sel) <= 0)
+    for a, b in zip(range(7), range(1, 8)):
+        if sel[a] == sel[b]:
+            assert ids[0, a] < ids[0, b]
+
+
+def test_moe_route_random_rows_and_rejections(orc):
+    rng = np.random.default_rng(5)
+    lg = rng.normal(0, 2, (37, 200)).astype(np.float32)
+    lg[:, 7] = lg[:, 150]  # ties across lanes
+    sc = rng.uniform(0.5, 2, 200).astype(np.float32)
+    for norm in (True, False):
+        ids, w = orc.moe_route(lg, 6, sc, norm)
+        wi, ww = _independent_route(lg, 6, sc, norm)
+        assert np.array_equal(ids, wi) and np.abs(w - ww).max() < 2e-7
+    for bad in (np.nan, np.inf, -np.inf):
+        x = lg.copy()
+        x[3, 5] = bad
+        with pytest.raises(orc.OracleError):
+            orc.moe_route(x, 6)
+    with pytest.raises(orc.OracleError):
+        orc.moe_route(lg, 0)
+    with pytest.raises(orc.OracleError):
+        orc.moe_route(lg, 201)
+
+
+def test_moe_combine_fp32_and_bf16_steps(orc):
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(6)
+    rows, top_k, n = 5, 8, 33
+    y = rng.normal(0, 1, (rows * top_k, n)).astype(np.float32)
+    w = rng.uniform(0, 1, rows * top_k).astype(np.float32)
+    got = orc.moe_combine(y, w, rows, top_k, n)
+    # float32 products summed in rank order: the library's float32 arithmetic, rank by rank
+    ty, tw = torch.from_numpy(y).reshape(rows, top_k, n), torch.from_numpy(w).reshape(rows, top_k, 1)
+    acc = torch.zeros(rows, n)
+    for r in range(top_k):
+        acc = acc + ty[:, r] * tw[:, r]
+    assert np.array_equal(got, acc.numpy())
+    assert np.abs(got - (y.reshape(rows, top_k, n).astype(np.float64) * w.reshape(rows, top_k, 1)).sum(1)).max() < 1e-5
+    # bf16 steps: torch.bfloat16 rounds after every multiply and add
+    yb = torch.from_numpy(y).bfloat16().reshape(rows, top_k, n)
+    wb = torch.from_numpy(w).bfloat16().reshape(rows, top_k, 1)
+    accb = yb[:, 0] * wb[:, 0]
+    for r in range(1, top_k):
+        accb = accb + yb[:, r] * wb[:, r]
+    gotb = orc.moe_combine(yb.float().numpy().reshape(rows * top_k, n), w, rows, top_k, n, bf16_steps=True)
+    assert np.array_equal(F.f32_to_bf16_bits(gotb), accb.view(torch.int16).numpy().view(np.uint16))
+    # one route with weight one is the identity
+    assert np.array_equal(orc.moe_combine(y[:3], np.ones(3, np.float32), 3, 1, n), y[:3])
