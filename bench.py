@@ -443,6 +443,48 @@ def main():
         for t in (hg, hu, hh):
             t.free()
 
+    # ---- extra: lm_head (vocabulary projection) with the argmax / top-k fused on the device ---------
+    head = None
+    if not args.no_extras:
+        HN, HK, HG = 262144, 1536, 32     # the head the reference times (go/engine/metal/qmv_head_bench_test.go:14-57)
+        hw = F.synthetic_affine(HN, HK, BITS, HG, seed=F.BASE_SEED + 60)
+        pool = [tuple(ctx.to_device(t) for t in hw)]
+        second = tuple(ctx.alloc(t.nbytes) for t in pool[0])
+        for d, t in zip(second, pool[0]):
+            ctx._check(ctx.lib.aq_d2d(ctx.handle, d.ptr, t.ptr, t.nbytes))
+        pool.append(second)
+        hx = ctx.to_device(F.synthetic_x(1, HK, seed=F.BASE_SEED + 1300))
+        h_logits, h_best, h_scores, h_top = ctx.alloc(HN * 2), ctx.alloc(8), ctx.alloc(HN * 8), ctx.alloc(40 * 8)
+        head_bytes = HN * HK * BITS // 8 + 2 * HN * (HK // HG) * 2 + HK * 2
+
+        def head_time(fn, n=40):
+            for i in range(4):
+                fn(pool[i % 2])
+            ctx.sync()
+            ctx.timer_start()
+            for i in range(n):
+                fn(pool[i % 2])
+            return ctx.timer_stop() * 1e3 / n
+
+        us_logits = head_time(lambda t: ctx.qmv(hx, t[0], t[1], t[2], h_logits, 1, HK, HN, HG, BITS))
+        k_logits = ctx.last_variant(0)
+        us_greedy = head_time(lambda t: ctx.qmv_greedy(hx, t[0], t[1], t[2], h_best, 1, HK, HN, HG, BITS))
+
+        def topk40(t):
+            ctx.qmv_scores(hx, t[0], t[1], t[2], h_scores, 1, HK, HN, HG, BITS)
+            ctx.packed_topk(h_scores, HN, 40, h_top)
+
+        us_topk = head_time(topk40)
+        head = {"N": HN, "K": HK, "group": HG, "bits": BITS, "weight_bytes": head_bytes,
+                "logits": {"us": round(us_logits, 2), "GBps": round((head_bytes + HN * 2) / us_logits / 1e3, 1), "kernel": k_logits},
+                "greedy_fused": {"us": round(us_greedy, 2), "GBps": round(head_bytes / us_greedy / 1e3, 1),
+                                 "pct_of_hbm_peak": round(head_bytes / us_greedy / 1e3 / HBM_PEAK_GBPS * 100, 2)},
+                "scores_then_top40": {"us": round(us_topk, 2), "GBps": round((head_bytes + HN * 8) / us_topk / 1e3, 1)},
+                "note": "lm_head 262144 x 1536, 4-bit group 32 (251 MB), two copies alternated; greedy_fused = aq_qmv_greedy "
+                        "(8 bytes out); scores_then_top40 = aq_qmv_scores + aq_packed_topk"}
+        for t in pool[0] + pool[1] + (hx, h_logits, h_best, h_scores, h_top):
+            t.free()
+
     # ---- CPU baseline: the reference's CPU path (oracle port of matNTQuantHost), bounded sample ----
     cpu = None
     if not args.no_cpu:
@@ -500,6 +542,7 @@ def main():
         "small_m": small_m,
         "gather": gather,
         "mlp_fused": mlp,
+        "lm_head": head,
     }
     print(json.dumps(out))
     ctx.close()

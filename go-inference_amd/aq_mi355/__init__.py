@@ -70,6 +70,11 @@ PROTOTYPES = {
     "aq_act_mul": (_i, [_vp, _vp, _vp, _vp, _c.c_int64, _i]),
     "aq_moe_route": (_i, [_vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _u]),
     "aq_moe_combine": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _u]),
+    "aq_qmv_greedy": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i]),
+    "aq_qmv_scores": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i]),
+    "aq_packed_topk": (_i, [_vp, _vp, _c.c_int64, _i, _vp]),
+    "aq_pack_best": (_c.c_uint64, [_f, _i]),
+    "aq_unpack_best": (_i, [_c.c_uint64, _f, _i, _c.POINTER(_i), _c.POINTER(_f)]),
     "aq_dequant_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _c.c_int64, _i, _i, _i]),
     "aq_matvec_host": (_i, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _i, _i, _i, _i, _vp, _sz]),
     "aq_proj_quant_matmul_host": (_i, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _i, _i, _i, _i, _i]),
@@ -280,6 +285,17 @@ class Context:
         self._check(self.lib.aq_moe_combine(self.handle, _ptr(route_rows), _ptr(weights), _ptr(out), rows, top_k, n,
                                             flags))
 
+    def qmv_greedy(self, x, w, s, b, best, M, K, N, group_size=64, bits=4, suppress=None, suppress_count=0):
+        self._check(self.lib.aq_qmv_greedy(self.handle, _ptr(x), _ptr(w), _ptr(s), _ptr(b), _ptr(suppress), suppress_count,
+                                           _ptr(best), M, K, N, group_size, bits))
+
+    def qmv_scores(self, x, w, s, b, scores, M, K, N, group_size=64, bits=4, suppress=None, suppress_count=0):
+        self._check(self.lib.aq_qmv_scores(self.handle, _ptr(x), _ptr(w), _ptr(s), _ptr(b), _ptr(suppress), suppress_count,
+                                           _ptr(scores), M, K, N, group_size, bits))
+
+    def packed_topk(self, scores, count, top_k, out):
+        self._check(self.lib.aq_packed_topk(self.handle, _ptr(scores), count, top_k, _ptr(out)))
+
     def dequant_f32(self, w, s, b, out, N, K, group_size=64, bits=4):
         self._check(self.lib.aq_dequant_f32(self.handle, _ptr(w), _ptr(s), _ptr(b), _ptr(out), N, K, group_size,
                                             bits))
@@ -310,6 +326,20 @@ class Context:
                                                        scales.size, biases.ctypes.data, biases.size, M, K, N,
                                                        group_size, bits))
         return out.reshape(M, N)
+
+
+def pack_best(score, token):
+    return int(load().aq_pack_best(score, token))
+
+
+def unpack_best(packed, softcap=0.0, vocab_size=2 ** 31 - 1):
+    """(token, score) of a packed greedy / top-k value; raises AqError as the Go helper returns errors."""
+    lib = load()
+    tok, sc = _c.c_int(0), _c.c_float(0)
+    rc = lib.aq_unpack_best(packed, softcap, vocab_size, ctypes.byref(tok), ctypes.byref(sc))
+    if rc != AQ_OK:
+        raise AqError(rc, lib.aq_last_error().decode())
+    return tok.value, sc.value
 
 
 def variant_names(op):

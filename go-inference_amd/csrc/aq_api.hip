@@ -6,6 +6,7 @@
 #include <hip/hip_runtime.h>
 
 #include <climits>
+#include <cmath>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -61,7 +62,9 @@ struct aq_ctx {
     int forced[2] = {-1, -1};
     const char* last_variant[2] = {"", ""};
     int cu_count = 0;
-    aq::Workspace ws;  // scratch of the matmul path (aq_qmm.h)
+    aq::Workspace ws;       // scratch of the matmul path and of the unfused fallbacks (aq_qmm.h)
+    aq::Workspace head_ws;         // per-wavefront maxima of aq_qmv_greedy; sized at creation for common vocabularies
+    void* head_fold = nullptr;     // aq_qmv_greedy's fold tickets and slots (aq::kHeadFoldBytes, kept zeroed by the kernel)
     char name[256] = {0};
 };
 
@@ -277,6 +280,13 @@ int aq_create(int device, aq_ctx** out) {
     rc = hipStreamCreateWithFlags(&ctx->own_stream, hipStreamNonBlocking);
     if (rc == hipSuccess) rc = hipEventCreate(&ctx->ev0);
     if (rc == hipSuccess) rc = hipEventCreate(&ctx->ev1);
+    if (rc == hipSuccess) rc = hipMalloc(&ctx->head_fold, aq::kHeadFoldBytes);
+    if (rc == hipSuccess) rc = hipMemset(ctx->head_fold, 0, aq::kHeadFoldBytes);
+    if (rc == hipSuccess) {
+        // room for the argmax partials of a 1M-row vocabulary at two rows per wavefront
+        rc = hipMalloc(&ctx->head_ws.ptr, (size_t)4 << 20);
+        if (rc == hipSuccess) ctx->head_ws.bytes = (size_t)4 << 20;
+    }
     if (rc != hipSuccess) {
         aq_destroy(ctx);
         return hip_fail(rc, "hipStreamCreate");
@@ -293,6 +303,8 @@ void aq_destroy(aq_ctx* ctx) {
         (void)hipStreamDestroy(ctx->own_stream);
     }
     if (ctx->ws.ptr) (void)hipFree(ctx->ws.ptr);
+    if (ctx->head_ws.ptr) (void)hipFree(ctx->head_ws.ptr);
+    if (ctx->head_fold) (void)hipFree(ctx->head_fold);
     if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
     if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
     delete ctx;
@@ -912,6 +924,149 @@ int aq_moe_combine(aq_ctx* ctx, const void* route_rows, const float* weights, vo
     a.out_f32 = out_f32 ? 1 : 0;
     a.bf16_steps = (flags & AQ_BF16_STEPS) ? 1 : 0;
     AQ_HIP(aq::moe_combine_launch(a, ctx->stream), "hipLaunchKernel");
+    return AQ_OK;
+}
+
+namespace {
+
+// Shared front of aq_qmv_greedy / aq_qmv_scores.  fuse 3: best[M]; fuse 4: scores[M, N].
+int head_call(aq_ctx* ctx, const char* op, int fuse, const void* x, const void* packed, const void* scales,
+              const void* biases, const int32_t* suppress, int suppress_count, uint64_t* out, int M, int K, int N,
+              int group_size, int bits) {
+    if (!ctx) return fail(AQ_ERR_ARG, "%s: ctx is null", op);
+    if (M < 0 || K < 0 || N < 0 || suppress_count < 0) return fail(AQ_ERR_SHAPE, "%s: M, K, N, suppress_count must be non-negative", op);
+    if (M == 0) return AQ_OK;
+    if (!out) return fail(AQ_ERR_ARG, "%s: null output", op);
+    if (!aligned(out, 8)) return fail(AQ_ERR_ARG, "%s: output pointer is not 8-byte aligned", op);
+    if (suppress_count > 0 && !suppress) return fail(AQ_ERR_ARG, "%s: suppress_count without a suppress list", op);
+    if (suppress && !aligned(suppress, 4)) return fail(AQ_ERR_ARG, "%s: operand pointer is not element-aligned", op);
+    const bool fused = M == 1 && N > 0 && K > 0 && ctx->forced[0] < 0 && (bits == 4 || bits == 8) && x && packed &&
+                       dot2_eligible(K, group_size, bits, x, packed, (size_t)K * 2);
+    if (fuse == 3 && !fused) {
+        // the unfused reduction accumulates with atomics and starts from "no result"
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        AQ_HIP(aq::fill_zero_launch(out, (size_t)M * 8, ctx->stream), "hipLaunchKernel");
+    }
+    if (N == 0) return AQ_OK;
+    if (K == 0) return fail(AQ_ERR_SHAPE, "%s: K must be positive when there are rows to score", op);
+    if (int rc = check_geometry(op, K, group_size, bits)) return rc;
+    if (!x || !packed || !scales || !biases) return fail(AQ_ERR_ARG, "%s: null operand", op);
+    if (!aligned(x, 2) || !aligned(packed, 4) || !aligned(scales, 2) || !aligned(biases, 2))
+        return fail(AQ_ERR_ARG, "%s: operand pointer is not element-aligned", op);
+    if (fused) {
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        const int idx = pick_qmv_variant(ctx, bits, 1, false, N, K, 1);
+        int rows = idx >= 0 ? aq::qmv_variant(idx)->rows : 1;
+        while (rows > 1 && !aq::qmv_head_supported(bits, fuse, rows)) rows >>= 1;
+        if (!aq::qmv_head_supported(bits, fuse, rows)) return fail(AQ_ERR_UNSUPPORTED, "%s: no kernel for bits=%d", op, bits);
+        if (fuse == 3) {
+            AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+            if (int rc = aq::workspace_reserve(ctx->stream, &ctx->head_ws, aq::qmv_head_partials(N, rows) * 8, fail)) return rc;
+        }
+        {
+            aq::QmvArgs a{};
+            a.x = static_cast<const uint16_t*>(x);
+            a.w = static_cast<const uint32_t*>(packed);
+            a.s = static_cast<const uint16_t*>(scales);
+            a.b = static_cast<const uint16_t*>(biases);
+            a.y = out;
+            a.K = K;
+            a.N = N;
+            a.M = 1;
+            a.gs_shift = ilog2(group_size);
+            a.routes = 1;
+            a.suppress = suppress;
+            a.suppress_count = suppress_count;
+            a.partial = static_cast<unsigned long long*>(ctx->head_ws.ptr);
+            a.fold = static_cast<unsigned long long*>(ctx->head_fold);
+            ctx->last_variant[0] = fuse == 3 ? "qmv_greedy_dot2" : "qmv_scores_dot2";
+            AQ_HIP(aq::qmv_head_launch(bits, fuse, rows, a, ctx->stream), "hipLaunchKernel");
+            return AQ_OK;
+        }
+    }
+    // the projection as fp32 into scratch, then the same epilogue over it
+    const size_t region = qmm_region(M, K);
+    {
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+        if (int rc = aq::workspace_reserve(ctx->stream, &ctx->ws, region + (size_t)M * N * 4, fail)) return rc;
+    }
+    float* logits = reinterpret_cast<float*>(static_cast<char*>(ctx->ws.ptr) + region);
+    if (int rc = aq_qmv(ctx, x, packed, scales, biases, logits, M, K, N, group_size, bits, AQ_OUT_F32)) return rc;
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    unsigned long long* o = reinterpret_cast<unsigned long long*>(out);
+    AQ_HIP(aq::pack_scores_launch(logits, M, N, suppress, suppress_count, fuse == 3 ? o : nullptr, fuse == 4 ? o : nullptr,
+                                  ctx->stream),
+           "hipLaunchKernel");
+    return AQ_OK;
+}
+
+uint32_t ordered_key_host(float v) {
+    uint32_t bits;
+    memcpy(&bits, &v, 4);
+    return (bits & 0x80000000u) ? ~bits : (bits ^ 0x80000000u);
+}
+
+}  // namespace
+
+int aq_qmv_greedy(aq_ctx* ctx, const void* x, const void* packed, const void* scales, const void* biases,
+                  const int32_t* suppress, int suppress_count, uint64_t* best, int M, int K, int N, int group_size,
+                  int bits) {
+    return head_call(ctx, "aq_qmv_greedy", 3, x, packed, scales, biases, suppress, suppress_count, best, M, K, N,
+                     group_size, bits);
+}
+
+int aq_qmv_scores(aq_ctx* ctx, const void* x, const void* packed, const void* scales, const void* biases,
+                  const int32_t* suppress, int suppress_count, uint64_t* scores, int M, int K, int N, int group_size,
+                  int bits) {
+    return head_call(ctx, "aq_qmv_scores", 4, x, packed, scales, biases, suppress, suppress_count, scores, M, K, N,
+                     group_size, bits);
+}
+
+int aq_packed_topk(aq_ctx* ctx, const uint64_t* scores, int64_t count, int top_k, uint64_t* out) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_packed_topk: ctx is null");
+    if (count < 0) return fail(AQ_ERR_SHAPE, "aq_packed_topk: count must be non-negative");
+    if (top_k <= 0) return fail(AQ_ERR_SHAPE, "aq_packed_topk: top-k must be positive");
+    if (top_k > aq::kTopKMax) return fail(AQ_ERR_UNSUPPORTED, "aq_packed_topk: top-k is at most %d", aq::kTopKMax);
+    if (!out || (count > 0 && !scores)) return fail(AQ_ERR_ARG, "aq_packed_topk: null operand");
+    if (!aligned(out, 8) || !aligned(scores, 8)) return fail(AQ_ERR_ARG, "aq_packed_topk: operand pointer is not 8-byte aligned");
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    if (count == 0) {
+        AQ_HIP(aq::fill_zero_launch(out, (size_t)top_k * 8, ctx->stream), "hipLaunchKernel");
+        return AQ_OK;
+    }
+    const size_t need = aq::packed_topk_scratch_entries(count, top_k) * 8;
+    if (need) {
+        AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+        if (int rc = aq::workspace_reserve(ctx->stream, &ctx->ws, need, fail)) return rc;
+    }
+    AQ_HIP(aq::packed_topk_launch(reinterpret_cast<const unsigned long long*>(scores), count, top_k,
+                                  reinterpret_cast<unsigned long long*>(out),
+                                  static_cast<unsigned long long*>(ctx->ws.ptr), ctx->stream),
+           "hipLaunchKernel");
+    return AQ_OK;
+}
+
+uint64_t aq_pack_best(float score, int token) {
+    return ((uint64_t)ordered_key_host(score) << 32) | (uint64_t)(~(uint32_t)token);
+}
+
+int aq_unpack_best(uint64_t packed, float softcap, int vocab_size, int* token, float* score) {
+    // order and wording of hipUnpackGreedyBest (hip_projection_launch.go:2397-2416)
+    if (vocab_size <= 0) return fail(AQ_ERR_SHAPE, "aq_unpack_best: vocab size must be positive");
+    if (packed == 0) return fail(AQ_ERR_INDEX, "aq_unpack_best: greedy projection did not produce a result");
+    if (softcap < 0 || softcap != softcap || softcap - softcap != 0)
+        return fail(AQ_ERR_ARG, "aq_unpack_best: softcap must be non-negative and finite");
+    const uint32_t low = (uint32_t)packed;
+    const int64_t id = (int64_t)(int32_t)(~low);
+    if (id < 0 || id >= vocab_size) return fail(AQ_ERR_INDEX, "aq_unpack_best: greedy projection token is out of range");
+    const uint32_t key = (uint32_t)(packed >> 32);
+    const uint32_t bits = (key & 0x80000000u) ? (key ^ 0x80000000u) : ~key;
+    float s;
+    memcpy(&s, &bits, 4);
+    if (softcap > 0) s = (float)tanh((double)(s / softcap)) * softcap;
+    if (token) *token = (int)id;
+    if (score) *score = s;
     return AQ_OK;
 }
 

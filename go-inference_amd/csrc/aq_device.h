@@ -112,6 +112,24 @@ __device__ __forceinline__ uint4 act_mul_bf16x8(uint4 g, uint4 u, int act) {
     return o;
 }
 
+// Score and row index packed so that an unsigned 64-bit maximum picks the highest score and, among equal
+// scores, the lowest index: rocm_ordered_float_key / rocm_pack_score_index
+// (go/engine/hip/kernels/common/numeric.hipinc:84-96; host side hipPackGreedyBest,
+// go/engine/hip/hip_projection_launch.go:2393-2395).  0 means "no candidate".
+__device__ __forceinline__ uint32_t ordered_float_key(float v) {
+    const uint32_t bits = __float_as_uint(v);
+    return (bits & 0x80000000u) ? ~bits : (bits ^ 0x80000000u);
+}
+__device__ __forceinline__ unsigned long long pack_score_index(float score, uint32_t index) {
+    return ((unsigned long long)ordered_float_key(score) << 32) | (unsigned long long)(~index);
+}
+// rocm_mlx_q4_token_suppressed (go/engine/hip/kernels/quant/affine_fused_validate.hipinc:3-15)
+__device__ __forceinline__ bool token_suppressed(uint32_t row, const int32_t* suppress, int count) {
+    for (int i = 0; i < count; i++)
+        if (suppress[i] == (int32_t)row) return true;
+    return false;
+}
+
 // Sum over the 64 lanes of a wavefront; every lane returns the total.
 // Four DPP adds fold each 16-lane row, then the four row totals are read
 // through SGPRs.

@@ -35,6 +35,11 @@ struct QmvArgs {
     const uint16_t* b2;
     int row_base2;       // pair fusion + gather: first `up` row inside an expert's slab
     int act;             // kActGeluTanh or kActSilu
+    // head kernels only (aq_qmv_head.hip): y is uint64 best[M] (argmax) or uint64 scores[M, N]
+    const int32_t* suppress;  // token ids that may not win, or nullptr
+    int suppress_count;
+    unsigned long long* partial;  // argmax: one slot per wavefront of the grid (qmv_head_partials)
+    unsigned long long* fold;     // argmax: kHeadFoldBytes of zeroed device memory that the fold leaves zeroed
 };
 
 constexpr int kActGeluTanh = 1;
@@ -134,6 +139,30 @@ int qmvs_variant_count();
 const QmvVariant* qmvs_variant(int idx);
 bool qmvs_plan(const QmvArgs& a, int bits, int group_size, bool gather, int cu_count, int forced_idx, StreamPlan* out);
 hipError_t qmvs_launch(const StreamPlan& p, const QmvArgs& a, hipStream_t stream);
+
+// lm_head kernels (aq_qmv_head.hip), one activation row: the projection with its epilogue replaced by
+//   fuse 3: best[0] = max over rows of pack(score, row): every wavefront stores its own maximum into
+//           a.partial (no contention); a second kernel of kHeadFoldGroups workgroups folds the partials,
+//           and the last of those to finish (a ticket in a.fold) writes a.y[0]
+//   fuse 4: scores[row] = pack(score, row)
+// Non-finite scores and suppressed rows pack to 0.
+constexpr int kHeadFoldGroups = 64;
+constexpr size_t kHeadFoldBytes = 128 + (size_t)kHeadFoldGroups * 8;  // ticket counter on its own line, then the group maxima
+bool qmv_head_supported(int bits, int fuse, int rows);
+// Slots a.partial must hold for the argmax of N rows at `rows` rows per wavefront.
+size_t qmv_head_partials(int N, int rows);
+hipError_t qmv_head_launch(int bits, int fuse, int rows, const QmvArgs& a, hipStream_t stream);
+// The same two epilogues over fp32 scores that are already in memory: scores [M, N] -> best[M] / packed[M, N].
+hipError_t pack_scores_launch(const float* scores, int M, int N, const int32_t* suppress, int suppress_count,
+                              unsigned long long* best_or_null, unsigned long long* packed_or_null, hipStream_t stream);
+// Largest top_k (<= kTopKMax) of `count` packed values, sorted descending, into out[top_k]; scratch holds
+// packed_topk_scratch_entries(count, top_k) values.
+constexpr int kTopKMax = 64;
+constexpr int kTopKPerLane = 16;                    // values a lane sorts in registers
+constexpr int kTopKSegment = 64 * kTopKPerLane;     // values one wavefront reduces to top_k
+size_t packed_topk_scratch_entries(int64_t count, int top_k);
+hipError_t packed_topk_launch(const unsigned long long* in, int64_t count, int top_k, unsigned long long* out,
+                              unsigned long long* scratch, hipStream_t stream);
 
 // MoE router and combine (aq_moe.hip).
 constexpr int kMoeMaxExperts = 1024;

@@ -24,15 +24,27 @@
 
 namespace aq {
 
+// Wave-wide maximum / minimum through DPP inside each row of 16 lanes (old value = the identity for lanes a
+// pattern leaves without a source) and SGPR reads across the four rows.
 __device__ __forceinline__ float wave_max_f32(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
-    return v;
+    const int ninf = __float_as_int(-INFINITY);
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(ninf, __float_as_int(v), 0xB1, 0xF, 0xF, false)));
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(ninf, __float_as_int(v), 0x4E, 0xF, 0xF, false)));
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(ninf, __float_as_int(v), 0x141, 0xF, 0xF, false)));
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(ninf, __float_as_int(v), 0x140, 0xF, 0xF, false)));
+    const float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    const float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    const float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    const float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    return fmaxf(fmaxf(a, b), fmaxf(c, d));
 }
 __device__ __forceinline__ int wave_min_i32(int v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = min(v, __shfl_xor(v, o, kWave));
-    return v;
+    v = min(v, __builtin_amdgcn_update_dpp(INT_MAX, v, 0xB1, 0xF, 0xF, false));
+    v = min(v, __builtin_amdgcn_update_dpp(INT_MAX, v, 0x4E, 0xF, 0xF, false));
+    v = min(v, __builtin_amdgcn_update_dpp(INT_MAX, v, 0x141, 0xF, 0xF, false));
+    v = min(v, __builtin_amdgcn_update_dpp(INT_MAX, v, 0x140, 0xF, 0xF, false));
+    return min(min(__builtin_amdgcn_readlane(v, 0), __builtin_amdgcn_readlane(v, 16)),
+               min(__builtin_amdgcn_readlane(v, 32), __builtin_amdgcn_readlane(v, 48)));
 }
 
 template <int PER>
@@ -125,6 +137,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const MoeCombineArgs a
         const int row = (int)(i / a.n);
         const int col = (int)(i - (int64_t)row * a.n);
         float acc = 0.0f;
+#pragma unroll 8
         for (int r = 0; r < a.top_k; r++) {
             const int64_t pair = (int64_t)row * a.top_k + r;
             const float y = a.in_f32 ? static_cast<const float*>(a.route_rows)[pair * a.n + col]

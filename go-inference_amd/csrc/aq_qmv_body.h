@@ -40,6 +40,10 @@ struct Slice {
 //         (go/engine/hip/kernels/quant/affine_gelu_tanh.hipinc:3-182; gathered: kernels/moe/routing.hipinc:312).
 // FUSE 2: the activations are bf16(act(x) * x2), formed while x is staged, as lthn_gather_qmv_gelu does
 //         (go/engine/metal/kernels/moe/lthn_gather_qmv.metal:98-132, lthn_gelu_qmv_impl.h:24-33).
+// FUSE 3: nothing but each wavefront's best packed (score, row) leaves the kernel; their maximum is what
+//         rocm_mlx_q4_projection_greedy accumulates with atomicMax
+//         (kernels/quant/affine_projection_fused.hipinc:190-248).
+// FUSE 4: every row's packed (score, row) is stored, as rocm_mlx_q4_projection_scores does (:411-446).
 template <int BITS, int M, int R, int NW, int DEPTH, bool GATHER, int XMODE, int FUSE = 0>
 __device__ __forceinline__ void qmv_dot2_body(const QmvArgs& a, const int bx) {
     using C = Codec<BITS>;
@@ -287,6 +291,29 @@ __device__ __forceinline__ void qmv_dot2_body(const QmvArgs& a, const int bx) {
         }
     }
 
+    if constexpr (FUSE == 3 || FUSE == 4) {
+        static_assert(FUSE < 3 || (M == 1 && !GATHER), "the head epilogues take one activation row");
+        unsigned long long wave_best = 0;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const float tot = wave_sum(acc[r][0]);
+            const int row = row_first + r;
+            unsigned long long packed = 0;
+            if (row < N && isfinite(tot) && !token_suppressed((uint32_t)row, a.suppress, a.suppress_count))
+                packed = pack_score_index(tot, (uint32_t)row);
+            if constexpr (FUSE == 4) {
+                if (lane == 0 && row < N) reinterpret_cast<unsigned long long*>(a.y)[row] = packed;
+            } else {
+                wave_best = packed > wave_best ? packed : wave_best;
+            }
+        }
+        if constexpr (FUSE == 3) {
+            // one private slot per wavefront: tens of thousands of wavefronts meeting on one address, be it
+            // only to read it or to take a ticket, cost more than the projection itself (measured)
+            if (lane == 0) a.partial[(size_t)bx * NW + wave] = wave_best;
+        }
+        return;
+    }
 #pragma unroll
     for (int r = 0; r < R; r++) {
 #pragma unroll

@@ -1,0 +1,254 @@
+// lm_head: the vocabulary projection whose consumer wants a token, not 262 144 logits.
+//
+//   greedy   the projection with the argmax as its epilogue: each wavefront keeps the best packed (score, row)
+//            of its rows and a small second kernel folds those; no logit is ever stored.  Replaces
+//            rocm_mlx_q4_projection_greedy (go/engine/hip/kernels/quant/affine_projection_fused.hipinc:190-248).
+//   scores   every row's (score, row) packed into 64 bits, the input of top-k sampling:
+//            rocm_mlx_q4_projection_scores (:411-446).
+//   top-k    the k largest packed values, sorted descending: what rocm_packed_topk
+//            (go/engine/hip/kernels/sampling/topk.hipinc:45-84) yields per chunk, here per wavefront segment
+//            and repeated until one segment is left.
+//
+// The streaming part is the dot2 body; only the epilogue differs.  pack_scores_kernel applies the same two
+// epilogues to fp32 scores already in memory (shapes the dot2 kernels do not take, several rows).
+#include "aq_qmv_body.h"
+
+namespace aq {
+
+template <int BITS, int R, int FUSE>
+__global__ __launch_bounds__(4 * kWave) void qmv_head_kernel(const QmvArgs a) {
+    qmv_dot2_body<BITS, 1, R, 4, 2, false, 0, FUSE>(a, blockIdx.x);
+}
+
+typedef void (*QmvHeadKernel)(const QmvArgs);
+struct QmvHeadEntry {
+    int bits, fuse, rows;
+    QmvHeadKernel fn;
+};
+#define AQ_HEAD(BITS, FUSE, R) {BITS, FUSE, R, qmv_head_kernel<BITS, R, FUSE>}
+#define AQ_HEAD_SET(BITS) \
+    AQ_HEAD(BITS, 3, 1), AQ_HEAD(BITS, 3, 2), AQ_HEAD(BITS, 3, 4), AQ_HEAD(BITS, 4, 1), AQ_HEAD(BITS, 4, 2), AQ_HEAD(BITS, 4, 4)
+static const QmvHeadEntry kHeadTable[] = {AQ_HEAD_SET(4), AQ_HEAD_SET(8)};
+
+static const QmvHeadEntry* find_head(int bits, int fuse, int rows) {
+    for (const QmvHeadEntry& e : kHeadTable)
+        if (e.bits == bits && e.fuse == fuse && e.rows == rows) return &e;
+    return nullptr;
+}
+
+bool qmv_head_supported(int bits, int fuse, int rows) { return find_head(bits, fuse, rows) != nullptr; }
+
+size_t qmv_head_partials(int N, int rows) { return (size_t)((N + rows * 4 - 1) / (rows * 4)) * 4; }
+
+// Folds the per-wavefront maxima into best[0]: kHeadFoldGroups workgroups each fold a slice into their own
+// slot, take a ticket, and the one that draws the last ticket folds the slots and zeroes the ticket counter
+// again.  Sixty-four tickets on one address are cheap; one ticket per wavefront of the projection is not.
+__global__ __launch_bounds__(256) void fold_best_kernel(const unsigned long long* __restrict__ partial, int count,
+                                                        unsigned long long* fold, unsigned long long* __restrict__ best) {
+    unsigned int* tickets = reinterpret_cast<unsigned int*>(fold);
+    unsigned long long* slots = fold + 16;
+    const int per_group = (count + kHeadFoldGroups - 1) / kHeadFoldGroups;
+    const int begin = blockIdx.x * per_group;
+    const int end = min(begin + per_group, count);
+    unsigned long long mine = 0;
+    constexpr int U = 4;
+    for (int base = begin; base < end; base += 256 * U) {
+        unsigned long long t[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int i = base + u * 256 + (int)threadIdx.x;
+            // clamped, not predicated: reading a value twice does not change a maximum, and the loads stay
+            // unconditional so that all of them are issued before the first is waited for
+            t[u] = partial[min(i, end - 1)];
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) mine = t[u] > mine ? t[u] : mine;
+    }
+    if (begin >= end) mine = 0;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const unsigned long long other = __shfl_xor(mine, o, kWave);
+        mine = other > mine ? other : mine;
+    }
+    __shared__ unsigned long long wave_best[4];
+    __shared__ int last;
+    if ((threadIdx.x & (kWave - 1)) == 0) wave_best[threadIdx.x >> 6] = mine;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned long long b = wave_best[0];
+        for (int i = 1; i < 4; i++) b = wave_best[i] > b ? wave_best[i] : b;
+        __atomic_store_n(&slots[blockIdx.x], b, __ATOMIC_RELAXED);
+        __threadfence();
+        last = atomicAdd(tickets, 1u) == (unsigned int)kHeadFoldGroups - 1u;
+    }
+    __syncthreads();
+    if (!last || threadIdx.x >= kWave) return;
+    __threadfence();
+    unsigned long long m = __atomic_load_n(&slots[threadIdx.x], __ATOMIC_RELAXED);  // kHeadFoldGroups == 64 lanes
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const unsigned long long other = __shfl_xor(m, o, kWave);
+        m = other > m ? other : m;
+    }
+    if (threadIdx.x == 0) {
+        best[0] = m;
+        atomicExch(tickets, 0u);
+    }
+}
+
+hipError_t qmv_head_launch(int bits, int fuse, int rows, const QmvArgs& a, hipStream_t stream) {
+    const QmvHeadEntry* e = find_head(bits, fuse, rows);
+    if (!e || a.M != 1) return hipErrorInvalidValue;
+    const int rows_per_wg = rows * 4;
+    const size_t lds = (size_t)a.K * 2;
+    if (lds > 48 * 1024) {
+        hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e->fn),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (rc != hipSuccess) return rc;
+    }
+    if (fuse == 3 && (!a.partial || !a.fold)) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(e->fn, dim3((unsigned)((a.N + rows_per_wg - 1) / rows_per_wg)), dim3(4 * kWave), lds, stream, a);
+    hipError_t rc = hipGetLastError();
+    if (rc != hipSuccess || fuse != 3) return rc;
+    static_assert(kHeadFoldGroups == kWave, "the last workgroup reads one slot per lane");
+    hipLaunchKernelGGL(fold_best_kernel, dim3(kHeadFoldGroups), dim3(256), 0, stream, a.partial,
+                       (int)qmv_head_partials(a.N, rows), a.fold, reinterpret_cast<unsigned long long*>(a.y));
+    return hipGetLastError();
+}
+
+// grid.y = activation row; a workgroup folds its share of a row before touching the shared maximum
+__global__ __launch_bounds__(256) void pack_scores_kernel(const float* __restrict__ scores, int N, const int32_t* suppress,
+                                                          int suppress_count, unsigned long long* best,
+                                                          unsigned long long* packed_out) {
+    const int m = blockIdx.y;
+    const float* row_scores = scores + (int64_t)m * N;
+    unsigned long long mine = 0;
+    for (int n = blockIdx.x * 256 + threadIdx.x; n < N; n += gridDim.x * 256) {
+        const float v = row_scores[n];
+        unsigned long long p = 0;
+        if (isfinite(v) && !token_suppressed((uint32_t)n, suppress, suppress_count)) p = pack_score_index(v, (uint32_t)n);
+        if (packed_out) packed_out[(int64_t)m * N + n] = p;
+        mine = p > mine ? p : mine;
+    }
+    if (!best) return;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const unsigned long long other = __shfl_xor(mine, o, kWave);
+        mine = other > mine ? other : mine;
+    }
+    __shared__ unsigned long long wave_best[4];
+    if ((threadIdx.x & (kWave - 1)) == 0) wave_best[threadIdx.x >> 6] = mine;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned long long b = wave_best[0];
+        for (int i = 1; i < 4; i++) b = wave_best[i] > b ? wave_best[i] : b;
+        if (b != 0) atomicMax(best + m, b);
+    }
+}
+
+hipError_t pack_scores_launch(const float* scores, int M, int N, const int32_t* suppress, int suppress_count,
+                              unsigned long long* best_or_null, unsigned long long* packed_or_null, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return hipSuccess;
+    int bx = (N + 255) / 256;
+    if (bx > 1024) bx = 1024;
+    hipLaunchKernelGGL(pack_scores_kernel, dim3((unsigned)bx, (unsigned)M), dim3(256), 0, stream, scores, N, suppress,
+                       suppress_count, best_or_null, packed_or_null);
+    return hipGetLastError();
+}
+
+// Maximum over the 64 lanes, unsigned: DPP folds inside each row of 16 lanes (a lane out of range reads 0,
+// the identity), then the four row results meet through SGPRs.
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+    v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, true));
+    v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xF, 0xF, true));
+    v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xF, 0xF, true));
+    v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x140, 0xF, 0xF, true));
+    const uint32_t a = (uint32_t)__builtin_amdgcn_readlane((int)v, 0), b = (uint32_t)__builtin_amdgcn_readlane((int)v, 16);
+    const uint32_t c = (uint32_t)__builtin_amdgcn_readlane((int)v, 32), d = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+    return max(max(a, b), max(c, d));
+}
+
+// One wavefront reduces kTopKSegment packed values to their top_k largest, sorted descending.  Every lane
+// sorts its kTopKPerLane values in registers; then, top_k times, the wavefront takes the largest of the 64
+// list heads (high words first, then the low words of the lanes that hold that high word) and the winning
+// lane drops its head.  Entries past `count` read as 0, which is also the "no candidate" value.
+__global__ __launch_bounds__(256) void packed_topk_kernel(const unsigned long long* __restrict__ in, int64_t count, int top_k,
+                                                          unsigned long long* __restrict__ out) {
+    constexpr int V = kTopKPerLane;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t segment = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t begin = segment * kTopKSegment;
+    if (begin >= count) return;  // whole wavefronts
+    unsigned long long v[V];
+#pragma unroll
+    for (int j = 0; j < V; j++) {
+        const int64_t i = begin + j * kWave + lane;
+        v[j] = i < count ? in[i] : 0ull;
+    }
+    // bitonic network over the lane's own values, fully unrolled: descending order
+#pragma unroll
+    for (int width = 2; width <= V; width <<= 1) {
+#pragma unroll
+        for (int stride = width >> 1; stride > 0; stride >>= 1) {
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                const int j = i ^ stride;
+                if (j > i) {
+                    const bool descending = (i & width) == 0;
+                    const unsigned long long a = v[i], b = v[j];
+                    const bool swap = descending ? a < b : a > b;
+                    v[i] = swap ? b : a;
+                    v[j] = swap ? a : b;
+                }
+            }
+        }
+    }
+    unsigned long long mine = 0;
+    for (int it = 0; it < top_k; it++) {
+        const uint32_t hi = (uint32_t)(v[0] >> 32), lo = (uint32_t)v[0];
+        const uint32_t best_hi = wave_max_u32(hi);
+        const uint32_t best_lo = wave_max_u32(hi == best_hi ? lo : 0u);
+        const unsigned long long best = ((unsigned long long)best_hi << 32) | best_lo;
+        if (best == 0) break;  // nothing but "no candidate" left; uniform over the wavefront
+        const unsigned long long holders = __ballot(v[0] == best);
+        if (lane == __ffsll((long long)holders) - 1) {  // equal values: one lane at a time gives its copy
+#pragma unroll
+            for (int j = 0; j + 1 < V; j++) v[j] = v[j + 1];
+            v[V - 1] = 0;
+        }
+        if (lane == it) mine = best;
+    }
+    if (lane < top_k) out[segment * top_k + lane] = mine;
+}
+
+static int64_t topk_segments(int64_t count) { return (count + kTopKSegment - 1) / kTopKSegment; }
+
+size_t packed_topk_scratch_entries(int64_t count, int top_k) {
+    if (count <= kTopKSegment) return 0;
+    // first round's output, then the second round's beside it (every later round is smaller)
+    const int64_t c1 = topk_segments(count) * top_k;
+    const int64_t c2 = c1 > kTopKSegment ? topk_segments(c1) * top_k : 0;
+    return (size_t)(c1 + c2);
+}
+
+hipError_t packed_topk_launch(const unsigned long long* in, int64_t count, int top_k, unsigned long long* out,
+                              unsigned long long* scratch, hipStream_t stream) {
+    if (top_k <= 0 || top_k > kTopKMax || count <= 0) return hipErrorInvalidValue;
+    const int64_t c1 = topk_segments(count) * top_k;
+    unsigned long long* bufs[2] = {scratch, scratch + c1};
+    int which = 0;
+    const unsigned long long* src = in;
+    int64_t n = count;
+    while (true) {
+        const int64_t segments = topk_segments(n);
+        unsigned long long* dst = segments == 1 ? out : bufs[which];
+        hipLaunchKernelGGL(packed_topk_kernel, dim3((unsigned)((segments + 3) / 4)), dim3(256), 0, stream, src, n, top_k, dst);
+        hipError_t rc = hipGetLastError();
+        if (rc != hipSuccess || segments == 1) return rc;
+        src = dst;
+        n = segments * top_k;
+        which ^= 1;
+    }
+}
+
+}  // namespace aq

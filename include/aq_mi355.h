@@ -224,6 +224,38 @@ int aq_moe_route(aq_ctx *ctx, const void *logits, int rows, int num_experts, int
 int aq_moe_combine(aq_ctx *ctx, const void *route_rows, const float *weights, void *out, int rows, int top_k, int n,
                    unsigned flags);
 
+/* lm_head with the argmax fused in: best[m] = max over vocabulary rows n of pack(score[m,n], n), where
+ * score = x[m,:] . dequant(w)[n,:] in fp32 and pack() is aq_pack_best's layout (score key in the high word,
+ * ~n in the low word, so the highest score wins and equal scores go to the lowest token id, the order of
+ * hipReferenceGreedySample, go/engine/hip/hip_transformer_reference.go:401-437).  Non-finite scores and the
+ * token ids listed in `suppress` (device int32[suppress_count], may be NULL) never win; best[m] == 0 means no
+ * row qualified.  best is device uint64[M]; the call clears it itself.  Replaces
+ * rocm_mlx_q4_projection_greedy / _greedy_batch (go/engine/hip/kernels/quant/affine_projection_fused.hipinc:190-410):
+ * for M == 1 and 4/8-bit codes 8 bytes leave the kernel instead of N logits; other shapes run the projection
+ * into the context's workspace and reduce it there. */
+int aq_qmv_greedy(aq_ctx *ctx, const void *x, const void *packed, const void *scales, const void *biases,
+                  const int32_t *suppress, int suppress_count, uint64_t *best, int M, int K, int N, int group_size,
+                  int bits);
+
+/* The same projection storing every row's packed (score, row): scores is device uint64[M, N]; suppressed or
+ * non-finite rows hold 0.  rocm_mlx_q4_projection_scores (affine_projection_fused.hipinc:411-446), the input
+ * of top-k sampling. */
+int aq_qmv_scores(aq_ctx *ctx, const void *x, const void *packed, const void *scales, const void *biases,
+                  const int32_t *suppress, int suppress_count, uint64_t *scores, int M, int K, int N, int group_size,
+                  int bits);
+
+/* The top_k (1..64) largest of `count` packed values, sorted descending, into device out[top_k]; fewer than
+ * top_k non-zero inputs leave zeros at the end.  rocm_packed_topk (go/engine/hip/kernels/sampling/topk.hipinc:45-84)
+ * applied chunk by chunk until one chunk is left; scratch comes from the context's workspace. */
+int aq_packed_topk(aq_ctx *ctx, const uint64_t *scores, int64_t count, int top_k, uint64_t *out);
+
+/* Host-side codec of the packed values: hipPackGreedyBest / hipUnpackGreedyBest
+ * (go/engine/hip/hip_projection_launch.go:2393-2416).  Unpacking rejects packed == 0 ("did not produce a
+ * result"), a token outside [0, vocab_size) and a negative or non-finite softcap; softcap > 0 returns
+ * tanh(score / softcap) * softcap. */
+uint64_t aq_pack_best(float score, int token);
+int aq_unpack_best(uint64_t packed, float softcap, int vocab_size, int *token, float *score);
+
 /* mlxaffine.DequantizeTensor on device (go/model/quant/mlxaffine/mlxaffine.go:178-208):
  * out_f32[N,K] = scale*code + bias, bit-exact with the CPU path. */
 int aq_dequant_f32(aq_ctx *ctx, const void *packed, const void *scales, const void *biases, float *out_f32, int64_t N,

@@ -544,6 +544,57 @@ int orc_moe_combine(const float *route_rows, const float *weights, int rows, int
     return ORC_OK;
 }
 
+/* hip_projection_launch.go:2375-2395 */
+static uint32_t ordered_float32_key(float value) {
+    uint32_t bits;
+    memcpy(&bits, &value, 4);
+    if (bits & 0x80000000u) return ~bits;
+    return bits ^ 0x80000000u;
+}
+
+uint64_t orc_pack_greedy_best(float score, int token) {
+    return ((uint64_t)ordered_float32_key(score) << 32) | (uint64_t)(~(uint32_t)token);
+}
+
+/* hip_projection_launch.go:2386-2416 */
+int orc_unpack_greedy_best(uint64_t packed, float softcap, int vocab_size, int *token, float *score) {
+    if (vocab_size <= 0) return ORC_ERR_DIMS;
+    if (packed == 0) return ORC_ERR_INDEX;
+    if (softcap < 0 || isnan(softcap) || isinf(softcap)) return ORC_ERR_SIZE;
+    const int64_t id = (int64_t)(int32_t)(~(uint32_t)packed);
+    if (id < 0 || id >= vocab_size) return ORC_ERR_INDEX;
+    const uint32_t key = (uint32_t)(packed >> 32);
+    const uint32_t bits = (key & 0x80000000u) ? (key ^ 0x80000000u) : ~key;
+    float s;
+    memcpy(&s, &bits, 4);
+    if (softcap > 0) s = (float)tanh((double)(s / softcap)) * softcap;
+    *token = (int)id;
+    *score = s;
+    return ORC_OK;
+}
+
+/* hip_transformer_reference.go:401-437 */
+int orc_greedy_sample_suppress(const float *logits, int n, const int32_t *suppress, int suppress_count, int *index,
+                               float *value) {
+    if (n <= 0) return ORC_ERR_DIMS;
+    int best = -1;
+    float best_value = 0;
+    for (int i = 0; i < n; i++) {
+        int skip = 0;
+        for (int s = 0; s < suppress_count; s++)
+            if (suppress[s] == i) skip = 1;
+        if (skip) continue;
+        if (best < 0 || logits[i] > best_value) {
+            best = i;
+            best_value = logits[i];
+        }
+    }
+    if (best < 0) return ORC_ERR_INDEX;
+    *index = best;
+    *value = best_value;
+    return ORC_OK;
+}
+
 int orc_max_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

@@ -146,6 +146,20 @@ int orc_moe_route(const float *logits, int rows, int num_experts, int top_k, con
 int orc_moe_combine(const float *route_rows, const float *weights, int rows, int top_k, int n, int bf16_steps,
                     float *out);
 
+/* Packed (score, token) values of the fused lm_head kernels: hipOrderedFloat32Key / hipPackGreedyBest /
+ * hipUnpackGreedyBest, go/engine/hip/hip_projection_launch.go:2375-2416 (device side
+ * kernels/common/numeric.hipinc:84-104).  Unsigned comparison of packed values orders by score, then by
+ * lower token id.  Unpack returns ORC_ERR_DIMS for a non-positive vocab, ORC_ERR_INDEX for packed == 0 or
+ * a token outside the vocab, ORC_ERR_SIZE for a bad softcap. */
+uint64_t orc_pack_greedy_best(float score, int token);
+int orc_unpack_greedy_best(uint64_t packed, float softcap, int vocab_size, int *token, float *score);
+
+/* hipReferenceGreedySample / hipReferenceGreedySampleSuppress, go/engine/hip/hip_transformer_reference.go:401-437:
+ * first maximum wins; suppressed tokens are skipped; ORC_ERR_DIMS without logits, ORC_ERR_INDEX when every
+ * token is suppressed. */
+int orc_greedy_sample_suppress(const float *logits, int n, const int32_t *suppress, int suppress_count, int *index,
+                               float *value);
+
 /* Number of hardware threads OpenMP would use (for reporting). */
 int orc_max_threads(void);
 

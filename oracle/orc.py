@@ -212,5 +212,29 @@ def moe_combine(route_rows_f32, weights_f32, rows, top_k, n, bf16_steps=False):
     return out
 
 
+def pack_greedy_best(score, token):
+    fn = lib().orc_pack_greedy_best
+    fn.restype = ctypes.c_uint64
+    fn.argtypes = [ctypes.c_float, ctypes.c_int]
+    return int(fn(score, token))
+
+
+def unpack_greedy_best(packed, softcap=0.0, vocab_size=2 ** 31 - 1):
+    fn = lib().orc_unpack_greedy_best
+    fn.argtypes = [ctypes.c_uint64, ctypes.c_float, ctypes.c_int, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_float)]
+    tok, sc = ctypes.c_int(0), ctypes.c_float(0)
+    _check(fn(packed, softcap, vocab_size, ctypes.byref(tok), ctypes.byref(sc)))
+    return tok.value, sc.value
+
+
+def greedy_sample_suppress(logits_f32, suppress=None):
+    lg = np.ascontiguousarray(logits_f32, dtype=np.float32).reshape(-1)
+    sup = None if suppress is None else np.ascontiguousarray(suppress, dtype=np.int32)
+    idx, val = ctypes.c_int(0), ctypes.c_float(0)
+    _check(lib().orc_greedy_sample_suppress(_p(lg), lg.size, _p(sup), 0 if sup is None else sup.size, ctypes.byref(idx),
+                                            ctypes.byref(val)))
+    return idx.value, val.value
+
+
 def max_threads():
     return int(lib().orc_max_threads())

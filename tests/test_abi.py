@@ -84,3 +84,22 @@ def test_affine_geometry(aqlib, in_dim, scales_last, packed_last, want):
     gs, bits = ctypes.c_int(-1), ctypes.c_int(-1)
     aqlib.aqh_affine_geometry(in_dim, scales_last, packed_last, ctypes.byref(gs), ctypes.byref(bits))
     assert (gs.value, bits.value) == want
+
+
+def test_pack_and_unpack_best_match_the_oracle(aqlib, orc):
+    """aq_pack_best / aq_unpack_best are host code (hipPackGreedyBest / hipUnpackGreedyBest,
+    go/engine/hip/hip_projection_launch.go:2393-2416)."""
+    import aq_mi355
+    for score, token in [(1.0, 2), (-3.5, 0), (0.0, 262143), (-0.0, 1), (1e-40, 5), (3.4e38, 77)]:
+        p = aq_mi355.pack_best(score, token)
+        assert p == orc.pack_greedy_best(score, token)
+        assert aq_mi355.unpack_best(p, 0.0, 262144) == orc.unpack_greedy_best(p, 0.0, 262144)
+    p = aq_mi355.pack_best(45.0, 9)
+    assert aq_mi355.unpack_best(p, 30.0, 100) == orc.unpack_greedy_best(p, 30.0, 100)
+    for args, code in [((0, 0.0, 10), aq_mi355.AQ_ERR_INDEX), ((aq_mi355.pack_best(1.0, 10), 0.0, 10), aq_mi355.AQ_ERR_INDEX),
+                       ((aq_mi355.pack_best(1.0, 1), -1.0, 10), aq_mi355.AQ_ERR_ARG),
+                       ((aq_mi355.pack_best(1.0, 1), float("inf"), 10), aq_mi355.AQ_ERR_ARG),
+                       ((aq_mi355.pack_best(1.0, 1), 0.0, 0), aq_mi355.AQ_ERR_SHAPE)]:
+        with pytest.raises(aq_mi355.AqError) as e:
+            aq_mi355.unpack_best(*args)
+        assert e.value.code == code

@@ -1,0 +1,187 @@
+"""GPU parity of the lm_head entry points (projection with fused argmax, packed scores, packed top-k)
+through the C ABI against the CPU oracle.  The winning token must be the oracle's greedy token for the
+device's own fp32 scores (exact), and the device scores must sit within the matvec tolerance of the
+float64 reference; where two float64 reference scores are closer than that tolerance either may win."""
+import numpy as np
+import pytest
+
+import fixtures as F
+from gpu_util import MAX_ABS, DeviceAffine, check_accumulators, run_qmv, say
+
+pytestmark = pytest.mark.gpu
+
+
+def _u64(buf, n):
+    return buf.download(np.uint64, n)
+
+
+def _unpack(packed):
+    import aq_mi355
+    return aq_mi355.unpack_best(int(packed))
+
+
+def _unpack_all(packed):
+    """numpy form of the unpack, for whole score vectors (spot-checked against aq_unpack_best below)."""
+    key = (packed >> np.uint64(32)).astype(np.uint32)
+    bits = np.where(key & np.uint32(0x80000000), key ^ np.uint32(0x80000000), ~key)
+    toks = (~packed.astype(np.uint32)).astype(np.int64)      # low word
+    return toks, bits.view(np.float32).copy()
+
+
+def _scores(ctx, x, dw, M, K, N, gs, bits, suppress=None):
+    dx = ctx.to_device(np.ascontiguousarray(x, np.uint16))
+    ds = None if suppress is None else ctx.to_device(np.asarray(suppress, np.int32))
+    out = ctx.alloc(M * N * 8)
+    ctx.qmv_scores(dx, dw.w, dw.s, dw.b, out, M, K, N, gs, bits, ds, 0 if suppress is None else len(suppress))
+    ctx.sync()
+    got = _u64(out, M * N).reshape(M, N)
+    for t in (dx, ds, out):
+        if t is not None:
+            t.free()
+    return got
+
+
+def _greedy(ctx, x, dw, M, K, N, gs, bits, suppress=None):
+    dx = ctx.to_device(np.ascontiguousarray(x, np.uint16))
+    ds = None if suppress is None else ctx.to_device(np.asarray(suppress, np.int32))
+    best = ctx.to_device(np.full(M, 0xDEADBEEF, np.uint64))   # the call clears it itself
+    ctx.qmv_greedy(dx, dw.w, dw.s, dw.b, best, M, K, N, gs, bits, ds, 0 if suppress is None else len(suppress))
+    ctx.sync()
+    got = _u64(best, M)
+    for t in (dx, ds, best):
+        if t is not None:
+            t.free()
+    return got
+
+
+@pytest.mark.parametrize("bits,gs,M,K,N,fused", [(4, 32, 1, 1536, 32768, True), (4, 64, 1, 4096, 20011, True),
+                                                 (8, 64, 1, 1024, 4096, True), (4, 64, 1, 512, 37, True),
+                                                 (6, 32, 1, 192, 301, False), (4, 64, 3, 512, 1000, False),
+                                                 (4, 64, 20, 1024, 515, False)])
+def test_greedy_and_scores_against_oracle(ctx, orc, bits, gs, M, K, N, fused):
+    say("head", bits, gs, M, K, N)
+    if 32 % bits == 0:
+        words, s, b = F.synthetic_affine(N, K, bits, gs, seed=F.BASE_SEED + 100)
+    else:
+        rng = np.random.default_rng(3)
+        words = F.pack_codes(rng.integers(0, 1 << bits, size=(N, K)), bits)
+        s = F.f32_to_bf16_bits((np.abs(rng.normal(0, 0.02, (N, K // gs))) + 1e-3).astype(np.float32))
+        b = F.f32_to_bf16_bits(rng.normal(0, 0.05, (N, K // gs)).astype(np.float32))
+    x = F.synthetic_x(M, K, seed=F.BASE_SEED + 101)
+    dw = DeviceAffine(ctx, words, s, b)
+    ref = F.reference_f64(x, words, s, b, bits, gs, K)
+    suppress = [int(np.argmax(ref[0])), 5, N - 1]
+    for sup in (None, suppress):
+        packed = _scores(ctx, x, dw, M, K, N, gs, bits, sup)
+        if fused:
+            assert ctx.last_variant(0) == "qmv_scores_dot2"
+        toks, dev = _unpack_all(packed)
+        live = packed != 0
+        if sup is not None:
+            assert not live[:, sup].any()
+            live[:, sup] = True
+            dev[:, sup] = ref[:, sup]
+            toks[:, sup] = np.asarray(sup)
+        assert live.all() and np.array_equal(toks, np.broadcast_to(np.arange(N), (M, N)))
+        for n in np.random.default_rng(1).integers(0, N, 40):      # the vectorised unpack against the library's
+            if packed[0, n]:
+                assert _unpack(packed[0, n]) == (int(toks[0, n]), float(dev[0, n]))
+        check_accumulators(dev, ref, "packed scores")
+        best = _greedy(ctx, x, dw, M, K, N, gs, bits, sup)
+        if fused:
+            assert ctx.last_variant(0) == "qmv_greedy_dot2"
+        for m in range(M):
+            tok, sc = _unpack(best[m])
+            want_tok, want_sc = orc.greedy_sample_suppress(dev[m], sup)
+            assert (tok, np.float32(sc)) == (want_tok, np.float32(want_sc)), (m, sup)
+            assert best[m] == packed[m].max()
+            # against the float64 reference: the winner's reference score is within tolerance of the best one
+            r = ref[m].copy()
+            if sup is not None:
+                r[sup] = -np.inf
+            assert r[tok] >= r.max() - 2 * MAX_ABS
+    dw.free()
+
+
+def test_greedy_ties_and_nonfinite_rows(ctx, orc):
+    """Equal rows give equal scores: the lowest token id wins.  A row whose sum overflows is skipped."""
+    say("head ties")
+    K, N, gs, bits = 512, 64, 64, 4
+    words, s, b = F.synthetic_affine(N, K, bits, gs, seed=F.BASE_SEED + 102)
+    x = F.synthetic_x(1, K, seed=F.BASE_SEED + 103)
+    ref = F.reference_f64(x, words, s, b, bits, gs, K)[0]
+    top = int(np.argmax(ref))
+    for dup in (3, 40, 63):            # copies of the winning row at other ids
+        words[dup], s[dup], b[dup] = words[top], s[top], b[top]
+    # a row of +inf scales times positive x sums would need signs; use a NaN bias instead: never a candidate
+    b[10, 0] = 0x7FC0
+    dw = DeviceAffine(ctx, words, s, b)
+    best = _greedy(ctx, x, dw, 1, K, N, gs, bits)
+    tok, _ = _unpack(best[0])
+    assert tok == min(top, 3)
+    packed = _scores(ctx, x, dw, 1, K, N, gs, bits)
+    assert packed[0, 10] == 0
+    best = _greedy(ctx, x, dw, 1, K, N, gs, bits, [min(top, 3)])
+    assert _unpack(best[0])[0] == sorted({top, 3, 40, 63})[1]
+    # everything suppressed: no result
+    best = _greedy(ctx, x, dw, 1, K, N, gs, bits, list(range(N)))
+    assert best[0] == 0
+    dw.free()
+
+
+@pytest.mark.parametrize("count,top_k", [(1, 1), (100, 8), (2048, 64), (2049, 5), (262144, 40), (70000, 64), (5, 8)])
+def test_packed_topk_sorted_descending(ctx, count, top_k):
+    import aq_mi355
+    say("packed topk", count, top_k)
+    rng = np.random.default_rng(count + top_k)
+    scores = rng.normal(0, 4, count).astype(np.float32)
+    scores[rng.integers(0, count, max(1, count // 50))] = scores.max()     # ties at the top
+    packed = np.array([aq_mi355.pack_best(float(v), t) for t, v in enumerate(scores)], dtype=np.uint64)
+    packed[rng.integers(0, count, count // 10)] = 0                          # suppressed entries
+    din, dout = ctx.to_device(packed), ctx.alloc(top_k * 8)
+    ctx.packed_topk(din, count, top_k, dout)
+    ctx.sync()
+    got = _u64(dout, top_k)
+    want = np.sort(packed)[::-1][:top_k]
+    want = np.concatenate([want, np.zeros(top_k - want.size, np.uint64)])
+    assert np.array_equal(got, want)
+    din.free()
+    dout.free()
+
+
+def test_head_top_k_pipeline_and_errors(ctx, orc):
+    """scores -> top-k: the k best tokens of the projection, in order, without the logits leaving the device."""
+    import aq_mi355
+    say("head topk pipeline")
+    K, N, gs, bits, k = 1536, 50000, 32, 4, 16
+    words, s, b = F.synthetic_affine(N, K, bits, gs, seed=F.BASE_SEED + 104)
+    x = F.synthetic_x(1, K, seed=F.BASE_SEED + 105)
+    dw = DeviceAffine(ctx, words, s, b)
+    dx, dsc, dtop = ctx.to_device(x), ctx.alloc(N * 8), ctx.alloc(k * 8)
+    ctx.qmv_scores(dx, dw.w, dw.s, dw.b, dsc, 1, K, N, gs, bits)
+    ctx.packed_topk(dsc, N, k, dtop)
+    ctx.sync()
+    top = _u64(dtop, k)
+    logits = run_qmv(ctx, x, dw, 1, K, N, gs, bits, True)[0]
+    order = np.lexsort((np.arange(N), -logits.astype(np.float64)))[:k]
+    assert [(_unpack(p)[0]) for p in top] == order.tolist()
+    assert [np.float32(_unpack(p)[1]) for p in top] == [logits[i] for i in order]
+    buf = ctx.alloc(4096)
+    for call, code in [(lambda: ctx.qmv_greedy(buf, buf, buf, buf, None, 1, 64, 8), aq_mi355.AQ_ERR_ARG),
+                       (lambda: ctx.qmv_greedy(buf, buf, buf, buf, buf, 1, 64, 8, 3), aq_mi355.AQ_ERR_SHAPE),
+                       (lambda: ctx.qmv_greedy(buf, buf, buf, buf, buf, 1, 64, 8, 64, 4, None, 2), aq_mi355.AQ_ERR_ARG),
+                       (lambda: ctx.qmv_scores(buf, buf, buf, buf, buf, 1, 0, 8), aq_mi355.AQ_ERR_SHAPE),
+                       (lambda: ctx.packed_topk(buf, 10, 0, buf), aq_mi355.AQ_ERR_SHAPE),
+                       (lambda: ctx.packed_topk(buf, 10, 65, buf), aq_mi355.AQ_ERR_UNSUPPORTED),
+                       (lambda: ctx.packed_topk(None, 10, 4, buf), aq_mi355.AQ_ERR_ARG)]:
+        with pytest.raises(aq_mi355.AqError) as e:
+            call()
+        assert e.value.code == code
+    ctx.qmv_greedy(None, None, None, None, None, 0, 64, 8)     # no rows: nothing to do
+    best = ctx.to_device(np.full(1, 7, np.uint64))
+    ctx.qmv_greedy(None, None, None, None, best, 1, 64, 0)     # no vocabulary: best is cleared, no result
+    ctx.sync()
+    assert _u64(best, 1)[0] == 0
+    for t in (dx, dsc, dtop, buf, best):
+        t.free()
+    dw.free()

@@ -556,3 +556,55 @@ def test_moe_combine_fp32_and_bf16_steps(orc):
     assert np.array_equal(F.f32_to_bf16_bits(gotb), accb.view(torch.int16).numpy().view(np.uint16))
     # one route with weight one is the identity
     assert np.array_equal(orc.moe_combine(y[:3], np.ones(3, np.float32), 3, 1, n), y[:3])
+
+
+# ---- packed (score, token) values and the greedy reference --------------------------------------------
+
+def test_greedy_sample_reference_known_answer(orc):
+    # go/engine/hip/hip_transformer_reference_test.go:182-188
+    assert orc.greedy_sample_suppress([-1, 0.25, 0.2]) == (1, 0.25)
+    assert orc.greedy_sample_suppress([3, 7, 7, 1])[0] == 1                  # first maximum wins
+    assert orc.greedy_sample_suppress([3, 7, 7, 1], [1])[0] == 2             # suppressed tokens are skipped
+    assert orc.greedy_sample_suppress([-5, -2, -9], [1]) == (0, -5.0)
+    with pytest.raises(orc.OracleError):
+        orc.greedy_sample_suppress([1, 2], [0, 1])
+    with pytest.raises(orc.OracleError):
+        orc.greedy_sample_suppress([])
+
+
+def test_packed_best_orders_like_the_greedy_reference(orc):
+    """max over pack(score, token) == (first) argmax: brute force over value sets that include negatives,
+    signed zeros, denormals, equal scores and the float32 extremes."""
+    vals = np.array([0.0, -0.0, 1e-45, -1e-45, 1.0, -1.0, 0.25, 0.2, 3.4e38, -3.4e38, 1e-30, -1e-30, 65504.0, 2.5, 2.5],
+                    dtype=np.float32)
+    for i, a in enumerate(vals):
+        for j, b in enumerate(vals):
+            pa, pb = orc.pack_greedy_best(float(a), 7), orc.pack_greedy_best(float(b), 7)
+            if a < b:
+                assert pa < pb, (a, b)
+            elif a > b:
+                assert pa > pb, (a, b)
+    # equal scores: the lower token id packs higher
+    assert orc.pack_greedy_best(2.5, 3) > orc.pack_greedy_best(2.5, 4)
+    rng = np.random.default_rng(9)
+    for _ in range(50):
+        lg = rng.normal(0, 3, 40).astype(np.float32)
+        lg[rng.integers(0, 40, 6)] = lg.max()        # ties for the maximum
+        best = max(orc.pack_greedy_best(float(v), t) for t, v in enumerate(lg))
+        tok, sc = orc.unpack_greedy_best(best)
+        assert (tok, np.float32(sc)) == orc.greedy_sample_suppress(lg)
+    # explicit layout: hipPackGreedyBest(1, 2) = key(1.0) << 32 | ^2
+    assert orc.pack_greedy_best(1.0, 2) == ((0x3F800000 ^ 0x80000000) << 32) | 0xFFFFFFFD
+    assert orc.pack_greedy_best(-1.0, 0) == ((~0xBF800000 & 0xFFFFFFFF) << 32) | 0xFFFFFFFF
+
+
+def test_unpack_best_round_trip_softcap_and_errors(orc):
+    for score, token in [(1.0, 2), (-3.5, 0), (0.0, 262143), (1e-40, 5)]:
+        tok, sc = orc.unpack_greedy_best(orc.pack_greedy_best(score, token), 0.0, 262144)
+        assert tok == token and np.float32(sc) == np.float32(score)
+    tok, sc = orc.unpack_greedy_best(orc.pack_greedy_best(45.0, 9), 30.0, 100)
+    assert tok == 9 and abs(sc - math.tanh(45.0 / 30.0) * 30.0) < 1e-5
+    for args in [(0, 0.0, 10), (orc.pack_greedy_best(1.0, 10), 0.0, 10), (orc.pack_greedy_best(1.0, 1), -1.0, 10),
+                 (orc.pack_greedy_best(1.0, 1), float("nan"), 10), (orc.pack_greedy_best(1.0, 1), 0.0, 0)]:
+        with pytest.raises(orc.OracleError):
+            orc.unpack_greedy_best(*args)
