@@ -34,6 +34,27 @@ _c = ctypes
 _vp, _i, _u, _sz, _f = _c.c_void_p, _c.c_int, _c.c_uint, _c.c_size_t, _c.c_float
 _cp = _c.c_char_p
 
+class HostLinear(ctypes.Structure):
+    """aqh_linear (include/aq_mi355_host.h)."""
+    _fields_ = [("weight", _vp), ("scales", _vp), ("biases", _vp), ("bias", _vp),
+                ("weight_len", _sz), ("scales_len", _sz), ("biases_len", _sz), ("bias_len", _sz),
+                ("out_dim", _i), ("in_dim", _i), ("group_size", _i), ("bits", _i), ("quantised", _i),
+                ("experts", _i), ("expert_rows", _i)]
+
+    def view(self, which):
+        """numpy uint8 view of weight / scales / biases / bias (valid while the file stays open)."""
+        ptr, n = getattr(self, which), getattr(self, which + "_len")
+        if not ptr:
+            return None
+        return np.ctypeslib.as_array(ctypes.cast(ptr, ctypes.POINTER(ctypes.c_uint8)), shape=(n,))
+
+
+class DeviceLinear(ctypes.Structure):
+    """aq_device_linear (include/aq_mi355.h)."""
+    _fields_ = [("weight", _vp), ("scales", _vp), ("biases", _vp), ("rows", _i), ("in_dim", _i), ("group_size", _i),
+                ("bits", _i), ("experts", _i)]
+
+
 # name -> (restype, argtypes); every symbol include/*.h declares
 PROTOTYPES = {
     "aq_version": (_cp, []),
@@ -75,6 +96,9 @@ PROTOTYPES = {
     "aq_packed_topk": (_i, [_vp, _vp, _c.c_int64, _i, _vp]),
     "aq_pack_best": (_c.c_uint64, [_f, _i]),
     "aq_unpack_best": (_i, [_c.c_uint64, _f, _i, _c.POINTER(_i), _c.POINTER(_f)]),
+    "aq_upload_linear": (_i, [_vp, _c.POINTER(HostLinear), _c.POINTER(DeviceLinear)]),
+    "aq_upload_fused_gate_up": (_i, [_vp, _c.POINTER(HostLinear), _c.POINTER(HostLinear), _c.POINTER(DeviceLinear)]),
+    "aq_free_device_linear": (_i, [_vp, _c.POINTER(DeviceLinear)]),
     "aq_dequant_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _c.c_int64, _i, _i, _i]),
     "aq_matvec_host": (_i, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _i, _i, _i, _i, _vp, _sz]),
     "aq_proj_quant_matmul_host": (_i, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _i, _i, _i, _i, _i]),
@@ -91,6 +115,14 @@ PROTOTYPES = {
     "aqh_proj_quant_matmul_into": (_i, [_vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _i, _i, _i, _i, _i]),
     "aqh_concat_quant_rows": (_i, [_vp, _sz, _vp, _sz, _vp, _i, _vp, _sz, _vp, _sz, _vp, _i, _i, _i, _i, _i, _i, _i,
                                    _vp, _vp, _vp, _c.POINTER(_i)]),
+    "aqh_safetensors_open": (_i, [_cp, _c.POINTER(_vp)]),
+    "aqh_safetensors_close": (None, [_vp]),
+    "aqh_safetensors_count": (_i, [_vp]),
+    "aqh_safetensors_name": (_i, [_vp, _i, _cp, _sz]),
+    "aqh_safetensors_tensor": (_i, [_vp, _cp, _cp, _c.POINTER(_c.c_int64), _c.POINTER(_i), _c.POINTER(_vp),
+                                    _c.POINTER(_sz)]),
+    "aqh_load_linear": (_i, [_vp, _cp, _i, _c.POINTER(HostLinear)]),
+    "aqh_repack_b1_to_b2": (_i, [_vp, _sz, _sz, _sz, _i, _i, _i, _vp, _sz]),
     "aqh_affine_geometry": (None, [_i, _i, _i, _c.POINTER(_i), _c.POINTER(_i)]),
 }
 
@@ -296,6 +328,19 @@ class Context:
     def packed_topk(self, scores, count, top_k, out):
         self._check(self.lib.aq_packed_topk(self.handle, _ptr(scores), count, top_k, _ptr(out)))
 
+    def upload_linear(self, host_linear):
+        out = DeviceLinear()
+        self._check(self.lib.aq_upload_linear(self.handle, ctypes.byref(host_linear), ctypes.byref(out)))
+        return out
+
+    def upload_fused_gate_up(self, gate, up):
+        out = DeviceLinear()
+        self._check(self.lib.aq_upload_fused_gate_up(self.handle, ctypes.byref(gate), ctypes.byref(up), ctypes.byref(out)))
+        return out
+
+    def free_device_linear(self, dev_linear):
+        self._check(self.lib.aq_free_device_linear(self.handle, ctypes.byref(dev_linear)))
+
     def dequant_f32(self, w, s, b, out, N, K, group_size=64, bits=4):
         self._check(self.lib.aq_dequant_f32(self.handle, _ptr(w), _ptr(s), _ptr(b), _ptr(out), N, K, group_size,
                                             bits))
@@ -326,6 +371,55 @@ class Context:
                                                        scales.size, biases.ctypes.data, biases.size, M, K, N,
                                                        group_size, bits))
         return out.reshape(M, N)
+
+
+class SafetensorsFile:
+    """aqh_safetensors_* : a memory-mapped safetensors file read by the library's own loader."""
+
+    def __init__(self, path):
+        self.lib = load()
+        h = _vp()
+        rc = self.lib.aqh_safetensors_open(os.fsencode(path), ctypes.byref(h))
+        if rc != AQ_OK:
+            raise AqError(rc, self.lib.aqh_last_error().decode())
+        self.handle = h
+
+    def close(self):
+        if self.handle:
+            self.lib.aqh_safetensors_close(self.handle)
+            self.handle = None
+
+    def names(self):
+        out = []
+        buf = ctypes.create_string_buffer(1024)
+        for i in range(self.lib.aqh_safetensors_count(self.handle)):
+            if self.lib.aqh_safetensors_name(self.handle, i, buf, 1024) != AQ_OK:
+                raise AqError(AQ_ERR_SIZE, self.lib.aqh_last_error().decode())
+            out.append(buf.value.decode())
+        return out
+
+    def tensor(self, name):
+        """(dtype, shape, uint8 view)"""
+        dtype = ctypes.create_string_buffer(16)
+        shape = (_c.c_int64 * 8)()
+        rank, data, n = _i(0), _vp(), _sz(0)
+        rc = self.lib.aqh_safetensors_tensor(self.handle, name.encode(), dtype, shape, ctypes.byref(rank), ctypes.byref(data),
+                                             ctypes.byref(n))
+        if rc != AQ_OK:
+            raise AqError(rc, self.lib.aqh_last_error().decode())
+        view = (np.ctypeslib.as_array(ctypes.cast(data, ctypes.POINTER(ctypes.c_uint8)), shape=(n.value,))
+                if n.value else np.zeros(0, np.uint8))
+        return dtype.value.decode(), [int(shape[i]) for i in range(rank.value)], view
+
+    def load_linear(self, prefix, in_dim):
+        """model.LoadLinear; None when prefix.weight is absent."""
+        out = HostLinear()
+        rc = self.lib.aqh_load_linear(self.handle, prefix.encode(), in_dim, ctypes.byref(out))
+        if rc == AQ_ERR_INDEX:
+            return None
+        if rc != AQ_OK:
+            raise AqError(rc, self.lib.aqh_last_error().decode())
+        return out
 
 
 def pack_best(score, token):

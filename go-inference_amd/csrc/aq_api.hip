@@ -2,6 +2,7 @@
 // validation, kernel selection and launch.  See include/aq_mi355.h for the
 // contract of each entry point and the reference interface it replaces.
 #include "../../include/aq_mi355.h"
+#include "../../include/aq_mi355_host.h"
 
 #include <hip/hip_runtime.h>
 
@@ -252,6 +253,17 @@ int launch_qmv_rows(aq_ctx* ctx, aq::QmvArgs a, int group_size, int bits, bool g
     return AQ_OK;
 }
 
+}  // namespace
+
+namespace {
+// Scoped device allocations for the host-slice entry points.
+struct DevBuf {
+    void* p = nullptr;
+    ~DevBuf() {
+        if (p) (void)hipFree(p);
+    }
+    hipError_t alloc(size_t n) { return hipMalloc(&p, n ? n : 1); }
+};
 }  // namespace
 
 extern "C" {
@@ -1070,6 +1082,94 @@ int aq_unpack_best(uint64_t packed, float softcap, int vocab_size, int* token, f
     return AQ_OK;
 }
 
+namespace {
+
+// Geometry a loaded weight must satisfy before it may be handed to the kernels.
+int check_linear(const char* op, const aqh_linear* l) {
+    if (!l) return fail(AQ_ERR_ARG, "%s: null weight", op);
+    if (!l->quantised || !l->scales || !l->biases || !l->weight)
+        return fail(AQ_ERR_UNSUPPORTED, "%s: only affine-quantised weights (with scales and biases) are uploaded", op);
+    if (l->expert_rows <= 0 || l->experts < 0 || l->in_dim <= 0) return fail(AQ_ERR_SHAPE, "%s: invalid dimensions", op);
+    if (int rc = check_geometry(op, l->in_dim, l->group_size, l->bits)) return rc;
+    const size_t e = l->experts > 0 ? (size_t)l->experts : 1;
+    const size_t want_w = e * (size_t)l->expert_rows * ((size_t)l->in_dim * l->bits / 32) * 4;
+    const size_t want_sb = e * (size_t)l->expert_rows * (size_t)(l->in_dim / l->group_size) * 2;
+    if (l->weight_len != want_w || l->scales_len != want_sb || l->biases_len != want_sb)
+        return fail(AQ_ERR_SIZE, "%s: packed/scales/biases size mismatch", op);
+    return AQ_OK;
+}
+
+}  // namespace
+
+int aq_upload_linear(aq_ctx* ctx, const struct aqh_linear* lin, aq_device_linear* out) {
+    if (!ctx || !out) return fail(AQ_ERR_ARG, "aq_upload_linear: bad argument");
+    memset(out, 0, sizeof *out);
+    if (int rc = check_linear("aq_upload_linear", lin)) return rc;
+    AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    DevBuf w, s, b;
+    AQ_HIP(w.alloc(lin->weight_len), "hipMalloc");
+    AQ_HIP(s.alloc(lin->scales_len), "hipMalloc");
+    AQ_HIP(b.alloc(lin->biases_len), "hipMalloc");
+    if (int rc = aq_h2d(ctx, w.p, lin->weight, lin->weight_len)) return rc;
+    if (int rc = aq_h2d(ctx, s.p, lin->scales, lin->scales_len)) return rc;
+    if (int rc = aq_h2d(ctx, b.p, lin->biases, lin->biases_len)) return rc;
+    out->weight = w.p, out->scales = s.p, out->biases = b.p;
+    w.p = s.p = b.p = nullptr;
+    out->rows = lin->expert_rows;
+    out->in_dim = lin->in_dim;
+    out->group_size = lin->group_size;
+    out->bits = lin->bits;
+    out->experts = lin->experts;
+    return AQ_OK;
+}
+
+int aq_upload_fused_gate_up(aq_ctx* ctx, const struct aqh_linear* gate, const struct aqh_linear* up, aq_device_linear* out) {
+    if (!ctx || !out) return fail(AQ_ERR_ARG, "aq_upload_fused_gate_up: bad argument");
+    memset(out, 0, sizeof *out);
+    if (int rc = check_linear("aq_upload_fused_gate_up", gate)) return rc;
+    if (int rc = check_linear("aq_upload_fused_gate_up", up)) return rc;
+    // model.ConcatQuantRows' conditions (quant_weight.go:46-48), plus equal row and expert counts
+    if (gate->in_dim != up->in_dim || gate->bits != up->bits || gate->group_size != up->group_size ||
+        gate->expert_rows != up->expert_rows || gate->experts != up->experts)
+        return fail(AQ_ERR_SHAPE, "aq_upload_fused_gate_up: gate and up differ in geometry");
+    AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    const size_t experts = gate->experts > 0 ? (size_t)gate->experts : 1;
+    const size_t w_part = gate->weight_len / experts, sb_part = gate->scales_len / experts;
+    DevBuf w, s, b;
+    AQ_HIP(w.alloc(2 * gate->weight_len), "hipMalloc");
+    AQ_HIP(s.alloc(2 * gate->scales_len), "hipMalloc");
+    AQ_HIP(b.alloc(2 * gate->biases_len), "hipMalloc");
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    // one strided copy per part and array: expert e's rows go to [e][part]
+    struct Job {
+        void* dst;
+        const uint8_t* src;
+        size_t part;
+    } jobs[6] = {{w.p, gate->weight, w_part},  {static_cast<char*>(w.p) + w_part, up->weight, w_part},
+                 {s.p, gate->scales, sb_part}, {static_cast<char*>(s.p) + sb_part, up->scales, sb_part},
+                 {b.p, gate->biases, sb_part}, {static_cast<char*>(b.p) + sb_part, up->biases, sb_part}};
+    for (const Job& j : jobs)
+        AQ_HIP(hipMemcpy2DAsync(j.dst, 2 * j.part, j.src, j.part, j.part, experts, hipMemcpyHostToDevice, ctx->stream),
+               "hipMemcpy2D");
+    AQ_HIP(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+    out->weight = w.p, out->scales = s.p, out->biases = b.p;
+    w.p = s.p = b.p = nullptr;
+    out->rows = 2 * gate->expert_rows;
+    out->in_dim = gate->in_dim;
+    out->group_size = gate->group_size;
+    out->bits = gate->bits;
+    out->experts = gate->experts;
+    return AQ_OK;
+}
+
+int aq_free_device_linear(aq_ctx* ctx, aq_device_linear* lin) {
+    if (!ctx || !lin) return fail(AQ_ERR_ARG, "aq_free_device_linear: bad argument");
+    for (void* p : {lin->weight, lin->scales, lin->biases})
+        if (p) AQ_HIP(hipFree(p), "hipFree");
+    memset(lin, 0, sizeof *lin);
+    return AQ_OK;
+}
+
 int aq_dequant_f32(aq_ctx* ctx, const void* packed, const void* scales, const void* biases, float* out_f32, int64_t N,
                    int K, int group_size, int bits) {
     if (!ctx) return fail(AQ_ERR_ARG, "aq_dequant_f32: ctx is null");
@@ -1086,17 +1186,6 @@ int aq_dequant_f32(aq_ctx* ctx, const void* packed, const void* scales, const vo
            "hipLaunchKernel");
     return AQ_OK;
 }
-
-namespace {
-// Scoped device allocations for the host-slice entry points.
-struct DevBuf {
-    void* p = nullptr;
-    ~DevBuf() {
-        if (p) (void)hipFree(p);
-    }
-    hipError_t alloc(size_t n) { return hipMalloc(&p, n ? n : 1); }
-};
-}  // namespace
 
 int aq_matvec_host(aq_ctx* ctx, const uint8_t* x, size_t x_len, const uint8_t* packed, size_t packed_len,
                    const uint8_t* scales, size_t scales_len, const uint8_t* biases, size_t biases_len, int out_dim,

@@ -2,11 +2,13 @@
 // FFI caller) can drive model.BackendQuant(...).MatVec and attn.ProjQuantMatMulInto
 // exactly as Go code would.  Declared in include/aq_mi355_host.h.
 #include <cstring>
+#include <iterator>
 
 #include "../../../include/aq_mi355.h"
 #include "../../../include/aq_mi355_host.h"
 #include "model_quant.h"
 #include "rocm_affine.h"
+#include "safetensors.h"
 
 namespace {
 thread_local std::string g_err;
@@ -88,6 +90,85 @@ void aqh_affine_geometry(int in_dim, int scales_last_dim, int weight_last_dim, i
     if (scales_last_dim >= 0) s = {1, scales_last_dim};
     if (weight_last_dim >= 0) w = {1, weight_last_dim};
     model::affineGeometry(in_dim, s, w, group_size, bits);
+}
+
+int aqh_safetensors_open(const char* path, aqh_safetensors** out) {
+    if (!path || !out) return report(model::Error::make(AQ_ERR_ARG, "aqh_safetensors_open: bad argument"));
+    *out = nullptr;
+    std::unique_ptr<safetensors::File> f;
+    model::Error e = safetensors::File::Open(path, &f);
+    if (!e.ok()) return report(e);
+    *out = reinterpret_cast<aqh_safetensors*>(f.release());
+    return AQ_OK;
+}
+
+void aqh_safetensors_close(aqh_safetensors* f) { delete reinterpret_cast<safetensors::File*>(f); }
+
+int aqh_safetensors_count(const aqh_safetensors* f) {
+    return f ? (int)reinterpret_cast<const safetensors::File*>(f)->Tensors.size() : 0;
+}
+
+int aqh_safetensors_name(const aqh_safetensors* f, int index, char* buf, size_t buf_len) {
+    if (!f || !buf) return report(model::Error::make(AQ_ERR_ARG, "aqh_safetensors_name: bad argument"));
+    const auto& m = reinterpret_cast<const safetensors::File*>(f)->Tensors;
+    if (index < 0 || (size_t)index >= m.size()) return report(model::Error::make(AQ_ERR_INDEX, "tensor index out of range"));
+    auto it = m.begin();
+    std::advance(it, index);
+    if (it->first.size() + 1 > buf_len) return report(model::Error::make(AQ_ERR_SIZE, "name buffer too small"));
+    memcpy(buf, it->first.c_str(), it->first.size() + 1);
+    return AQ_OK;
+}
+
+int aqh_safetensors_tensor(const aqh_safetensors* f, const char* name, char dtype[16], int64_t shape[8], int* rank,
+                           const uint8_t** data, size_t* len) {
+    if (!f || !name) return report(model::Error::make(AQ_ERR_ARG, "aqh_safetensors_tensor: bad argument"));
+    const auto& m = reinterpret_cast<const safetensors::File*>(f)->Tensors;
+    auto it = m.find(name);
+    if (it == m.end()) return report(model::Error::make(AQ_ERR_INDEX, std::string("no tensor named ") + name));
+    const safetensors::Tensor& t = it->second;
+    if (t.Shape.size() > 8 || t.Dtype.size() > 15) return report(model::Error::make(AQ_ERR_UNSUPPORTED, "tensor rank or dtype name too long"));
+    if (dtype) {
+        memset(dtype, 0, 16);
+        memcpy(dtype, t.Dtype.c_str(), t.Dtype.size());
+    }
+    if (shape)
+        for (size_t i = 0; i < t.Shape.size(); i++) shape[i] = t.Shape[i];
+    if (rank) *rank = (int)t.Shape.size();
+    if (data) *data = t.Data;
+    if (len) *len = t.Len;
+    return AQ_OK;
+}
+
+int aqh_load_linear(aqh_safetensors* f, const char* prefix, int in_dim, aqh_linear* out) {
+    if (!f || !prefix || !out) return report(model::Error::make(AQ_ERR_ARG, "aqh_load_linear: bad argument"));
+    memset(out, 0, sizeof *out);
+    auto lin = model::LoadLinear(reinterpret_cast<safetensors::File*>(f), prefix, in_dim, "affine");
+    if (!lin) return report(model::Error::make(AQ_ERR_INDEX, std::string("no weight at ") + prefix));
+    out->weight = lin->Weight, out->weight_len = lin->WeightLen;
+    out->scales = lin->Scales, out->scales_len = lin->ScalesLen;
+    out->biases = lin->Biases, out->biases_len = lin->BiasesLen;
+    out->bias = lin->Bias, out->bias_len = lin->BiasLen;
+    out->out_dim = lin->OutDim, out->in_dim = lin->InDim, out->group_size = lin->GroupSize, out->bits = lin->Bits;
+    out->quantised = lin->Quantised() ? 1 : 0;
+    if (lin->WeightShape.size() == 3) {
+        out->experts = lin->WeightShape[0];
+        out->expert_rows = lin->WeightShape[1];
+    } else {
+        out->experts = 0;
+        out->expert_rows = lin->OutDim;
+    }
+    return AQ_OK;
+}
+
+int aqh_repack_b1_to_b2(const uint8_t* packed, size_t packed_len, size_t scales_len, size_t biases_len, int out_dim,
+                        int in_dim, int group_size, uint8_t* packed2, size_t packed2_len) {
+    if (!packed || !packed2) return report(model::Error::make(AQ_ERR_ARG, "aqh_repack_b1_to_b2: bad argument"));
+    model::Bytes p2;
+    model::Error e = model::RepackB1ToB2(packed, packed_len, scales_len, biases_len, out_dim, in_dim, group_size, &p2);
+    if (!e.ok()) return report(e);
+    if (p2.size() != packed2_len) return report(model::Error::make(AQ_ERR_SIZE, "aqh_repack_b1_to_b2: packed2 must hold out_dim*in_dim/4 bytes"));
+    memcpy(packed2, p2.data(), p2.size());
+    return AQ_OK;
 }
 
 }  // extern "C"

@@ -256,6 +256,30 @@ int aq_packed_topk(aq_ctx *ctx, const uint64_t *scores, int64_t count, int top_k
 uint64_t aq_pack_best(float score, int token);
 int aq_unpack_best(uint64_t packed, float softcap, int vocab_size, int *token, float *score);
 
+/* A quantised weight resident on the device, the three arrays every kernel entry point takes.
+ * experts == 0: [rows, ...]; experts > 0: an expert slab [experts, rows, ...] for the gathers. */
+typedef struct aq_device_linear {
+    void *weight, *scales, *biases;
+    int rows, in_dim, group_size, bits, experts;
+} aq_device_linear;
+struct aqh_linear; /* include/aq_mi355_host.h */
+
+/* Uploads one loaded weight (aqh_load_linear) straight from its file mapping: the device-binding half of the
+ * loader (the reference hands model.Linear's mmap views to hipUploadByteBuffer,
+ * go/engine/hip/hip_projection_launch.go:3086-3124 deviceBuffers).  Synchronous.  Dense (unquantised) weights are
+ * rejected with AQ_ERR_UNSUPPORTED. */
+int aq_upload_linear(aq_ctx *ctx, const struct aqh_linear *lin, aq_device_linear *out);
+
+/* Uploads gate and up as ONE slab whose experts hold [gate rows | up rows] (rank-2 weights: one "expert"), the
+ * layout aq_qmv_gate_up / aq_gather_qmv_gate_up read with up_row_base = rows.  This is the fused expert
+ * gate+up tensor the reference synthesises on the heap at load when a checkpoint ships them apart
+ * (Arch.FuseExpertGateUp, go/model/arch.go:167; row concatenation model.ConcatQuantRows,
+ * go/model/quant_weight.go:45-63); here the interleave happens in the copy itself (strided H2D), with no
+ * host copy of the weights.  out->rows is 2 * the rows of each part. */
+int aq_upload_fused_gate_up(aq_ctx *ctx, const struct aqh_linear *gate, const struct aqh_linear *up, aq_device_linear *out);
+
+int aq_free_device_linear(aq_ctx *ctx, aq_device_linear *lin);
+
 /* mlxaffine.DequantizeTensor on device (go/model/quant/mlxaffine/mlxaffine.go:178-208):
  * out_f32[N,K] = scale*code + bias, bit-exact with the CPU path. */
 int aq_dequant_f32(aq_ctx *ctx, const void *packed, const void *scales, const void *biases, float *out_f32, int64_t N,

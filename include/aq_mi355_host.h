@@ -9,6 +9,9 @@
  *   attn.ProjQuantMatMulInto                                          go/model/attn/gated_delta.go:46-58
  *   model.ConcatQuantRows                                             go/model/quant_weight.go:45-63
  *   model affineGeometry                                              go/model/linear.go:91-102
+ *   safetensors.ReadSafetensors / tensor views                        go/model/safetensors/safetensors.go:53-95
+ *   model.LoadLinear                                                  go/model/linear.go:42-84
+ *   mlxaffine.RepackB1ToB2                                            go/model/quant/mlxaffine/repack.go:27-62
  *
  * Return value: 0 ok, otherwise the AQ_ERR_* / hipError_t code; aqh_last_error() gives
  * the message (the Go `error` string).
@@ -58,6 +61,40 @@ int aqh_concat_quant_rows(const uint8_t *a_packed, size_t a_packed_len, const ui
 /* affineGeometry(inDim, scalesShape, weightShape) with the shapes' last dims (negative = empty shape)
  * (go/model/linear.go:91-110). */
 void aqh_affine_geometry(int in_dim, int scales_last_dim, int weight_last_dim, int *group_size, int *bits);
+
+/* A safetensors file, memory-mapped; tensors are views into the mapping and stay valid until
+ * aqh_safetensors_close (go/model/safetensors/safetensors.go:53-95; entry rules
+ * go/model/safetensors/header_parse.go:343-437: dtype, shape and data_offsets are required, unknown keys are
+ * skipped, offsets must be ordered and inside the file). */
+typedef struct aqh_safetensors aqh_safetensors;
+int aqh_safetensors_open(const char *path, aqh_safetensors **out);
+void aqh_safetensors_close(aqh_safetensors *f);
+int aqh_safetensors_count(const aqh_safetensors *f);
+/* Name of tensor `index` in sorted order; AQ_ERR_INDEX past the end, AQ_ERR_SIZE if buf is too short. */
+int aqh_safetensors_name(const aqh_safetensors *f, int index, char *buf, size_t buf_len);
+/* dtype (at most 15 characters), shape (at most 8 dims), bytes.  AQ_ERR_INDEX when the tensor is absent. */
+int aqh_safetensors_tensor(const aqh_safetensors *f, const char *name, char dtype[16], int64_t shape[8], int *rank,
+                           const uint8_t **data, size_t *len);
+
+/* model.Linear (go/model/linear.go:21-33) as plain data: views into the file (or, after the 1-bit -> 2-bit
+ * widening, into a buffer the file object owns).  scales == NULL means dense bf16.  experts / expert_rows
+ * describe a rank-3 [experts, expert_rows, words] weight (an MoE expert stack); experts == 0 for rank 2. */
+typedef struct aqh_linear {
+    const uint8_t *weight, *scales, *biases, *bias;
+    size_t weight_len, scales_len, biases_len, bias_len;
+    int out_dim, in_dim, group_size, bits;
+    int quantised;
+    int experts, expert_rows;
+} aqh_linear;
+
+/* model.LoadLinear(tensors, prefix, inDim, "affine") (go/model/linear.go:42-84): ".scales" present means
+ * quantised, geometry from the shapes, a 1-bit pack is widened to 2 bits and written back into the file
+ * object's tensor map.  AQ_ERR_INDEX when prefix + ".weight" is absent (Go returns nil). */
+int aqh_load_linear(aqh_safetensors *f, const char *prefix, int in_dim, aqh_linear *out);
+
+/* mlxaffine.RepackB1ToB2 on caller buffers: packed2 holds out_dim * in_dim / 4 bytes. */
+int aqh_repack_b1_to_b2(const uint8_t *packed, size_t packed_len, size_t scales_len, size_t biases_len, int out_dim,
+                        int in_dim, int group_size, uint8_t *packed2, size_t packed2_len);
 
 #ifdef __cplusplus
 }
