@@ -46,6 +46,10 @@ int qmmt_variant_count();
 const QmmVariant* qmmt_variant(int idx);
 // Device bytes the tile kernels need beside their operands for an M x K activation matrix.
 size_t qmmt_workspace_bytes(int M, int K);
+// Variants named *_q move scales, biases and block sums through LDS as well; they take group size 64,
+// K a multiple of 512 and 16-byte aligned scale / bias arrays.
+bool qmmt_quad_staging_ok(const QmmArgs& a);
+bool qmmt_variant_stages_quads(int idx);
 // Pass over x + tile kernel `idx`; `workspace` holds at least qmmt_workspace_bytes(M, K).
 hipError_t qmmt_launch(int idx, const QmmArgs& a, void* workspace, hipStream_t stream);
 

@@ -465,6 +465,8 @@ int qmm_dispatch(hipStream_t stream, Workspace* ws, int cu_count, int forced, co
         tile_idx = idx - n_direct;
         const QmmVariant* v = qmmt_variant(tile_idx);
         if (!v || v->bits != bits) return fail(AQ_ERR_ARG, "aq_qmm: forced variant %d does not fit bits=%d", idx, bits);
+        if (qmmt_variant_stages_quads(tile_idx) && !qmmt_quad_staging_ok(a))
+            return fail(AQ_ERR_ARG, "aq_qmm: forced variant %d needs group size 64, K %% 512 == 0 and 16-byte aligned scales", idx);
     } else if (idx < 0 && M >= 64) {
         // prefill sizes: the LDS-staged 128 x 128 tiles (four 64 x 64 wavefront tiles, two workgroups a CU);
         // the 128 x 64 wavefront tiles need more registers than two wavefronts a SIMD leave and measure slower

@@ -63,8 +63,11 @@ __device__ __forceinline__ uint32_t dup16(uint32_t h) { return (h & 0xffffu) | (
 // orders them itself with counted waits.  Hidden from the compiler, a copy can only make the
 // compiler's own waits for ordinary loads stricter, never weaker (completion is in order).
 // m0 is reserved by the compiler (it sets it before each of its own uses), so writing it here is safe.
-__device__ __forceinline__ void copy16_to_lds(const void* src_lane, uint32_t lds_base_uniform) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src_lane), "s"(lds_base_uniform)
+// The source address is a wave-uniform 64-bit base in SGPRs plus a 32-bit byte offset per lane, so the address
+// arithmetic of the main loop runs on the scalar unit.
+__device__ __forceinline__ void copy16_to_lds(const void* base_uniform, uint32_t lane_offset, uint32_t lds_base_uniform) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(base_uniform),
+                 "s"(lds_base_uniform)
                  : "memory");
 }
 __device__ __forceinline__ uint32_t lds_offset(const void* p) {
@@ -126,8 +129,13 @@ __global__ __launch_bounds__(256) void qmm_prep_kernel(const uint16_t* __restric
 
 // ---- main kernel ----------------------------------------------------------------------------
 // Wavefront tiles of at most 64 x 64 keep under 256 registers, so two wavefronts share a SIMD.
-template <int BITS, int MB, int NB, int WM, int WN>
+// SBL: scales, biases and block sums also travel global -> LDS by copy instructions (then the loop holds no
+// load the compiler has to wait for: it cannot count the copies, so any wait of its own drains them all).
+// Needs group size 64, K a multiple of 512 and 16-byte aligned scale / bias rows.
+template <int BITS, int MB, int NB, int WM, int WN, int STAGES, bool SBL>
 __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTileArgs a) {
+    static_assert(STAGES == 3 || STAGES == 4, "LDS stages");
+    constexpr int AHEAD = STAGES - 1;  // iteration g requests block g + AHEAD
     constexpr int BM = WM * MB * 32;
     constexpr int BN = WN * NB * 32;
     constexpr int NWAVE = WM * WN;
@@ -148,8 +156,16 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
     static_assert(W_PIECES % kWave == 0, "a copy instruction moves 64 pieces");
 
     extern __shared__ __align__(16) uint8_t lds[];
-    uint8_t* const abuf = lds;                // [3][A_STAGE]
-    uint8_t* const bbuf = lds + 3 * A_STAGE;  // [3][B_STAGE]
+    uint8_t* const abuf = lds;                     // [STAGES][A_STAGE]
+    uint8_t* const bbuf = lds + STAGES * A_STAGE;  // [STAGES][B_STAGE]
+    // SBL: one quad ahead of (hi, lo) sums per tile row, and 16 bytes (eight blocks) of scales and of biases
+    // per tile column
+    uint8_t* const xsq = bbuf + STAGES * B_STAGE;  // [BM][16]
+    uint8_t* const sq = xsq + BM * 16;             // [BN][16]
+    uint8_t* const bq = sq + BN * 16;              // [BN][16]
+    constexpr int SB_SLOTS = BM / 64 + 2 * (BN / 64);           // 1 KiB copies per quad and workgroup
+    constexpr int SBE = SBL ? (SB_SLOTS + NWAVE - 1) / NWAVE : 0;  // per wavefront (spare slots repeat one)
+    static_assert(!SBL || (BM % 64 == 0 && BN % 64 == 0), "quad staging moves 64 rows per copy");
 
     // tile of this workgroup: workgroups are dealt to the 8 XCDs round-robin, so every 8th one
     // shares an L2; give each XCD a contiguous run of tiles in row-band-major order
@@ -185,27 +201,65 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
             const int blk = wave + q * NWAVE;
             int mblk = m0 / 32 + (blk >> 2);
             mblk = mblk < a.mblks ? mblk : a.mblks - 1;  // past the end: any valid rows, never stored
-            const uint16_t* src = a.xf + ((int64_t)mblk * ksteps + g * 4 + (blk & 3)) * 512 + lane * 8;
-            copy16_to_lds(src, __builtin_amdgcn_readfirstlane(lds_offset(dst + blk * 1024)));
+            const uint16_t* src = a.xf + ((int64_t)mblk * ksteps + g * 4 + (blk & 3)) * 512;
+            copy16_to_lds(src, (uint32_t)lane * 16u, lds_offset(dst + blk * 1024));
         }
     };
 
     // B: the tile's packed rows, 16-byte pieces; copy instruction i of this wavefront moves pieces
     // (i * NWAVE + wave) * 64 + lane to consecutive LDS slots, which leaves row r at r * (WPB * 4) bytes
-    const uint32_t* wsrc[WPT];
+    // (rows past N repeat the last row; a tile spans well under 4 GiB, so the lane part fits 32 bits)
+    const uint32_t* const wtile = a.w + (int64_t)min(n0, N - 1) * words_per_row;
+    uint32_t woff[WPT];
 #pragma unroll
     for (int i = 0; i < WPT; i++) {
         const int p = (i * NWAVE + wave) * kWave + lane;
         constexpr int PPR = WPB / 4;  // pieces per row
         const int r = p / PPR, q = p % PPR;
         const int n = min(n0 + r, N - 1);
-        wsrc[i] = a.w + (int64_t)n * words_per_row + q * 4;
+        woff[i] = (uint32_t)(n - min(n0, N - 1)) * (uint32_t)(words_per_row * 4) + (uint32_t)q * 16u;
     }
     auto issue_b = [&](int g, int stage) {
         uint8_t* dst = bbuf + stage * B_STAGE;
 #pragma unroll
         for (int i = 0; i < WPT; i++)
-            copy16_to_lds(wsrc[i] + (int64_t)g * WPB, __builtin_amdgcn_readfirstlane(lds_offset(dst + (i * NWAVE + wave) * 1024)));
+            copy16_to_lds(wtile + (int64_t)g * WPB, woff[i], lds_offset(dst + (i * NWAVE + wave) * 1024));
+    };
+    // SBL: slot e of this wavefront: which array, which 64 rows
+    const uint8_t* sb_src[SBE > 0 ? SBE : 1];
+    uint32_t sb_off[SBE > 0 ? SBE : 1];
+    uint32_t sb_dst[SBE > 0 ? SBE : 1];
+    bool sb_is_xs[SBE > 0 ? SBE : 1];
+    if constexpr (SBL) {
+#pragma unroll
+        for (int e = 0; e < SBE; e++) {
+            const int slot = (wave * SBE + e) % SB_SLOTS;
+            if (slot < BM / 64) {
+                int row = m0 + slot * 64 + lane;
+                row = row < a.mblks * 32 ? row : a.mblks * 32 - 1;
+                sb_src[e] = reinterpret_cast<const uint8_t*>(a.xs);
+                sb_off[e] = (uint32_t)row * (uint32_t)G4 * 16u;
+                sb_dst[e] = lds_offset(xsq + slot * 1024);
+                sb_is_xs[e] = true;
+            } else {
+                const int t = slot - BM / 64;
+                const bool bias = t >= BN / 64;
+                const int n = min(n0 + (bias ? t - BN / 64 : t) * 64 + lane, N - 1);
+                sb_src[e] = reinterpret_cast<const uint8_t*>(bias ? a.b : a.s);
+                sb_off[e] = (uint32_t)n * (uint32_t)sb_per_row * 2u;
+                sb_dst[e] = lds_offset((bias ? bq : sq) + (bias ? t - BN / 64 : t) * 1024);
+                sb_is_xs[e] = false;
+            }
+        }
+    }
+    // requests quad `quad` (clamped to the last one) into the staging rows
+    auto issue_quad = [&](int quad) {
+        if constexpr (SBL) {
+            const int nq = quad < G4 ? quad : G4 - 1;
+#pragma unroll
+            for (int e = 0; e < SBE; e++)
+                copy16_to_lds(sb_src[e] + (sb_is_xs[e] ? nq * 16 : (nq >> 1) * 16), sb_off[e], sb_dst[e]);
+        }
     };
     const uint32_t mask_s = opaque_s(kMask16);
     const uint32_t magic_v = opaque_v(kMagic16);
@@ -285,7 +339,20 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
     auto iteration = [&](auto q_tag, int g) {
         constexpr int Q = decltype(q_tag)::value;
         const bool more = g + 1 < G;
-        if constexpr (Q == 0) {
+        if constexpr (Q == 0 && SBL) {
+            // the quad's scales, biases and sums landed in LDS two blocks ago (the first quad: before the loop)
+            const int half = ((g >> 2) & 1) * 8;
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) {
+                const int col = (wave_n * NB + nb) * 32 + j;
+                s_cur[nb] = *reinterpret_cast<const uint2*>(sq + col * 16 + half);
+                b_cur[nb] = *reinterpret_cast<const uint2*>(bq + col * 16 + half);
+            }
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++)
+                xs_cur[mb] = *reinterpret_cast<const uint4*>(xsq + ((wave_m * MB + mb) * 32 + j) * 16);
+        }
+        if constexpr (Q == 0 && !SBL) {
             // the quad's scales, biases and sums were requested three blocks ago (the first quad: before
             // the loop).  Taken over here, before this iteration's copies are issued: the compiler waits
             // for every request it cannot count before the first use of a loaded register.
@@ -297,15 +364,16 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
 #pragma unroll
             for (int mb = 0; mb < MB; mb++) xs_cur[mb] = xs_nxt[mb];
         }
-        if constexpr (Q == 1) {
+        if constexpr (Q == 1 && SBL) issue_quad((g >> 2) + 1);  // every wavefront read the staging rows in the block before
+        if constexpr (Q == 1 && !SBL) {
             // ordinary loads first: the wait at the end of the iteration counts the copies behind them
             const int nq = (g >> 2) + 1 < G4 ? (g >> 2) + 1 : G4 - 1;
             load_quad(nq, s_nxt, b_nxt);
             load_xs(nq, xs_nxt);
         }
         {
-            const int g2 = g + 2 < G ? g + 2 : glast;
-            const int s2 = sa == 0 ? 2 : sa - 1;  // stage (sa + 2) % 3: read last in iteration g-1
+            const int g2 = g + AHEAD < G ? g + AHEAD : glast;
+            const int s2 = sa == 0 ? STAGES - 1 : sa - 1;  // stage (sa + AHEAD) % STAGES: read last in iteration g-1
             issue_a(g2, s2);
             issue_b(g2, s2);
         }
@@ -378,23 +446,30 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
             }
         }
 
-        sa = sa == 2 ? 0 : sa + 1;
-        // Block g+1 has landed once at most this iteration's own copies (of block g+2) are outstanding;
+        sa = sa == STAGES - 1 ? 0 : sa + 1;
+        // Block g+1 has landed once at most the copies of the AHEAD-1 newest blocks are outstanding;
         // this iteration's LDS reads have returned.  A bare s_barrier on purpose: __syncthreads() carries
         // a workgroup fence, for which the compiler drains ALL outstanding copies into LDS.
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(GROUP_OPS) : "memory");
+        // (the quad copies of block Q == 1 stay countable as long as they are among the AHEAD-1 newest groups)
+        constexpr int QUAD_OPS = (SBL && Q >= 1 && Q <= AHEAD - 1) ? SBE : 0;
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((AHEAD - 1) * GROUP_OPS + QUAD_OPS) : "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
     };
 
-    // the first quad and blocks 0 and 1 are requested up front
-    load_quad(0, s_nxt, b_nxt);
-    load_xs(0, xs_nxt);
-    issue_a(0, 0);
-    issue_b(0, 0);
-    issue_a(1 < G ? 1 : glast, 1);
-    issue_b(1 < G ? 1 : glast, 1);
-    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(GROUP_OPS) : "memory");  // block 0 has landed
+    // the first quad and blocks 0 .. AHEAD-1 are requested up front
+    if constexpr (SBL) {
+        issue_quad(0);
+    } else {
+        load_quad(0, s_nxt, b_nxt);
+        load_xs(0, xs_nxt);
+    }
+#pragma unroll
+    for (int d = 0; d < AHEAD; d++) {
+        issue_a(d < G ? d : glast, d);
+        issue_b(d < G ? d : glast, d);
+    }
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((AHEAD - 1) * GROUP_OPS) : "memory");  // block 0 has landed
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 
@@ -437,17 +512,22 @@ struct QmmTileEntry {
     QmmVariant v;
     QmmTileKernel fn;
     int lds_bytes;
+    bool sbl;  // stages scales, biases and sums through LDS: needs qmmt_quad_staging_ok()
 };
 
-#define AQ_QMMT(BITS, MB, NB, WM, WN)                                                    \
-    {                                                                                    \
-        {"qmmt_b" #BITS "_mb" #MB "_nb" #NB "_wm" #WM "_wn" #WN, BITS, MB, NB, WM, WN},  \
-            qmm_tile_kernel<BITS, MB, NB, WM, WN>, 3 * (WM * MB * 4096 + WN * NB * 32 * (BITS == 4 ? 32 : 64))        \
+#define AQ_QMMT_S(BITS, MB, NB, WM, WN, ST, SBL, SUFFIX)                                                  \
+    {                                                                                                    \
+        {"qmmt_b" #BITS "_mb" #MB "_nb" #NB "_wm" #WM "_wn" #WN SUFFIX, BITS, MB, NB, WM, WN},           \
+            qmm_tile_kernel<BITS, MB, NB, WM, WN, ST, SBL>,                                              \
+            ST * (WM * MB * 4096 + WN * NB * 32 * (BITS == 4 ? 32 : 64)) + (SBL ? (WM * MB * 32 + 2 * WN * NB * 32) * 16 : 0), SBL \
     }
+#define AQ_QMMT(BITS, MB, NB, WM, WN) AQ_QMMT_S(BITS, MB, NB, WM, WN, 3, false, "")
 #define AQ_QMMT_SET(BITS)                                                                        \
     AQ_QMMT(BITS, 4, 2, 2, 2), AQ_QMMT(BITS, 4, 2, 1, 2), AQ_QMMT(BITS, 2, 2, 2, 2),             \
         AQ_QMMT(BITS, 2, 2, 1, 2), AQ_QMMT(BITS, 4, 2, 1, 4),         \
-        AQ_QMMT(BITS, 2, 2, 2, 4), AQ_QMMT(BITS, 1, 2, 1, 4)
+        AQ_QMMT(BITS, 2, 2, 2, 4), AQ_QMMT(BITS, 1, 2, 1, 4), AQ_QMMT_S(BITS, 2, 2, 2, 2, 4, false, "_s4"), \
+        AQ_QMMT_S(BITS, 2, 2, 1, 4, 4, false, "_s4"), AQ_QMMT_S(BITS, 2, 2, 1, 4, 3, false, ""),       \
+        AQ_QMMT_S(BITS, 2, 2, 2, 2, 3, true, "_q"), AQ_QMMT_S(BITS, 2, 2, 1, 4, 3, true, "_q")
 
 static const QmmTileEntry kQmmTileTable[] = {AQ_QMMT_SET(4), AQ_QMMT_SET(8)};
 
@@ -463,9 +543,15 @@ size_t qmmt_workspace_bytes(int M, int K) {
     return mblks * 32 * (size_t)K * 2 + mblks * 32 * g4 * 16;
 }
 
+bool qmmt_quad_staging_ok(const QmmArgs& q) {
+    return q.gs_blocks == 1 && q.K % 512 == 0 && ((reinterpret_cast<uintptr_t>(q.s) | reinterpret_cast<uintptr_t>(q.b)) & 15) == 0;
+}
+bool qmmt_variant_stages_quads(int idx) { return idx >= 0 && idx < qmmt_variant_count() && kQmmTileTable[idx].sbl; }
+
 hipError_t qmmt_launch(int idx, const QmmArgs& q, void* workspace, hipStream_t stream) {
     if (idx < 0 || idx >= qmmt_variant_count()) return hipErrorInvalidValue;
     const QmmTileEntry& e = kQmmTileTable[idx];
+    if (e.sbl && !qmmt_quad_staging_ok(q)) return hipErrorInvalidValue;
     const int mblks = (q.M + 31) / 32;
     uint16_t* xf = static_cast<uint16_t*>(workspace);
     uint16_t* xs = xf + (size_t)mblks * 32 * q.K;

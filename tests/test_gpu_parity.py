@@ -567,21 +567,27 @@ def test_qmm_small_cases(ctx, orc, M, K, N, bits, gs):
 def test_qmm_every_variant(ctx, orc):
     import aq_mi355
     names = aq_mi355.variant_names(1)
-    M, K, N = 150, 704, 200
+    M, N = 150, 200
     data = {}
     try:
         for idx, name in enumerate(names):
             say("qmm variant", idx, name)
             bits = int(name.split("_")[1][1:])
-            if bits not in data:
+            # variants that stage scales through LDS take K in multiples of 512 (1536: three quads, the last
+            # octet half used); the others get a K that ends in the middle of a quad
+            K = 1536 if name.endswith("_q") else 704
+            if (bits, K) not in data:
                 words, s, b = F.synthetic_affine(N, K, bits, 64, seed=700 + bits)
                 x = F.synthetic_x(M, K, seed=800 + bits)
-                data[bits] = (DeviceAffine(ctx, words, s, b), x, F.reference_f64(x, words, s, b, bits, 64, K))
-            dw, x, ref = data[bits]
+                data[(bits, K)] = (DeviceAffine(ctx, words, s, b), x, F.reference_f64(x, words, s, b, bits, 64, K))
+            dw, x, ref = data[(bits, K)]
             ctx.force_variant(1, idx)
             acc = run_qmv(ctx, x, dw, M, K, N, 64, bits, True, "qmm")
             assert ctx.last_variant(1) == name
             check_accumulators(acc, ref, name)
+            if name.endswith("_q"):
+                with pytest.raises(aq_mi355.AqError):      # a K the staging cannot take is refused, not mangled
+                    run_qmv(ctx, x[:, :704].copy(), dw, M, 704, N, 64, bits, True, "qmm")
     finally:
         ctx.force_variant(1, -1)
     for dw, _, _ in data.values():
