@@ -313,7 +313,7 @@ def main():
         ctx.reserve_workspace(64, K)
         for bits in (4, 8):
             pool = pools[bits]
-            for M in (1, 2, 4, 8, 16, 32):
+            for M in (1, 2, 4, 8, 16, 32, 64):
                 xm = ctx.to_device(F.synthetic_x(M, K, seed=F.BASE_SEED + 1100 + M))
                 ym = ctx.alloc(M * N * 2)
                 n = 60

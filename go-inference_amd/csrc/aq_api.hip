@@ -484,14 +484,26 @@ int aq_qmv(aq_ctx* ctx, const void* x, const void* packed, const void* scales, c
     a.out_f32 = (flags & AQ_OUT_F32) ? 1 : 0;
     a.routes = 1;
     if (M > aq::kQmvMaxRows && ctx->forced[0] < 0) {
-        // more rows than the dot2 kernels take: the block-MFMA family where the shape fits (it takes 4
-        // rows a launch whenever it takes any), else the matmul tiles
+        // More rows than the dot2 kernels take.  The block-MFMA family streams the weights once per launch of
+        // up to 16 rows (4 where K is long); when the call fits one such launch it is the fastest.  Beyond that
+        // the matmul tiles with K shared out over workgroups read the weights once for all rows.
         aq::BlkPlan plan;
         aq::QmvArgs probe = a;
-        probe.M = 4;
-        if (M > 64 || !aq::qmvb_plan(probe, bits, group_size, false, ctx->cu_count, -1, &plan))
-            return aq::qmm_dispatch(ctx->stream, &ctx->ws, ctx->cu_count, ctx->forced[1], &ctx->last_variant[1], x, packed,
-                                    scales, biases, y, M, K, N, group_size, bits, (flags & AQ_OUT_F32) != 0, fail);
+        int rows_per_launch = 0;
+        for (int rows : {16, 4}) {
+            probe.M = M < rows ? M : rows;
+            if (aq::qmvb_plan(probe, bits, group_size, false, ctx->cu_count, -1, &plan)) {
+                rows_per_launch = rows;
+                break;
+            }
+        }
+        if (rows_per_launch == 0 || M > 64 || M > rows_per_launch) {
+            const int rc = aq::qmm_dispatch(ctx->stream, &ctx->ws, ctx->cu_count, ctx->forced[1], &ctx->last_variant[1], x,
+                                            packed, scales, biases, y, M, K, N, group_size, bits,
+                                            (flags & AQ_OUT_F32) != 0, fail);
+            if (rc == AQ_OK) ctx->last_variant[0] = ctx->last_variant[1];  // the kernel this aq_qmv call ran
+            return rc;
+        }
     }
     return launch_qmv_rows(ctx, a, group_size, bits, false);
 }
@@ -575,6 +587,14 @@ int aq_reserve_workspace(aq_ctx* ctx, int M, int K) {
     return aq::qmm_reserve(ctx->stream, &ctx->ws, M, K, fail);
 }
 
+int aq_reserve_workspace_bytes(aq_ctx* ctx, size_t bytes) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_reserve_workspace_bytes: ctx is null");
+    if (bytes == 0) return AQ_OK;
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    return aq::workspace_reserve(ctx->stream, &ctx->ws, bytes, fail);
+}
+
 int aq_gather_qmv(aq_ctx* ctx, const void* x, const void* packed, const void* scales, const void* biases,
                   const int32_t* lhs, const int32_t* rhs, void* y, int routes, int x_rows, int K, int N,
                   int num_experts, int expert_rows, int row_base, int group_size, int bits, unsigned flags) {
@@ -618,9 +638,9 @@ namespace {
 
 bool act_ok(int act) { return act == AQ_ACT_GELU_TANH || act == AQ_ACT_SILU; }
 
-// Bytes of the workspace the matmul path may claim for an M x K activation matrix, rounded so that
-// whatever follows it stays 256-byte aligned.
-size_t qmm_region(int M, int K) { return (aq::qmmt_workspace_bytes(M, K) + 255) & ~(size_t)255; }
+// Bytes of the workspace the matmul path may claim for an M x K by N call (activations in fragment order,
+// partial tiles of a K split), 256-byte aligned: the unfused fallbacks keep their intermediates behind it.
+size_t qmm_region(int M, int K, int N) { return aq::qmm_scratch_bytes(M, K, N); }
 
 // Rows per wavefront for the activation-fused dot2 kernels: `slots` row streams a wavefront of the
 // plain kernel would take for this much work, shared between the two matrices of a pair.
@@ -692,7 +712,7 @@ int aq_qmv_gate_up(aq_ctx* ctx, const void* x, const void* gate_packed, const vo
         }
     }
     // two projections into fp32 scratch, then the element-wise step
-    const size_t region = qmm_region(M, K);
+    const size_t region = qmm_region(M, K, N);
     const size_t each = (((size_t)M * N * 4) + 255) & ~(size_t)255;
     {
         std::lock_guard<std::mutex> lk(ctx->mu);
@@ -813,7 +833,7 @@ int aq_qmv_act(aq_ctx* ctx, const void* gate_x, const void* up_x, const void* pa
             return AQ_OK;
         }
     }
-    const size_t region = qmm_region(M, K);
+    const size_t region = qmm_region(M, K, N);
     {
         std::lock_guard<std::mutex> lk(ctx->mu);
         AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
@@ -997,7 +1017,7 @@ int head_call(aq_ctx* ctx, const char* op, int fuse, const void* x, const void* 
         }
     }
     // the projection as fp32 into scratch, then the same epilogue over it
-    const size_t region = qmm_region(M, K);
+    const size_t region = qmm_region(M, K, N);
     {
         std::lock_guard<std::mutex> lk(ctx->mu);
         AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");

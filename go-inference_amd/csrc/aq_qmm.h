@@ -40,6 +40,9 @@ struct QmmTileArgs {
     int out_f32;
     int mblks;             // ceil(M / 32)
     int tiles_m, tiles_n;  // workgroup tiles along M and N
+    int ksplit;            // workgroups that share a tile along K (1: none)
+    int gsplit;            // 64-code blocks of K per workgroup (a multiple of 4)
+    float* partial;        // ksplit > 1: fp32 partial tiles [ksplit][M][N]
 };
 
 int qmmt_variant_count();
@@ -52,6 +55,10 @@ bool qmmt_quad_staging_ok(const QmmArgs& a);
 bool qmmt_variant_stages_quads(int idx);
 // Pass over x + tile kernel `idx`; `workspace` holds at least qmmt_workspace_bytes(M, K).
 hipError_t qmmt_launch(int idx, const QmmArgs& a, void* workspace, hipStream_t stream);
+// The same with K shared out over ksplit workgroups per tile and a second kernel that adds the partial
+// tiles: for few rows of x, where M x N tiles alone leave most of the chip idle.
+size_t qmmt_splitk_bytes(int M, int N, int ksplit);
+hipError_t qmmt_launch_splitk(int idx, const QmmArgs& a, void* workspace, int ksplit, hipStream_t stream);
 
 // Scratch memory a context lends to the matmul path; grown on demand, never while a capture is open.
 struct Workspace {
@@ -70,6 +77,11 @@ typedef int (*FailFn)(int code, const char* fmt, ...);
 // Makes ws hold at least `need` bytes (drains the stream and reallocates when it must grow; refused
 // while the stream is being captured).
 int workspace_reserve(hipStream_t stream, Workspace* ws, size_t need, FailFn fail);
+
+// Upper bound (256-byte aligned) of the workspace bytes qmm_dispatch may use for an M x K by N call: the
+// rewritten activations and, for few rows, the fp32 partial tiles of the K split.  Callers that keep their
+// own data in the same workspace place it behind this.
+size_t qmm_scratch_bytes(int M, int K, int N);
 
 // Sizes ws for activations of M x K ahead of time (not during capture).
 int qmm_reserve(hipStream_t stream, Workspace* ws, int M, int K, FailFn fail);

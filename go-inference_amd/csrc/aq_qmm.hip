@@ -411,6 +411,12 @@ int workspace_reserve(hipStream_t stream, Workspace* ws, size_t need, FailFn fai
     return grow_workspace(ws, need, stream, fail);
 }
 
+size_t qmm_scratch_bytes(int M, int K, int N) {
+    const size_t xbytes = (qmmt_workspace_bytes(M, K) + 255) & ~(size_t)255;
+    const size_t partial = (M > 4 && M <= 64) ? qmmt_splitk_bytes(M, N, 16) : 0;
+    return xbytes + ((partial + 255) & ~(size_t)255);
+}
+
 int qmm_reserve(hipStream_t stream, Workspace* ws, int M, int K, FailFn fail) {
     return grow_workspace(ws, qmmt_workspace_bytes(M, K), stream, fail);
 }
@@ -426,7 +432,6 @@ static int find_qmmt(int bits, int mb, int nb, int wm, int wn) {
 int qmm_dispatch(hipStream_t stream, Workspace* ws, int cu_count, int forced, const char** last_variant, const void* x,
                  const void* packed, const void* scales, const void* biases, void* y, int M, int K, int N,
                  int group_size, int bits, bool out_f32, FailFn fail) {
-    (void)cu_count;
     const bool mfma_ok = (bits == 4 || bits == 8) && (group_size == 64 || group_size == 128) && K % 64 == 0 &&
                          (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(packed) & 15) == 0;
     if (!mfma_ok) {
@@ -472,10 +477,30 @@ int qmm_dispatch(hipStream_t stream, Workspace* ws, int cu_count, int forced, co
         // the 128 x 64 wavefront tiles need more registers than two wavefronts a SIMD leave and measure slower
         tile_idx = find_qmmt(bits, 2, 2, 2, 2);
     }
+    // Few rows of x: M x N tiles alone would occupy a fraction of the chip (56 workgroups for 32 x 14336), so
+    // K is shared out as well and a small kernel adds the partial tiles.
+    int ksplit = 1;
+    if (idx < 0 && M > 4 && M <= 64 && (K / 64) % 4 == 0) {
+        const int want = find_qmmt(bits, M <= 32 ? 1 : 2, 2, 1, 4);
+        if (want >= 0) {
+            const int bm = M <= 32 ? 32 : 64;
+            const int tiles = ((M + bm - 1) / bm) * ((N + 255) / 256);
+            const int cus = cu_count > 0 ? cu_count : 256;
+            int ks = 1;
+            // (measured: one workgroup a CU is the sweet spot; more splits cost more in partial tiles than they
+            // gain in parallel streams)
+            while (ks < 16 && tiles * ks * 2 <= 2 * cus && (K / 64) % (8 * ks) == 0) ks *= 2;
+            if (ks > 1) {
+                tile_idx = want;
+                ksplit = ks;
+            }
+        }
+    }
     if (tile_idx >= 0) {
-        if (int rc = grow_workspace(ws, qmmt_workspace_bytes(M, K), stream, fail)) return rc;
+        const size_t xbytes = (qmmt_workspace_bytes(M, K) + 255) & ~(size_t)255;
+        if (int rc = grow_workspace(ws, xbytes + qmmt_splitk_bytes(M, N, ksplit), stream, fail)) return rc;
         *last_variant = qmmt_variant(tile_idx)->name;
-        hipError_t rc = qmmt_launch(tile_idx, a, ws->ptr, stream);
+        hipError_t rc = qmmt_launch_splitk(tile_idx, a, ws->ptr, ksplit, stream);
         if (rc != hipSuccess) return fail((int)rc, "rocm.hip.hipLaunchKernel: HIP returned %d (%s)", (int)rc, hipGetErrorString(rc));
         return AQ_OK;
     }

@@ -128,6 +128,12 @@ int aq_qmm(aq_ctx *ctx, const void *x, const void *packed, const void *scales, c
  * own scratch the same way at model load (hipMLXQ4DeviceWeightConfig and the batch scratch of
  * go/engine/hip/hip_projection_launch.go:2671-2720). */
 int aq_reserve_workspace(aq_ctx *ctx, int M, int K);
+/* The same by size.  Besides the prefill copy of x the workspace holds: the fp32 partial tiles of calls with
+ * 5..64 rows whose K is shared out over workgroups (up to 64*M*N bytes), the intermediates of the unfused
+ * fallbacks of the fused MLP / lm_head entry points, and the scratch of aq_packed_topk.  A call that needs
+ * more than is there grows it (not possible while a capture is open): run such a call once before capturing,
+ * or reserve its bytes here. */
+int aq_reserve_workspace_bytes(aq_ctx *ctx, size_t bytes);
 
 /* gather_qmv: for each route z, y[z,:N] = x[lhs[z] or 0, :K] . dequant(W_e)^T with
  * e = rhs[z] read ON DEVICE; W_e = rows [row_base, row_base+N) of expert e's slab.
@@ -309,7 +315,8 @@ int aq_proj_quant_matmul_host(aq_ctx *ctx, float *out, const float *x, size_t x_
 int aq_variant_count(int op);
 const char *aq_variant_name(int op, int variant);
 int aq_force_variant(aq_ctx *ctx, int op, int variant);
-/* Name of the kernel variant the last launch of `op` on this context used. */
+/* Name of the kernel variant the last launch of `op` on this context used; an aq_qmv call with more than
+ * four rows that ran on the matmul tiles reports the tile kernel under both ops. */
 const char *aq_last_variant(aq_ctx *ctx, int op);
 
 #ifdef __cplusplus

@@ -575,7 +575,8 @@ def test_qmm_every_variant(ctx, orc):
             bits = int(name.split("_")[1][1:])
             # variants that stage scales through LDS take K in multiples of 512 (1536: three quads, the last
             # octet half used); the others get a K that ends in the middle of a quad
-            K = 1536 if name.endswith("_q") else 704
+            staged = name.endswith("_q") or name.endswith("_pq")
+            K = 1536 if staged else 704
             if (bits, K) not in data:
                 words, s, b = F.synthetic_affine(N, K, bits, 64, seed=700 + bits)
                 x = F.synthetic_x(M, K, seed=800 + bits)
@@ -585,13 +586,32 @@ def test_qmm_every_variant(ctx, orc):
             acc = run_qmv(ctx, x, dw, M, K, N, 64, bits, True, "qmm")
             assert ctx.last_variant(1) == name
             check_accumulators(acc, ref, name)
-            if name.endswith("_q"):
+            if staged:
                 with pytest.raises(aq_mi355.AqError):      # a K the staging cannot take is refused, not mangled
                     run_qmv(ctx, x[:, :704].copy(), dw, M, 704, N, 64, bits, True, "qmm")
     finally:
         ctx.force_variant(1, -1)
     for dw, _, _ in data.values():
         dw.free()
+
+
+@pytest.mark.parametrize("fn", ["qmv", "qmm"])
+@pytest.mark.parametrize("M,K,N,bits", [(5, 256, 70, 4), (17, 1024, 130, 4), (32, 4096, 1000, 4), (33, 2048, 516, 8),
+                                        (64, 4096, 257, 4), (48, 14336, 96, 4), (20, 768, 64, 8), (64, 512, 40, 4)])
+def test_few_rows_k_shared_over_workgroups(ctx, orc, fn, M, K, N, bits):
+    """5..64 activation rows: the tile kernels share K out over several workgroups per output tile and a
+    second kernel adds the fp32 partial tiles in a fixed order.  Through both doors, fp32 and bf16 stores,
+    widths 4 and 8, N that ends inside a tile, K whose group count allows 1, 2, 4 .. 16 splits; two calls
+    give the same bytes (the order of the additions does not depend on which workgroup finishes first)."""
+    say("few rows, split K", fn, M, K, N, bits)
+    acc, ref, (words, s, b, x) = _qmv_case(ctx, orc, M, K, N, bits, 64, 4000 + M + K, fn=fn)
+    say("  ran on", ctx.last_variant(0), ctx.last_variant(1))
+    if M > 16 and fn == "qmv":
+        assert ctx.last_variant(1).startswith("qmm"), ctx.last_variant(1)
+    dw = DeviceAffine(ctx, words, s, b)
+    again = run_qmv(ctx, x, dw, M, K, N, 64, bits, True, fn)
+    assert np.array_equal(again.view(np.uint32), acc.view(np.uint32))
+    dw.free()
 
 
 def test_qmm_hardware_fixture_q4_g64_tokens16(ctx, orc):
