@@ -31,6 +31,7 @@ struct QmmVariant {
 struct QmmTileArgs {
     const uint16_t* xf;  // activations in A-fragment order, rows padded to a multiple of 32
     const uint16_t* xs;  // per 64-code block sums of x as (hi, lo) bf16, four blocks per 16 bytes
+    const float* rs;     // fp16-operand kernels: per row of x, the inverse of the power of two it was scaled by
     const uint32_t* w;
     const uint16_t* s;
     const uint16_t* b;
@@ -45,6 +46,7 @@ struct QmmTileArgs {
     float* partial;        // ksplit > 1: fp32 partial tiles [ksplit][M][N]
 };
 
+// (the variants of the fp16-operand kernels, aq_qmm_half.hip, are listed behind those of the tile kernels)
 int qmmt_variant_count();
 const QmmVariant* qmmt_variant(int idx);
 // Device bytes the tile kernels need beside their operands for an M x K activation matrix.
@@ -59,6 +61,11 @@ hipError_t qmmt_launch(int idx, const QmmArgs& a, void* workspace, hipStream_t s
 // tiles: for few rows of x, where M x N tiles alone leave most of the chip idle.
 size_t qmmt_splitk_bytes(int M, int N, int ksplit);
 hipError_t qmmt_launch_splitk(int idx, const QmmArgs& a, void* workspace, int ksplit, hipStream_t stream);
+
+// 4-bit kernels whose matrix-core operand carries scale * (code - 8) as fp16 (aq_qmm_half.hip); same workspace.
+int qmmh_variant_count();
+const QmmVariant* qmmh_variant(int idx);
+hipError_t qmmh_launch(int idx, const QmmArgs& a, void* workspace, hipStream_t stream);
 
 // Scratch memory a context lends to the matmul path; grown on demand, never while a capture is open.
 struct Workspace {

@@ -24,6 +24,7 @@
 //     rows of x across N: the band's A tile stays in that XCD's L2 while the weights stream by.
 #include "aq_device.h"
 #include "aq_kernels.h"
+#include "aq_lds_copy.h"
 #include "aq_qmm.h"
 
 #include "../../include/aq_mi355.h"
@@ -55,24 +56,6 @@ __device__ __forceinline__ uint4 unpack_words8(uint32_t w0, uint32_t w1) {
 }
 
 __device__ __forceinline__ uint32_t dup16(uint32_t h) { return (h & 0xffffu) | (h << 16); }
-
-// One global -> LDS copy of 16 bytes per lane (64 lanes fill 1 KiB at lds_base + 16 * lane), written as
-// inline asm on purpose.  The compiler knows that the builtin form writes LDS and, unable to tell the
-// target from the stages being read, drains EVERY outstanding copy (s_waitcnt vmcnt(0)) before the
-// next LDS access; the loop below needs the copies of block g+2 in flight while block g is read and
-// orders them itself with counted waits.  Hidden from the compiler, a copy can only make the
-// compiler's own waits for ordinary loads stricter, never weaker (completion is in order).
-// m0 is reserved by the compiler (it sets it before each of its own uses), so writing it here is safe.
-// The source address is a wave-uniform 64-bit base in SGPRs plus a 32-bit byte offset per lane, so the address
-// arithmetic of the main loop runs on the scalar unit.
-__device__ __forceinline__ void copy16_to_lds(const void* base_uniform, uint32_t lane_offset, uint32_t lds_base_uniform) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(base_uniform),
-                 "s"(__builtin_amdgcn_readfirstlane(lds_base_uniform))
-                 : "memory");
-}
-__device__ __forceinline__ uint32_t lds_offset(const void* p) {
-    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t*)p;
-}
 
 }  // namespace
 
@@ -757,22 +740,24 @@ struct QmmTileEntry {
 
 static const QmmTileEntry kQmmTileTable[] = {AQ_QMMT_SET(4), AQ_QMMT_SET(8)};
 
-int qmmt_variant_count() { return (int)(sizeof(kQmmTileTable) / sizeof(kQmmTileTable[0])); }
+static int tile_variants() { return (int)(sizeof(kQmmTileTable) / sizeof(kQmmTileTable[0])); }
+int qmmt_variant_count() { return tile_variants() + qmmh_variant_count(); }
 const QmmVariant* qmmt_variant(int idx) {
     if (idx < 0 || idx >= qmmt_variant_count()) return nullptr;
-    return &kQmmTileTable[idx].v;
+    return idx < tile_variants() ? &kQmmTileTable[idx].v : qmmh_variant(idx - tile_variants());
 }
 
+// fragments of x, block sums, one fp32 factor per row (the fp16-operand kernels)
 size_t qmmt_workspace_bytes(int M, int K) {
     const size_t mblks = ((size_t)M + 31) / 32;
     const size_t g4 = ((size_t)K / 64 + 3) / 4;
-    return mblks * 32 * (size_t)K * 2 + mblks * 32 * g4 * 16;
+    return mblks * 32 * (size_t)K * 2 + mblks * 32 * g4 * 16 + mblks * 32 * 4;
 }
 
 bool qmmt_quad_staging_ok(const QmmArgs& q) {
     return q.gs_blocks == 1 && q.K % 512 == 0 && ((reinterpret_cast<uintptr_t>(q.s) | reinterpret_cast<uintptr_t>(q.b)) & 15) == 0;
 }
-bool qmmt_variant_stages_quads(int idx) { return idx >= 0 && idx < qmmt_variant_count() && kQmmTileTable[idx].sbl; }
+bool qmmt_variant_stages_quads(int idx) { return idx >= 0 && idx < tile_variants() && kQmmTileTable[idx].sbl; }
 
 // Adds the ksplit partial tiles [ksplit][M*N] in split order and stores bf16 or fp32.
 __global__ __launch_bounds__(256) void qmm_splitk_reduce_kernel(const float* __restrict__ partial, int ksplit, int64_t mn,
@@ -798,6 +783,7 @@ hipError_t qmmt_launch(int idx, const QmmArgs& q, void* workspace, hipStream_t s
 // rewritten activations (qmmt_workspace_bytes(M, K) rounded up to 256, then qmmt_splitk_bytes).
 hipError_t qmmt_launch_splitk(int idx, const QmmArgs& q, void* workspace, int ksplit, hipStream_t stream) {
     if (idx < 0 || idx >= qmmt_variant_count()) return hipErrorInvalidValue;
+    if (idx >= tile_variants()) return ksplit == 1 ? qmmh_launch(idx - tile_variants(), q, workspace, stream) : hipErrorInvalidValue;
     const QmmTileEntry& e = kQmmTileTable[idx];
     if (e.sbl && !qmmt_quad_staging_ok(q)) return hipErrorInvalidValue;
     if (ksplit < 1 || (ksplit > 1 && (q.K / 64) % (4 * ksplit) != 0)) return hipErrorInvalidValue;

@@ -614,6 +614,75 @@ def test_few_rows_k_shared_over_workgroups(ctx, orc, fn, M, K, N, bits):
     dw.free()
 
 
+def _half_variants():
+    import aq_mi355
+    return [(i, n) for i, n in enumerate(aq_mi355.variant_names(1)) if n.startswith("qmmh_")]
+
+
+def test_qmm_fp16_operand_kernels_power_of_two_factors(ctx, orc):
+    """The qmmh kernels multiply fp16 operands: rows of x and rows of the weights are brought into fp16 range by
+    powers of two that the epilogue takes off again.  So scaling a row of x, or the scales and biases of a row of
+    the weights, by a power of two must scale the fp32 outputs by exactly that power (bit for bit), wherever the
+    row sits in bf16's range; an all-zero row gives zeros; and a row whose elements differ by many orders of
+    magnitude still meets the reference to fp32 accumulation accuracy."""
+    M, K, N = 130, 1024, 300
+    words, s, b = F.synthetic_affine(N, K, 4, 64, seed=611)
+    x = F.synthetic_x(M, K, seed=612)
+    xf = F.bf16_bits_to_f32(x).reshape(M, K)
+    row_pow = np.zeros(M, dtype=np.int64)
+    row_pow[1:9] = [40, -40, 100, -100, 14, -14, 1, -1]
+    x2 = (xf * np.exp2(row_pow)[:, None].astype(np.float32)).astype(np.float32)
+    x2[9] = 0.0
+    x2_bits = F.f32_to_bf16_bits(x2)
+    col_pow = np.zeros(N, dtype=np.int64)
+    col_pow[2:8] = [30, -30, 60, -60, 7, -7]
+    sf, bf = F.bf16_bits_to_f32(s).reshape(N, -1), F.bf16_bits_to_f32(b).reshape(N, -1)
+    s2 = F.f32_to_bf16_bits(sf * np.exp2(col_pow)[:, None].astype(np.float32)).reshape(s.shape)
+    b2 = F.f32_to_bf16_bits(bf * np.exp2(col_pow)[:, None].astype(np.float32)).reshape(b.shape)
+    # a row of x with a few very large elements among ordinary ones
+    x3 = xf.copy()
+    x3[11, ::97] *= 3000.0
+    x3_bits = F.f32_to_bf16_bits(x3)
+    dw, dw2 = DeviceAffine(ctx, words, s, b), DeviceAffine(ctx, words, s2, b2)
+    try:
+        for idx, name in _half_variants():
+            say("qmmh scaling", name)
+            ctx.force_variant(1, idx)
+            base = run_qmv(ctx, x, dw, M, K, N, 64, 4, True, "qmm").reshape(M, N)
+            assert ctx.last_variant(1) == name
+            check_accumulators(base, F.reference_f64(x, words, s, b, 4, 64, K), name)
+            rows = run_qmv(ctx, x2_bits, dw, M, K, N, 64, 4, True, "qmm").reshape(M, N)
+            want = (base.astype(np.float64) * np.exp2(row_pow)[:, None]).astype(np.float32)
+            want[9] = 0.0
+            assert np.array_equal(rows.view(np.uint32), want.view(np.uint32)), name
+            cols = run_qmv(ctx, x, dw2, M, K, N, 64, 4, True, "qmm").reshape(M, N)
+            want = (base.astype(np.float64) * np.exp2(col_pow)[None, :]).astype(np.float32)
+            assert np.array_equal(cols.view(np.uint32), want.view(np.uint32)), name
+            wide = run_qmv(ctx, x3_bits, dw, M, K, N, 64, 4, True, "qmm").reshape(M, N)
+            ref = F.reference_f64(x3_bits, words, s, b, 4, 64, K)
+            wabs = np.abs(F.numpy_dequant(words, s, b, 4, 64, K).astype(np.float64))
+            mass = np.abs(x3.astype(np.float64)) @ wabs.T
+            assert (np.abs(wide - ref) <= 4e-6 * mass + 1e-6).all(), name
+    finally:
+        ctx.force_variant(1, -1)
+    dw.free()
+    dw2.free()
+
+
+@pytest.mark.parametrize("M,K,N,gs", [(1, 64, 1, 64), (33, 192, 257, 64), (300, 2048, 520, 128), (70, 4096, 96, 64)])
+def test_qmm_fp16_operand_kernels_shapes(ctx, orc, M, K, N, gs):
+    """qmmh variants on shapes that end inside a tile, K of one block, K that ends inside a quad of blocks (192),
+    and group size 128, fp32 and bf16 stores."""
+    try:
+        for idx, name in _half_variants():
+            say("qmmh shape", name, M, K, N, gs)
+            ctx.force_variant(1, idx)
+            _qmv_case(ctx, orc, M, K, N, 4, gs, 7000 + M + K, fn="qmm")
+            assert ctx.last_variant(1) == name
+    finally:
+        ctx.force_variant(1, -1)
+
+
 def test_qmm_hardware_fixture_q4_g64_tokens16(ctx, orc):
     """17 x 704 x 16 batch fixture of go/engine/hip/hip_hardware_test.go:7822-7878 (reference tolerance 1e-3)."""
     say("qmm hw fixture")
