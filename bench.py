@@ -62,7 +62,7 @@ def traffic_from_profiles():
         return None
 
 
-def run_probe(which):
+def run_probe(which, variant=None):
     import numpy as np
     import aq_mi355
     import fixtures as F
@@ -95,7 +95,9 @@ def run_probe(which):
         x = ctx.to_device(F.synthetic_x(M, K, seed=F.BASE_SEED + 1003))
         y = ctx.alloc(M * N * 2)
         ctx.reserve_workspace(M, K)
-        for i in range(6):
+        if variant:
+            ctx.force_variant(1, aq_mi355.variant_names(1).index(variant))
+        for i in range(40):  # the first dozen calls run before the clocks have settled
             ww, ss, bb = pool[i % ncopy]
             ctx.qmm(x, ww, ss, bb, y, M, K, N, GROUP, BITS)
     ctx.sync()
@@ -116,6 +118,7 @@ def main():
     ap.add_argument("--probe", choices=["dominant", "qmm"], help="run only the named kernel a few times, preceded by two "
                     "kernels of known traffic (a 256 MiB zero fill, a dequantisation of the gate tensor): the workload "
                     "of the rocprofv3 --pmc passes behind roofline.traffic")
+    ap.add_argument("--variant", help="with --probe qmm: force this kernel variant (a name aq_variant_name lists)")
     ap.add_argument("--pmc-summary", metavar="DIR", help="print per-kernel averages of the counters a rocprofv3 --pmc "
                     "--output-format csv run left under DIR, and exit")
     args = ap.parse_args()
@@ -128,7 +131,7 @@ def main():
         sys.exit(2)
 
     if args.probe:
-        run_probe(args.probe)
+        run_probe(args.probe, args.variant)
         return
 
     import numpy as np
@@ -273,9 +276,9 @@ def main():
         ym = ctx.alloc(M * N * 2)
         ctx.reserve_workspace(M, K)
         pool = [layers[c]["gate"] for c in range(copies)]
-        # a prefill call takes a third of a millisecond and the first dozen run before the clocks have settled:
-        # 16 untimed calls, then the mean over 48
-        for i in range(16):
+        # a prefill call takes a third of a millisecond and the first few dozen run before the clocks have settled:
+        # 64 untimed calls, then the mean over 48
+        for i in range(64):
             w, s, b = pool[i % copies]
             ctx.qmm(xm, w, s, b, ym, M, K, N, GROUP, BITS)
         ctx.sync()
@@ -290,6 +293,24 @@ def main():
         qmm = {"M": M, "K": K, "N": N, "ms": round(q_ms, 4), "TFLOPs": round(tf, 1), "kernel": ctx.last_variant(1),
                "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                             "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None}}
+        # the same call on the other kernel family: bare codes as bf16 operands and one fp32 FMA per output element
+        # and 64-code block (the default is the family whose MFMA operand carries scale * (code - 8) as fp16)
+        other = "qmmt_b4_mb2_nb2_wm2_wn2"
+        names = aq_mi355.variant_names(1)
+        if other in names:
+            ctx.force_variant(1, names.index(other))
+            for i in range(8):
+                w, s, b = pool[i % copies]
+                ctx.qmm(xm, w, s, b, ym, M, K, N, GROUP, BITS)
+            ctx.sync()
+            ctx.timer_start()
+            for i in range(n):
+                w, s, b = pool[i % copies]
+                ctx.qmm(xm, w, s, b, ym, M, K, N, GROUP, BITS)
+            o_ms = ctx.timer_stop() / n
+            ctx.force_variant(1, -1)
+            qmm["bf16_code_variant"] = {"kernel": other, "ms": round(o_ms, 4),
+                                           "TFLOPs": round(flops / (o_ms * 1e-3) / 1e12, 1)}
         xm.free()
         ym.free()
 

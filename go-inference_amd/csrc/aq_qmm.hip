@@ -25,6 +25,8 @@
 #include "aq_kernels.h"
 #include "aq_qmm.h"
 
+#include <cstring>
+
 #include "../../include/aq_mi355.h"
 
 namespace aq {
@@ -394,7 +396,7 @@ static int grow_workspace(Workspace* ws, size_t need, hipStream_t stream, FailFn
     if (stream != nullptr && hipStreamIsCapturing(stream, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone)
         return fail(AQ_ERR_UNSUPPORTED,
                     "the context's workspace must grow to %zu bytes, which cannot happen during stream capture; "
-                    "call aq_reserve_workspace before capturing", need);
+                    "run the call once, or call aq_reserve_workspace / aq_reserve_workspace_bytes, before capturing", need);
     hipError_t rc = hipStreamSynchronize(stream);
     if (rc != hipSuccess) return fail((int)rc, "rocm.hip.hipStreamSynchronize: HIP returned %d", (int)rc);
     if (ws->ptr) (void)hipFree(ws->ptr);
@@ -426,6 +428,12 @@ static int find_qmmt(int bits, int mb, int nb, int wm, int wn) {
         const QmmVariant* v = qmmt_variant(i);
         if (v->bits == bits && v->mb == mb && v->nb == nb && v->wm == wm && v->wn == wn) return i;
     }
+    return -1;
+}
+
+static int find_qmmt_named(const char* name) {
+    for (int i = 0; i < qmmt_variant_count(); i++)
+        if (strcmp(qmmt_variant(i)->name, name) == 0) return i;
     return -1;
 }
 
@@ -476,6 +484,12 @@ int qmm_dispatch(hipStream_t stream, Workspace* ws, int cu_count, int forced, co
         // prefill sizes: the LDS-staged 128 x 128 tiles (four 64 x 64 wavefront tiles, two workgroups a CU);
         // the 128 x 64 wavefront tiles need more registers than two wavefronts a SIMD leave and measure slower
         tile_idx = find_qmmt(bits, 2, 2, 2, 2);
+        // 4 bit, enough 128 x 256 tiles to fill the chip twice over: the kernels whose MFMA operand carries
+        // scale * (code - 8) as fp16 (half the vector instructions per MFMA; measured 5-9 % faster at 2048 x 14336)
+        if (bits == 4 && (int64_t)((M + 127) / 128) * ((N + 255) / 256) >= 2 * (cu_count > 0 ? cu_count : 256)) {
+            const int half = find_qmmt_named("qmmh_b4_mb4_nb2_wm1_wn4_c");
+            if (half >= 0) tile_idx = half;
+        }
     }
     // Few rows of x: M x N tiles alone would occupy a fraction of the chip (56 workgroups for 32 x 14336), so
     // K is shared out as well and a small kernel adds the partial tiles.

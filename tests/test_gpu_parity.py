@@ -614,6 +614,52 @@ def test_few_rows_k_shared_over_workgroups(ctx, orc, fn, M, K, N, bits):
     dw.free()
 
 
+def test_few_rows_call_in_a_graph_after_reserving_workspace(orc):
+    """A call with 32 rows keeps fp32 partial tiles in the context's workspace.  On a fresh context the workspace
+    cannot grow while a capture is open: the call is refused with an error, not mangled; after
+    aq_reserve_workspace_bytes the same call is captured and every replay equals the eager result."""
+    import aq_mi355
+    M, K, N = 32, 2048, 1000
+    say("few rows in a graph", M, K, N)
+    words, s, b = F.synthetic_affine(N, K, 4, 64, seed=931)
+    x = F.synthetic_x(M, K, seed=932)
+    ref = F.reference_f64(x, words, s, b, 4, 64, K)
+    fresh = aq_mi355.Context(0)
+    try:
+        dw = DeviceAffine(fresh, words, s, b)
+        dx, dy = fresh.to_device(x), fresh.alloc(M * N * 4)
+        fresh.capture_begin()
+        with pytest.raises(aq_mi355.AqError):
+            fresh.qmv(dx, dw.w, dw.s, dw.b, dy, M, K, N, 64, 4, aq_mi355.AQ_OUT_F32)
+        try:
+            fresh.graph_destroy(fresh.capture_end())
+        except aq_mi355.AqError:
+            pass
+        fresh.reserve_workspace_bytes(64 << 20)
+        fresh.capture_begin()
+        fresh.qmv(dx, dw.w, dw.s, dw.b, dy, M, K, N, 64, 4, aq_mi355.AQ_OUT_F32)
+        graph = fresh.capture_end()
+        first = None
+        for i in range(3):
+            fresh.fill_zero(dy)
+            fresh.graph_launch(graph)
+            fresh.sync()
+            got = dy.download(np.float32, M * N).copy()
+            check_accumulators(got, ref, "replay %d" % i)
+            if first is None:
+                first = got
+            assert np.array_equal(got.view(np.uint32), first.view(np.uint32)), i
+        fresh.graph_destroy(graph)
+        fresh.qmv(dx, dw.w, dw.s, dw.b, dy, M, K, N, 64, 4, aq_mi355.AQ_OUT_F32)
+        fresh.sync()
+        assert np.array_equal(dy.download(np.float32, M * N).view(np.uint32), first.view(np.uint32))
+        dw.free()
+        dx.free()
+        dy.free()
+    finally:
+        fresh.close()
+
+
 def _half_variants():
     import aq_mi355
     return [(i, n) for i, n in enumerate(aq_mi355.variant_names(1)) if n.startswith("qmmh_")]
