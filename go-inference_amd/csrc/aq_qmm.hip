@@ -484,10 +484,11 @@ int qmm_dispatch(hipStream_t stream, Workspace* ws, int cu_count, int forced, co
         // prefill sizes: the LDS-staged 128 x 128 tiles (four 64 x 64 wavefront tiles, two workgroups a CU);
         // the 128 x 64 wavefront tiles need more registers than two wavefronts a SIMD leave and measure slower
         tile_idx = find_qmmt(bits, 2, 2, 2, 2);
-        // 4 bit, enough 128 x 256 tiles to fill the chip twice over: the kernels whose MFMA operand carries
-        // scale * (code - 8) as fp16 (half the vector instructions per MFMA; measured 5-9 % faster at 2048 x 14336)
-        if (bits == 4 && (int64_t)((M + 127) / 128) * ((N + 255) / 256) >= 2 * (cu_count > 0 ? cu_count : 256)) {
-            const int half = find_qmmt_named("qmmh_b4_mb4_nb2_wm1_wn4_c");
+        // 4 bit, enough 256 x 128 tiles to fill the chip twice over: the kernels whose MFMA operand carries
+        // scale * (code - 8) as fp16 (half the vector instructions per MFMA, no fp32 work on the accumulators;
+        // measured 10 % faster at 2048 x 14336)
+        if (bits == 4 && (int64_t)((M + 255) / 256) * ((N + 127) / 128) >= 2 * (cu_count > 0 ? cu_count : 256)) {
+            const int half = find_qmmt_named("qmmh_b4_mb4_nb2_wm2_wn2_s2c");
             if (half >= 0) tile_idx = half;
         }
     }

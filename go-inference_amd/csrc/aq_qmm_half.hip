@@ -621,33 +621,73 @@ __global__ __launch_bounds__(WM* WN* kWave, OCC) void qmmh_kernel(const QmmTileA
     // the copies requested past the end of K must not outlive the wavefront's use of LDS
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-    // D layout of v_mfma_f32_32x32x*: lane (j, h), register r -> row 8*(r/4) + 4*h + r%4, column j.
-    // Both powers of two come off here: exact, whatever the order.
+    // D layout of v_mfma_f32_32x32x*: lane (j, h), register r -> row 8*(r/4) + 4*h + r%4, column j: a lane holds
+    // single elements of 16 rows, and storing them as they lie means 2-byte stores to 64-byte pieces of rows
+    // (measured: a third of a tile's time).  Each 32-row block of the wavefront's tile therefore goes through a
+    // staging area in LDS that belongs to the wavefront (the stages are free: every copy has landed, every read of
+    // the loop has returned, and the barrier says so for all wavefronts), scaled by the two inverse powers of two
+    // (exact, whatever the order), and leaves it row-major, eight consecutive columns per lane: 16-byte bf16
+    // stores, whole 128-byte lines per eight lanes.
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    constexpr int CW = NB * 32;       // columns of the wavefront's tile
+    constexpr int LPR = CW / 8;       // lanes that share a row, eight columns each
+    constexpr int RPP = kWave / LPR;  // rows per pass
+    static_assert(NWAVE * 32 * CW * 4 <= STAGES * (A_STAGE + B_STAGE), "staging area fits the stages");
+    float* const stage = reinterpret_cast<float*>(lds) + wave * (32 * CW);
+    const bool wide = (reinterpret_cast<uintptr_t>(a.y) & 15) == 0 && (a.out_f32 ? (N & 3) == 0 : (N & 7) == 0);
+    const int row_in = lane / LPR, c8 = (lane % LPR) * 8;
+    const int n = n0 + wave_n * CW + c8;
 #pragma unroll
     for (int mb = 0; mb < MB; mb++) {
-        const int mbase = m0 + (wave_m * MB + mb) * 32 + 4 * h;  // < mblks * 32 unless the whole block lies past M
+        const int mtop = m0 + (wave_m * MB + mb) * 32;  // < mblks * 32 unless the whole block lies past M
         float4 down[4];
 #pragma unroll
         for (int q = 0; q < 4; q++) {
-            const int m = mbase + 8 * q;
+            const int m = mtop + 4 * h + 8 * q;
             down[q] = m < a.mblks * 32 ? *reinterpret_cast<const float4*>(a.rs + m) : make_float4(0.f, 0.f, 0.f, 0.f);
         }
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) {
-            const int n = n0 + (wave_n * NB + nb) * 32 + j;
             const float col_down = 1.0f / col_up[nb];
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const int m = mbase + 8 * (r >> 2) + (r & 3);
                 const float4 d4 = down[r >> 2];
                 const float dm = (r & 3) == 0 ? d4.x : (r & 3) == 1 ? d4.y : (r & 3) == 2 ? d4.z : d4.w;
-                if (m < M && n < N) {
-                    const float v = out[mb][nb][r] * dm * col_down;
-                    const int64_t o = (int64_t)m * N + n;
-                    if (a.out_f32) {
-                        reinterpret_cast<float*>(a.y)[o] = v;
-                    } else {
-                        reinterpret_cast<uint16_t*>(a.y)[o] = f32_to_bf16_bits(v);
+                stage[(8 * (r >> 2) + 4 * h + (r & 3)) * CW + nb * 32 + j] = out[mb][nb][r] * dm * col_down;
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < 32 / RPP; p++) {
+            const int row = p * RPP + row_in;
+            const int m = mtop + row;
+            const float4 lo = *reinterpret_cast<const float4*>(stage + row * CW + c8);
+            const float4 hi = *reinterpret_cast<const float4*>(stage + row * CW + c8 + 4);
+            if (m >= M || n >= N) continue;
+            const int64_t o = (int64_t)m * N + n;
+            if (wide && n + 8 <= N) {
+                if (a.out_f32) {
+                    float4* dst = reinterpret_cast<float4*>(reinterpret_cast<float*>(a.y) + o);
+                    dst[0] = lo;
+                    dst[1] = hi;
+                } else {
+                    uint4 u;
+                    u.x = f32_to_bf16_bits(lo.x) | ((uint32_t)f32_to_bf16_bits(lo.y) << 16);
+                    u.y = f32_to_bf16_bits(lo.z) | ((uint32_t)f32_to_bf16_bits(lo.w) << 16);
+                    u.z = f32_to_bf16_bits(hi.x) | ((uint32_t)f32_to_bf16_bits(hi.y) << 16);
+                    u.w = f32_to_bf16_bits(hi.z) | ((uint32_t)f32_to_bf16_bits(hi.w) << 16);
+                    *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(a.y) + o) = u;
+                }
+            } else {
+                const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    if (n + e < N) {
+                        if (a.out_f32) {
+                            reinterpret_cast<float*>(a.y)[o + e] = v[e];
+                        } else {
+                            reinterpret_cast<uint16_t*>(a.y)[o + e] = f32_to_bf16_bits(v[e]);
+                        }
                     }
                 }
             }

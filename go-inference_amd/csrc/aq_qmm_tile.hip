@@ -686,23 +686,75 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
     // the copies requested past the end of K must not outlive the wavefront's use of LDS
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-    // D layout of v_mfma_f32_32x32x*: lane (j, h), register r -> row 8*(r/4) + 4*h + r%4, column j
+    // D layout of v_mfma_f32_32x32x*: lane (j, h), register r -> row 8*(r/4) + 4*h + r%4, column j: a lane holds
+    // single elements of 16 rows.  Partial tiles of a K split are stored as they lie (fp32: 128-byte pieces of
+    // rows).  Final values go through a staging area in LDS that belongs to the wavefront (the stages are free:
+    // every copy has landed, every read of the loop has returned, and the barrier says so for all wavefronts) and
+    // leave it row-major, eight consecutive columns per lane: 16-byte bf16 stores instead of 2-byte ones to
+    // 64-byte pieces of rows, which took a third of a tile's time.
+    if (a.partial) {
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) {
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) {
+                const int n = n0 + (wave_n * NB + nb) * 32 + j;
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int m = m0 + (wave_m * MB + mb) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+                    if (m < M && n < N) a.partial[(int64_t)split * M * N + (int64_t)m * N + n] = out[mb][nb][r];
+                }
+            }
+        }
+        return;
+    }
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    constexpr int CW = NB * 32;       // columns of the wavefront's tile
+    constexpr int LPR = CW / 8;       // lanes that share a row, eight columns each
+    constexpr int RPP = kWave / LPR;  // rows per pass
+    static_assert(NWAVE * 32 * CW * 4 <= STAGES * A_STAGE + BST * B_STAGE, "staging area fits the stages");
+    float* const stage = reinterpret_cast<float*>(lds) + wave * (32 * CW);
+    const bool wide = (reinterpret_cast<uintptr_t>(a.y) & 15) == 0 && (a.out_f32 ? (N & 3) == 0 : (N & 7) == 0);
+    const int row_in = lane / LPR, c8 = (lane % LPR) * 8;
+    const int n = n0 + wave_n * CW + c8;
 #pragma unroll
     for (int mb = 0; mb < MB; mb++) {
+        const int mtop = m0 + (wave_m * MB + mb) * 32;
 #pragma unroll
-        for (int nb = 0; nb < NB; nb++) {
-            const int n = n0 + (wave_n * NB + nb) * 32 + j;
+        for (int nb = 0; nb < NB; nb++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int m = m0 + (wave_m * MB + mb) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                if (m < M && n < N) {
-                    const int64_t o = (int64_t)m * N + n;
-                    if (a.partial) {
-                        a.partial[(int64_t)split * M * N + o] = out[mb][nb][r];
-                    } else if (a.out_f32) {
-                        reinterpret_cast<float*>(a.y)[o] = out[mb][nb][r];
-                    } else {
-                        reinterpret_cast<uint16_t*>(a.y)[o] = f32_to_bf16_bits(out[mb][nb][r]);
+            for (int r = 0; r < 16; r++) stage[(8 * (r >> 2) + 4 * h + (r & 3)) * CW + nb * 32 + j] = out[mb][nb][r];
+#pragma unroll
+        for (int p = 0; p < 32 / RPP; p++) {
+            const int row = p * RPP + row_in;
+            const int m = mtop + row;
+            const float4 lo = *reinterpret_cast<const float4*>(stage + row * CW + c8);
+            const float4 hi = *reinterpret_cast<const float4*>(stage + row * CW + c8 + 4);
+            if (m >= M || n >= N) continue;
+            const int64_t o = (int64_t)m * N + n;
+            if (wide && n + 8 <= N) {
+                if (a.out_f32) {
+                    float4* dst = reinterpret_cast<float4*>(reinterpret_cast<float*>(a.y) + o);
+                    dst[0] = lo;
+                    dst[1] = hi;
+                } else {
+                    uint4 u;
+                    u.x = f32_to_bf16_bits(lo.x) | ((uint32_t)f32_to_bf16_bits(lo.y) << 16);
+                    u.y = f32_to_bf16_bits(lo.z) | ((uint32_t)f32_to_bf16_bits(lo.w) << 16);
+                    u.z = f32_to_bf16_bits(hi.x) | ((uint32_t)f32_to_bf16_bits(hi.y) << 16);
+                    u.w = f32_to_bf16_bits(hi.z) | ((uint32_t)f32_to_bf16_bits(hi.w) << 16);
+                    *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(a.y) + o) = u;
+                }
+            } else {
+                const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    if (n + e < N) {
+                        if (a.out_f32) {
+                            reinterpret_cast<float*>(a.y)[o + e] = v[e];
+                        } else {
+                            reinterpret_cast<uint16_t*>(a.y)[o + e] = f32_to_bf16_bits(v[e]);
+                        }
                     }
                 }
             }
