@@ -246,6 +246,14 @@ __global__ __launch_bounds__(WM* WN* kWave, OCC) void qmmh_kernel(const QmmTileA
     };
     const uint32_t mask_s = opaque_s(kMaskH);
     const uint32_t magic_v = opaque_v(kMagicH);
+    // the first blocks are on their way while the prologue scans the scale rows
+    if constexpr (!PIPE) {
+#pragma unroll
+        for (int d = 0; d < AHEAD; d++) {
+            issue_a(d < K / 64 ? d : K / 64 - 1, d);
+            issue_b(d < K / 64 ? d : K / 64 - 1, d);
+        }
+    }
 
     // this lane's weight rows (one per column block), and the power of two that brings the row's largest scale
     // into [2^10, 2^11): lane half h scans its half of the row's scales
@@ -463,16 +471,12 @@ __global__ __launch_bounds__(WM* WN* kWave, OCC) void qmmh_kernel(const QmmTileA
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
     };
-    // the first quad's scales (used at once, so the wait comes before any copy) and blocks 0 .. AHEAD-1
+    // the first quad's scales; blocks 0 .. AHEAD-1 were requested before the scan of the scale rows (any wait of
+    // the compiler's for the loads since then has drained those copies too: all the better)
     load_quad(a.s, 0, s_nxt);
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) asm volatile("" : "+v"(s_nxt[nb].x), "+v"(s_nxt[nb].y));
     __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int d = 0; d < AHEAD; d++) {
-        issue_a(d < G ? d : glast, d);
-        issue_b(d < G ? d : glast, d);
-    }
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((AHEAD - 1) * GROUP_OPS) : "memory");  // block 0 has landed
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
@@ -672,10 +676,10 @@ __global__ __launch_bounds__(WM* WN* kWave, OCC) void qmmh_kernel(const QmmTileA
                     dst[1] = hi;
                 } else {
                     uint4 u;
-                    u.x = f32_to_bf16_bits(lo.x) | ((uint32_t)f32_to_bf16_bits(lo.y) << 16);
-                    u.y = f32_to_bf16_bits(lo.z) | ((uint32_t)f32_to_bf16_bits(lo.w) << 16);
-                    u.z = f32_to_bf16_bits(hi.x) | ((uint32_t)f32_to_bf16_bits(hi.y) << 16);
-                    u.w = f32_to_bf16_bits(hi.z) | ((uint32_t)f32_to_bf16_bits(hi.w) << 16);
+                    u.x = pack_bf16x2(lo.x, lo.y);
+                    u.y = pack_bf16x2(lo.z, lo.w);
+                    u.z = pack_bf16x2(hi.x, hi.y);
+                    u.w = pack_bf16x2(hi.z, hi.w);
                     *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(a.y) + o) = u;
                 }
             } else {

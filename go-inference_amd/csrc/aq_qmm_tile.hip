@@ -739,10 +739,10 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
                     dst[1] = hi;
                 } else {
                     uint4 u;
-                    u.x = f32_to_bf16_bits(lo.x) | ((uint32_t)f32_to_bf16_bits(lo.y) << 16);
-                    u.y = f32_to_bf16_bits(lo.z) | ((uint32_t)f32_to_bf16_bits(lo.w) << 16);
-                    u.z = f32_to_bf16_bits(hi.x) | ((uint32_t)f32_to_bf16_bits(hi.y) << 16);
-                    u.w = f32_to_bf16_bits(hi.z) | ((uint32_t)f32_to_bf16_bits(hi.w) << 16);
+                    u.x = pack_bf16x2(lo.x, lo.y);
+                    u.y = pack_bf16x2(lo.z, lo.w);
+                    u.z = pack_bf16x2(hi.x, hi.y);
+                    u.w = pack_bf16x2(hi.z, hi.w);
                     *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(a.y) + o) = u;
                 }
             } else {
