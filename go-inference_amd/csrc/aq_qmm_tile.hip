@@ -687,26 +687,12 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
     // D layout of v_mfma_f32_32x32x*: lane (j, h), register r -> row 8*(r/4) + 4*h + r%4, column j: a lane holds
-    // single elements of 16 rows.  Partial tiles of a K split are stored as they lie (fp32: 128-byte pieces of
-    // rows).  Final values go through a staging area in LDS that belongs to the wavefront (the stages are free:
-    // every copy has landed, every read of the loop has returned, and the barrier says so for all wavefronts) and
-    // leave it row-major, eight consecutive columns per lane: 16-byte bf16 stores instead of 2-byte ones to
-    // 64-byte pieces of rows, which took a third of a tile's time.
-    if (a.partial) {
-#pragma unroll
-        for (int mb = 0; mb < MB; mb++) {
-#pragma unroll
-            for (int nb = 0; nb < NB; nb++) {
-                const int n = n0 + (wave_n * NB + nb) * 32 + j;
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int m = m0 + (wave_m * MB + mb) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                    if (m < M && n < N) a.partial[(int64_t)split * M * N + (int64_t)m * N + n] = out[mb][nb][r];
-                }
-            }
-        }
-        return;
-    }
+    // single elements of 16 rows.  Stored as they lie that is one store instruction per element, to 64-byte
+    // (bf16) or 128-byte (fp32) pieces of rows, which took a third of a big tile's time and most of a small one's.
+    // So every 32-row block goes through a staging area in LDS that belongs to the wavefront (the stages are
+    // free: every copy has landed, every read of the loop has returned, and the barrier says so for all
+    // wavefronts) and leaves it row-major, eight consecutive columns per lane, as 16-byte stores.  The fp32
+    // partial tile of a K split takes the same way into its slot of the workspace.
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     constexpr int CW = NB * 32;       // columns of the wavefront's tile
@@ -714,7 +700,9 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
     constexpr int RPP = kWave / LPR;  // rows per pass
     static_assert(NWAVE * 32 * CW * 4 <= STAGES * A_STAGE + BST * B_STAGE, "staging area fits the stages");
     float* const stage = reinterpret_cast<float*>(lds) + wave * (32 * CW);
-    const bool wide = (reinterpret_cast<uintptr_t>(a.y) & 15) == 0 && (a.out_f32 ? (N & 3) == 0 : (N & 7) == 0);
+    void* const ybase = a.partial ? static_cast<void*>(a.partial + (int64_t)split * M * N) : a.y;
+    const bool y_f32 = a.partial != nullptr || a.out_f32 != 0;
+    const bool wide = (reinterpret_cast<uintptr_t>(ybase) & 15) == 0 && (y_f32 ? (N & 3) == 0 : (N & 7) == 0);
     const int row_in = lane / LPR, c8 = (lane % LPR) * 8;
     const int n = n0 + wave_n * CW + c8;
 #pragma unroll
@@ -733,8 +721,8 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
             if (m >= M || n >= N) continue;
             const int64_t o = (int64_t)m * N + n;
             if (wide && n + 8 <= N) {
-                if (a.out_f32) {
-                    float4* dst = reinterpret_cast<float4*>(reinterpret_cast<float*>(a.y) + o);
+                if (y_f32) {
+                    float4* dst = reinterpret_cast<float4*>(reinterpret_cast<float*>(ybase) + o);
                     dst[0] = lo;
                     dst[1] = hi;
                 } else {
@@ -743,17 +731,17 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
                     u.y = pack_bf16x2(lo.z, lo.w);
                     u.z = pack_bf16x2(hi.x, hi.y);
                     u.w = pack_bf16x2(hi.z, hi.w);
-                    *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(a.y) + o) = u;
+                    *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(ybase) + o) = u;
                 }
             } else {
                 const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
                     if (n + e < N) {
-                        if (a.out_f32) {
-                            reinterpret_cast<float*>(a.y)[o + e] = v[e];
+                        if (y_f32) {
+                            reinterpret_cast<float*>(ybase)[o + e] = v[e];
                         } else {
-                            reinterpret_cast<uint16_t*>(a.y)[o + e] = f32_to_bf16_bits(v[e]);
+                            reinterpret_cast<uint16_t*>(ybase)[o + e] = f32_to_bf16_bits(v[e]);
                         }
                     }
                 }
