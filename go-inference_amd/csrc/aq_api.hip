@@ -485,8 +485,8 @@ int aq_qmv(aq_ctx* ctx, const void* x, const void* packed, const void* scales, c
     a.routes = 1;
     if (M > aq::kQmvMaxRows && ctx->forced[0] < 0) {
         // More rows than the dot2 kernels take.  The block-MFMA family streams the weights once per launch of
-        // up to 16 rows (4 where K is long); when the call fits one such launch it is the fastest.  Beyond that
-        // the matmul tiles with K shared out over workgroups read the weights once for all rows.
+        // up to 16 rows (4 where K is long); when the call fits one such launch it is the fastest up to 8 rows.
+        // Beyond that the matmul tiles with K shared out over workgroups read the weights once for all rows.
         aq::BlkPlan plan;
         aq::QmvArgs probe = a;
         int rows_per_launch = 0;
@@ -497,7 +497,9 @@ int aq_qmv(aq_ctx* ctx, const void* x, const void* packed, const void* scales, c
                 break;
             }
         }
-        if (rows_per_launch == 0 || M > 64 || M > rows_per_launch) {
+        // (9..16 rows of a large matrix: the 16-row block-MFMA kernel is bound by its 4x4x4 MFMAs, the tiles are not)
+        const bool tiles_win = M > 8 && M <= 64 && (K / 64) % 4 == 0 && (int64_t)N * K >= (int64_t)16 << 20;
+        if (rows_per_launch == 0 || M > 64 || M > rows_per_launch || tiles_win) {
             const int rc = aq::qmm_dispatch(ctx->stream, &ctx->ws, ctx->cu_count, ctx->forced[1], &ctx->last_variant[1], x,
                                             packed, scales, biases, y, M, K, N, group_size, bits,
                                             (flags & AQ_OUT_F32) != 0, fail);

@@ -62,6 +62,12 @@ hipError_t qmmt_launch(int idx, const QmmArgs& a, void* workspace, hipStream_t s
 size_t qmmt_splitk_bytes(int M, int N, int ksplit);
 hipError_t qmmt_launch_splitk(int idx, const QmmArgs& a, void* workspace, int ksplit, hipStream_t stream);
 
+// Kernels for 5..64 rows of x whose LDS stages hold four blocks of K (aq_qmm_few.hip): listed behind the
+// fp16-operand variants; they take the operands the tile kernels take and are launched through qmmt_launch_splitk.
+int qmmf_variant_count();
+const QmmVariant* qmmf_variant(int idx);
+hipError_t qmmf_launch_kernel(int idx, const QmmTileArgs& a, hipStream_t stream);
+
 // 4-bit kernels whose matrix-core operand carries scale * (code - 8) as fp16 (aq_qmm_half.hip); same workspace.
 int qmmh_variant_count();
 const QmmVariant* qmmh_variant(int idx);

@@ -496,19 +496,18 @@ int qmm_dispatch(hipStream_t stream, Workspace* ws, int cu_count, int forced, co
     // K is shared out as well and a small kernel adds the partial tiles.
     int ksplit = 1;
     if (idx < 0 && M > 4 && M <= 64 && (K / 64) % 4 == 0) {
-        const int want = find_qmmt(bits, M <= 32 ? 1 : 2, 2, 1, 4);
+        // the kernels whose LDS stages hold four blocks of K: 32 or 64 rows by 256 (8 bit: 128) columns per workgroup
+        const int bm = M <= 32 ? 32 : 64, bn = bits == 4 ? 256 : 128;
+        const int want = find_qmmt_named(bits == 4 ? (M <= 32 ? "qmmf_b4_mb1_nb2_wm1_wn4" : "qmmf_b4_mb2_nb2_wm1_wn4")
+                                                   : (M <= 32 ? "qmmf_b8_mb1_nb1_wm1_wn4" : "qmmf_b8_mb2_nb1_wm1_wn4"));
         if (want >= 0) {
-            const int bm = M <= 32 ? 32 : 64;
-            const int tiles = ((M + bm - 1) / bm) * ((N + 255) / 256);
+            const int tiles = ((M + bm - 1) / bm) * ((N + bn - 1) / bn);
             const int cus = cu_count > 0 ? cu_count : 256;
             int ks = 1;
-            // (measured: one workgroup a CU is the sweet spot; more splits cost more in partial tiles than they
-            // gain in parallel streams)
-            while (ks < 16 && tiles * ks * 2 <= 2 * cus && (K / 64) % (8 * ks) == 0) ks *= 2;
-            if (ks > 1) {
-                tile_idx = want;
-                ksplit = ks;
-            }
+            // one workgroup a CU (their LDS allows no more); every workgroup keeps at least two quads of K
+            while (ks < 16 && tiles * ks * 2 <= cus && (K / 64) % (8 * ks) == 0 && (K / 64) / (2 * ks) >= 8) ks *= 2;
+            tile_idx = want;
+            ksplit = ks;
         }
     }
     if (tile_idx >= 0) {

@@ -781,10 +781,12 @@ struct QmmTileEntry {
 static const QmmTileEntry kQmmTileTable[] = {AQ_QMMT_SET(4), AQ_QMMT_SET(8)};
 
 static int tile_variants() { return (int)(sizeof(kQmmTileTable) / sizeof(kQmmTileTable[0])); }
-int qmmt_variant_count() { return tile_variants() + qmmh_variant_count(); }
+int qmmt_variant_count() { return tile_variants() + qmmh_variant_count() + qmmf_variant_count(); }
 const QmmVariant* qmmt_variant(int idx) {
     if (idx < 0 || idx >= qmmt_variant_count()) return nullptr;
-    return idx < tile_variants() ? &kQmmTileTable[idx].v : qmmh_variant(idx - tile_variants());
+    if (idx < tile_variants()) return &kQmmTileTable[idx].v;
+    idx -= tile_variants();
+    return idx < qmmh_variant_count() ? qmmh_variant(idx) : qmmf_variant(idx - qmmh_variant_count());
 }
 
 // fragments of x, block sums, one fp32 factor per row (the fp16-operand kernels)
@@ -823,8 +825,12 @@ hipError_t qmmt_launch(int idx, const QmmArgs& q, void* workspace, hipStream_t s
 // rewritten activations (qmmt_workspace_bytes(M, K) rounded up to 256, then qmmt_splitk_bytes).
 hipError_t qmmt_launch_splitk(int idx, const QmmArgs& q, void* workspace, int ksplit, hipStream_t stream) {
     if (idx < 0 || idx >= qmmt_variant_count()) return hipErrorInvalidValue;
-    if (idx >= tile_variants()) return ksplit == 1 ? qmmh_launch(idx - tile_variants(), q, workspace, stream) : hipErrorInvalidValue;
-    const QmmTileEntry& e = kQmmTileTable[idx];
+    if (idx >= tile_variants() && idx < tile_variants() + qmmh_variant_count())
+        return ksplit == 1 ? qmmh_launch(idx - tile_variants(), q, workspace, stream) : hipErrorInvalidValue;
+    const int few = idx >= tile_variants() ? idx - tile_variants() - qmmh_variant_count() : -1;
+    static const QmmTileEntry kNone{};
+    const QmmTileEntry& e = few < 0 ? kQmmTileTable[idx] : kNone;
+    const QmmVariant& v = few < 0 ? e.v : *qmmf_variant(few);
     if (e.sbl && !qmmt_quad_staging_ok(q)) return hipErrorInvalidValue;
     if (ksplit < 1 || (ksplit > 1 && (q.K / 64) % (4 * ksplit) != 0)) return hipErrorInvalidValue;
     const int mblks = (q.M + 31) / 32;
@@ -832,7 +838,7 @@ hipError_t qmmt_launch_splitk(int idx, const QmmArgs& q, void* workspace, int ks
     uint16_t* xs = xf + (size_t)mblks * 32 * q.K;
     const int64_t pieces = (int64_t)mblks * 32 * (q.K / 64) * 8;
     const unsigned prep_blocks = (unsigned)((pieces + 255) / 256);
-    if (e.v.bits == 4)
+    if (v.bits == 4)
         hipLaunchKernelGGL(qmm_prep_kernel<4>, dim3(prep_blocks), dim3(256), 0, stream, q.x, xf, xs, q.M, q.K, mblks);
     else
         hipLaunchKernelGGL(qmm_prep_kernel<8>, dim3(prep_blocks), dim3(256), 0, stream, q.x, xf, xs, q.M, q.K, mblks);
@@ -852,7 +858,7 @@ hipError_t qmmt_launch_splitk(int idx, const QmmArgs& q, void* workspace, int ks
     a.gs_blocks = q.gs_blocks;
     a.out_f32 = q.out_f32;
     a.mblks = mblks;
-    const int bm = e.v.wm * e.v.mb * 32, bn = e.v.wn * e.v.nb * 32;
+    const int bm = v.wm * v.mb * 32, bn = v.wn * v.nb * 32;
     a.tiles_m = (q.M + bm - 1) / bm;
     a.tiles_n = (q.N + bn - 1) / bn;
     a.ksplit = ksplit;
@@ -864,13 +870,17 @@ hipError_t qmmt_launch_splitk(int idx, const QmmArgs& q, void* workspace, int ks
     }
     const int T = a.tiles_m * a.tiles_n * ksplit;
     const unsigned grid = (unsigned)(((T + 7) / 8) * 8);
-    if (e.lds_bytes > 48 * 1024) {
-        rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e.fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                 e.lds_bytes);
-        if (rc != hipSuccess) return rc;
+    if (few >= 0) {
+        rc = qmmf_launch_kernel(few, a, stream);
+    } else {
+        if (e.lds_bytes > 48 * 1024) {
+            rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e.fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     e.lds_bytes);
+            if (rc != hipSuccess) return rc;
+        }
+        hipLaunchKernelGGL(e.fn, dim3(grid), dim3((unsigned)(e.v.wm * e.v.wn * kWave)), (size_t)e.lds_bytes, stream, a);
+        rc = hipGetLastError();
     }
-    hipLaunchKernelGGL(e.fn, dim3(grid), dim3((unsigned)(e.v.wm * e.v.wn * kWave)), (size_t)e.lds_bytes, stream, a);
-    rc = hipGetLastError();
     if (rc != hipSuccess || ksplit == 1) return rc;
     const int64_t mn = (int64_t)q.M * q.N;
     int64_t blocks = (mn + 255) / 256;
