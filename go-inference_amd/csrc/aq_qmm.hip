@@ -503,9 +503,11 @@ int qmm_dispatch(hipStream_t stream, Workspace* ws, int cu_count, int forced, co
         if (want >= 0) {
             const int tiles = ((M + bm - 1) / bm) * ((N + bn - 1) / bn);
             const int cus = cu_count > 0 ? cu_count : 256;
+            // as many workgroups as CUs at most (their LDS allows one each); every workgroup takes whole quads of K
+            // and at least two of them; at most 16 partial tiles per output tile
             int ks = 1;
-            // one workgroup a CU (their LDS allows no more); every workgroup keeps at least two quads of K
-            while (ks < 16 && tiles * ks * 2 <= cus && (K / 64) % (8 * ks) == 0 && (K / 64) / (2 * ks) >= 8) ks *= 2;
+            for (int k = 2; k <= 16; k++)
+                if ((K / 64) % (4 * k) == 0 && tiles * k <= cus && (K / 64) / k >= 8) ks = k;
             tile_idx = want;
             ksplit = ks;
         }

@@ -18,6 +18,8 @@
 #include "aq_lds_copy.h"
 #include "aq_qmm.h"
 
+#include <type_traits>
+
 namespace aq {
 
 namespace {
@@ -184,12 +186,19 @@ __global__ __launch_bounds__(4 * kWave, 1) void qmm_few_kernel(const QmmTileArgs
 #pragma unroll
             for (int r = 0; r < 16; r++) out[mb][nb][r] = 0.0f;
 
+    // Order of the loop, chosen around one fact: the compiler cannot count the copy instructions (inline asm), so
+    // wherever it waits for one of its own loads it waits until nothing at all is outstanding.  Scales, biases and
+    // block sums of quad q+2 are therefore requested right behind the end-of-quad wait of quad q (nothing in
+    // flight, the next copies not yet issued) and first used right behind the end-of-quad wait of quad q+1, which
+    // has covered them anyway; the copies of quad q+1 are issued at the top of quad q.
     const int quad0 = gb >> 2, quad_end = (G + 3) >> 2;
-#pragma unroll
-    for (int nb = 0; nb < NB; nb++) s_nxt[nb] = b_nxt[nb] = make_uint2(0u, 0u);
-#pragma unroll
-    for (int mb = 0; mb < MB; mb++) xs_nxt[mb] = make_uint4(0u, 0u, 0u, 0u);
     load_all(quad0, s_cur, b_cur, xs_cur);
+    load_all(quad0 + 1, s_nxt, b_nxt, xs_nxt);
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) asm volatile("" : "+v"(s_cur[nb].x), "+v"(s_cur[nb].y), "+v"(b_cur[nb].x), "+v"(b_cur[nb].y));
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) asm volatile("" : "+v"(xs_cur[mb].x), "+v"(xs_cur[mb].y), "+v"(xs_cur[mb].z), "+v"(xs_cur[mb].w));
+    __builtin_amdgcn_sched_barrier(0);
     issue_quad(quad0, 0);
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
@@ -197,52 +206,60 @@ __global__ __launch_bounds__(4 * kWave, 1) void qmm_few_kernel(const QmmTileArgs
 
     int st = 0;
     for (int quad = quad0; quad < quad_end; quad++) {
-        if (quad + 1 < quad_end) {  // uniform
-            load_all(quad + 1, s_nxt, b_nxt, xs_nxt);
-            issue_quad(quad + 1, st ^ 1);  // that stage was read last in the quad before this one
-        }
+        if (quad + 1 < quad_end) issue_quad(quad + 1, st ^ 1);  // uniform; that stage was read last in the quad before
         const int blocks = min(4, G - quad * 4);  // 4 except where K ends inside a quad
+        // one block of the quad in stage st; q static.  A whole quad is written as straight-line code so that the
+        // scheduler can run the blocks' independent MFMA chains back to back: with so few rows a block alone is two
+        // chains of four dependent MFMAs, and a wavefront that is alone on its SIMD idles between them.
+        auto block = [&](auto q_tag) {
+            constexpr int q = decltype(q_tag)::value;
+            const uint8_t* ab = abuf + st * A_QUAD + q * A_BLK + lane * 16;
+            // this lane's codes: row (wave * NB + nb) * 32 + j, words 4h .. 4h+3 (8 bit: 8h .. 8h+7)
+            const uint8_t* bb = bbuf + st * B_QUAD + q * B_BLK + ((wave * NB) * 32 + j) * (WPB * 4) + h * (WPB * 2);
+            bf16x8_t bfrag[NB][4];
+            float sc[NB];
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            if (q < blocks) {
-                const uint8_t* ab = abuf + st * A_QUAD + q * A_BLK + lane * 16;
-                // this lane's codes: row (wave * NB + nb) * 32 + j, words 4h .. 4h+3 (8 bit: 8h .. 8h+7)
-                const uint8_t* bb = bbuf + st * B_QUAD + q * B_BLK + ((wave * NB) * 32 + j) * (WPB * 4) + h * (WPB * 2);
-                bf16x8_t bfrag[NB][4];
-                float sc[NB];
+            for (int nb = 0; nb < NB; nb++) {
+                if constexpr (BITS == 4) {
+                    const uint4 cw = *reinterpret_cast<const uint4*>(bb + nb * 32 * 32);
+                    bfrag[nb][0] = __builtin_bit_cast(bf16x8_t, unpack_word4(cw.x, mask_s, magic_v));
+                    bfrag[nb][1] = __builtin_bit_cast(bf16x8_t, unpack_word4(cw.y, mask_s, magic_v));
+                    bfrag[nb][2] = __builtin_bit_cast(bf16x8_t, unpack_word4(cw.z, mask_s, magic_v));
+                    bfrag[nb][3] = __builtin_bit_cast(bf16x8_t, unpack_word4(cw.w, mask_s, magic_v));
+                } else {
+                    const uint4 c0 = *reinterpret_cast<const uint4*>(bb + nb * 32 * 64);
+                    const uint4 c1 = *reinterpret_cast<const uint4*>(bb + nb * 32 * 64 + 16);
+                    bfrag[nb][0] = __builtin_bit_cast(bf16x8_t, unpack_words8(c0.x, c0.y));
+                    bfrag[nb][1] = __builtin_bit_cast(bf16x8_t, unpack_words8(c0.z, c0.w));
+                    bfrag[nb][2] = __builtin_bit_cast(bf16x8_t, unpack_words8(c1.x, c1.y));
+                    bfrag[nb][3] = __builtin_bit_cast(bf16x8_t, unpack_words8(c1.z, c1.w));
+                }
+                sc[nb] = __uint_as_float(quad_hi(s_cur[nb], q));
+            }
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++) {
+                bf16x8_t afrag[4];
+#pragma unroll
+                for (int t = 0; t < 4; t++) afrag[t] = *reinterpret_cast<const bf16x8_t*>(ab + (mb * 4 + t) * 1024);
 #pragma unroll
                 for (int nb = 0; nb < NB; nb++) {
-                    if constexpr (BITS == 4) {
-                        const uint4 cw = *reinterpret_cast<const uint4*>(bb + nb * 32 * 32);
-                        bfrag[nb][0] = __builtin_bit_cast(bf16x8_t, unpack_word4(cw.x, mask_s, magic_v));
-                        bfrag[nb][1] = __builtin_bit_cast(bf16x8_t, unpack_word4(cw.y, mask_s, magic_v));
-                        bfrag[nb][2] = __builtin_bit_cast(bf16x8_t, unpack_word4(cw.z, mask_s, magic_v));
-                        bfrag[nb][3] = __builtin_bit_cast(bf16x8_t, unpack_word4(cw.w, mask_s, magic_v));
-                    } else {
-                        const uint4 c0 = *reinterpret_cast<const uint4*>(bb + nb * 32 * 64);
-                        const uint4 c1 = *reinterpret_cast<const uint4*>(bb + nb * 32 * 64 + 16);
-                        bfrag[nb][0] = __builtin_bit_cast(bf16x8_t, unpack_words8(c0.x, c0.y));
-                        bfrag[nb][1] = __builtin_bit_cast(bf16x8_t, unpack_words8(c0.z, c0.w));
-                        bfrag[nb][2] = __builtin_bit_cast(bf16x8_t, unpack_words8(c1.x, c1.y));
-                        bfrag[nb][3] = __builtin_bit_cast(bf16x8_t, unpack_words8(c1.z, c1.w));
-                    }
-                    sc[nb] = __uint_as_float(quad_hi(s_cur[nb], q));
-                }
+                    f32x16_t p = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int mb = 0; mb < MB; mb++) {
-                    bf16x8_t afrag[4];
+                    for (int t = 0; t < 4; t++) p = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag[t], bfrag[nb][t], p, 0, 0, 0);
 #pragma unroll
-                    for (int t = 0; t < 4; t++) afrag[t] = *reinterpret_cast<const bf16x8_t*>(ab + (mb * 4 + t) * 1024);
-#pragma unroll
-                    for (int nb = 0; nb < NB; nb++) {
-                        f32x16_t p = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                        for (int t = 0; t < 4; t++) p = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag[t], bfrag[nb][t], p, 0, 0, 0);
-#pragma unroll
-                        for (int r = 0; r < 16; r++) out[mb][nb][r] = __fmaf_rn(sc[nb], p[r], out[mb][nb][r]);
-                    }
+                    for (int r = 0; r < 16; r++) out[mb][nb][r] = __fmaf_rn(sc[nb], p[r], out[mb][nb][r]);
                 }
             }
+        };
+        if (blocks == 4) {
+            block(std::integral_constant<int, 0>{});
+            block(std::integral_constant<int, 1>{});
+            block(std::integral_constant<int, 2>{});
+            block(std::integral_constant<int, 3>{});
+        } else {
+            block(std::integral_constant<int, 0>{});
+            if (blocks > 1) block(std::integral_constant<int, 1>{});
+            if (blocks > 2) block(std::integral_constant<int, 2>{});
         }
         {
             // affine terms of the quad's blocks in one MFMA: k-slots (2q, 2q+1) carry (Sx_hi, Sx_lo) of block q on
@@ -275,8 +292,6 @@ __global__ __launch_bounds__(4 * kWave, 1) void qmm_few_kernel(const QmmTileArgs
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         st ^= 1;
-        // first use of the next quad's registers HERE, where nothing is outstanding: the compiler cannot count the
-        // copy instructions, and a wait of its own further down would drain the copies of the quad after next
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) {
             asm volatile("" : "+v"(s_nxt[nb].x), "+v"(s_nxt[nb].y), "+v"(b_nxt[nb].x), "+v"(b_nxt[nb].y));
@@ -288,6 +303,9 @@ __global__ __launch_bounds__(4 * kWave, 1) void qmm_few_kernel(const QmmTileArgs
             asm volatile("" : "+v"(xs_nxt[mb].x), "+v"(xs_nxt[mb].y), "+v"(xs_nxt[mb].z), "+v"(xs_nxt[mb].w));
             xs_cur[mb] = xs_nxt[mb];
         }
+        __builtin_amdgcn_sched_barrier(0);
+        load_all(quad + 2, s_nxt, b_nxt, xs_nxt);  // clamped to the last quad of K
+        __builtin_amdgcn_sched_barrier(0);
     }
 
     // D layout of v_mfma_f32_32x32x*: lane (j, h), register r -> row 8*(r/4) + 4*h + r%4, column j.  Every 32-row
