@@ -50,11 +50,11 @@ def pmc_summary(root):
         print("%-90s %-12s n=%-4d mean=%.6g" % (k[:90], c, len(v), sum(v) / len(v)))
 
 
-def traffic_from_profiles():
-    """HBM bytes per launch of the dominant kernel as recorded in profiles/ (from rocprofv3 --pmc
-    FETCH_SIZE and WRITE_SIZE passes, scaled by the kernels of known traffic in the same passes)."""
+def traffic_from_profiles(name="qmv_dominant_traffic.md"):
+    """Bytes per launch of a kernel as recorded in profiles/ (from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
+    passes, scaled by the kernels of known traffic in the same passes)."""
     import re
-    path = os.path.join(ROOT, "profiles", "qmv_dominant_traffic.md")
+    path = os.path.join(ROOT, "profiles", name)
     try:
         m = re.search(r"traffic_bytes_per_launch:\s*([0-9]+)", open(path).read())
         return int(m.group(1)) if m else None
@@ -292,7 +292,8 @@ def main():
         tf = flops / (q_ms * 1e-3) / 1e12
         qmm = {"M": M, "K": K, "N": N, "ms": round(q_ms, 4), "TFLOPs": round(tf, 1), "kernel": ctx.last_variant(1),
                "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                            "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None}}
+                            "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
+                            "traffic": traffic_from_profiles("qmm_cfg3_traffic.md")}}
         # the same call on the other kernel family: bare codes as bf16 operands and one fp32 FMA per output element
         # and 64-code block (the default is the family whose MFMA operand carries scale * (code - 8) as fp16)
         other = "qmmt_b4_mb2_nb2_wm2_wn2"
