@@ -275,6 +275,21 @@ class Context:
         self._check(self.lib.aq_qmv_multi(self.handle, _ptr(x), n, arr(ws), arr(ss), arr(bs), arr(ys),
                                           (_c.c_int * n)(*Ns), M, K, group_size, bits, flags))
 
+    def prepared_qmv(self, x, w, s, b, y, M, K, N, group_size=64, bits=4, flags=0):
+        """The same call as qmv with every argument converted once: returns a function of no arguments.  For loops
+        whose per-call host work would otherwise be this wrapper's argument handling."""
+        fn, check, h = self.lib.aq_qmv, self._check, self.handle
+        args = (_ptr(x), _ptr(w), _ptr(s), _ptr(b), _ptr(y), M, K, N, group_size, bits, flags)
+        return lambda: check(fn(h, *args))
+
+    def prepared_qmv_multi(self, x, ws, ss, bs, ys, Ns, M, K, group_size=64, bits=4, flags=0):
+        """qmv_multi with its pointer arrays built once: returns a function of no arguments."""
+        n = len(ws)
+        arr = lambda seq: (_c.c_void_p * n)(*[_ptr(t) for t in seq])
+        fn, check, h = self.lib.aq_qmv_multi, self._check, self.handle
+        args = (_ptr(x), n, arr(ws), arr(ss), arr(bs), arr(ys), (_c.c_int * n)(*Ns), M, K, group_size, bits, flags)
+        return lambda: check(fn(h, *args))
+
     def reserve_workspace(self, M, K):
         self._check(self.lib.aq_reserve_workspace(self.handle, M, K))
 

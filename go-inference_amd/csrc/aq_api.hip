@@ -125,9 +125,10 @@ int pick_qmv_variant(const aq_ctx* ctx, int bits, int m, bool gather, int N, int
 }
 
 // One index space over the matvec kernel families: dot2 variants first, then the 32x32 MFMA
-// variants, then the block-MFMA variants, then the streaming dot2 variants.
+// variants, then the block-MFMA variants, then the streaming dot2 variants, then the diagonal-MFMA variants.
 int qmv_total_variants() {
-    return aq::qmv_variant_count() + aq::qmvx_variant_count() + aq::qmvb_variant_count() + aq::qmvs_variant_count();
+    return aq::qmv_variant_count() + aq::qmvx_variant_count() + aq::qmvb_variant_count() + aq::qmvs_variant_count() +
+           aq::qmvd_variant_count();
 }
 const aq::QmvVariant* qmv_any_variant(int idx) {
     const int nd = aq::qmv_variant_count();
@@ -136,7 +137,9 @@ const aq::QmvVariant* qmv_any_variant(int idx) {
     if (idx < nd + nx) return aq::qmvx_variant(idx - nd);
     const int nb = aq::qmvb_variant_count();
     if (idx < nd + nx + nb) return aq::qmvb_variant(idx - nd - nx);
-    return aq::qmvs_variant(idx - nd - nx - nb);
+    const int ns = aq::qmvs_variant_count();
+    if (idx < nd + nx + nb + ns) return aq::qmvs_variant(idx - nd - nx - nb);
+    return aq::qmvd_variant(idx - nd - nx - nb - ns);
 }
 
 constexpr size_t kMaxLds = 160 * 1024;
@@ -164,6 +167,26 @@ int launch_qmv_rows(aq_ctx* ctx, aq::QmvArgs a, int group_size, int bits, bool g
     const int nx = aq::qmvx_variant_count();
     int forced = ctx->forced[0];
     const int nbk = aq::qmvb_variant_count();
+    const int nst = aq::qmvs_variant_count();
+    if (forced >= nd + nx + nbk + nst) {
+        // diagonal-MFMA family, forced
+        const int di = forced - nd - nx - nbk - nst;
+        if (!aq::qmvd_fits(a, bits, group_size, gather, di))
+            return fail(AQ_ERR_ARG, "aq_qmv: forced variant %d does not fit bits=%d gather=%d rows=%d K=%d N=%d", forced,
+                        bits, (int)gather, M, a.K, a.N);
+        ctx->last_variant[0] = aq::qmvd_variant(di)->name;
+        AQ_HIP(aq::qmvd_launch(di, a, ctx->stream), "hipLaunchKernel");
+        return AQ_OK;
+    }
+    if (forced < 0 && !gather) {
+        // 4-bit group-64 codes, up to 4 rows, K of 2..4 steps of 1024: the diagonal-MFMA kernels
+        const int di = aq::qmvd_pick(M, a.K);
+        if (di >= 0 && aq::qmvd_fits(a, bits, group_size, gather, di)) {
+            ctx->last_variant[0] = aq::qmvd_variant(di)->name;
+            AQ_HIP(aq::qmvd_launch(di, a, ctx->stream), "hipLaunchKernel");
+            return AQ_OK;
+        }
+    }
     if (forced >= nd + nx + nbk || (forced < 0 && M == 1 && kStreamDefault)) {
         // streaming dot2 family: forced, or the default for one activation row wherever K fits it
         aq::StreamPlan plan;
@@ -537,6 +560,38 @@ int aq_qmv_multi(aq_ctx* ctx, const void* x, int count, const void* const* packe
         fused = fused && total < (int64_t)1 << 30;
         if (fused) {
             std::lock_guard<std::mutex> lk(ctx->mu);
+            // the kernels aq_qmv would pick for each member, in one grid
+            const int di = aq::qmvd_pick(1, K);
+            if (di >= 0 && aq::qmvd_multi_supported(di)) {
+                bool fits = true;
+                aq::QmvMultiArgs ma{};
+                ma.common.x = static_cast<const uint16_t*>(x);
+                ma.common.K = K;
+                ma.common.M = 1;
+                ma.common.gs_shift = ilog2(group_size);
+                ma.common.out_f32 = (flags & AQ_OUT_F32) ? 1 : 0;
+                ma.common.routes = 1;
+                ma.count = count;
+                for (int i = 0; i < count; i++) {
+                    ma.w[i] = static_cast<const uint32_t*>(packed[i]);
+                    ma.s[i] = static_cast<const uint16_t*>(scales[i]);
+                    ma.b[i] = static_cast<const uint16_t*>(biases[i]);
+                    ma.y[i] = y[i];
+                    ma.N[i] = N[i];
+                    aq::QmvArgs one = ma.common;
+                    one.w = ma.w[i];
+                    one.s = ma.s[i];
+                    one.b = ma.b[i];
+                    one.y = y[i];
+                    one.N = N[i];
+                    fits = fits && aq::qmvd_fits(one, bits, group_size, false, di);
+                }
+                if (fits) {
+                    ctx->last_variant[0] = "qmv_multi_diag";
+                    AQ_HIP(aq::qmvd_multi_launch(di, ma, ctx->stream), "hipLaunchKernel");
+                    return AQ_OK;
+                }
+            }
             const int idx = pick_qmv_variant(ctx, bits, 1, false, (int)total, K, 1);
             const int rows = idx >= 0 ? aq::qmv_variant(idx)->rows : 0;
             if (rows > 0 && aq::qmv_multi_supported(bits, 1, rows)) {

@@ -85,6 +85,7 @@ struct QmvVariant {
     int kind;    // 0: VALU dot2 kernel (aq_qmv.hip), 1: MFMA kernel (aq_qmv_mfma.hip; m = most rows it takes),
                  // 2: block-MFMA kernel (aq_qmv_blk.hip; m = most rows, depth = K pieces per wavefront),
                  // 3: streaming dot2 kernel (aq_qmv_stream.hip; depth = rows in flight, xmode = slices per row)
+                 // 4: diagonal-MFMA kernel (aq_qmv_diag.hip; m = most rows, rows = rows per workgroup)
 };
 
 int qmv_variant_count();
@@ -139,6 +140,16 @@ int qmvs_variant_count();
 const QmvVariant* qmvs_variant(int idx);
 bool qmvs_plan(const QmvArgs& a, int bits, int group_size, bool gather, int cu_count, int forced_idx, StreamPlan* out);
 hipError_t qmvs_launch(const StreamPlan& p, const QmvArgs& a, hipStream_t stream);
+
+// Diagonal-MFMA matvec kernels (aq_qmv_diag.hip; 4-bit group-64 codes, M <= 4, K a multiple of 256).
+int qmvd_variant_count();
+const QmvVariant* qmvd_variant(int idx);
+bool qmvd_fits(const QmvArgs& a, int bits, int group_size, bool gather, int idx);
+hipError_t qmvd_launch(int idx, const QmvArgs& a, hipStream_t stream);
+// The variant the library picks for M rows and this K, or -1 when another family takes the shape.
+int qmvd_pick(int M, int K);
+bool qmvd_multi_supported(int idx);
+hipError_t qmvd_multi_launch(int idx, QmvMultiArgs ma, hipStream_t stream);
 
 // lm_head kernels (aq_qmv_head.hip), one activation row: the projection with its epilogue replaced by
 //   fuse 3: best[0] = max over rows of pack(score, row): every wavefront stores its own maximum into

@@ -1,0 +1,411 @@
+// affine_qmv for gfx950, M = 1..4 activation rows of 4-bit group-64 codes: the diagonal-MFMA kernel.
+//
+// Same contract as the dot2 kernel (aq_qmv.hip): replaces rocm_mlx_q4_projection*
+// (go/engine/hip/kernels/quant/affine_projection.hipinc:3-266), semantics of MLX affine_qmv
+// (go/engine/metal/qmv.go:354-421).
+//
+// The dot2 kernel pays, per packed word of a lane, 7 vector instructions to expand the codes and 4 more
+// to multiply them, then a cross-lane reduction per row; it is bound by those issue slots.  Here only the
+// expansion stays on the vector unit:
+//   * v_mfma_f32_16x16x32_bf16 contracts over (lane group, element): lane (n = lane % 16, j = lane / 16)
+//     supplies as B eight codes of weight row n, so the sum over the 64 lanes that the dot2 kernel does
+//     with DPP adds happens inside the instruction;
+//   * the 16 rows of A are (token t, group slot g): row (t, g) carries the activations of token t in the
+//     lane groups whose codes belong to 64-group g of the current chunk and zeros elsewhere, so
+//     D[(t, g)][n] is the code . activation sum of exactly one quantisation group, for up to four tokens
+//     at the cost of one.  D lands as lane (t, n), register g;
+//   * per 256-code chunk of 16 rows: two 16-byte loads per lane (64 contiguous bytes per row and
+//     instruction), 8 MFMAs, and per lane `acc += scale[g] * D[g]` (four FMAs);
+//   * the affine term needs no vector work either: the group sums X of the activations are split into
+//     three bf16 terms when x is staged (exact: 3 x 8 bits), and one more MFMA per chunk accumulates
+//     bias * X - 128 * scale * X from B = (b, b, b, s, s, s, 0, 0), A = (X0, X1, X2, -128 X0, -128 X1,
+//     -128 X2, 0, 0), every product exact (the codes travel as 128 + code, see aq_device.h);
+//   * the NW wavefronts of a workgroup take the chunks of the same 16 rows in turn and meet in LDS.
+#include "aq_device.h"
+#include "aq_kernels.h"
+
+namespace aq {
+
+namespace {
+
+typedef const __attribute__((address_space(1))) char* gptr_t;
+__device__ __forceinline__ gptr_t uniform_ptr(const void* p) {
+    const uint64_t u = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)u);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(u >> 32));
+    return reinterpret_cast<gptr_t>(((uint64_t)hi << 32) | lo);
+}
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint4 load_u128_at(gptr_t base, uint32_t off) {
+    const u32x4_t v = *reinterpret_cast<const __attribute__((address_space(1))) u32x4_t*>(base + off);
+    return make_uint4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ uint2 load_u64_at(gptr_t base, uint32_t off) {
+    const u32x2_t v = *reinterpret_cast<const __attribute__((address_space(1))) u32x2_t*>(base + off);
+    return make_uint2(v[0], v[1]);
+}
+
+__device__ __forceinline__ bf16x8_t as_bf16x8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+    const uint4 v = make_uint4(a, b, c, d);
+    return __builtin_bit_cast(bf16x8_t, v);
+}
+
+}  // namespace
+
+constexpr int kDiagRows = 16;      // weight rows per workgroup
+constexpr int kDiagChunk = 256;    // codes of a row per MFMA chain (four groups of 64)
+constexpr int kDiagSuper = 1024;   // codes of a row per wavefront step (four chunks)
+constexpr int kDiagZeroBytes = 64;
+
+// LDS: activations in expansion order [M][K] bf16, the split group sums [M][K/1024][4] x 48 B, 64 zero bytes,
+// the partial sums of the wavefronts [NW][64] fp32.
+__host__ __device__ inline size_t qmvd_lds_bytes_for(int M, int K, int nw) {
+    return (size_t)M * K * 2 + (size_t)M * (K / kDiagChunk) * 48 + kDiagZeroBytes + (size_t)nw * 64 * 4;
+}
+
+// NR sets of NW wavefronts (a set per 16 rows), each wavefront takes SUP steps of 1024 codes (steps wave, wave + NW, ...) of the same 16 rows and requests
+// everything it will read up front.
+template <int NW, int SUP, int NR>
+__device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave_wg = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave = wave_wg % NW;  // which steps of K
+    const int rg = wave_wg / NW;    // which 16 rows of the workgroup's NR x 16
+    const int K = a.K, N = a.N, M = a.M;
+    const int groups = K >> 6;
+    const int supers = K / kDiagSuper;
+    const uint32_t xs_off = 0;
+    const uint32_t a2_off = (uint32_t)M * K * 2;
+    const uint32_t zero_off = a2_off + (uint32_t)M * (K / kDiagChunk) * 48;
+    const uint32_t red_off = zero_off + kDiagZeroBytes;
+
+    // ---- stage x: expansion order within every 8 values, group sums split into three bf16 terms ----
+    const gptr_t xg = uniform_ptr(a.x);
+    const int pieces = M * (K >> 3);  // 16-byte pieces of all tokens (K % 1024 == 0: a token is whole pieces)
+    auto stage = [&](int p, const uint4 v) {
+        uint4 o;
+        o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);  // (x0, x4)
+        o.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);  // (x1, x5)
+        o.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);  // (x2, x6)
+        o.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);  // (x3, x7)
+        *reinterpret_cast<uint4*>(lds_raw + xs_off + (uint32_t)p * 16) = o;
+        const uint32_t ones = 0x3f803f80u;
+        float sum = dot2_bf16(v.x, ones, 0.0f);
+        sum = dot2_bf16(v.y, ones, sum);
+        sum = dot2_bf16(v.z, ones, sum);
+        sum = dot2_bf16(v.w, ones, sum);
+        // the eight pieces of a group sit in eight consecutive lanes
+        sum += __shfl_xor(sum, 1);
+        sum += __shfl_xor(sum, 2);
+        sum += __shfl_xor(sum, 4);
+        if ((p & 7) == 0) {
+            const uint32_t u0 = __float_as_uint(sum) & 0xffff0000u;
+            const float r1 = sum - __uint_as_float(u0);
+            const uint32_t u1 = __float_as_uint(r1) & 0xffff0000u;
+            const float r2 = r1 - __uint_as_float(u1);
+            const uint32_t u2 = __float_as_uint(r2) & 0xffff0000u;
+            const uint32_t n0 = __float_as_uint(-128.0f * __uint_as_float(u0));
+            const uint32_t n1 = __float_as_uint(-128.0f * __uint_as_float(u1));
+            const uint32_t n2 = __float_as_uint(-128.0f * __uint_as_float(u2));
+            // group g of a token: 12 bytes at [chunk g / 4][g % 4] of that token's table
+            const uint32_t g = (uint32_t)p >> 3;
+            uint32_t* e = reinterpret_cast<uint32_t*>(lds_raw + a2_off + (g >> 2) * 48 + (g & 3) * 12);
+            e[0] = (u0 >> 16) | u1;  // (X0, X1)
+            e[1] = (u2 >> 16) | n0;  // (X2, -128 X0)
+            e[2] = (n1 >> 16) | n2;  // (-128 X1, -128 X2)
+        }
+    };
+    // the first pieces of a thread are requested before the weights, so that they arrive first
+    constexpr int PRE = 2;
+    uint4 pre[PRE];
+#pragma unroll
+    for (int q = 0; q < PRE; q++) {
+        int p = tid + q * NR * NW * kWave;
+        if (p >= pieces) p = pieces - 1;
+        pre[q] = load_u128_at(xg, (uint32_t)p * 16);
+    }
+    if (tid < kDiagZeroBytes / 16) *reinterpret_cast<uint4*>(lds_raw + zero_off + tid * 16) = make_uint4(0, 0, 0, 0);
+
+    // ---- per-lane constants ----
+    const int n = lane & 15;   // weight row of the lane (B operand, D column)
+    const int j = lane >> 4;   // lane group: which 16 bytes of a 64-byte row piece (B), token (D)
+    const int at = (lane & 15) >> 2;  // A operand: token of the lane's A row
+    const int ag = lane & 3;          // A operand: group slot of the lane's A row
+    const int row0 = (block * NR + rg) * kDiagRows;
+    int row = row0 + n;
+    if (row >= N) row = N - 1;
+    const gptr_t wg = uniform_ptr(a.w);
+    const gptr_t sg = uniform_ptr(a.s);
+    const gptr_t bg = uniform_ptr(a.b);
+    const uint32_t w_lane = (uint32_t)row * (uint32_t)(K >> 1) + (uint32_t)j * 16;  // bytes
+    // scales and biases: lane group j holds the four groups of chunk j of the step
+    const uint32_t sb_lane = (uint32_t)row * (uint32_t)groups * 2 + (uint32_t)j * 8;  // bytes
+
+    // A fragments: load L (0, 1) of a chunk holds groups 2L and 2L + 1; lane group j holds codes of group
+    // 2L + (j >> 1).  The lane's A row (at, ag) is non-zero in load L iff ag == 2L + (j >> 1).
+    const bool tok = at < M;
+    const bool d0 = tok && ag == (j >> 1);
+    const bool d1 = tok && ag == 2 + (j >> 1);
+    const uint32_t x_lane = xs_off + (uint32_t)at * K * 2 + (uint32_t)j * 64;  // codes j*32.. of a 128-code load
+    const uint32_t a_base0 = d0 ? x_lane : zero_off, a_base1 = d1 ? x_lane + 256 : zero_off;
+    const uint32_t a_mul0 = d0 ? 2048 : 0, a_mul1 = d1 ? 2048 : 0, a_chunk0 = d0 ? 512 : 0, a_chunk1 = d1 ? 512 : 0;
+    // affine-term A: rows (t, 0) carry the split sums of the four groups of chunk j of the step, 48 bytes
+    const bool d2 = tok && ag == 0;
+    const uint32_t a2_base = d2 ? a2_off + ((uint32_t)at * (K / kDiagChunk) + j) * 48 : zero_off;
+    const uint32_t a2_mul = d2 ? 4 * 48 : 0;
+    // the lane that holds the scales of chunk 0 of the step for this lane's row (ds_bpermute byte address)
+    const int sc_addr = n * 4;
+
+    const uint32_t mask = opaque_s(kNibbleMask);
+    const uint32_t magic = opaque_v(kMagic128);
+
+    uint4 wq[SUP][4][2];
+    uint2 sq[SUP], bq[SUP];
+#pragma unroll
+    for (int u = 0; u < SUP; u++) {
+        int sp = wave + u * NW;
+        if (sp >= supers) sp = supers - 1;  // past the end: a valid address, the result is not used
+        const uint32_t wo = w_lane + (uint32_t)sp * 512;
+#pragma unroll
+        for (int cc = 0; cc < 4; cc++) {
+            wq[u][cc][0] = load_u128_at(wg, wo + cc * 128);
+            wq[u][cc][1] = load_u128_at(wg, wo + cc * 128 + 64);
+        }
+        sq[u] = load_u64_at(sg, sb_lane + (uint32_t)sp * 32);
+        bq[u] = load_u64_at(bg, sb_lane + (uint32_t)sp * 32);
+    }
+
+#pragma unroll
+    for (int q = 0; q < PRE; q++) {
+        const int p = tid + q * NR * NW * kWave;
+        if (p < pieces) stage(p, pre[q]);
+    }
+    for (int p = tid + PRE * NR * NW * kWave; p < pieces; p += NR * NW * kWave) stage(p, load_u128_at(xg, (uint32_t)p * 16));
+    __syncthreads();  // x, sums and zeros are in LDS
+
+    float acc = 0.0f;
+    f32x4_t dsum = {0.0f, 0.0f, 0.0f, 0.0f};  // affine term, register 0 is the one that is used
+#pragma unroll
+    for (int u = 0; u < SUP; u++) {
+        const int sp = wave + u * NW;
+        if (sp < supers) {
+            const uint2 sv = sq[u], bv = bq[u];
+            // affine term of the 16 groups of the step: 24 k-slots per lane, three MFMAs
+            {
+                const uint32_t a2_addr = a2_base + (uint32_t)sp * a2_mul;
+                const bf16x8_t a20 = *reinterpret_cast<const bf16x8_t*>(lds_raw + a2_addr);
+                const bf16x8_t a21 = *reinterpret_cast<const bf16x8_t*>(lds_raw + a2_addr + 16);
+                const bf16x8_t a22 = *reinterpret_cast<const bf16x8_t*>(lds_raw + a2_addr + 32);
+                // (b0 b0 b0 s0 s0 s0 b1 b1 | b1 s1 s1 s1 b2 b2 b2 s2 | s2 s2 b3 b3 b3 s3 s3 s3)
+                const uint32_t lo2 = 0x01000100u, hi2 = 0x03020302u, lolo = 0x05040100u, hihi = 0x07060302u;
+                const uint32_t e0 = __builtin_amdgcn_perm(bv.x, bv.x, lo2), e1 = __builtin_amdgcn_perm(sv.x, bv.x, lolo);
+                const uint32_t e2 = __builtin_amdgcn_perm(sv.x, sv.x, lo2), e3 = __builtin_amdgcn_perm(bv.x, bv.x, hi2);
+                const uint32_t e4 = __builtin_amdgcn_perm(sv.x, bv.x, hihi), e5 = __builtin_amdgcn_perm(sv.x, sv.x, hi2);
+                const uint32_t e6 = __builtin_amdgcn_perm(bv.y, bv.y, lo2), e7 = __builtin_amdgcn_perm(sv.y, bv.y, lolo);
+                const uint32_t e8 = __builtin_amdgcn_perm(sv.y, sv.y, lo2), e9 = __builtin_amdgcn_perm(bv.y, bv.y, hi2);
+                const uint32_t e10 = __builtin_amdgcn_perm(sv.y, bv.y, hihi), e11 = __builtin_amdgcn_perm(sv.y, sv.y, hi2);
+                dsum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a20, as_bf16x8(e0, e1, e2, e3), dsum, 0, 0, 0);
+                dsum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a21, as_bf16x8(e4, e5, e6, e7), dsum, 0, 0, 0);
+                dsum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a22, as_bf16x8(e8, e9, e10, e11), dsum, 0, 0, 0);
+            }
+            const uint32_t a_addr0 = a_base0 + (uint32_t)sp * a_mul0, a_addr1 = a_base1 + (uint32_t)sp * a_mul1;
+#pragma unroll
+            for (int cc = 0; cc < 4; cc++) {
+                bf16x8_t af[2][4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    af[0][i] = *reinterpret_cast<const bf16x8_t*>(lds_raw + a_addr0 + cc * a_chunk0 + i * 16);
+                    af[1][i] = *reinterpret_cast<const bf16x8_t*>(lds_raw + a_addr1 + cc * a_chunk1 + i * 16);
+                }
+                // the four scales of chunk cc of this lane's row sit in lane group cc
+                const uint32_t sx = (uint32_t)__builtin_amdgcn_ds_bpermute(sc_addr + cc * 64, (int)sv.x);
+                const uint32_t sy = (uint32_t)__builtin_amdgcn_ds_bpermute(sc_addr + cc * 64, (int)sv.y);
+                f32x4_t dq = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int L = 0; L < 2; L++) {
+                    const uint32_t ww[4] = {wq[u][cc][L].x, wq[u][cc][L].y, wq[u][cc][L].z, wq[u][cc][L].w};
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        uint32_t p[4];
+                        unpack4_word(ww[i], mask, magic, p);
+                        dq = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[L][i], as_bf16x8(p[0], p[1], p[2], p[3]), dq, 0, 0, 0);
+                    }
+                }
+                acc = __builtin_fmaf(bf16_bits_to_f32(sx & 0xffffu), dq[0], acc);
+                acc = __builtin_fmaf(__uint_as_float(sx & 0xffff0000u), dq[1], acc);
+                acc = __builtin_fmaf(bf16_bits_to_f32(sy & 0xffffu), dq[2], acc);
+                acc = __builtin_fmaf(__uint_as_float(sy & 0xffff0000u), dq[3], acc);
+            }
+        }
+    }
+    acc += dsum[0];
+
+    // ---- the wavefronts' partial sums meet in LDS; lane (t, n) of wavefront 0 stores ----
+    float* red = reinterpret_cast<float*>(lds_raw + red_off);
+    red[wave_wg * 64 + lane] = acc;
+    __syncthreads();
+    if (wave == 0) {
+        float total = red[wave_wg * 64 + lane];
+#pragma unroll
+        for (int w2 = 1; w2 < NW; w2++) total += red[(wave_wg + w2) * 64 + lane];
+        const int t = j, r = row0 + n;
+        if (t < M && r < N) {
+            const size_t o = (size_t)t * N + r;
+            if (a.out_f32) {
+                static_cast<float*>(a.y)[o] = total;
+            } else {
+                static_cast<uint16_t*>(a.y)[o] = f32_to_bf16_bits(total);
+            }
+        }
+    }
+}
+
+template <int NW, int SUP, int NR>
+__global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_kernel(const QmvArgs a) {
+    qmv_diag_body<NW, SUP, NR>(a, (int)blockIdx.x);
+}
+
+// Several weight matrices against the same activations in one launch (q|k|v, gate|up): the workgroups of all
+// matrices form one grid, and each looks up which matrix it belongs to.
+template <int NW, int SUP, int NR>
+__global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_multi_kernel(const QmvMultiArgs ma) {
+    int set = 0;
+#pragma unroll
+    for (int i = 1; i < kQmvMultiMax; i++)
+        if (i < ma.count && (int)blockIdx.x >= ma.block_end[i - 1]) set = i;
+    QmvArgs a = ma.common;
+    a.w = ma.w[set];
+    a.s = ma.s[set];
+    a.b = ma.b[set];
+    a.y = ma.y[set];
+    a.N = ma.N[set];
+    qmv_diag_body<NW, SUP, NR>(a, (int)blockIdx.x - (set ? ma.block_end[set - 1] : 0));
+}
+
+// ---- variant table --------------------------------------------------------
+
+typedef void (*QmvDiagKernel)(const QmvArgs);
+struct QmvDiagEntry {
+    QmvVariant v;
+    QmvDiagKernel fn;
+};
+// name, bits, m (most rows), sets of 16 rows per workgroup, wavefronts per set, steps per wavefront, gather, xmode, kind
+// waves x depth steps of 1024 codes cover K
+#define AQ_QMVD(NW, SUP, NR)                                                                              \
+    {                                                                                                     \
+        {"qmvd_b4_m4_r" #NR "_w" #NW "_d" #SUP "_g0", 4, 4, NR, NW, SUP, 0, 0, 4}, qmv_diag_kernel<NW, SUP, NR> \
+    }
+static const QmvDiagEntry kQmvDiagTable[] = {
+    AQ_QMVD(4, 1, 1), AQ_QMVD(4, 1, 2), AQ_QMVD(4, 1, 4), AQ_QMVD(2, 2, 2), AQ_QMVD(2, 1, 2), AQ_QMVD(8, 1, 1),
+    AQ_QMVD(4, 2, 1), AQ_QMVD(2, 1, 4), AQ_QMVD(6, 1, 1), AQ_QMVD(10, 1, 1), AQ_QMVD(12, 1, 1),
+    AQ_QMVD(14, 1, 1), AQ_QMVD(16, 1, 1),
+};
+
+int qmvd_variant_count() { return (int)(sizeof(kQmvDiagTable) / sizeof(kQmvDiagTable[0])); }
+const QmvVariant* qmvd_variant(int idx) {
+    if (idx < 0 || idx >= qmvd_variant_count()) return nullptr;
+    return &kQmvDiagTable[idx].v;
+}
+
+bool qmvd_fits(const QmvArgs& a, int bits, int group_size, bool gather, int idx) {
+    const QmvVariant* v = qmvd_variant(idx);
+    if (!v || bits != 4 || group_size != 64 || gather) return false;
+    if (a.M < 1 || a.M > 4 || a.K <= 0 || a.K % kDiagSuper != 0 || a.N < 1) return false;
+    if (a.K / kDiagSuper > v->waves * v->depth) return false;
+    const uintptr_t al16 = reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.w);
+    const uintptr_t al8 = reinterpret_cast<uintptr_t>(a.s) | reinterpret_cast<uintptr_t>(a.b);
+    if ((al16 & 15) || (al8 & 7)) return false;
+    // 32-bit byte offsets into the packed matrix
+    if ((uint64_t)a.N * (uint64_t)(a.K / 2) >= (1ull << 32)) return false;
+    return qmvd_lds_bytes_for(a.M, a.K, v->waves * v->rows) <= 96 * 1024;
+}
+
+hipError_t qmvd_launch(int idx, const QmvArgs& a, hipStream_t stream) {
+    if (idx < 0 || idx >= qmvd_variant_count()) return hipErrorInvalidValue;
+    const QmvDiagEntry& e = kQmvDiagTable[idx];
+    const size_t lds = qmvd_lds_bytes_for(a.M, a.K, e.v.waves * e.v.rows);
+    if (lds > 48 * 1024) {
+        hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e.fn),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (rc != hipSuccess) return rc;
+    }
+    const int wg_rows = kDiagRows * e.v.rows;
+    dim3 grid((unsigned)((a.N + wg_rows - 1) / wg_rows), 1u, 1u);
+    hipLaunchKernelGGL(e.fn, grid, dim3((unsigned)(e.v.rows * e.v.waves * kWave)), lds, stream, a);
+    return hipGetLastError();
+}
+
+// The variant the library picks for M rows and this K, or -1: one step of 1024 codes per wavefront; up to 4 steps,
+// more rows per workgroup the more activation rows there are to stage.
+int qmvd_pick(int M, int K) {
+    if (M < 1 || M > 4 || K <= 0 || K % kDiagSuper != 0) return -1;
+    const int steps = K / kDiagSuper;
+    int nw, nr;
+    if (steps == 2) {
+        nw = 2;
+        nr = M == 1 ? 2 : 4;
+    } else if (steps == 3 || steps == 4) {
+        nw = 4;
+        nr = M == 1 ? 1 : M == 2 ? 2 : 4;
+    } else if (steps <= 16 && M == 1) {
+        // one step per wavefront (an idle one when the count is odd); more rows would stage too much x per workgroup
+        nw = (steps + 1) & ~1;
+        nr = 1;
+    } else {
+        return -1;
+    }
+    for (int i = 0; i < qmvd_variant_count(); i++) {
+        const QmvVariant& v = kQmvDiagTable[i].v;
+        if (v.waves == nw && v.depth == 1 && v.rows == nr) return i;
+    }
+    return -1;
+}
+
+typedef void (*QmvDiagMultiKernel)(const QmvMultiArgs);
+struct QmvDiagMultiEntry {
+    int nw, sup, nr;
+    QmvDiagMultiKernel fn;
+};
+#define AQ_QMVD_MULTI(NW, SUP, NR) {NW, SUP, NR, qmv_diag_multi_kernel<NW, SUP, NR>}
+static const QmvDiagMultiEntry kQmvDiagMultiTable[] = {
+    AQ_QMVD_MULTI(4, 1, 1), AQ_QMVD_MULTI(4, 1, 2), AQ_QMVD_MULTI(4, 1, 4), AQ_QMVD_MULTI(2, 1, 2), AQ_QMVD_MULTI(2, 1, 4),
+    AQ_QMVD_MULTI(6, 1, 1), AQ_QMVD_MULTI(8, 1, 1), AQ_QMVD_MULTI(10, 1, 1), AQ_QMVD_MULTI(12, 1, 1), AQ_QMVD_MULTI(14, 1, 1),
+    AQ_QMVD_MULTI(16, 1, 1),
+};
+
+// The multi-matrix launch of variant idx (the same arithmetic, so the same bytes, as one launch per matrix).
+bool qmvd_multi_supported(int idx) {
+    const QmvVariant* v = qmvd_variant(idx);
+    if (!v) return false;
+    for (const QmvDiagMultiEntry& e : kQmvDiagMultiTable)
+        if (e.nw == v->waves && e.sup == v->depth && e.nr == v->rows) return true;
+    return false;
+}
+
+hipError_t qmvd_multi_launch(int idx, QmvMultiArgs ma, hipStream_t stream) {
+    const QmvVariant* v = qmvd_variant(idx);
+    const QmvDiagMultiEntry* e = nullptr;
+    if (v)
+        for (const QmvDiagMultiEntry& c : kQmvDiagMultiTable)
+            if (c.nw == v->waves && c.sup == v->depth && c.nr == v->rows) e = &c;
+    if (!e || ma.count < 1 || ma.count > kQmvMultiMax) return hipErrorInvalidValue;
+    const int wg_rows = kDiagRows * e->nr;
+    int blocks = 0;
+    for (int i = 0; i < ma.count; i++) {
+        blocks += (ma.N[i] + wg_rows - 1) / wg_rows;
+        ma.block_end[i] = blocks;
+    }
+    const size_t lds = qmvd_lds_bytes_for(ma.common.M, ma.common.K, e->nw * e->nr);
+    if (lds > 48 * 1024) {
+        hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e->fn),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (rc != hipSuccess) return rc;
+    }
+    hipLaunchKernelGGL(e->fn, dim3((unsigned)blocks), dim3((unsigned)(e->nw * e->nr * kWave)), lds, stream, ma);
+    return hipGetLastError();
+}
+
+}  // namespace aq

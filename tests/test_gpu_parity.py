@@ -134,6 +134,8 @@ def _parse_variant(name):
         return "blk", parts["b"], parts["m"], parts["g"]
     if name.startswith("qmvs_"):
         return "stream", parts["b"], 1, parts["g"]
+    if name.startswith("qmvd_"):
+        return "diag", parts["b"], parts["m"], parts["g"]
     return "dot2", parts["b"], parts["m"], parts["g"]
 
 
@@ -152,8 +154,8 @@ def test_qmv_every_variant(ctx, orc):
     try:
         for idx, name in enumerate(names):
             fam, bits, m, gather = _parse_variant(name)
-            if gather or fam in ("blk", "stream"):
-                continue  # covered by test_gather_every_variant / test_qmvb_every_variant / test_qmvs_every_variant
+            if gather or fam in ("blk", "stream", "diag"):
+                continue  # covered by test_gather_every_variant / test_qmvb_every_variant / test_qmvs_every_variant / test_qmvd_every_variant
             say("variant", idx, name)
             if bits not in data:
                 words, s, b = F.synthetic_affine(N, K, bits, 64, seed=500 + bits)
@@ -331,6 +333,89 @@ def test_qmvs_every_variant(ctx, orc):
         dw.free()
 
 
+def test_qmvd_every_variant(ctx, orc):
+    """Each diagonal-MFMA matvec variant, forced: 1..4 activation rows, K = all the steps of 1024 codes its
+    wavefronts take and one step fewer (an idle wavefront), ragged N; fp32 and bf16 stores; a K that is no multiple
+    of 1024, or more steps than the variant takes, is refused."""
+    import aq_mi355
+    names = aq_mi355.variant_names(0)
+    N = 150
+    data = {}
+    try:
+        for idx, name in enumerate(names):
+            fam, bits, m, gather = _parse_variant(name)
+            if fam != "diag":
+                continue
+            waves = int(name.split("_w")[1].split("_")[0])
+            steps = waves * int(name.split("_d")[1].split("_")[0])
+            wg_waves = waves * int(name.split("_r")[1].split("_")[0])
+            for K in sorted({1024 * steps, 1024 * max(1, steps - 1)}):
+                say("variant", idx, name, "K", K)
+                if K not in data:
+                    words, s, b = F.synthetic_affine(N, K, bits, 64, seed=530 + K // 1024)
+                    x = F.synthetic_x(4, K, seed=630 + K // 1024)
+                    data[K] = (DeviceAffine(ctx, words, s, b), x, F.reference_f64(x, words, s, b, bits, 64, K))
+                dw, x, ref = data[K]
+                ctx.force_variant(0, idx)
+                for rows in (1, 2, 3, 4):
+                    if rows * K * 2 + rows * (K // 256) * 48 + 64 + wg_waves * 256 > 96 * 1024:
+                        # the activations of all rows and their group sums sit in LDS: beyond 96 KiB the variant refuses
+                        with pytest.raises(aq_mi355.AqError) as ei:
+                            run_qmv(ctx, x[:rows], dw, rows, K, N, 64, bits, True)
+                        assert ei.value.code == aq_mi355.AQ_ERR_ARG
+                        continue
+                    acc = run_qmv(ctx, x[:rows], dw, rows, K, N, 64, bits, True)
+                    assert ctx.last_variant(0) == name
+                    check_accumulators(acc, ref[:rows], "%s rows=%d" % (name, rows))
+                out = run_qmv(ctx, x[:2], dw, 2, K, N, 64, bits, False)
+                check_bf16_store(out, ref[:2], name)
+            dw, x, ref = data[1024 * steps]
+            for bad_k in (1024 * steps - 256, 1024 * (steps + 1)):
+                with pytest.raises(aq_mi355.AqError) as ei:
+                    run_qmv(ctx, np.zeros((1, bad_k), np.uint16), dw, 1, bad_k, N, 64, bits, True)
+                assert ei.value.code == aq_mi355.AQ_ERR_ARG
+    finally:
+        ctx.force_variant(0, -1)
+    for dw, _, _ in data.values():
+        dw.free()
+
+
+def test_qmvd_is_the_default_for_few_rows(ctx, orc):
+    """4-bit group-64 codes: 1..4 activation rows with K of 2, 3 or 4 steps of 1024 codes, and one row with up to 16
+    steps, land on the diagonal-MFMA kernels without forcing, rows beyond the last full 16 included; other K, more
+    rows at a long K, and 8 bit do not."""
+    for K, N in ((4096, 16 * 9 + 5), (3072, 64), (2048, 33)):
+        words, s, b = F.synthetic_affine(N, K, 4, 64, seed=810 + K // 1024)
+        x = F.synthetic_x(4, K, seed=820 + K // 1024)
+        ref = F.reference_f64(x, words, s, b, 4, 64, K)
+        dw = DeviceAffine(ctx, words, s, b)
+        for rows in (1, 2, 3, 4):
+            say("default few rows", K, N, rows)
+            acc = run_qmv(ctx, x[:rows], dw, rows, K, N, 64, 4, True)
+            assert ctx.last_variant(0).startswith("qmvd_"), ctx.last_variant(0)
+            check_accumulators(acc, ref[:rows], "diag default K=%d rows=%d" % (K, rows))
+            out = run_qmv(ctx, x[:rows], dw, rows, K, N, 64, 4, False)
+            check_bf16_store(out, ref[:rows], "diag default bf16 K=%d rows=%d" % (K, rows))
+        dw.free()
+    for K in (5120, 7168, 14336, 16384):
+        words, s, b = F.synthetic_affine(40, K, 4, 64, seed=840 + K // 1024)
+        x = F.synthetic_x(1, K, seed=850 + K // 1024)
+        dw = DeviceAffine(ctx, words, s, b)
+        say("default one row", K)
+        acc = run_qmv(ctx, x, dw, 1, K, 40, 64, 4, True)
+        assert ctx.last_variant(0).startswith("qmvd_"), ctx.last_variant(0)
+        check_accumulators(acc, F.reference_f64(x, words, s, b, 4, 64, K), "diag default K=%d" % K)
+        dw.free()
+    for K, bits, rows in ((17408, 4, 1), (1024, 4, 1), (4096, 8, 1), (8192, 4, 2)):
+        words, s, b = F.synthetic_affine(32, K, bits, 64, seed=830)
+        x = F.synthetic_x(rows, K, seed=831)
+        dw = DeviceAffine(ctx, words, s, b)
+        acc = run_qmv(ctx, x, dw, rows, K, 32, 64, bits, True)
+        assert not ctx.last_variant(0).startswith("qmvd_"), ctx.last_variant(0)
+        check_accumulators(acc, F.reference_f64(x, words, s, b, bits, 64, K), "not diag K=%d bits=%d" % (K, bits))
+        dw.free()
+
+
 def test_qmvb_gather_every_variant(ctx, orc):
     """Each gather-capable block-MFMA variant, forced, against the oracle (batched x, row_base slab
     offset)."""
@@ -391,15 +476,16 @@ def test_concat_rows_is_byte_identical(ctx, orc):
         d.free()
 
 
-@pytest.mark.parametrize("M,bits,Ns", [(1, 4, (96, 160, 40)), (1, 4, (4096, 1024, 1024)), (1, 4, (50,)), (1, 4, (7, 9, 300, 64)),
-                                        (2, 4, (96, 160)), (1, 8, (64, 200)), (1, 4, (96, 0, 32))])
-def test_qmv_multi_matches_separate_calls(ctx, orc, M, bits, Ns):
+@pytest.mark.parametrize("M,bits,Ns,K", [(1, 4, (96, 160, 40), 1024), (1, 4, (4096, 1024, 1024), 1024), (1, 4, (50,), 1024),
+                                          (1, 4, (7, 9, 300, 64), 1024), (2, 4, (96, 160), 1024), (1, 8, (64, 200), 1024),
+                                          (1, 4, (96, 0, 32), 1024), (1, 4, (96, 160, 40), 2048), (1, 4, (4096, 1024, 1030), 4096),
+                                          (1, 4, (7, 300), 3072), (2, 4, (96, 160), 4096), (1, 8, (64, 200), 4096)])
+def test_qmv_multi_matches_separate_calls(ctx, orc, M, bits, Ns, K):
     """aq_qmv_multi (q|k|v, gate|up in one launch) is byte-identical to one aq_qmv per matrix, the
     contract ConcatQuantRows states (go/model/quant_weight.go:32-44); members that the fused kernels
     do not take (more rows, 8 bit, empty) run as separate launches behind the same call."""
     import aq_mi355
-    say("qmv multi", M, bits, Ns)
-    K = 1024
+    say("qmv multi", M, bits, Ns, K)
     x = F.synthetic_x(M, K, seed=333)
     dx = ctx.to_device(x)
     mats = [F.synthetic_affine(max(n, 1), K, bits, 64, seed=340 + i) for i, n in enumerate(Ns)]
@@ -423,7 +509,8 @@ def test_qmv_multi_matches_separate_calls(ctx, orc, M, bits, Ns):
             if f32:
                 check_accumulators(got, ref, "multi member %d" % i)
         if M == 1 and bits == 4 and all(n > 0 for n in Ns):
-            assert fused_name == "qmv_multi_dot2", fused_name
+            # K of 2..4 steps of 1024 codes goes to the diagonal-MFMA kernels, like the single calls
+            assert fused_name == ("qmv_multi_diag" if K >= 2048 else "qmv_multi_dot2"), fused_name
         for t in ys:
             t.free()
     with pytest.raises(aq_mi355.AqError):
