@@ -742,6 +742,38 @@ int aq_qmv_gate_up(aq_ctx* ctx, const void* x, const void* gate_packed, const vo
         !aligned(gate_biases, 2) || !aligned(up_scales, 2) || !aligned(up_biases, 2) || !aligned(y, 2))
         return fail(AQ_ERR_ARG, "aq_qmv_gate_up: operand pointer is not element-aligned");
     const bool out_f32 = (flags & AQ_OUT_F32) != 0;
+    if (M <= 4 && ctx->forced[0] < 0) {
+        // the diagonal-MFMA kernels with one set of wavefronts per matrix
+        const int di = aq::qmvd_pick(1, K);  // the split of K that a single row gets; any row count shares its bytes
+        aq::QmvArgs a{};
+        a.x = static_cast<const uint16_t*>(x);
+        a.w = static_cast<const uint32_t*>(gate_packed);
+        a.s = static_cast<const uint16_t*>(gate_scales);
+        a.b = static_cast<const uint16_t*>(gate_biases);
+        a.w2 = static_cast<const uint32_t*>(up_packed);
+        a.s2 = static_cast<const uint16_t*>(up_scales);
+        a.b2 = static_cast<const uint16_t*>(up_biases);
+        a.y = y;
+        a.K = K;
+        a.N = N;
+        a.M = M;
+        a.gs_shift = is_pow2(group_size) ? ilog2(group_size) : 0;
+        a.out_f32 = out_f32 ? 1 : 0;
+        a.routes = 1;
+        a.act = act;
+        aq::QmvArgs up = a;
+        up.w = a.w2;
+        up.s = a.s2;
+        up.b = a.b2;
+        if (di >= 0 && aq::qmvd_pair_supported(di) && aq::qmvd_fits(a, bits, group_size, false, di) &&
+            aq::qmvd_fits(up, bits, group_size, false, di) &&
+            (size_t)M * K * 2 + (size_t)M * (K / 256) * 48 + 64 + (size_t)2 * aq::qmvd_variant(di)->waves * 256 <= 96 * 1024) {
+            std::lock_guard<std::mutex> lk(ctx->mu);
+            ctx->last_variant[0] = "qmv_gate_up_diag";
+            AQ_HIP(aq::qmvd_pair_launch(di, a, ctx->stream), "hipLaunchKernel");
+            return AQ_OK;
+        }
+    }
     if (M == 1 && ctx->forced[0] < 0 && dot2_eligible(K, group_size, bits, x, gate_packed, (size_t)K * 2) &&
         aligned(up_packed, 16)) {
         std::lock_guard<std::mutex> lk(ctx->mu);

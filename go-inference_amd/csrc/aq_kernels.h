@@ -148,6 +148,10 @@ bool qmvd_fits(const QmvArgs& a, int bits, int group_size, bool gather, int idx)
 hipError_t qmvd_launch(int idx, const QmvArgs& a, hipStream_t stream);
 // The variant the library picks for M rows and this K, or -1 when another family takes the shape.
 int qmvd_pick(int M, int K);
+// y = act(gate . x) * (up . x) with variant idx's split of K (a.w2, a.s2, a.b2: the `up` matrix; a.act); the two
+// dot products are the bytes qmvd_launch computes for each matrix.
+bool qmvd_pair_supported(int idx);
+hipError_t qmvd_pair_launch(int idx, const QmvArgs& a, hipStream_t stream);
 bool qmvd_multi_supported(int idx);
 hipError_t qmvd_multi_launch(int idx, QmvMultiArgs ma, hipStream_t stream);
 

@@ -16,11 +16,19 @@
 //     at the cost of one.  D lands as lane (t, n), register g;
 //   * per 256-code chunk of 16 rows: two 16-byte loads per lane (64 contiguous bytes per row and
 //     instruction), 8 MFMAs, and per lane `acc += scale[g] * D[g]` (four FMAs);
+//   * a wavefront works in steps of 1024 codes (four chunks) and requests everything it will read up front.
+//     The scales and biases of a step are ONE 8-byte load each per lane: lane group j takes the four groups of
+//     chunk j (16 rows x 32 contiguous bytes per instruction; a load per chunk touched as many cache lines as
+//     the weights themselves and cost 2 us on the headline shape).  The lanes that need the scales of chunk c
+//     for the FMAs fetch them from lane group c with ds_bpermute (no vector instruction);
 //   * the affine term needs no vector work either: the group sums X of the activations are split into
-//     three bf16 terms when x is staged (exact: 3 x 8 bits), and one more MFMA per chunk accumulates
-//     bias * X - 128 * scale * X from B = (b, b, b, s, s, s, 0, 0), A = (X0, X1, X2, -128 X0, -128 X1,
-//     -128 X2, 0, 0), every product exact (the codes travel as 128 + code, see aq_device.h);
-//   * the NW wavefronts of a workgroup take the chunks of the same 16 rows in turn and meet in LDS.
+//     three bf16 terms when x is staged (exact: 3 x 8 bits), and three more MFMAs per step accumulate
+//     bias * X - 128 * scale * X over its 16 groups from B = (b, b, b, s, s, s) and A = (X0, X1, X2, -128 X0,
+//     -128 X1, -128 X2) per group, every product exact (the codes travel as 128 + code, see aq_device.h);
+//   * the NW wavefronts of a set take the steps of the same 16 rows in turn and meet in LDS; a workgroup
+//     holds NR sets (more rows per workgroup when more activation rows have to be staged).
+// Every variant of one (NW, steps per wavefront) pair computes the same bytes for a row, whatever NR and
+// whatever the number of activation rows, and so does the multi-matrix launch.
 #include "aq_device.h"
 #include "aq_kernels.h"
 
@@ -64,10 +72,13 @@ __host__ __device__ inline size_t qmvd_lds_bytes_for(int M, int K, int nw) {
     return (size_t)M * K * 2 + (size_t)M * (K / kDiagChunk) * 48 + kDiagZeroBytes + (size_t)nw * 64 * 4;
 }
 
-// NR sets of NW wavefronts (a set per 16 rows), each wavefront takes SUP steps of 1024 codes (steps wave, wave + NW, ...) of the same 16 rows and requests
-// everything it will read up front.
-template <int NW, int SUP, int NR>
+// NR sets of NW wavefronts (a set per 16 rows); each wavefront takes SUP steps of 1024 codes (steps wave,
+// wave + NW, ...) of its set's rows.
+// PAIR (NR = 2): set 0 works on the `gate` matrix (a.w, a.s, a.b), set 1 on the `up` matrix (a.w2, a.s2, a.b2), both
+// on the same 16 rows, and the store is act(gate . x) * (up . x).
+template <int NW, int SUP, int NR, bool PAIR>
 __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block) {
+    static_assert(!PAIR || NR == 2, "the pair kernel runs one set per matrix");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -134,12 +145,13 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     const int j = lane >> 4;   // lane group: which 16 bytes of a 64-byte row piece (B), token (D)
     const int at = (lane & 15) >> 2;  // A operand: token of the lane's A row
     const int ag = lane & 3;          // A operand: group slot of the lane's A row
-    const int row0 = (block * NR + rg) * kDiagRows;
+    const int row0 = (PAIR ? block : block * NR + rg) * kDiagRows;
     int row = row0 + n;
     if (row >= N) row = N - 1;
-    const gptr_t wg = uniform_ptr(a.w);
-    const gptr_t sg = uniform_ptr(a.s);
-    const gptr_t bg = uniform_ptr(a.b);
+    const bool second = PAIR && rg == 1;
+    const gptr_t wg = uniform_ptr(second ? a.w2 : a.w);
+    const gptr_t sg = uniform_ptr(second ? a.s2 : a.s);
+    const gptr_t bg = uniform_ptr(second ? a.b2 : a.b);
     const uint32_t w_lane = (uint32_t)row * (uint32_t)(K >> 1) + (uint32_t)j * 16;  // bytes
     // scales and biases: lane group j holds the four groups of chunk j of the step
     const uint32_t sb_lane = (uint32_t)row * (uint32_t)groups * 2 + (uint32_t)j * 8;  // bytes
@@ -247,10 +259,16 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     float* red = reinterpret_cast<float*>(lds_raw + red_off);
     red[wave_wg * 64 + lane] = acc;
     __syncthreads();
-    if (wave == 0) {
+    if (wave == 0 && !second) {
         float total = red[wave_wg * 64 + lane];
 #pragma unroll
         for (int w2 = 1; w2 < NW; w2++) total += red[(wave_wg + w2) * 64 + lane];
+        if constexpr (PAIR) {
+            float up = red[NW * 64 + lane];
+#pragma unroll
+            for (int w2 = 1; w2 < NW; w2++) up += red[(NW + w2) * 64 + lane];
+            total = fmul_unfused(act_value(a.act, total), up);
+        }
         const int t = j, r = row0 + n;
         if (t < M && r < N) {
             const size_t o = (size_t)t * N + r;
@@ -265,7 +283,12 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
 
 template <int NW, int SUP, int NR>
 __global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_kernel(const QmvArgs a) {
-    qmv_diag_body<NW, SUP, NR>(a, (int)blockIdx.x);
+    qmv_diag_body<NW, SUP, NR, false>(a, (int)blockIdx.x);
+}
+
+template <int NW, int SUP>
+__global__ __launch_bounds__(2 * NW* kWave) void qmv_diag_pair_kernel(const QmvArgs a) {
+    qmv_diag_body<NW, SUP, 2, true>(a, (int)blockIdx.x);
 }
 
 // Several weight matrices against the same activations in one launch (q|k|v, gate|up): the workgroups of all
@@ -282,7 +305,7 @@ __global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_multi_kernel(const Qmv
     a.b = ma.b[set];
     a.y = ma.y[set];
     a.N = ma.N[set];
-    qmv_diag_body<NW, SUP, NR>(a, (int)blockIdx.x - (set ? ma.block_end[set - 1] : 0));
+    qmv_diag_body<NW, SUP, NR, false>(a, (int)blockIdx.x - (set ? ma.block_end[set - 1] : 0));
 }
 
 // ---- variant table --------------------------------------------------------
@@ -362,6 +385,38 @@ int qmvd_pick(int M, int K) {
         if (v.waves == nw && v.depth == 1 && v.rows == nr) return i;
     }
     return -1;
+}
+
+// act(gate . x) * (up . x) with the variant's (wavefronts, steps) split of K; a.w2 / a.s2 / a.b2 are the `up` matrix.
+struct QmvDiagPairEntry {
+    int nw, sup;
+    QmvDiagKernel fn;
+};
+#define AQ_QMVD_PAIR(NW, SUP) {NW, SUP, qmv_diag_pair_kernel<NW, SUP>}
+static const QmvDiagPairEntry kQmvDiagPairTable[] = {
+    AQ_QMVD_PAIR(2, 1), AQ_QMVD_PAIR(4, 1), AQ_QMVD_PAIR(6, 1), AQ_QMVD_PAIR(8, 1),
+};
+static const QmvDiagPairEntry* find_pair(int idx) {
+    const QmvVariant* v = qmvd_variant(idx);
+    if (v)
+        for (const QmvDiagPairEntry& e : kQmvDiagPairTable)
+            if (e.nw == v->waves && e.sup == v->depth) return &e;
+    return nullptr;
+}
+bool qmvd_pair_supported(int idx) { return find_pair(idx) != nullptr; }
+
+hipError_t qmvd_pair_launch(int idx, const QmvArgs& a, hipStream_t stream) {
+    const QmvDiagPairEntry* e = find_pair(idx);
+    if (!e) return hipErrorInvalidValue;
+    const size_t lds = qmvd_lds_bytes_for(a.M, a.K, 2 * e->nw);
+    if (lds > 48 * 1024) {
+        hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e->fn),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (rc != hipSuccess) return rc;
+    }
+    dim3 grid((unsigned)((a.N + kDiagRows - 1) / kDiagRows), 1u, 1u);
+    hipLaunchKernelGGL(e->fn, grid, dim3((unsigned)(2 * e->nw * kWave)), lds, stream, a);
+    return hipGetLastError();
 }
 
 typedef void (*QmvDiagMultiKernel)(const QmvMultiArgs);

@@ -77,7 +77,8 @@ def _run_gate_up(ctx, x, dg, du, M, K, N, gs, bits, act, f32=True):
 @pytest.mark.parametrize("act", ACTS)
 @pytest.mark.parametrize("bits,gs,M,K,N", [(4, 64, 1, 4096, 14336), (4, 64, 1, 2048, 1001), (4, 64, 1, 2816, 1408),
                                            (8, 64, 1, 2560, 640), (4, 32, 1, 512, 40), (4, 128, 1, 1024, 7),
-                                           (8, 32, 1, 256, 3), (4, 64, 1, 14336, 256)])
+                                           (8, 32, 1, 256, 3), (4, 64, 1, 14336, 256), (4, 64, 3, 4096, 203),
+                                           (4, 64, 4, 3072, 48), (4, 64, 1, 8192, 130), (4, 64, 2, 2048, 77)])
 def test_gate_up_single_row(ctx, orc, act, bits, gs, M, K, N):
     say("gate_up", act, bits, gs, M, K, N)
     gw, gsb, gb = F.synthetic_affine(N, K, bits, gs, seed=F.BASE_SEED + 70)
@@ -85,10 +86,18 @@ def test_gate_up_single_row(ctx, orc, act, bits, gs, M, K, N):
     x = F.synthetic_x(M, K, seed=F.BASE_SEED + 72)
     dg, du = DeviceAffine(ctx, gw, gsb, gb), DeviceAffine(ctx, uw, usb, ub)
     got = _run_gate_up(ctx, x, dg, du, M, K, N, gs, bits, act)
-    assert ctx.last_variant(0) == "qmv_gate_up_dot2"
-    with _dot2_family(ctx, bits, False):
+    # 4-bit group-64 codes with K of 2..8 steps of 1024: the diagonal-MFMA pair kernel (up to 4 rows), whose two sums
+    # are those of the library's own choice for a plain call; otherwise the dot2 pair kernel (one row)
+    diag = bits == 4 and gs == 64 and K % 1024 == 0 and 2 <= K // 1024 <= 8
+    assert ctx.last_variant(0) == ("qmv_gate_up_diag" if diag else "qmv_gate_up_dot2")
+    if diag:
         g_gpu = run_qmv(ctx, x, dg, M, K, N, gs, bits, True)
+        assert ctx.last_variant(0).startswith("qmvd_")
         u_gpu = run_qmv(ctx, x, du, M, K, N, gs, bits, True)
+    else:
+        with _dot2_family(ctx, bits, False):
+            g_gpu = run_qmv(ctx, x, dg, M, K, N, gs, bits, True)
+            u_gpu = run_qmv(ctx, x, du, M, K, N, gs, bits, True)
     _check_fused(got, g_gpu, u_gpu, F.reference_f64(x, gw, gsb, gb, bits, gs, K), F.reference_f64(x, uw, usb, ub, bits, gs, K),
                  act, orc, "gate_up")
     out = _run_gate_up(ctx, x, dg, du, M, K, N, gs, bits, act, f32=False)
