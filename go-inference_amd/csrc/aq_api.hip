@@ -180,7 +180,7 @@ int launch_qmv_rows(aq_ctx* ctx, aq::QmvArgs a, int group_size, int bits, bool g
     }
     if (forced < 0 && !gather) {
         // 4-bit group-64 codes, up to 4 rows, K of 2..4 steps of 1024: the diagonal-MFMA kernels
-        const int di = aq::qmvd_pick(M, a.K);
+        const int di = aq::qmvd_pick(M, a.K, a.N);
         if (di >= 0 && aq::qmvd_fits(a, bits, group_size, gather, di)) {
             ctx->last_variant[0] = aq::qmvd_variant(di)->name;
             AQ_HIP(aq::qmvd_launch(di, a, ctx->stream), "hipLaunchKernel");
@@ -510,6 +510,9 @@ int aq_qmv(aq_ctx* ctx, const void* x, const void* packed, const void* scales, c
         // More rows than the dot2 kernels take.  The block-MFMA family streams the weights once per launch of
         // up to 16 rows (4 where K is long); when the call fits one such launch it is the fastest up to 8 rows.
         // Beyond that the matmul tiles with K shared out over workgroups read the weights once for all rows.
+        // (up to 8 rows of 4-bit codes at a K of 2..4 steps of 1024: the diagonal-MFMA kernels, one launch)
+        const int di = aq::qmvd_pick(M, K, N);
+        if (di >= 0 && aq::qmvd_fits(a, bits, group_size, false, di)) return launch_qmv_rows(ctx, a, group_size, bits, false);
         aq::BlkPlan plan;
         aq::QmvArgs probe = a;
         int rows_per_launch = 0;
@@ -561,7 +564,7 @@ int aq_qmv_multi(aq_ctx* ctx, const void* x, int count, const void* const* packe
         if (fused) {
             std::lock_guard<std::mutex> lk(ctx->mu);
             // the kernels aq_qmv would pick for each member, in one grid
-            const int di = aq::qmvd_pick(1, K);
+            const int di = aq::qmvd_pick(1, K, 1 << 20);
             if (di >= 0 && aq::qmvd_multi_supported(di)) {
                 bool fits = true;
                 aq::QmvMultiArgs ma{};
@@ -744,7 +747,7 @@ int aq_qmv_gate_up(aq_ctx* ctx, const void* x, const void* gate_packed, const vo
     const bool out_f32 = (flags & AQ_OUT_F32) != 0;
     if (M <= 4 && ctx->forced[0] < 0) {
         // the diagonal-MFMA kernels with one set of wavefronts per matrix
-        const int di = aq::qmvd_pick(1, K);  // the split of K that a single row gets; any row count shares its bytes
+        const int di = aq::qmvd_pick(1, K, 1 << 20);  // the split of K that a single row gets; any row count shares its bytes
         aq::QmvArgs a{};
         a.x = static_cast<const uint16_t*>(x);
         a.w = static_cast<const uint32_t*>(gate_packed);

@@ -141,13 +141,13 @@ const QmvVariant* qmvs_variant(int idx);
 bool qmvs_plan(const QmvArgs& a, int bits, int group_size, bool gather, int cu_count, int forced_idx, StreamPlan* out);
 hipError_t qmvs_launch(const StreamPlan& p, const QmvArgs& a, hipStream_t stream);
 
-// Diagonal-MFMA matvec kernels (aq_qmv_diag.hip; 4-bit group-64 codes, M <= 4, K a multiple of 256).
+// Diagonal-MFMA matvec kernels (aq_qmv_diag.hip; 4-bit group-64 codes, M <= 8, K a multiple of 1024).
 int qmvd_variant_count();
 const QmvVariant* qmvd_variant(int idx);
 bool qmvd_fits(const QmvArgs& a, int bits, int group_size, bool gather, int idx);
 hipError_t qmvd_launch(int idx, const QmvArgs& a, hipStream_t stream);
 // The variant the library picks for M rows and this K, or -1 when another family takes the shape.
-int qmvd_pick(int M, int K);
+int qmvd_pick(int M, int K, int N);
 // y = act(gate . x) * (up . x) with variant idx's split of K (a.w2, a.s2, a.b2: the `up` matrix; a.act); the two
 // dot products are the bytes qmvd_launch computes for each matrix.
 bool qmvd_pair_supported(int idx);

@@ -67,16 +67,18 @@ constexpr int kDiagSuper = 1024;   // codes of a row per wavefront step (four ch
 constexpr int kDiagZeroBytes = 64;
 
 // LDS: activations in expansion order [M][K] bf16, the split group sums [M][K/1024][4] x 48 B, 64 zero bytes,
-// the partial sums of the wavefronts [NW][64] fp32.
-__host__ __device__ inline size_t qmvd_lds_bytes_for(int M, int K, int nw) {
-    return (size_t)M * K * 2 + (size_t)M * (K / kDiagChunk) * 48 + kDiagZeroBytes + (size_t)nw * 64 * 4;
+// the partial sums of the wavefronts [NW][sets of four activation rows][64] fp32.
+__host__ __device__ inline size_t qmvd_lds_bytes_for(int M, int K, int nw, int mt = 1) {
+    return (size_t)M * K * 2 + (size_t)M * (K / kDiagChunk) * 48 + kDiagZeroBytes + (size_t)nw * mt * 64 * 4;
 }
 
 // NR sets of NW wavefronts (a set per 16 rows); each wavefront takes SUP steps of 1024 codes (steps wave,
 // wave + NW, ...) of its set's rows.
 // PAIR (NR = 2): set 0 works on the `gate` matrix (a.w, a.s, a.b), set 1 on the `up` matrix (a.w2, a.s2, a.b2), both
 // on the same 16 rows, and the store is act(gate . x) * (up . x).
-template <int NW, int SUP, int NR, bool PAIR>
+// MT: sets of four activation rows (the 16 rows of A hold four tokens; a second set reuses the expanded codes with
+// eight more MFMAs per chunk).
+template <int NW, int SUP, int NR, bool PAIR, int MT = 1>
 __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block) {
     static_assert(!PAIR || NR == 2, "the pair kernel runs one set per matrix");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
@@ -158,16 +160,25 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
 
     // A fragments: load L (0, 1) of a chunk holds groups 2L and 2L + 1; lane group j holds codes of group
     // 2L + (j >> 1).  The lane's A row (at, ag) is non-zero in load L iff ag == 2L + (j >> 1).
-    const bool tok = at < M;
-    const bool d0 = tok && ag == (j >> 1);
-    const bool d1 = tok && ag == 2 + (j >> 1);
-    const uint32_t x_lane = xs_off + (uint32_t)at * K * 2 + (uint32_t)j * 64;  // codes j*32.. of a 128-code load
-    const uint32_t a_base0 = d0 ? x_lane : zero_off, a_base1 = d1 ? x_lane + 256 : zero_off;
-    const uint32_t a_mul0 = d0 ? 2048 : 0, a_mul1 = d1 ? 2048 : 0, a_chunk0 = d0 ? 512 : 0, a_chunk1 = d1 ? 512 : 0;
     // affine-term A: rows (t, 0) carry the split sums of the four groups of chunk j of the step, 48 bytes
-    const bool d2 = tok && ag == 0;
-    const uint32_t a2_base = d2 ? a2_off + ((uint32_t)at * (K / kDiagChunk) + j) * 48 : zero_off;
-    const uint32_t a2_mul = d2 ? 4 * 48 : 0;
+    uint32_t a_base0[MT], a_base1[MT], a_mul0[MT], a_mul1[MT], a_chunk0[MT], a_chunk1[MT], a2_base[MT], a2_mul[MT];
+#pragma unroll
+    for (int tg = 0; tg < MT; tg++) {
+        const int token = tg * 4 + at;
+        const bool tok = token < M;
+        const bool d0 = tok && ag == (j >> 1);
+        const bool d1 = tok && ag == 2 + (j >> 1);
+        const uint32_t x_lane = xs_off + (uint32_t)token * K * 2 + (uint32_t)j * 64;  // codes j*32.. of a 128-code load
+        a_base0[tg] = d0 ? x_lane : zero_off;
+        a_base1[tg] = d1 ? x_lane + 256 : zero_off;
+        a_mul0[tg] = d0 ? 2048 : 0;
+        a_mul1[tg] = d1 ? 2048 : 0;
+        a_chunk0[tg] = d0 ? 512 : 0;
+        a_chunk1[tg] = d1 ? 512 : 0;
+        const bool d2 = tok && ag == 0;
+        a2_base[tg] = d2 ? a2_off + ((uint32_t)token * (K / kDiagChunk) + j) * 48 : zero_off;
+        a2_mul[tg] = d2 ? 4 * 48 : 0;
+    }
     // the lane that holds the scales of chunk 0 of the step for this lane's row (ds_bpermute byte address)
     const int sc_addr = n * 4;
 
@@ -198,8 +209,13 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     for (int p = tid + PRE * NR * NW * kWave; p < pieces; p += NR * NW * kWave) stage(p, load_u128_at(xg, (uint32_t)p * 16));
     __syncthreads();  // x, sums and zeros are in LDS
 
-    float acc = 0.0f;
-    f32x4_t dsum = {0.0f, 0.0f, 0.0f, 0.0f};  // affine term, register 0 is the one that is used
+    float acc[MT];
+    f32x4_t dsum[MT];  // affine term, register 0 is the one that is used
+#pragma unroll
+    for (int tg = 0; tg < MT; tg++) {
+        acc[tg] = 0.0f;
+        dsum[tg] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    }
 #pragma unroll
     for (int u = 0; u < SUP; u++) {
         const int sp = wave + u * NW;
@@ -207,10 +223,6 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
             const uint2 sv = sq[u], bv = bq[u];
             // affine term of the 16 groups of the step: 24 k-slots per lane, three MFMAs
             {
-                const uint32_t a2_addr = a2_base + (uint32_t)sp * a2_mul;
-                const bf16x8_t a20 = *reinterpret_cast<const bf16x8_t*>(lds_raw + a2_addr);
-                const bf16x8_t a21 = *reinterpret_cast<const bf16x8_t*>(lds_raw + a2_addr + 16);
-                const bf16x8_t a22 = *reinterpret_cast<const bf16x8_t*>(lds_raw + a2_addr + 32);
                 // (b0 b0 b0 s0 s0 s0 b1 b1 | b1 s1 s1 s1 b2 b2 b2 s2 | s2 s2 b3 b3 b3 s3 s3 s3)
                 const uint32_t lo2 = 0x01000100u, hi2 = 0x03020302u, lolo = 0x05040100u, hihi = 0x07060302u;
                 const uint32_t e0 = __builtin_amdgcn_perm(bv.x, bv.x, lo2), e1 = __builtin_amdgcn_perm(sv.x, bv.x, lolo);
@@ -219,23 +231,40 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
                 const uint32_t e6 = __builtin_amdgcn_perm(bv.y, bv.y, lo2), e7 = __builtin_amdgcn_perm(sv.y, bv.y, lolo);
                 const uint32_t e8 = __builtin_amdgcn_perm(sv.y, sv.y, lo2), e9 = __builtin_amdgcn_perm(bv.y, bv.y, hi2);
                 const uint32_t e10 = __builtin_amdgcn_perm(sv.y, bv.y, hihi), e11 = __builtin_amdgcn_perm(sv.y, sv.y, hi2);
-                dsum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a20, as_bf16x8(e0, e1, e2, e3), dsum, 0, 0, 0);
-                dsum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a21, as_bf16x8(e4, e5, e6, e7), dsum, 0, 0, 0);
-                dsum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a22, as_bf16x8(e8, e9, e10, e11), dsum, 0, 0, 0);
+#pragma unroll
+                for (int tg = 0; tg < MT; tg++) {
+                    const uint32_t a2_addr = a2_base[tg] + (uint32_t)sp * a2_mul[tg];
+                    const bf16x8_t a20 = *reinterpret_cast<const bf16x8_t*>(lds_raw + a2_addr);
+                    const bf16x8_t a21 = *reinterpret_cast<const bf16x8_t*>(lds_raw + a2_addr + 16);
+                    const bf16x8_t a22 = *reinterpret_cast<const bf16x8_t*>(lds_raw + a2_addr + 32);
+                    dsum[tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a20, as_bf16x8(e0, e1, e2, e3), dsum[tg], 0, 0, 0);
+                    dsum[tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a21, as_bf16x8(e4, e5, e6, e7), dsum[tg], 0, 0, 0);
+                    dsum[tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a22, as_bf16x8(e8, e9, e10, e11), dsum[tg], 0, 0, 0);
+                }
             }
-            const uint32_t a_addr0 = a_base0 + (uint32_t)sp * a_mul0, a_addr1 = a_base1 + (uint32_t)sp * a_mul1;
+            uint32_t a_addr0[MT], a_addr1[MT];
+#pragma unroll
+            for (int tg = 0; tg < MT; tg++) {
+                a_addr0[tg] = a_base0[tg] + (uint32_t)sp * a_mul0[tg];
+                a_addr1[tg] = a_base1[tg] + (uint32_t)sp * a_mul1[tg];
+            }
 #pragma unroll
             for (int cc = 0; cc < 4; cc++) {
-                bf16x8_t af[2][4];
+                bf16x8_t af[MT][2][4];
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    af[0][i] = *reinterpret_cast<const bf16x8_t*>(lds_raw + a_addr0 + cc * a_chunk0 + i * 16);
-                    af[1][i] = *reinterpret_cast<const bf16x8_t*>(lds_raw + a_addr1 + cc * a_chunk1 + i * 16);
+                for (int tg = 0; tg < MT; tg++) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        af[tg][0][i] = *reinterpret_cast<const bf16x8_t*>(lds_raw + a_addr0[tg] + cc * a_chunk0[tg] + i * 16);
+                        af[tg][1][i] = *reinterpret_cast<const bf16x8_t*>(lds_raw + a_addr1[tg] + cc * a_chunk1[tg] + i * 16);
+                    }
                 }
                 // the four scales of chunk cc of this lane's row sit in lane group cc
                 const uint32_t sx = (uint32_t)__builtin_amdgcn_ds_bpermute(sc_addr + cc * 64, (int)sv.x);
                 const uint32_t sy = (uint32_t)__builtin_amdgcn_ds_bpermute(sc_addr + cc * 64, (int)sv.y);
-                f32x4_t dq = {0.0f, 0.0f, 0.0f, 0.0f};
+                f32x4_t dq[MT];
+#pragma unroll
+                for (int tg = 0; tg < MT; tg++) dq[tg] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                 for (int L = 0; L < 2; L++) {
                     const uint32_t ww[4] = {wq[u][cc][L].x, wq[u][cc][L].y, wq[u][cc][L].z, wq[u][cc][L].w};
@@ -243,47 +272,60 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
                     for (int i = 0; i < 4; i++) {
                         uint32_t p[4];
                         unpack4_word(ww[i], mask, magic, p);
-                        dq = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[L][i], as_bf16x8(p[0], p[1], p[2], p[3]), dq, 0, 0, 0);
+                        const bf16x8_t bfrag = as_bf16x8(p[0], p[1], p[2], p[3]);
+#pragma unroll
+                        for (int tg = 0; tg < MT; tg++)
+                            dq[tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[tg][L][i], bfrag, dq[tg], 0, 0, 0);
                     }
                 }
-                acc = __builtin_fmaf(bf16_bits_to_f32(sx & 0xffffu), dq[0], acc);
-                acc = __builtin_fmaf(__uint_as_float(sx & 0xffff0000u), dq[1], acc);
-                acc = __builtin_fmaf(bf16_bits_to_f32(sy & 0xffffu), dq[2], acc);
-                acc = __builtin_fmaf(__uint_as_float(sy & 0xffff0000u), dq[3], acc);
+                const float s0 = bf16_bits_to_f32(sx & 0xffffu), s1 = __uint_as_float(sx & 0xffff0000u);
+                const float s2 = bf16_bits_to_f32(sy & 0xffffu), s3 = __uint_as_float(sy & 0xffff0000u);
+#pragma unroll
+                for (int tg = 0; tg < MT; tg++) {
+                    acc[tg] = __builtin_fmaf(s0, dq[tg][0], acc[tg]);
+                    acc[tg] = __builtin_fmaf(s1, dq[tg][1], acc[tg]);
+                    acc[tg] = __builtin_fmaf(s2, dq[tg][2], acc[tg]);
+                    acc[tg] = __builtin_fmaf(s3, dq[tg][3], acc[tg]);
+                }
             }
         }
     }
-    acc += dsum[0];
+#pragma unroll
+    for (int tg = 0; tg < MT; tg++) acc[tg] += dsum[tg][0];
 
-    // ---- the wavefronts' partial sums meet in LDS; lane (t, n) of wavefront 0 stores ----
+    // ---- the wavefronts' partial sums meet in LDS; lane (t, n) of the first wavefront of a set stores ----
     float* red = reinterpret_cast<float*>(lds_raw + red_off);
-    red[wave_wg * 64 + lane] = acc;
+#pragma unroll
+    for (int tg = 0; tg < MT; tg++) red[(wave_wg * MT + tg) * 64 + lane] = acc[tg];
     __syncthreads();
     if (wave == 0 && !second) {
-        float total = red[wave_wg * 64 + lane];
 #pragma unroll
-        for (int w2 = 1; w2 < NW; w2++) total += red[(wave_wg + w2) * 64 + lane];
-        if constexpr (PAIR) {
-            float up = red[NW * 64 + lane];
+        for (int tg = 0; tg < MT; tg++) {
+            float total = red[(wave_wg * MT + tg) * 64 + lane];
 #pragma unroll
-            for (int w2 = 1; w2 < NW; w2++) up += red[(NW + w2) * 64 + lane];
-            total = fmul_unfused(act_value(a.act, total), up);
-        }
-        const int t = j, r = row0 + n;
-        if (t < M && r < N) {
-            const size_t o = (size_t)t * N + r;
-            if (a.out_f32) {
-                static_cast<float*>(a.y)[o] = total;
-            } else {
-                static_cast<uint16_t*>(a.y)[o] = f32_to_bf16_bits(total);
+            for (int w2 = 1; w2 < NW; w2++) total += red[((wave_wg + w2) * MT + tg) * 64 + lane];
+            if constexpr (PAIR) {
+                float up = red[(NW * MT + tg) * 64 + lane];
+#pragma unroll
+                for (int w2 = 1; w2 < NW; w2++) up += red[((NW + w2) * MT + tg) * 64 + lane];
+                total = fmul_unfused(act_value(a.act, total), up);
+            }
+            const int t = tg * 4 + j, r = row0 + n;
+            if (t < M && r < N) {
+                const size_t o = (size_t)t * N + r;
+                if (a.out_f32) {
+                    static_cast<float*>(a.y)[o] = total;
+                } else {
+                    static_cast<uint16_t*>(a.y)[o] = f32_to_bf16_bits(total);
+                }
             }
         }
     }
 }
 
-template <int NW, int SUP, int NR>
+template <int NW, int SUP, int NR, int MT>
 __global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_kernel(const QmvArgs a) {
-    qmv_diag_body<NW, SUP, NR, false>(a, (int)blockIdx.x);
+    qmv_diag_body<NW, SUP, NR, false, MT>(a, (int)blockIdx.x);
 }
 
 template <int NW, int SUP>
@@ -317,14 +359,18 @@ struct QmvDiagEntry {
 };
 // name, bits, m (most rows), sets of 16 rows per workgroup, wavefronts per set, steps per wavefront, gather, xmode, kind
 // waves x depth steps of 1024 codes cover K
-#define AQ_QMVD(NW, SUP, NR)                                                                              \
-    {                                                                                                     \
-        {"qmvd_b4_m4_r" #NR "_w" #NW "_d" #SUP "_g0", 4, 4, NR, NW, SUP, 0, 0, 4}, qmv_diag_kernel<NW, SUP, NR> \
+#define AQ_QMVD(NW, SUP, NR)                                                                                 \
+    {                                                                                                        \
+        {"qmvd_b4_m4_r" #NR "_w" #NW "_d" #SUP "_g0", 4, 4, NR, NW, SUP, 0, 0, 4}, qmv_diag_kernel<NW, SUP, NR, 1> \
+    }
+#define AQ_QMVD8(NW, SUP, NR)                                                                                \
+    {                                                                                                        \
+        {"qmvd_b4_m8_r" #NR "_w" #NW "_d" #SUP "_g0", 4, 8, NR, NW, SUP, 0, 0, 4}, qmv_diag_kernel<NW, SUP, NR, 2> \
     }
 static const QmvDiagEntry kQmvDiagTable[] = {
     AQ_QMVD(4, 1, 1), AQ_QMVD(4, 1, 2), AQ_QMVD(4, 1, 4), AQ_QMVD(2, 2, 2), AQ_QMVD(2, 1, 2), AQ_QMVD(8, 1, 1),
     AQ_QMVD(4, 2, 1), AQ_QMVD(2, 1, 4), AQ_QMVD(6, 1, 1), AQ_QMVD(10, 1, 1), AQ_QMVD(12, 1, 1),
-    AQ_QMVD(14, 1, 1), AQ_QMVD(16, 1, 1),
+    AQ_QMVD(14, 1, 1), AQ_QMVD(16, 1, 1), AQ_QMVD8(4, 1, 4), AQ_QMVD8(4, 1, 2), AQ_QMVD8(2, 1, 4),
 };
 
 int qmvd_variant_count() { return (int)(sizeof(kQmvDiagTable) / sizeof(kQmvDiagTable[0])); }
@@ -336,20 +382,20 @@ const QmvVariant* qmvd_variant(int idx) {
 bool qmvd_fits(const QmvArgs& a, int bits, int group_size, bool gather, int idx) {
     const QmvVariant* v = qmvd_variant(idx);
     if (!v || bits != 4 || group_size != 64 || gather) return false;
-    if (a.M < 1 || a.M > 4 || a.K <= 0 || a.K % kDiagSuper != 0 || a.N < 1) return false;
+    if (a.M < 1 || a.M > v->m || a.K <= 0 || a.K % kDiagSuper != 0 || a.N < 1) return false;
     if (a.K / kDiagSuper > v->waves * v->depth) return false;
     const uintptr_t al16 = reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.w);
     const uintptr_t al8 = reinterpret_cast<uintptr_t>(a.s) | reinterpret_cast<uintptr_t>(a.b);
     if ((al16 & 15) || (al8 & 7)) return false;
     // 32-bit byte offsets into the packed matrix
     if ((uint64_t)a.N * (uint64_t)(a.K / 2) >= (1ull << 32)) return false;
-    return qmvd_lds_bytes_for(a.M, a.K, v->waves * v->rows) <= 96 * 1024;
+    return qmvd_lds_bytes_for(a.M, a.K, v->waves * v->rows, v->m / 4) <= 96 * 1024;
 }
 
 hipError_t qmvd_launch(int idx, const QmvArgs& a, hipStream_t stream) {
     if (idx < 0 || idx >= qmvd_variant_count()) return hipErrorInvalidValue;
     const QmvDiagEntry& e = kQmvDiagTable[idx];
-    const size_t lds = qmvd_lds_bytes_for(a.M, a.K, e.v.waves * e.v.rows);
+    const size_t lds = qmvd_lds_bytes_for(a.M, a.K, e.v.waves * e.v.rows, e.v.m / 4);
     if (lds > 48 * 1024) {
         hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e.fn),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -363,9 +409,10 @@ hipError_t qmvd_launch(int idx, const QmvArgs& a, hipStream_t stream) {
 
 // The variant the library picks for M rows and this K, or -1: one step of 1024 codes per wavefront; up to 4 steps,
 // more rows per workgroup the more activation rows there are to stage.
-int qmvd_pick(int M, int K) {
-    if (M < 1 || M > 4 || K <= 0 || K % kDiagSuper != 0) return -1;
+int qmvd_pick(int M, int K, int N) {
+    if (M < 1 || M > 8 || K <= 0 || K % kDiagSuper != 0) return -1;
     const int steps = K / kDiagSuper;
+    const int cap = M <= 4 ? 4 : 8;
     int nw, nr;
     if (steps == 2) {
         nw = 2;
@@ -380,9 +427,13 @@ int qmvd_pick(int M, int K) {
     } else {
         return -1;
     }
+    // fewer rows per workgroup while that leaves under 128 workgroups (the 8-row kernels exist for 2 and 4 sets)
+    const int min_nr = (cap == 8 || nw == 2) ? 2 : 1;
+    while (nr > min_nr && (N + kDiagRows * nr - 1) / (kDiagRows * nr) < 128) nr >>= 1;
+    if (cap == 8 && nw == 2) nr = 4;
     for (int i = 0; i < qmvd_variant_count(); i++) {
         const QmvVariant& v = kQmvDiagTable[i].v;
-        if (v.waves == nw && v.depth == 1 && v.rows == nr) return i;
+        if (v.waves == nw && v.depth == 1 && v.rows == nr && v.m == cap) return i;
     }
     return -1;
 }

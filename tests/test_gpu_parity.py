@@ -334,7 +334,7 @@ def test_qmvs_every_variant(ctx, orc):
 
 
 def test_qmvd_every_variant(ctx, orc):
-    """Each diagonal-MFMA matvec variant, forced: 1..4 activation rows, K = all the steps of 1024 codes its
+    """Each diagonal-MFMA matvec variant, forced: 1..4 (1..8) activation rows, K = all the steps of 1024 codes its
     wavefronts take and one step fewer (an idle wavefront), ragged N; fp32 and bf16 stores; a K that is no multiple
     of 1024, or more steps than the variant takes, is refused."""
     import aq_mi355
@@ -353,12 +353,12 @@ def test_qmvd_every_variant(ctx, orc):
                 say("variant", idx, name, "K", K)
                 if K not in data:
                     words, s, b = F.synthetic_affine(N, K, bits, 64, seed=530 + K // 1024)
-                    x = F.synthetic_x(4, K, seed=630 + K // 1024)
+                    x = F.synthetic_x(8, K, seed=630 + K // 1024)
                     data[K] = (DeviceAffine(ctx, words, s, b), x, F.reference_f64(x, words, s, b, bits, 64, K))
                 dw, x, ref = data[K]
                 ctx.force_variant(0, idx)
-                for rows in (1, 2, 3, 4):
-                    if rows * K * 2 + rows * (K // 256) * 48 + 64 + wg_waves * 256 > 96 * 1024:
+                for rows in ((1, 2, 3, 4) if m == 4 else (1, 4, 5, 7, 8)):
+                    if rows * K * 2 + rows * (K // 256) * 48 + 64 + wg_waves * (m // 4) * 256 > 96 * 1024:
                         # the activations of all rows and their group sums sit in LDS: beyond 96 KiB the variant refuses
                         with pytest.raises(aq_mi355.AqError) as ei:
                             run_qmv(ctx, x[:rows], dw, rows, K, N, 64, bits, True)
@@ -381,15 +381,15 @@ def test_qmvd_every_variant(ctx, orc):
 
 
 def test_qmvd_is_the_default_for_few_rows(ctx, orc):
-    """4-bit group-64 codes: 1..4 activation rows with K of 2, 3 or 4 steps of 1024 codes, and one row with up to 16
+    """4-bit group-64 codes: 1..8 activation rows with K of 2, 3 or 4 steps of 1024 codes, and one row with up to 16
     steps, land on the diagonal-MFMA kernels without forcing, rows beyond the last full 16 included; other K, more
     rows at a long K, and 8 bit do not."""
     for K, N in ((4096, 16 * 9 + 5), (3072, 64), (2048, 33)):
         words, s, b = F.synthetic_affine(N, K, 4, 64, seed=810 + K // 1024)
-        x = F.synthetic_x(4, K, seed=820 + K // 1024)
+        x = F.synthetic_x(8, K, seed=820 + K // 1024)
         ref = F.reference_f64(x, words, s, b, 4, 64, K)
         dw = DeviceAffine(ctx, words, s, b)
-        for rows in (1, 2, 3, 4):
+        for rows in (1, 2, 3, 4, 5, 8):
             say("default few rows", K, N, rows)
             acc = run_qmv(ctx, x[:rows], dw, rows, K, N, 64, 4, True)
             assert ctx.last_variant(0).startswith("qmvd_"), ctx.last_variant(0)
