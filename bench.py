@@ -113,6 +113,9 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--stream-launches", action="store_true",
+                    help="time stream launches instead of graph replays (for runs under rocprofv3, whose kernel trace "
+                         "does not survive stream capture; its per-dispatch durations are what such a run is for)")
     ap.add_argument("--no-qmm", action="store_true", help="skip the prefill qmm extra")
     ap.add_argument("--no-extras", action="store_true", help="skip the small-M and MoE gather extras")
     ap.add_argument("--probe", choices=["dominant", "qmm"], help="run only the named kernel a few times, preceded by two "
@@ -198,6 +201,12 @@ def main():
         replays after an untimed one).  A launch from this Python harness costs the host about as much time as the
         kernel runs, so stream launches measure the harness as soon as a kernel gets faster than that; a replay
         measures the GPU, and is how a decode loop would issue these launches."""
+        if args.stream_launches:
+            ctx.sync()
+            ctx.timer_start()
+            for i in range(reps):
+                launch(i)
+            return ctx.timer_stop() / reps
         ctx.capture_begin()
         for i in range(reps):
             launch(i)
