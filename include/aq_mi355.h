@@ -163,7 +163,8 @@ int aq_gather_qmv(aq_ctx *ctx, const void *x, const void *packed, const void *sc
  * launch go/engine/hip/hip_projection_launch.go:3086-3160, packet contract/launch_abi.hipinc:634-657).
  * gate and up are [N, K*bits/32] with their own scales/biases; for a row-concatenated gate|up slab
  * (model.ConcatQuantRows, go/model/quant_weight.go:32-62) pass the slab for gate and slab + N rows for up.
- * M == 1 with 4/8-bit codes runs as ONE launch that reads every weight once; other shapes run the two
+ * M == 1 with 4/8-bit codes (up to 4 rows of 4-bit group-64 codes when K is 2..8 times 1024) runs as ONE launch
+ * that reads every weight once; other shapes run the two
  * projections and the element-wise step as separate launches through the context's workspace (which grows
  * on demand like aq_qmm's; not while a capture is open). */
 int aq_qmv_gate_up(aq_ctx *ctx, const void *x, const void *gate_packed, const void *gate_scales,
@@ -309,7 +310,7 @@ int aq_proj_quant_matmul_host(aq_ctx *ctx, float *out, const float *x, size_t x_
                               size_t biases_len, int M, int K, int N, int group_size, int bits);
 
 /* Kernel-variant introspection and override, for tuning sweeps and profiles.
- * op: 0 = qmv/gather (dot2 kernels), 1 = qmm (MFMA kernels).  variant -1 restores automatic
+ * op: 0 = qmv/gather (matvec kernel families), 1 = qmm (matmul kernel families).  variant -1 restores automatic
  * selection (the counterpart of the reference's shape->kernel selector tables,
  * go/engine/hip/hip_projection_launch.go:4925-5064 and its GO_ROCM_* route switches :107-137). */
 int aq_variant_count(int op);
