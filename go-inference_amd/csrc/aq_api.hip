@@ -179,7 +179,7 @@ int launch_qmv_rows(aq_ctx* ctx, aq::QmvArgs a, int group_size, int bits, bool g
         return AQ_OK;
     }
     if (forced < 0 && !gather) {
-        // 4-bit group-64 codes, up to 4 rows, K of 2..4 steps of 1024: the diagonal-MFMA kernels
+        // 4-bit group-64 codes: up to 8 rows at a K of 2..4 steps of 1024 codes, one row up to 16 steps: the diagonal-MFMA kernels
         const int di = aq::qmvd_pick(M, a.K, a.N);
         if (di >= 0 && aq::qmvd_fits(a, bits, group_size, gather, di)) {
             ctx->last_variant[0] = aq::qmvd_variant(di)->name;

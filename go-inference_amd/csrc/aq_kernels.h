@@ -141,7 +141,7 @@ const QmvVariant* qmvs_variant(int idx);
 bool qmvs_plan(const QmvArgs& a, int bits, int group_size, bool gather, int cu_count, int forced_idx, StreamPlan* out);
 hipError_t qmvs_launch(const StreamPlan& p, const QmvArgs& a, hipStream_t stream);
 
-// Diagonal-MFMA matvec kernels (aq_qmv_diag.hip; 4-bit group-64 codes, M <= 8, K a multiple of 1024).
+// Diagonal-MFMA matvec kernels (aq_qmv_diag.hip; 4-bit group-64 codes, M <= 8, K a multiple of 256 in 2..16 steps of 1024).
 int qmvd_variant_count();
 const QmvVariant* qmvd_variant(int idx);
 bool qmvd_fits(const QmvArgs& a, int bits, int group_size, bool gather, int idx);

@@ -16,7 +16,8 @@
 //     at the cost of one.  D lands as lane (t, n), register g;
 //   * per 256-code chunk of 16 rows: two 16-byte loads per lane (64 contiguous bytes per row and
 //     instruction), 8 MFMAs, and per lane `acc += scale[g] * D[g]` (four FMAs);
-//   * a wavefront works in steps of 1024 codes (four chunks) and requests everything it will read up front.
+//   * a wavefront works in steps of 1024 codes (four chunks; the last step of a row may hold fewer) and requests
+//     everything it will read up front.
 //     The scales and biases of a step are ONE 8-byte load each per lane: lane group j takes the four groups of
 //     chunk j (16 rows x 32 contiguous bytes per instruction; a load per chunk touched as many cache lines as
 //     the weights themselves and cost 2 us on the headline shape).  The lanes that need the scales of chunk c
@@ -89,7 +90,8 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     const int rg = wave_wg / NW;    // which 16 rows of the workgroup's NR x 16
     const int K = a.K, N = a.N, M = a.M;
     const int groups = K >> 6;
-    const int supers = K / kDiagSuper;
+    const int chunks = K / kDiagChunk;
+    const int supers = (chunks + 3) >> 2;  // the last step may hold fewer than four chunks
     const uint32_t xs_off = 0;
     const uint32_t a2_off = (uint32_t)M * K * 2;
     const uint32_t zero_off = a2_off + (uint32_t)M * (K / kDiagChunk) * 48;
@@ -97,7 +99,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
 
     // ---- stage x: expansion order within every 8 values, group sums split into three bf16 terms ----
     const gptr_t xg = uniform_ptr(a.x);
-    const int pieces = M * (K >> 3);  // 16-byte pieces of all tokens (K % 1024 == 0: a token is whole pieces)
+    const int pieces = M * (K >> 3);  // 16-byte pieces of all tokens (K % 256 == 0: a token is whole pieces)
     auto stage = [&](int p, const uint4 v) {
         uint4 o;
         o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);  // (x0, x4)
@@ -191,14 +193,17 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     for (int u = 0; u < SUP; u++) {
         int sp = wave + u * NW;
         if (sp >= supers) sp = supers - 1;  // past the end: a valid address, the result is not used
+        const int valid = min(4, chunks - 4 * sp);  // chunks of this step; the others re-read chunk 0 and are not used
         const uint32_t wo = w_lane + (uint32_t)sp * 512;
 #pragma unroll
         for (int cc = 0; cc < 4; cc++) {
-            wq[u][cc][0] = load_u128_at(wg, wo + cc * 128);
-            wq[u][cc][1] = load_u128_at(wg, wo + cc * 128 + 64);
+            const uint32_t co = cc < valid ? cc * 128 : 0;
+            wq[u][cc][0] = load_u128_at(wg, wo + co);
+            wq[u][cc][1] = load_u128_at(wg, wo + co + 64);
         }
-        sq[u] = load_u64_at(sg, sb_lane + (uint32_t)sp * 32);
-        bq[u] = load_u64_at(bg, sb_lane + (uint32_t)sp * 32);
+        const uint32_t so = sb_lane + (uint32_t)sp * 32 - (j < valid ? 0u : (uint32_t)j * 8);
+        sq[u] = load_u64_at(sg, so);
+        bq[u] = load_u64_at(bg, so);
     }
 
 #pragma unroll
@@ -220,6 +225,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     for (int u = 0; u < SUP; u++) {
         const int sp = wave + u * NW;
         if (sp < supers) {
+            const int valid = min(4, chunks - 4 * sp);
             const uint2 sv = sq[u], bv = bq[u];
             // affine term of the 16 groups of the step: 24 k-slots per lane, three MFMAs
             {
@@ -233,7 +239,8 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
                 const uint32_t e10 = __builtin_amdgcn_perm(sv.y, bv.y, hihi), e11 = __builtin_amdgcn_perm(sv.y, sv.y, hi2);
 #pragma unroll
                 for (int tg = 0; tg < MT; tg++) {
-                    const uint32_t a2_addr = a2_base[tg] + (uint32_t)sp * a2_mul[tg];
+                    // (lane groups past the last chunk of the row contribute zeros)
+                    const uint32_t a2_addr = j < valid ? a2_base[tg] + (uint32_t)sp * a2_mul[tg] : zero_off;
                     const bf16x8_t a20 = *reinterpret_cast<const bf16x8_t*>(lds_raw + a2_addr);
                     const bf16x8_t a21 = *reinterpret_cast<const bf16x8_t*>(lds_raw + a2_addr + 16);
                     const bf16x8_t a22 = *reinterpret_cast<const bf16x8_t*>(lds_raw + a2_addr + 32);
@@ -250,6 +257,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
             }
 #pragma unroll
             for (int cc = 0; cc < 4; cc++) {
+                if (cc >= valid) break;
                 bf16x8_t af[MT][2][4];
 #pragma unroll
                 for (int tg = 0; tg < MT; tg++) {
@@ -382,8 +390,8 @@ const QmvVariant* qmvd_variant(int idx) {
 bool qmvd_fits(const QmvArgs& a, int bits, int group_size, bool gather, int idx) {
     const QmvVariant* v = qmvd_variant(idx);
     if (!v || bits != 4 || group_size != 64 || gather) return false;
-    if (a.M < 1 || a.M > v->m || a.K <= 0 || a.K % kDiagSuper != 0 || a.N < 1) return false;
-    if (a.K / kDiagSuper > v->waves * v->depth) return false;
+    if (a.M < 1 || a.M > v->m || a.K <= 0 || a.K % kDiagChunk != 0 || a.N < 1) return false;
+    if ((a.K + kDiagSuper - 1) / kDiagSuper > v->waves * v->depth) return false;
     const uintptr_t al16 = reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.w);
     const uintptr_t al8 = reinterpret_cast<uintptr_t>(a.s) | reinterpret_cast<uintptr_t>(a.b);
     if ((al16 & 15) || (al8 & 7)) return false;
@@ -410,8 +418,8 @@ hipError_t qmvd_launch(int idx, const QmvArgs& a, hipStream_t stream) {
 // The variant the library picks for M rows and this K, or -1: one step of 1024 codes per wavefront; up to 4 steps,
 // more rows per workgroup the more activation rows there are to stage.
 int qmvd_pick(int M, int K, int N) {
-    if (M < 1 || M > 8 || K <= 0 || K % kDiagSuper != 0) return -1;
-    const int steps = K / kDiagSuper;
+    if (M < 1 || M > 8 || K <= 0 || K % kDiagChunk != 0) return -1;
+    const int steps = (K + kDiagSuper - 1) / kDiagSuper;
     const int cap = M <= 4 ? 4 : 8;
     int nw, nr;
     if (steps == 2) {

@@ -163,7 +163,7 @@ int aq_gather_qmv(aq_ctx *ctx, const void *x, const void *packed, const void *sc
  * launch go/engine/hip/hip_projection_launch.go:3086-3160, packet contract/launch_abi.hipinc:634-657).
  * gate and up are [N, K*bits/32] with their own scales/biases; for a row-concatenated gate|up slab
  * (model.ConcatQuantRows, go/model/quant_weight.go:32-62) pass the slab for gate and slab + N rows for up.
- * M == 1 with 4/8-bit codes (up to 4 rows of 4-bit group-64 codes when K is 2..8 times 1024) runs as ONE launch
+ * M == 1 with 4/8-bit codes (up to 4 rows of 4-bit group-64 codes when K is a multiple of 256 between 1280 and 8192) runs as ONE launch
  * that reads every weight once; other shapes run the two
  * projections and the element-wise step as separate launches through the context's workspace (which grows
  * on demand like aq_qmm's; not while a capture is open). */

@@ -86,9 +86,9 @@ def test_gate_up_single_row(ctx, orc, act, bits, gs, M, K, N):
     x = F.synthetic_x(M, K, seed=F.BASE_SEED + 72)
     dg, du = DeviceAffine(ctx, gw, gsb, gb), DeviceAffine(ctx, uw, usb, ub)
     got = _run_gate_up(ctx, x, dg, du, M, K, N, gs, bits, act)
-    # 4-bit group-64 codes with K of 2..8 steps of 1024: the diagonal-MFMA pair kernel (up to 4 rows), whose two sums
+    # 4-bit group-64 codes with K a multiple of 256 in 2..8 steps of 1024: the diagonal-MFMA pair kernel (up to 4 rows), whose two sums
     # are those of the library's own choice for a plain call; otherwise the dot2 pair kernel (one row)
-    diag = bits == 4 and gs == 64 and K % 1024 == 0 and 2 <= K // 1024 <= 8
+    diag = bits == 4 and gs == 64 and K % 256 == 0 and 2 <= (K + 1023) // 1024 <= 8
     assert ctx.last_variant(0) == ("qmv_gate_up_diag" if diag else "qmv_gate_up_dot2")
     if diag:
         g_gpu = run_qmv(ctx, x, dg, M, K, N, gs, bits, True)

@@ -335,8 +335,9 @@ def test_qmvs_every_variant(ctx, orc):
 
 def test_qmvd_every_variant(ctx, orc):
     """Each diagonal-MFMA matvec variant, forced: 1..4 (1..8) activation rows, K = all the steps of 1024 codes its
-    wavefronts take and one step fewer (an idle wavefront), ragged N; fp32 and bf16 stores; a K that is no multiple
-    of 1024, or more steps than the variant takes, is refused."""
+    wavefronts take and one step fewer (an idle wavefront), a last step of three chunks and of one chunk of 256
+    codes, ragged N; fp32 and bf16 stores; a K that is no multiple of 256, or more steps than the variant takes, is
+    refused."""
     import aq_mi355
     names = aq_mi355.variant_names(0)
     N = 150
@@ -349,7 +350,7 @@ def test_qmvd_every_variant(ctx, orc):
             waves = int(name.split("_w")[1].split("_")[0])
             steps = waves * int(name.split("_d")[1].split("_")[0])
             wg_waves = waves * int(name.split("_r")[1].split("_")[0])
-            for K in sorted({1024 * steps, 1024 * max(1, steps - 1)}):
+            for K in sorted({1024 * steps, 1024 * max(1, steps - 1), 1024 * steps - 256, 1024 * (steps - 1) + 256}):
                 say("variant", idx, name, "K", K)
                 if K not in data:
                     words, s, b = F.synthetic_affine(N, K, bits, 64, seed=530 + K // 1024)
@@ -370,7 +371,7 @@ def test_qmvd_every_variant(ctx, orc):
                 out = run_qmv(ctx, x[:2], dw, 2, K, N, 64, bits, False)
                 check_bf16_store(out, ref[:2], name)
             dw, x, ref = data[1024 * steps]
-            for bad_k in (1024 * steps - 256, 1024 * (steps + 1)):
+            for bad_k in (1024 * steps - 64, 1024 * steps + 256):
                 with pytest.raises(aq_mi355.AqError) as ei:
                     run_qmv(ctx, np.zeros((1, bad_k), np.uint16), dw, 1, bad_k, N, 64, bits, True)
                 assert ei.value.code == aq_mi355.AQ_ERR_ARG
@@ -397,7 +398,7 @@ def test_qmvd_is_the_default_for_few_rows(ctx, orc):
             out = run_qmv(ctx, x[:rows], dw, rows, K, N, 64, 4, False)
             check_bf16_store(out, ref[:rows], "diag default bf16 K=%d rows=%d" % (K, rows))
         dw.free()
-    for K in (5120, 7168, 14336, 16384):
+    for K in (5120, 7168, 14336, 16384, 2816, 11008, 1280):
         words, s, b = F.synthetic_affine(40, K, 4, 64, seed=840 + K // 1024)
         x = F.synthetic_x(1, K, seed=850 + K // 1024)
         dw = DeviceAffine(ctx, words, s, b)
@@ -406,7 +407,7 @@ def test_qmvd_is_the_default_for_few_rows(ctx, orc):
         assert ctx.last_variant(0).startswith("qmvd_"), ctx.last_variant(0)
         check_accumulators(acc, F.reference_f64(x, words, s, b, 4, 64, K), "diag default K=%d" % K)
         dw.free()
-    for K, bits, rows in ((17408, 4, 1), (1024, 4, 1), (4096, 8, 1), (8192, 4, 2)):
+    for K, bits, rows in ((17408, 4, 1), (1024, 4, 1), (4096, 8, 1), (8192, 4, 2), (2880, 4, 1)):
         words, s, b = F.synthetic_affine(32, K, bits, 64, seed=830)
         x = F.synthetic_x(rows, K, seed=831)
         dw = DeviceAffine(ctx, words, s, b)
@@ -510,7 +511,7 @@ def test_qmv_multi_matches_separate_calls(ctx, orc, M, bits, Ns, K):
                 check_accumulators(got, ref, "multi member %d" % i)
         if M == 1 and bits == 4 and all(n > 0 for n in Ns):
             # K of 2..4 steps of 1024 codes goes to the diagonal-MFMA kernels, like the single calls
-            assert fused_name == ("qmv_multi_diag" if K >= 2048 else "qmv_multi_dot2"), fused_name
+            assert fused_name == ("qmv_multi_diag" if K > 1024 else "qmv_multi_dot2"), fused_name
         for t in ys:
             t.free()
     with pytest.raises(aq_mi355.AqError):
