@@ -178,6 +178,15 @@ int launch_qmv_rows(aq_ctx* ctx, aq::QmvArgs a, int group_size, int bits, bool g
         AQ_HIP(aq::qmvd_launch(di, a, ctx->stream), "hipLaunchKernel");
         return AQ_OK;
     }
+    if (forced < 0 && gather) {
+        // 4-bit group-64 codes, K a multiple of 128 in 2..8 steps of 1024: the gathered diagonal-MFMA kernels
+        const int di = aq::qmvd_pick_gather(a.K);
+        if (di >= 0 && aq::qmvd_fits(a, bits, group_size, true, di)) {
+            ctx->last_variant[0] = aq::qmvd_variant(di)->name;
+            AQ_HIP(aq::qmvd_launch(di, a, ctx->stream), "hipLaunchKernel");
+            return AQ_OK;
+        }
+    }
     if (forced < 0 && !gather) {
         // 4-bit group-64 codes: up to 8 rows at a K of 2..4 steps of 1024 codes, one row up to 16 steps: the diagonal-MFMA kernels
         const int di = aq::qmvd_pick(M, a.K, a.N);
@@ -770,10 +779,10 @@ int aq_qmv_gate_up(aq_ctx* ctx, const void* x, const void* gate_packed, const vo
         up.b = a.b2;
         if (di >= 0 && aq::qmvd_pair_supported(di) && aq::qmvd_fits(a, bits, group_size, false, di) &&
             aq::qmvd_fits(up, bits, group_size, false, di) &&
-            (size_t)M * K * 2 + (size_t)M * (K / 256) * 48 + 64 + (size_t)2 * aq::qmvd_variant(di)->waves * 256 <= 96 * 1024) {
+            (size_t)M * K * 2 + (size_t)M * ((K + 255) / 256) * 48 + 64 + (size_t)2 * aq::qmvd_variant(di)->waves * 256 <= 96 * 1024) {
             std::lock_guard<std::mutex> lk(ctx->mu);
             ctx->last_variant[0] = "qmv_gate_up_diag";
-            AQ_HIP(aq::qmvd_pair_launch(di, a, ctx->stream), "hipLaunchKernel");
+            AQ_HIP(aq::qmvd_pair_launch(di, a, false, ctx->stream), "hipLaunchKernel");
             return AQ_OK;
         }
     }
@@ -842,6 +851,36 @@ int aq_gather_qmv_gate_up(aq_ctx* ctx, const void* x, const void* packed, const 
         return fail(AQ_ERR_ARG, "aq_gather_qmv_gate_up: operand pointer is not element-aligned");
     if (routes > 65535) return fail(AQ_ERR_UNSUPPORTED, "aq_gather_qmv_gate_up: at most 65535 routes per call");
     const bool out_f32 = (flags & AQ_OUT_F32) != 0;
+    if (ctx->forced[0] < 0) {
+        // the gathered diagonal-MFMA pair kernel: one set of wavefronts on the gate rows, one on the up rows
+        const int di = aq::qmvd_pick_gather(K);
+        aq::QmvArgs a{};
+        a.x = static_cast<const uint16_t*>(x);
+        a.w = a.w2 = static_cast<const uint32_t*>(packed);
+        a.s = a.s2 = static_cast<const uint16_t*>(scales);
+        a.b = a.b2 = static_cast<const uint16_t*>(biases);
+        a.y = y;
+        a.lhs = lhs;
+        a.rhs = rhs;
+        a.K = K;
+        a.N = N;
+        a.M = 1;
+        a.gs_shift = is_pow2(group_size) ? ilog2(group_size) : 0;
+        a.out_f32 = out_f32 ? 1 : 0;
+        a.num_experts = num_experts;
+        a.expert_rows = expert_rows;
+        a.row_base = gate_row_base;
+        a.row_base2 = up_row_base;
+        a.x_rows = x_rows;
+        a.routes = routes;
+        a.act = act;
+        if (di >= 0 && aq::qmvd_pair_supported(di) && aq::qmvd_fits(a, bits, group_size, true, di)) {
+            std::lock_guard<std::mutex> lk(ctx->mu);
+            ctx->last_variant[0] = "gather_gate_up_diag";
+            AQ_HIP(aq::qmvd_pair_launch(di, a, true, ctx->stream), "hipLaunchKernel");
+            return AQ_OK;
+        }
+    }
     if (ctx->forced[0] < 0 && dot2_eligible(K, group_size, bits, x, packed, (size_t)K * 2)) {
         std::lock_guard<std::mutex> lk(ctx->mu);
         const int rows = act_rows(ctx, bits, 1, true, N, K, routes);

@@ -151,7 +151,9 @@ int qmvd_pick(int M, int K, int N);
 // y = act(gate . x) * (up . x) with variant idx's split of K (a.w2, a.s2, a.b2: the `up` matrix; a.act); the two
 // dot products are the bytes qmvd_launch computes for each matrix.
 bool qmvd_pair_supported(int idx);
-hipError_t qmvd_pair_launch(int idx, const QmvArgs& a, hipStream_t stream);
+hipError_t qmvd_pair_launch(int idx, const QmvArgs& a, bool gather, hipStream_t stream);
+// The gathered variant (one activation row per route, grid.y = routes) for this K, or -1.
+int qmvd_pick_gather(int K);
 bool qmvd_multi_supported(int idx);
 hipError_t qmvd_multi_launch(int idx, QmvMultiArgs ma, hipStream_t stream);
 

@@ -67,10 +67,10 @@ constexpr int kDiagChunk = 256;    // codes of a row per MFMA chain (four groups
 constexpr int kDiagSuper = 1024;   // codes of a row per wavefront step (four chunks)
 constexpr int kDiagZeroBytes = 64;
 
-// LDS: activations in expansion order [M][K] bf16, the split group sums [M][K/1024][4] x 48 B, 64 zero bytes,
+// LDS: activations in expansion order [M][K] bf16, the split group sums [M][chunks of 256 codes] x 48 B, 64 zero bytes,
 // the partial sums of the wavefronts [NW][sets of four activation rows][64] fp32.
 __host__ __device__ inline size_t qmvd_lds_bytes_for(int M, int K, int nw, int mt = 1) {
-    return (size_t)M * K * 2 + (size_t)M * (K / kDiagChunk) * 48 + kDiagZeroBytes + (size_t)nw * mt * 64 * 4;
+    return (size_t)M * K * 2 + (size_t)M * ((K + kDiagChunk - 1) / kDiagChunk) * 48 + kDiagZeroBytes + (size_t)nw * mt * 64 * 4;
 }
 
 // NR sets of NW wavefronts (a set per 16 rows); each wavefront takes SUP steps of 1024 codes (steps wave,
@@ -79,27 +79,47 @@ __host__ __device__ inline size_t qmvd_lds_bytes_for(int M, int K, int nw, int m
 // on the same 16 rows, and the store is act(gate . x) * (up . x).
 // MT: sets of four activation rows (the 16 rows of A hold four tokens; a second set reuses the expanded codes with
 // eight more MFMAs per chunk).
-template <int NW, int SUP, int NR, bool PAIR, int MT = 1>
+// GATHER: blockIdx.y is a route; the expert id and the activation row are read from a.rhs / a.lhs on the device
+// (kernels/moe/lthn_gather_qmv.metal:54-66 semantics), one activation row per route.
+template <int NW, int SUP, int NR, bool PAIR, int MT = 1, bool GATHER = false>
 __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block) {
     static_assert(!PAIR || NR == 2, "the pair kernel runs one set per matrix");
+    static_assert(!GATHER || MT == 1, "a route has one activation row");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave_wg = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wave = wave_wg % NW;  // which steps of K
     const int rg = wave_wg / NW;    // which 16 rows of the workgroup's NR x 16
-    const int K = a.K, N = a.N, M = a.M;
+    const int K = a.K, N = a.N, M = GATHER ? 1 : a.M;
     const int groups = K >> 6;
-    const int chunks = K / kDiagChunk;
+    const int halves = K >> 7;             // 128-code halves of a row (K % 128 == 0)
+    const int chunks = (halves + 1) >> 1;  // the last chunk may be a single half
     const int supers = (chunks + 3) >> 2;  // the last step may hold fewer than four chunks
     const uint32_t xs_off = 0;
     const uint32_t a2_off = (uint32_t)M * K * 2;
-    const uint32_t zero_off = a2_off + (uint32_t)M * (K / kDiagChunk) * 48;
+    const uint32_t zero_off = a2_off + (uint32_t)M * chunks * 48;
     const uint32_t red_off = zero_off + kDiagZeroBytes;
 
+    // gather: the route's expert slab and activation row
+    int64_t slab_row = 0, slab_row2 = 0, x_row = 0, y_row = 0;
+    bool route_ok = true;
+    if constexpr (GATHER) {
+        const int z = blockIdx.y;
+        const int e = a.rhs[z];
+        int xr = a.lhs ? a.lhs[z] : 0;
+        route_ok = (unsigned)e < (unsigned)a.num_experts && (unsigned)xr < (unsigned)a.x_rows;
+        if (!route_ok) xr = 0;
+        slab_row = route_ok ? (int64_t)e * a.expert_rows + a.row_base : 0;
+        slab_row2 = route_ok ? (int64_t)e * a.expert_rows + a.row_base2 : 0;
+        x_row = xr;
+        y_row = z;
+    }
+
     // ---- stage x: expansion order within every 8 values, group sums split into three bf16 terms ----
-    const gptr_t xg = uniform_ptr(a.x);
-    const int pieces = M * (K >> 3);  // 16-byte pieces of all tokens (K % 256 == 0: a token is whole pieces)
+    const gptr_t xg = uniform_ptr(reinterpret_cast<const char*>(a.x) + x_row * K * 2);
+    const int ppt = K >> 3;        // 16-byte pieces of a token (K % 128 == 0: whole groups of eight)
+    const int pieces = M * ppt;
     auto stage = [&](int p, const uint4 v) {
         uint4 o;
         o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);  // (x0, x4)
@@ -125,12 +145,18 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
             const uint32_t n0 = __float_as_uint(-128.0f * __uint_as_float(u0));
             const uint32_t n1 = __float_as_uint(-128.0f * __uint_as_float(u1));
             const uint32_t n2 = __float_as_uint(-128.0f * __uint_as_float(u2));
-            // group g of a token: 12 bytes at [chunk g / 4][g % 4] of that token's table
-            const uint32_t g = (uint32_t)p >> 3;
-            uint32_t* e = reinterpret_cast<uint32_t*>(lds_raw + a2_off + (g >> 2) * 48 + (g & 3) * 12);
+            // group g of token t: 12 bytes at [t][chunk g / 4][g % 4]
+            const uint32_t t = (uint32_t)p / (uint32_t)ppt;
+            const uint32_t g = ((uint32_t)p - t * (uint32_t)ppt) >> 3;
+            uint32_t* e = reinterpret_cast<uint32_t*>(lds_raw + a2_off + (t * chunks + (g >> 2)) * 48 + (g & 3) * 12);
             e[0] = (u0 >> 16) | u1;  // (X0, X1)
             e[1] = (u2 >> 16) | n0;  // (X2, -128 X0)
             e[2] = (n1 >> 16) | n2;  // (-128 X1, -128 X2)
+            if ((halves & 1) && (int)g == groups - 1) {
+                // a last chunk of one half: its two missing groups must add nothing to the affine term
+#pragma unroll
+                for (int q = 3; q < 9; q++) e[q] = 0;
+            }
         }
     };
     // the first pieces of a thread are requested before the weights, so that they arrive first
@@ -153,9 +179,11 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     int row = row0 + n;
     if (row >= N) row = N - 1;
     const bool second = PAIR && rg == 1;
-    const gptr_t wg = uniform_ptr(second ? a.w2 : a.w);
-    const gptr_t sg = uniform_ptr(second ? a.s2 : a.s);
-    const gptr_t bg = uniform_ptr(second ? a.b2 : a.b);
+    const bool other = second && !GATHER;  // gathered pairs: two row bases inside one expert slab
+    const int64_t srow = second ? slab_row2 : slab_row;
+    const gptr_t wg = uniform_ptr(reinterpret_cast<const char*>(other ? a.w2 : a.w) + srow * (K >> 1));
+    const gptr_t sg = uniform_ptr(reinterpret_cast<const char*>(other ? a.s2 : a.s) + srow * groups * 2);
+    const gptr_t bg = uniform_ptr(reinterpret_cast<const char*>(other ? a.b2 : a.b) + srow * groups * 2);
     const uint32_t w_lane = (uint32_t)row * (uint32_t)(K >> 1) + (uint32_t)j * 16;  // bytes
     // scales and biases: lane group j holds the four groups of chunk j of the step
     const uint32_t sb_lane = (uint32_t)row * (uint32_t)groups * 2 + (uint32_t)j * 8;  // bytes
@@ -178,7 +206,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
         a_chunk0[tg] = d0 ? 512 : 0;
         a_chunk1[tg] = d1 ? 512 : 0;
         const bool d2 = tok && ag == 0;
-        a2_base[tg] = d2 ? a2_off + ((uint32_t)token * (K / kDiagChunk) + j) * 48 : zero_off;
+        a2_base[tg] = d2 ? a2_off + ((uint32_t)token * chunks + j) * 48 : zero_off;
         a2_mul[tg] = d2 ? 4 * 48 : 0;
     }
     // the lane that holds the scales of chunk 0 of the step for this lane's row (ds_bpermute byte address)
@@ -199,11 +227,19 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
         for (int cc = 0; cc < 4; cc++) {
             const uint32_t co = cc < valid ? cc * 128 : 0;
             wq[u][cc][0] = load_u128_at(wg, wo + co);
-            wq[u][cc][1] = load_u128_at(wg, wo + co + 64);
+            // (the second half of a last chunk that is a single half: re-reads the first, not used)
+            wq[u][cc][1] = load_u128_at(wg, wo + co + (cc < valid && 2 * (4 * sp + cc) + 1 < halves ? 64 : 0));
         }
-        const uint32_t so = sb_lane + (uint32_t)sp * 32 - (j < valid ? 0u : (uint32_t)j * 8);
+        // A last chunk of one half has two groups: its 8 bytes are read 4 bytes early (inside the row) and the
+        // upper word, which holds the two groups, moves down.
+        const bool halfl = (halves & 1) && 4 * sp + j == chunks - 1;
+        const uint32_t so = sb_lane + (uint32_t)sp * 32 - (j < valid ? 0u : (uint32_t)j * 8) - (halfl ? 4u : 0u);
         sq[u] = load_u64_at(sg, so);
         bq[u] = load_u64_at(bg, so);
+        if (halves & 1) {
+            sq[u].x = halfl ? sq[u].y : sq[u].x;
+            bq[u].x = halfl ? bq[u].y : bq[u].x;
+        }
     }
 
 #pragma unroll
@@ -275,6 +311,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
                 for (int tg = 0; tg < MT; tg++) dq[tg] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                 for (int L = 0; L < 2; L++) {
+                    if (L == 1 && 2 * (4 * sp + cc) + 1 >= halves) break;  // a last chunk of one half
                     const uint32_t ww[4] = {wq[u][cc][L].x, wq[u][cc][L].y, wq[u][cc][L].z, wq[u][cc][L].w};
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
@@ -318,9 +355,12 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
                 for (int w2 = 1; w2 < NW; w2++) up += red[((NW + w2) * MT + tg) * 64 + lane];
                 total = fmul_unfused(act_value(a.act, total), up);
             }
+            if constexpr (GATHER) {
+                if (!route_ok) total = 0.0f;
+            }
             const int t = tg * 4 + j, r = row0 + n;
             if (t < M && r < N) {
-                const size_t o = (size_t)t * N + r;
+                const size_t o = (size_t)(GATHER ? y_row : t) * N + r;
                 if (a.out_f32) {
                     static_cast<float*>(a.y)[o] = total;
                 } else {
@@ -339,6 +379,16 @@ __global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_kernel(const QmvArgs a
 template <int NW, int SUP>
 __global__ __launch_bounds__(2 * NW* kWave) void qmv_diag_pair_kernel(const QmvArgs a) {
     qmv_diag_body<NW, SUP, 2, true>(a, (int)blockIdx.x);
+}
+
+// Gathered forms: grid.y = routes.
+template <int NW, int SUP, int NR>
+__global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_gather_kernel(const QmvArgs a) {
+    qmv_diag_body<NW, SUP, NR, false, 1, true>(a, (int)blockIdx.x);
+}
+template <int NW, int SUP>
+__global__ __launch_bounds__(2 * NW* kWave) void qmv_diag_gather_pair_kernel(const QmvArgs a) {
+    qmv_diag_body<NW, SUP, 2, true, 1, true>(a, (int)blockIdx.x);
 }
 
 // Several weight matrices against the same activations in one launch (q|k|v, gate|up): the workgroups of all
@@ -371,6 +421,10 @@ struct QmvDiagEntry {
     {                                                                                                        \
         {"qmvd_b4_m4_r" #NR "_w" #NW "_d" #SUP "_g0", 4, 4, NR, NW, SUP, 0, 0, 4}, qmv_diag_kernel<NW, SUP, NR, 1> \
     }
+#define AQ_QMVDG(NW, SUP, NR)                                                                                \
+    {                                                                                                        \
+        {"qmvd_b4_m1_r" #NR "_w" #NW "_d" #SUP "_g1", 4, 1, NR, NW, SUP, 1, 0, 4}, qmv_diag_gather_kernel<NW, SUP, NR> \
+    }
 #define AQ_QMVD8(NW, SUP, NR)                                                                                \
     {                                                                                                        \
         {"qmvd_b4_m8_r" #NR "_w" #NW "_d" #SUP "_g0", 4, 8, NR, NW, SUP, 0, 0, 4}, qmv_diag_kernel<NW, SUP, NR, 2> \
@@ -379,6 +433,7 @@ static const QmvDiagEntry kQmvDiagTable[] = {
     AQ_QMVD(4, 1, 1), AQ_QMVD(4, 1, 2), AQ_QMVD(4, 1, 4), AQ_QMVD(2, 2, 2), AQ_QMVD(2, 1, 2), AQ_QMVD(8, 1, 1),
     AQ_QMVD(4, 2, 1), AQ_QMVD(2, 1, 4), AQ_QMVD(6, 1, 1), AQ_QMVD(10, 1, 1), AQ_QMVD(12, 1, 1),
     AQ_QMVD(14, 1, 1), AQ_QMVD(16, 1, 1), AQ_QMVD8(4, 1, 4), AQ_QMVD8(4, 1, 2), AQ_QMVD8(2, 1, 4),
+    AQ_QMVDG(2, 1, 1), AQ_QMVDG(2, 1, 2), AQ_QMVDG(4, 1, 1), AQ_QMVDG(4, 1, 2), AQ_QMVDG(6, 1, 1), AQ_QMVDG(8, 1, 1),
 };
 
 int qmvd_variant_count() { return (int)(sizeof(kQmvDiagTable) / sizeof(kQmvDiagTable[0])); }
@@ -389,28 +444,29 @@ const QmvVariant* qmvd_variant(int idx) {
 
 bool qmvd_fits(const QmvArgs& a, int bits, int group_size, bool gather, int idx) {
     const QmvVariant* v = qmvd_variant(idx);
-    if (!v || bits != 4 || group_size != 64 || gather) return false;
-    if (a.M < 1 || a.M > v->m || a.K <= 0 || a.K % kDiagChunk != 0 || a.N < 1) return false;
+    if (!v || bits != 4 || group_size != 64 || gather != (v->gather != 0)) return false;
+    if (gather && (a.M != 1 || a.routes < 1 || a.routes > 65535)) return false;
+    if (a.M < 1 || a.M > v->m || a.K <= 0 || a.K % 128 != 0 || a.N < 1) return false;
     if ((a.K + kDiagSuper - 1) / kDiagSuper > v->waves * v->depth) return false;
     const uintptr_t al16 = reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.w);
     const uintptr_t al8 = reinterpret_cast<uintptr_t>(a.s) | reinterpret_cast<uintptr_t>(a.b);
     if ((al16 & 15) || (al8 & 7)) return false;
     // 32-bit byte offsets into the packed matrix
     if ((uint64_t)a.N * (uint64_t)(a.K / 2) >= (1ull << 32)) return false;
-    return qmvd_lds_bytes_for(a.M, a.K, v->waves * v->rows, v->m / 4) <= 96 * 1024;
+    return qmvd_lds_bytes_for(a.M, a.K, v->waves * v->rows, (v->m + 3) / 4) <= 96 * 1024;
 }
 
 hipError_t qmvd_launch(int idx, const QmvArgs& a, hipStream_t stream) {
     if (idx < 0 || idx >= qmvd_variant_count()) return hipErrorInvalidValue;
     const QmvDiagEntry& e = kQmvDiagTable[idx];
-    const size_t lds = qmvd_lds_bytes_for(a.M, a.K, e.v.waves * e.v.rows, e.v.m / 4);
+    const size_t lds = qmvd_lds_bytes_for(a.M, a.K, e.v.waves * e.v.rows, (e.v.m + 3) / 4);
     if (lds > 48 * 1024) {
         hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e.fn),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (rc != hipSuccess) return rc;
     }
     const int wg_rows = kDiagRows * e.v.rows;
-    dim3 grid((unsigned)((a.N + wg_rows - 1) / wg_rows), 1u, 1u);
+    dim3 grid((unsigned)((a.N + wg_rows - 1) / wg_rows), e.v.gather ? (unsigned)a.routes : 1u, 1u);
     hipLaunchKernelGGL(e.fn, grid, dim3((unsigned)(e.v.rows * e.v.waves * kWave)), lds, stream, a);
     return hipGetLastError();
 }
@@ -418,7 +474,7 @@ hipError_t qmvd_launch(int idx, const QmvArgs& a, hipStream_t stream) {
 // The variant the library picks for M rows and this K, or -1: one step of 1024 codes per wavefront; up to 4 steps,
 // more rows per workgroup the more activation rows there are to stage.
 int qmvd_pick(int M, int K, int N) {
-    if (M < 1 || M > 8 || K <= 0 || K % kDiagChunk != 0) return -1;
+    if (M < 1 || M > 8 || K <= 0 || K % 128 != 0) return -1;
     const int steps = (K + kDiagSuper - 1) / kDiagSuper;
     const int cap = M <= 4 ? 4 : 8;
     int nw, nr;
@@ -441,7 +497,7 @@ int qmvd_pick(int M, int K, int N) {
     if (cap == 8 && nw == 2) nr = 4;
     for (int i = 0; i < qmvd_variant_count(); i++) {
         const QmvVariant& v = kQmvDiagTable[i].v;
-        if (v.waves == nw && v.depth == 1 && v.rows == nr && v.m == cap) return i;
+        if (v.waves == nw && v.depth == 1 && v.rows == nr && v.m == cap && !v.gather) return i;
     }
     return -1;
 }
@@ -449,9 +505,9 @@ int qmvd_pick(int M, int K, int N) {
 // act(gate . x) * (up . x) with the variant's (wavefronts, steps) split of K; a.w2 / a.s2 / a.b2 are the `up` matrix.
 struct QmvDiagPairEntry {
     int nw, sup;
-    QmvDiagKernel fn;
+    QmvDiagKernel fn, gather_fn;
 };
-#define AQ_QMVD_PAIR(NW, SUP) {NW, SUP, qmv_diag_pair_kernel<NW, SUP>}
+#define AQ_QMVD_PAIR(NW, SUP) {NW, SUP, qmv_diag_pair_kernel<NW, SUP>, qmv_diag_gather_pair_kernel<NW, SUP>}
 static const QmvDiagPairEntry kQmvDiagPairTable[] = {
     AQ_QMVD_PAIR(2, 1), AQ_QMVD_PAIR(4, 1), AQ_QMVD_PAIR(6, 1), AQ_QMVD_PAIR(8, 1),
 };
@@ -464,18 +520,33 @@ static const QmvDiagPairEntry* find_pair(int idx) {
 }
 bool qmvd_pair_supported(int idx) { return find_pair(idx) != nullptr; }
 
-hipError_t qmvd_pair_launch(int idx, const QmvArgs& a, hipStream_t stream) {
+hipError_t qmvd_pair_launch(int idx, const QmvArgs& a, bool gather, hipStream_t stream) {
     const QmvDiagPairEntry* e = find_pair(idx);
     if (!e) return hipErrorInvalidValue;
-    const size_t lds = qmvd_lds_bytes_for(a.M, a.K, 2 * e->nw);
+    const QmvDiagKernel fn = gather ? e->gather_fn : e->fn;
+    const size_t lds = qmvd_lds_bytes_for(gather ? 1 : a.M, a.K, 2 * e->nw);
     if (lds > 48 * 1024) {
-        hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e->fn),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                            (int)lds);
         if (rc != hipSuccess) return rc;
     }
-    dim3 grid((unsigned)((a.N + kDiagRows - 1) / kDiagRows), 1u, 1u);
-    hipLaunchKernelGGL(e->fn, grid, dim3((unsigned)(2 * e->nw * kWave)), lds, stream, a);
+    dim3 grid((unsigned)((a.N + kDiagRows - 1) / kDiagRows), gather ? (unsigned)a.routes : 1u, 1u);
+    hipLaunchKernelGGL(fn, grid, dim3((unsigned)(2 * e->nw * kWave)), lds, stream, a);
     return hipGetLastError();
+}
+
+// The gathered variant for this K (one activation row per route), or -1.
+int qmvd_pick_gather(int K) {
+    if (K <= 0 || K % 128 != 0) return -1;
+    const int steps = (K + kDiagSuper - 1) / kDiagSuper;
+    if (steps < 2 || steps > 8) return -1;
+    const int nw = (steps + 1) & ~1;
+    const int nr = nw == 2 ? 2 : 1;
+    for (int i = 0; i < qmvd_variant_count(); i++) {
+        const QmvVariant& v = kQmvDiagTable[i].v;
+        if (v.gather && v.waves == nw && v.depth == 1 && v.rows == nr) return i;
+    }
+    return -1;
 }
 
 typedef void (*QmvDiagMultiKernel)(const QmvMultiArgs);

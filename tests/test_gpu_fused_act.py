@@ -178,7 +178,8 @@ def _gather_inputs(ctx, E, expert_rows, K, bits, gs, x_rows, lhs, rhs, seed):
 
 
 @pytest.mark.parametrize("act", ACTS)
-@pytest.mark.parametrize("bits,K,N,batched", [(4, 2816, 1408, True), (4, 512, 40, False), (8, 1024, 64, True)])
+@pytest.mark.parametrize("bits,K,N,batched", [(4, 2816, 1408, True), (4, 512, 40, False), (8, 1024, 64, True),
+                                              (4, 1408, 70, True), (4, 4096, 40, False)])
 def test_gather_gate_up_fused_slab(ctx, orc, act, bits, K, N, batched):
     """Experts hold a fused gate|up slab of 2N rows; expert ids and token rows are read on the device."""
     import aq_mi355
@@ -196,15 +197,20 @@ def test_gather_gate_up_fused_slab(ctx, orc, act, bits, K, N, batched):
     ctx.gather_qmv_gate_up(dev["x"], dw.w, dw.s, dw.b, dev["lhs"], dev["rhs"], dy, routes, x_rows, K, N, E, 2 * N, 0, N, gs,
                            bits, act, aq_mi355.AQ_OUT_F32)
     ctx.sync()
-    assert ctx.last_variant(0) == "gather_gate_up_dot2"
+    # 4-bit codes with K a multiple of 128 in 2..8 steps of 1024: the gathered diagonal-MFMA pair kernel, whose sums
+    # are those of the library's own choice for a plain gather; otherwise the dot2 pair kernel
+    diag = bits == 4 and K % 128 == 0 and 2 <= (K + 1023) // 1024 <= 8
+    assert ctx.last_variant(0) == ("gather_gate_up_diag" if diag else "gather_gate_up_dot2")
     got = dy.download(np.float32, routes * N).reshape(routes, N)
     parts = []
-    with _dot2_family(ctx, bits, True):
+    import contextlib
+    with (contextlib.nullcontext() if diag else _dot2_family(ctx, bits, True)):
         for base in (0, N):
             ctx.fill_zero(dy)
             ctx.gather_qmv(dev["x"], dw.w, dw.s, dw.b, dev["lhs"], dev["rhs"], dy, routes, x_rows, K, N, E, 2 * N, base, gs,
                            bits, aq_mi355.AQ_OUT_F32)
             ctx.sync()
+            assert ctx.last_variant(0).startswith("qmvd_") == diag
             parts.append(dy.download(np.float32, routes * N).reshape(routes, N))
     wq = F.numpy_dequant(words, s, b, bits, gs, K).astype(np.float64).reshape(E, 2 * N, K)
     xf = F.bf16_bits_to_f32(x).astype(np.float64).reshape(x_rows, K)
@@ -224,10 +230,11 @@ def test_gather_gate_up_fused_slab(ctx, orc, act, bits, K, N, batched):
     dw.free()
 
 
-def test_gather_gate_up_bad_ids_and_errors(ctx):
+@pytest.mark.parametrize("K", [512, 1408])
+def test_gather_gate_up_bad_ids_and_errors(ctx, K):
     import aq_mi355
-    say("gather gate_up bad ids")
-    E, N, K = 4, 32, 512
+    say("gather gate_up bad ids", K)
+    E, N = 4, 32
     words, s, b, x, dev = _gather_inputs(ctx, E, 2 * N, K, 4, 64, 1, None, [1, 9, -2], F.BASE_SEED + 78)
     dw = dev["w"]
     dy = ctx.alloc(3 * N * 4)

@@ -197,7 +197,7 @@ def test_gather_every_variant(ctx, orc):
     try:
         for idx, name in enumerate(names):
             fam, bits, m, gather = _parse_variant(name)
-            if not gather or fam in ("blk", "stream"):
+            if not gather or fam in ("blk", "stream", "diag"):
                 continue
             say("gather variant", idx, name)
             fx = F.gather_fixture(out_dim, in_dim, 64, bits, E, expert_rows, True, routes)
@@ -336,8 +336,8 @@ def test_qmvs_every_variant(ctx, orc):
 def test_qmvd_every_variant(ctx, orc):
     """Each diagonal-MFMA matvec variant, forced: 1..4 (1..8) activation rows, K = all the steps of 1024 codes its
     wavefronts take and one step fewer (an idle wavefront), a last step of three chunks and of one chunk of 256
-    codes, ragged N; fp32 and bf16 stores; a K that is no multiple of 256, or more steps than the variant takes, is
-    refused."""
+    codes, a last chunk that is a single half of 128 codes, ragged N; fp32 and bf16 stores; a K that is no multiple
+    of 128, or more steps than the variant takes, is refused."""
     import aq_mi355
     names = aq_mi355.variant_names(0)
     N = 150
@@ -345,12 +345,13 @@ def test_qmvd_every_variant(ctx, orc):
     try:
         for idx, name in enumerate(names):
             fam, bits, m, gather = _parse_variant(name)
-            if fam != "diag":
+            if fam != "diag" or gather:
                 continue
             waves = int(name.split("_w")[1].split("_")[0])
             steps = waves * int(name.split("_d")[1].split("_")[0])
             wg_waves = waves * int(name.split("_r")[1].split("_")[0])
-            for K in sorted({1024 * steps, 1024 * max(1, steps - 1), 1024 * steps - 256, 1024 * (steps - 1) + 256}):
+            for K in sorted({1024 * steps, 1024 * max(1, steps - 1), 1024 * steps - 256, 1024 * (steps - 1) + 256,
+                             1024 * steps - 128, 1024 * (steps - 1) + 128}):
                 say("variant", idx, name, "K", K)
                 if K not in data:
                     words, s, b = F.synthetic_affine(N, K, bits, 64, seed=530 + K // 1024)
@@ -381,6 +382,48 @@ def test_qmvd_every_variant(ctx, orc):
         dw.free()
 
 
+def test_qmvd_gather_every_variant(ctx, orc):
+    """Each gathered diagonal-MFMA variant, forced and as the default: K = all the steps its wavefronts take, a last
+    chunk that is a single half of 128 codes, a last step of one chunk; batched x, a row_base inside the slab, ragged
+    N, an expert id out of range (zeros for that route)."""
+    import aq_mi355
+    names = aq_mi355.variant_names(0)
+    E, routes, out_dim, expert_rows, row_base = 4, 6, 40, 96, 32
+    try:
+        for idx, name in enumerate(names):
+            fam, bits, m, gather = _parse_variant(name)
+            if fam != "diag" or not gather:
+                continue
+            steps = int(name.split("_w")[1].split("_")[0]) * int(name.split("_d")[1].split("_")[0])
+            for K in sorted({1024 * steps, 1024 * steps - 128, 1024 * (steps - 1) + 256, 1024 * (steps - 1) + 128}):
+                say("gather variant", idx, name, "K", K)
+                fx = F.gather_fixture(out_dim, K, 64, bits, E, expert_rows, True, routes)
+                _, s, b = F.synthetic_affine(E * expert_rows, K, bits, 64, seed=41 + bits)
+                fx["scales"], fx["biases"] = s, b
+                fx["rhs"] = fx["rhs"].copy()
+                fx["rhs"][4] = E + 3  # no such expert
+                ok = [z for z in range(routes) if z != 4]
+                ref64, _ = orc.gather_qmv(fx["x"], fx["x_rows"], fx["packed"], s, b, fx["lhs"][ok], fx["rhs"][ok], len(ok), E,
+                                          expert_rows, row_base, out_dim, K, 64, bits)
+                for forced in (True, False):
+                    ctx.force_variant(0, idx if forced else -1)
+                    acc, dw = _gather_run(ctx, fx, routes, E, expert_rows, row_base, out_dim, K, 64, bits, True)
+                    if forced:
+                        assert ctx.last_variant(0) == name
+                    else:
+                        assert ctx.last_variant(0).startswith("qmvd_") and ctx.last_variant(0).endswith("_g1"), ctx.last_variant(0)
+                    check_accumulators(acc[ok], ref64, name)
+                    assert np.all(acc[4] == 0)
+                    dw.free()
+                ctx.force_variant(0, idx)
+            fx = F.gather_fixture(out_dim, 1024 * steps + 128, 64, bits, E, expert_rows, True, routes)
+            with pytest.raises(aq_mi355.AqError) as ei:
+                _gather_run(ctx, fx, routes, E, expert_rows, row_base, out_dim, 1024 * steps + 128, 64, bits, True)
+            assert ei.value.code == aq_mi355.AQ_ERR_ARG
+    finally:
+        ctx.force_variant(0, -1)
+
+
 def test_qmvd_is_the_default_for_few_rows(ctx, orc):
     """4-bit group-64 codes: 1..8 activation rows with K of 2, 3 or 4 steps of 1024 codes, and one row with up to 16
     steps, land on the diagonal-MFMA kernels without forcing, rows beyond the last full 16 included; other K, more
@@ -398,7 +441,7 @@ def test_qmvd_is_the_default_for_few_rows(ctx, orc):
             out = run_qmv(ctx, x[:rows], dw, rows, K, N, 64, 4, False)
             check_bf16_store(out, ref[:rows], "diag default bf16 K=%d rows=%d" % (K, rows))
         dw.free()
-    for K in (5120, 7168, 14336, 16384, 2816, 11008, 1280):
+    for K in (5120, 7168, 14336, 16384, 2816, 11008, 1280, 1408, 2944):
         words, s, b = F.synthetic_affine(40, K, 4, 64, seed=840 + K // 1024)
         x = F.synthetic_x(1, K, seed=850 + K // 1024)
         dw = DeviceAffine(ctx, words, s, b)
