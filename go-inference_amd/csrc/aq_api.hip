@@ -553,7 +553,7 @@ int aq_qmv_multi(aq_ctx* ctx, const void* x, int count, const void* const* packe
     if (count == 0) return AQ_OK;
     if (!packed || !scales || !biases || !y || !N) return fail(AQ_ERR_ARG, "aq_qmv_multi: null array");
     if (M < 0 || K < 0) return fail(AQ_ERR_SHAPE, "aq_qmv_multi: M, K must be non-negative");
-    bool fused = M == 1 && K > 0 && bits == 4 && ctx->forced[0] < 0;
+    bool fused = M >= 1 && M <= 4 && K > 0 && bits == 4 && ctx->forced[0] < 0;
     for (int i = 0; i < count; i++) {
         if (N[i] < 0) return fail(AQ_ERR_SHAPE, "aq_qmv_multi: N[%d] must be non-negative", i);
         if (N[i] == 0) fused = false;  // an empty member: leave the bookkeeping to aq_qmv
@@ -573,13 +573,14 @@ int aq_qmv_multi(aq_ctx* ctx, const void* x, int count, const void* const* packe
         if (fused) {
             std::lock_guard<std::mutex> lk(ctx->mu);
             // the kernels aq_qmv would pick for each member, in one grid
-            const int di = aq::qmvd_pick(1, K, 1 << 20);
+            // (every variant with the same split of K computes the same bytes, whatever the rows per workgroup)
+            const int di = aq::qmvd_pick(M, K, (int)total);
             if (di >= 0 && aq::qmvd_multi_supported(di)) {
                 bool fits = true;
                 aq::QmvMultiArgs ma{};
                 ma.common.x = static_cast<const uint16_t*>(x);
                 ma.common.K = K;
-                ma.common.M = 1;
+                ma.common.M = M;
                 ma.common.gs_shift = ilog2(group_size);
                 ma.common.out_f32 = (flags & AQ_OUT_F32) ? 1 : 0;
                 ma.common.routes = 1;
@@ -604,7 +605,7 @@ int aq_qmv_multi(aq_ctx* ctx, const void* x, int count, const void* const* packe
                     return AQ_OK;
                 }
             }
-            const int idx = pick_qmv_variant(ctx, bits, 1, false, (int)total, K, 1);
+            const int idx = M == 1 ? pick_qmv_variant(ctx, bits, 1, false, (int)total, K, 1) : -1;
             const int rows = idx >= 0 ? aq::qmv_variant(idx)->rows : 0;
             if (rows > 0 && aq::qmv_multi_supported(bits, 1, rows)) {
                 aq::QmvMultiArgs ma{};

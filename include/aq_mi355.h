@@ -109,7 +109,8 @@ int aq_qmv(aq_ctx *ctx, const void *x, const void *packed, const void *scales, c
  * pointers.  Results are byte-identical to `count` separate aq_qmv calls.  This is the no-copy form of
  * running q|k|v or gate|up over model.ConcatQuantRows (go/model/quant_weight.go:32-62): at batch 1 the
  * narrow projections are bound by launch latency, not bandwidth, and one grid over all of them fills
- * the machine.  Shapes the fused kernels do not take are run as separate launches. */
+ * the machine.  One launch for one activation row (up to four when K is a multiple of 128 between 1152 and 16384);
+ * shapes the fused kernels do not take are run as separate launches. */
 int aq_qmv_multi(aq_ctx *ctx, const void *x, int count, const void *const *packed, const void *const *scales,
                  const void *const *biases, void *const *y, const int *N, int M, int K, int group_size, int bits,
                  unsigned flags);

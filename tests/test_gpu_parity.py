@@ -523,7 +523,8 @@ def test_concat_rows_is_byte_identical(ctx, orc):
 @pytest.mark.parametrize("M,bits,Ns,K", [(1, 4, (96, 160, 40), 1024), (1, 4, (4096, 1024, 1024), 1024), (1, 4, (50,), 1024),
                                           (1, 4, (7, 9, 300, 64), 1024), (2, 4, (96, 160), 1024), (1, 8, (64, 200), 1024),
                                           (1, 4, (96, 0, 32), 1024), (1, 4, (96, 160, 40), 2048), (1, 4, (4096, 1024, 1030), 4096),
-                                          (1, 4, (7, 300), 3072), (2, 4, (96, 160), 4096), (1, 8, (64, 200), 4096)])
+                                          (1, 4, (7, 300), 3072), (2, 4, (96, 160), 4096), (1, 8, (64, 200), 4096),
+                                          (4, 4, (4096, 1024, 1030), 4096), (3, 4, (50, 40, 33, 20), 2816), (5, 4, (96, 160), 4096)])
 def test_qmv_multi_matches_separate_calls(ctx, orc, M, bits, Ns, K):
     """aq_qmv_multi (q|k|v, gate|up in one launch) is byte-identical to one aq_qmv per matrix, the
     contract ConcatQuantRows states (go/model/quant_weight.go:32-44); members that the fused kernels
@@ -552,9 +553,11 @@ def test_qmv_multi_matches_separate_calls(ctx, orc, M, bits, Ns, K):
             ref = F.reference_f64(x, mats[i][0][:n], mats[i][1][:n], mats[i][2][:n], bits, 64, K)
             if f32:
                 check_accumulators(got, ref, "multi member %d" % i)
-        if M == 1 and bits == 4 and all(n > 0 for n in Ns):
-            # K of 2..4 steps of 1024 codes goes to the diagonal-MFMA kernels, like the single calls
+        if bits == 4 and all(n > 0 for n in Ns) and (M == 1 or (M <= 4 and K > 1024)):
+            # K beyond one step of 1024 codes goes to the diagonal-MFMA kernels (up to four rows), like the single calls
             assert fused_name == ("qmv_multi_diag" if K > 1024 else "qmv_multi_dot2"), fused_name
+        else:
+            assert not fused_name.startswith("qmv_multi"), fused_name
         for t in ys:
             t.free()
     with pytest.raises(aq_mi355.AqError):
