@@ -132,10 +132,11 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
         sum = dot2_bf16(v.y, ones, sum);
         sum = dot2_bf16(v.z, ones, sum);
         sum = dot2_bf16(v.w, ones, sum);
-        // the eight pieces of a group sit in eight consecutive lanes
-        sum += __shfl_xor(sum, 1);
-        sum += __shfl_xor(sum, 2);
-        sum += __shfl_xor(sum, 4);
+        // the eight pieces of a group sit in eight consecutive, aligned lanes: two quad swaps, then the mirror of the
+        // half row adds the other quad (DPP, no LDS round trips)
+        sum += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sum), 0xB1, 0xF, 0xF, true));
+        sum += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sum), 0x4E, 0xF, 0xF, true));
+        sum += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sum), 0x141, 0xF, 0xF, true));
         if ((p & 7) == 0) {
             const uint32_t u0 = __float_as_uint(sum) & 0xffff0000u;
             const float r1 = sum - __uint_as_float(u0);
@@ -159,16 +160,21 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
             }
         }
     };
+    // One activation row and one step per wavefront: every wavefront stages the 1024 activations of its own step
+    // (128 pieces, two per lane) and nobody waits for anybody before the arithmetic.  Otherwise the workgroup stages
+    // all of x together and meets at a barrier.
+    const bool wstage = SUP == 1 && M == 1;
     // the first pieces of a thread are requested before the weights, so that they arrive first
     constexpr int PRE = 2;
     uint4 pre[PRE];
+    int pre_p[PRE];
 #pragma unroll
     for (int q = 0; q < PRE; q++) {
-        int p = tid + q * NR * NW * kWave;
-        if (p >= pieces) p = pieces - 1;
-        pre[q] = load_u128_at(xg, (uint32_t)p * 16);
+        pre_p[q] = wstage ? wave * 128 + q * 64 + lane : tid + q * NR * NW * kWave;
+        pre[q] = load_u128_at(xg, (uint32_t)min(pre_p[q], pieces - 1) * 16);
     }
-    if (tid < kDiagZeroBytes / 16) *reinterpret_cast<uint4*>(lds_raw + zero_off + tid * 16) = make_uint4(0, 0, 0, 0);
+    if (lane < kDiagZeroBytes / 16 && (wstage || wave_wg == 0))
+        *reinterpret_cast<uint4*>(lds_raw + zero_off + lane * 16) = make_uint4(0, 0, 0, 0);
 
     // ---- per-lane constants ----
     const int n = lane & 15;   // weight row of the lane (B operand, D column)
@@ -243,12 +249,17 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     }
 
 #pragma unroll
-    for (int q = 0; q < PRE; q++) {
-        const int p = tid + q * NR * NW * kWave;
-        if (p < pieces) stage(p, pre[q]);
+    for (int q = 0; q < PRE; q++)
+        if (pre_p[q] < pieces) stage(pre_p[q], pre[q]);
+    if (wstage) {
+        // LDS operations of one wavefront complete in order: what its lanes wrote is there for its later reads
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    } else {
+        for (int p = tid + PRE * NR * NW * kWave; p < pieces; p += NR * NW * kWave) stage(p, load_u128_at(xg, (uint32_t)p * 16));
+        __syncthreads();  // x, sums and zeros are in LDS
     }
-    for (int p = tid + PRE * NR * NW * kWave; p < pieces; p += NR * NW * kWave) stage(p, load_u128_at(xg, (uint32_t)p * 16));
-    __syncthreads();  // x, sums and zeros are in LDS
 
     float acc[MT];
     f32x4_t dsum[MT];  // affine term, register 0 is the one that is used
