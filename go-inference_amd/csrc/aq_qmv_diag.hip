@@ -28,6 +28,9 @@
 //     -128 X1, -128 X2) per group, every product exact (the codes travel as 128 + code, see aq_device.h);
 //   * the NW wavefronts of a set take the steps of the same 16 rows in turn and meet in LDS; a workgroup
 //     holds NR sets (more rows per workgroup when more activation rows have to be staged).
+//   * one activation row: every wavefront stages the activations of its own step (no workgroup barrier before
+//     the arithmetic: with many wavefronts per workgroup the barrier made all wait for the one whose loads got out
+//     last); more rows: the workgroup stages x together.
 // Every variant of one (NW, steps per wavefront) pair computes the same bytes for a row, whatever NR and
 // whatever the number of activation rows, and so does the multi-matrix launch.
 #include "aq_device.h"
@@ -66,6 +69,9 @@ constexpr int kDiagRows = 16;      // weight rows per workgroup
 constexpr int kDiagChunk = 256;    // codes of a row per MFMA chain (four groups of 64)
 constexpr int kDiagSuper = 1024;   // codes of a row per wavefront step (four chunks)
 constexpr int kDiagZeroBytes = 64;
+#ifndef AQ_DIAG_WROWS
+#define AQ_DIAG_WROWS 1  // most activation rows a wavefront stages for itself (4 measured slower for every row count)
+#endif
 
 // LDS: activations in expansion order [M][K] bf16, the split group sums [M][chunks of 256 codes] x 48 B, 64 zero bytes,
 // the partial sums of the wavefronts [NW][sets of four activation rows][64] fp32.
@@ -160,18 +166,24 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
             }
         }
     };
-    // One activation row and one step per wavefront: every wavefront stages the 1024 activations of its own step
-    // (128 pieces, two per lane) and nobody waits for anybody before the arithmetic.  Otherwise the workgroup stages
-    // all of x together and meets at a barrier.
-    const bool wstage = SUP == 1 && M == 1;
+    // One step per wavefront and up to WROWS activation rows: every wavefront stages the 1024 activations per row of
+    // its own step (128 pieces per row, two per lane) and nobody waits for anybody before the arithmetic.  Otherwise
+    // the workgroup stages all of x together and meets at a barrier.
+    constexpr int WROWS = (SUP == 1 && MT == 1) ? AQ_DIAG_WROWS : 0;
+    const bool wstage = M <= WROWS;
     // the first pieces of a thread are requested before the weights, so that they arrive first
-    constexpr int PRE = 2;
+    constexpr int PRE = WROWS > 1 ? 2 * WROWS : 2;
     uint4 pre[PRE];
     int pre_p[PRE];
 #pragma unroll
     for (int q = 0; q < PRE; q++) {
-        pre_p[q] = wstage ? wave * 128 + q * 64 + lane : tid + q * NR * NW * kWave;
-        pre[q] = load_u128_at(xg, (uint32_t)min(pre_p[q], pieces - 1) * 16);
+        if (wstage) {
+            const int pl = wave * 128 + (q & 1) * 64 + lane;  // piece of row q / 2
+            pre_p[q] = (q >> 1) < M && pl < ppt ? (q >> 1) * ppt + pl : pieces;
+        } else {
+            pre_p[q] = q < 2 ? tid + q * NR * NW * kWave : pieces;
+        }
+        if (q < 2 || (wstage && (q >> 1) < M)) pre[q] = load_u128_at(xg, (uint32_t)min(pre_p[q], pieces - 1) * 16);
     }
     if (lane < kDiagZeroBytes / 16 && (wstage || wave_wg == 0))
         *reinterpret_cast<uint4*>(lds_raw + zero_off + lane * 16) = make_uint4(0, 0, 0, 0);
@@ -257,7 +269,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     } else {
-        for (int p = tid + PRE * NR * NW * kWave; p < pieces; p += NR * NW * kWave) stage(p, load_u128_at(xg, (uint32_t)p * 16));
+        for (int p = tid + 2 * NR * NW * kWave; p < pieces; p += NR * NW * kWave) stage(p, load_u128_at(xg, (uint32_t)p * 16));
         __syncthreads();  // x, sums and zeros are in LDS
     }
 
