@@ -67,7 +67,8 @@ __device__ __forceinline__ bf16x8_t as_bf16x8(uint32_t a, uint32_t b, uint32_t c
 
 constexpr int kDiagRows = 16;      // weight rows per workgroup
 constexpr int kDiagChunk = 256;    // codes of a row per MFMA chain (four groups of 64)
-constexpr int kDiagSuper = 1024;   // codes of a row per wavefront step (four chunks)
+// A wavefront step is CPS chunks (a template parameter: 4, or 3 where that shares K out more evenly, e.g. the 11
+// chunks of K = 2816 as 3 + 3 + 3 + 2 over four wavefronts instead of 4 + 4 + 3 + none).
 constexpr int kDiagZeroBytes = 64;
 #ifndef AQ_DIAG_WROWS
 #define AQ_DIAG_WROWS 1  // most activation rows a wavefront stages for itself (4 measured slower for every row count)
@@ -87,7 +88,7 @@ __host__ __device__ inline size_t qmvd_lds_bytes_for(int M, int K, int nw, int m
 // eight more MFMAs per chunk).
 // GATHER: blockIdx.y is a route; the expert id and the activation row are read from a.rhs / a.lhs on the device
 // (kernels/moe/lthn_gather_qmv.metal:54-66 semantics), one activation row per route.
-template <int NW, int SUP, int NR, bool PAIR, int MT = 1, bool GATHER = false>
+template <int NW, int SUP, int NR, bool PAIR, int MT = 1, bool GATHER = false, int CPS = 4>
 __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block) {
     static_assert(!PAIR || NR == 2, "the pair kernel runs one set per matrix");
     static_assert(!GATHER || MT == 1, "a route has one activation row");
@@ -101,7 +102,8 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     const int groups = K >> 6;
     const int halves = K >> 7;             // 128-code halves of a row (K % 128 == 0)
     const int chunks = (halves + 1) >> 1;  // the last chunk may be a single half
-    const int supers = (chunks + 3) >> 2;  // the last step may hold fewer than four chunks
+    static_assert(CPS >= 2 && CPS <= 4, "a step holds 2..4 chunks (one lane group per chunk for the scales)");
+    const int supers = (chunks + CPS - 1) / CPS;  // the last step may hold fewer chunks
     const uint32_t xs_off = 0;
     const uint32_t a2_off = (uint32_t)M * K * 2;
     const uint32_t zero_off = a2_off + (uint32_t)M * chunks * 48;
@@ -178,8 +180,8 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
 #pragma unroll
     for (int q = 0; q < PRE; q++) {
         if (wstage) {
-            const int pl = wave * 128 + (q & 1) * 64 + lane;  // piece of row q / 2
-            pre_p[q] = (q >> 1) < M && pl < ppt ? (q >> 1) * ppt + pl : pieces;
+            const int pl = wave * (CPS * 32) + (q & 1) * 64 + lane;  // piece of row q / 2
+            pre_p[q] = (q >> 1) < M && pl < ppt && (q & 1) * 64 + lane < CPS * 32 ? (q >> 1) * ppt + pl : pieces;
         } else {
             pre_p[q] = q < 2 ? tid + q * NR * NW * kWave : pieces;
         }
@@ -219,13 +221,13 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
         const uint32_t x_lane = xs_off + (uint32_t)token * K * 2 + (uint32_t)j * 64;  // codes j*32.. of a 128-code load
         a_base0[tg] = d0 ? x_lane : zero_off;
         a_base1[tg] = d1 ? x_lane + 256 : zero_off;
-        a_mul0[tg] = d0 ? 2048 : 0;
-        a_mul1[tg] = d1 ? 2048 : 0;
+        a_mul0[tg] = d0 ? CPS * 512 : 0;
+        a_mul1[tg] = d1 ? CPS * 512 : 0;
         a_chunk0[tg] = d0 ? 512 : 0;
         a_chunk1[tg] = d1 ? 512 : 0;
         const bool d2 = tok && ag == 0;
         a2_base[tg] = d2 ? a2_off + ((uint32_t)token * chunks + j) * 48 : zero_off;
-        a2_mul[tg] = d2 ? 4 * 48 : 0;
+        a2_mul[tg] = d2 ? CPS * 48 : 0;
     }
     // the lane that holds the scales of chunk 0 of the step for this lane's row (ds_bpermute byte address)
     const int sc_addr = n * 4;
@@ -233,25 +235,25 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     const uint32_t mask = opaque_s(kNibbleMask);
     const uint32_t magic = opaque_v(kMagic128);
 
-    uint4 wq[SUP][4][2];
+    uint4 wq[SUP][CPS][2];
     uint2 sq[SUP], bq[SUP];
 #pragma unroll
     for (int u = 0; u < SUP; u++) {
         int sp = wave + u * NW;
         if (sp >= supers) sp = supers - 1;  // past the end: a valid address, the result is not used
-        const int valid = min(4, chunks - 4 * sp);  // chunks of this step; the others re-read chunk 0 and are not used
-        const uint32_t wo = w_lane + (uint32_t)sp * 512;
+        const int valid = min(CPS, chunks - CPS * sp);  // chunks of this step; the others re-read chunk 0 and are not used
+        const uint32_t wo = w_lane + (uint32_t)sp * (CPS * 128);
 #pragma unroll
-        for (int cc = 0; cc < 4; cc++) {
+        for (int cc = 0; cc < CPS; cc++) {
             const uint32_t co = cc < valid ? cc * 128 : 0;
             wq[u][cc][0] = load_u128_at(wg, wo + co);
             // (the second half of a last chunk that is a single half: re-reads the first, not used)
-            wq[u][cc][1] = load_u128_at(wg, wo + co + (cc < valid && 2 * (4 * sp + cc) + 1 < halves ? 64 : 0));
+            wq[u][cc][1] = load_u128_at(wg, wo + co + (cc < valid && 2 * (CPS * sp + cc) + 1 < halves ? 64 : 0));
         }
         // A last chunk of one half has two groups: its 8 bytes are read 4 bytes early (inside the row) and the
         // upper word, which holds the two groups, moves down.
-        const bool halfl = (halves & 1) && 4 * sp + j == chunks - 1;
-        const uint32_t so = sb_lane + (uint32_t)sp * 32 - (j < valid ? 0u : (uint32_t)j * 8) - (halfl ? 4u : 0u);
+        const bool halfl = (halves & 1) && j < CPS && CPS * sp + j == chunks - 1;
+        const uint32_t so = sb_lane + (uint32_t)sp * (CPS * 8) - (j < valid ? 0u : (uint32_t)j * 8) - (halfl ? 4u : 0u);
         sq[u] = load_u64_at(sg, so);
         bq[u] = load_u64_at(bg, so);
         if (halves & 1) {
@@ -284,7 +286,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     for (int u = 0; u < SUP; u++) {
         const int sp = wave + u * NW;
         if (sp < supers) {
-            const int valid = min(4, chunks - 4 * sp);
+            const int valid = min(CPS, chunks - CPS * sp);
             const uint2 sv = sq[u], bv = bq[u];
             // affine term of the 16 groups of the step: 24 k-slots per lane, three MFMAs
             {
@@ -315,7 +317,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
                 a_addr1[tg] = a_base1[tg] + (uint32_t)sp * a_mul1[tg];
             }
 #pragma unroll
-            for (int cc = 0; cc < 4; cc++) {
+            for (int cc = 0; cc < CPS; cc++) {
                 if (cc >= valid) break;
                 bf16x8_t af[MT][2][4];
 #pragma unroll
@@ -334,7 +336,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
                 for (int tg = 0; tg < MT; tg++) dq[tg] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                 for (int L = 0; L < 2; L++) {
-                    if (L == 1 && 2 * (4 * sp + cc) + 1 >= halves) break;  // a last chunk of one half
+                    if (L == 1 && 2 * (CPS * sp + cc) + 1 >= halves) break;  // a last chunk of one half
                     const uint32_t ww[4] = {wq[u][cc][L].x, wq[u][cc][L].y, wq[u][cc][L].z, wq[u][cc][L].w};
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
@@ -394,29 +396,29 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     }
 }
 
-template <int NW, int SUP, int NR, int MT>
+template <int NW, int SUP, int NR, int MT, int CPS>
 __global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_kernel(const QmvArgs a) {
-    qmv_diag_body<NW, SUP, NR, false, MT>(a, (int)blockIdx.x);
+    qmv_diag_body<NW, SUP, NR, false, MT, false, CPS>(a, (int)blockIdx.x);
 }
 
-template <int NW, int SUP>
+template <int NW, int SUP, int CPS>
 __global__ __launch_bounds__(2 * NW* kWave) void qmv_diag_pair_kernel(const QmvArgs a) {
-    qmv_diag_body<NW, SUP, 2, true>(a, (int)blockIdx.x);
+    qmv_diag_body<NW, SUP, 2, true, 1, false, CPS>(a, (int)blockIdx.x);
 }
 
 // Gathered forms: grid.y = routes.
-template <int NW, int SUP, int NR>
+template <int NW, int SUP, int NR, int CPS>
 __global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_gather_kernel(const QmvArgs a) {
-    qmv_diag_body<NW, SUP, NR, false, 1, true>(a, (int)blockIdx.x);
+    qmv_diag_body<NW, SUP, NR, false, 1, true, CPS>(a, (int)blockIdx.x);
 }
-template <int NW, int SUP>
+template <int NW, int SUP, int CPS>
 __global__ __launch_bounds__(2 * NW* kWave) void qmv_diag_gather_pair_kernel(const QmvArgs a) {
-    qmv_diag_body<NW, SUP, 2, true, 1, true>(a, (int)blockIdx.x);
+    qmv_diag_body<NW, SUP, 2, true, 1, true, CPS>(a, (int)blockIdx.x);
 }
 
 // Several weight matrices against the same activations in one launch (q|k|v, gate|up): the workgroups of all
 // matrices form one grid, and each looks up which matrix it belongs to.
-template <int NW, int SUP, int NR>
+template <int NW, int SUP, int NR, int CPS>
 __global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_multi_kernel(const QmvMultiArgs ma) {
     int set = 0;
 #pragma unroll
@@ -428,7 +430,7 @@ __global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_multi_kernel(const Qmv
     a.b = ma.b[set];
     a.y = ma.y[set];
     a.N = ma.N[set];
-    qmv_diag_body<NW, SUP, NR, false>(a, (int)blockIdx.x - (set ? ma.block_end[set - 1] : 0));
+    qmv_diag_body<NW, SUP, NR, false, 1, false, CPS>(a, (int)blockIdx.x - (set ? ma.block_end[set - 1] : 0));
 }
 
 // ---- variant table --------------------------------------------------------
@@ -438,26 +440,52 @@ struct QmvDiagEntry {
     QmvVariant v;
     QmvDiagKernel fn;
 };
-// name, bits, m (most rows), sets of 16 rows per workgroup, wavefronts per set, steps per wavefront, gather, xmode, kind
-// waves x depth steps of 1024 codes cover K
-#define AQ_QMVD(NW, SUP, NR)                                                                                 \
-    {                                                                                                        \
-        {"qmvd_b4_m4_r" #NR "_w" #NW "_d" #SUP "_g0", 4, 4, NR, NW, SUP, 0, 0, 4}, qmv_diag_kernel<NW, SUP, NR, 1> \
+// name, bits, m (most rows), sets of 16 rows per workgroup, wavefronts per set, steps per wavefront, gather,
+// xmode = chunks per step when not 4, kind.  waves x depth steps cover K.
+#define AQ_QMVD(NW, SUP, NR)                                                                                    \
+    {                                                                                                           \
+        {"qmvd_b4_m4_r" #NR "_w" #NW "_d" #SUP "_g0", 4, 4, NR, NW, SUP, 0, 0, 4}, qmv_diag_kernel<NW, SUP, NR, 1, 4> \
     }
-#define AQ_QMVDG(NW, SUP, NR)                                                                                \
-    {                                                                                                        \
-        {"qmvd_b4_m1_r" #NR "_w" #NW "_d" #SUP "_g1", 4, 1, NR, NW, SUP, 1, 0, 4}, qmv_diag_gather_kernel<NW, SUP, NR> \
+#define AQ_QMVD3(NW, SUP, NR)                                                                                      \
+    {                                                                                                              \
+        {"qmvd_b4_m4_r" #NR "_w" #NW "_d" #SUP "_g0_c3", 4, 4, NR, NW, SUP, 0, 3, 4}, qmv_diag_kernel<NW, SUP, NR, 1, 3> \
     }
-#define AQ_QMVD8(NW, SUP, NR)                                                                                \
-    {                                                                                                        \
-        {"qmvd_b4_m8_r" #NR "_w" #NW "_d" #SUP "_g0", 4, 8, NR, NW, SUP, 0, 0, 4}, qmv_diag_kernel<NW, SUP, NR, 2> \
+#define AQ_QMVDG(NW, SUP, NR)                                                                                          \
+    {                                                                                                                  \
+        {"qmvd_b4_m1_r" #NR "_w" #NW "_d" #SUP "_g1", 4, 1, NR, NW, SUP, 1, 0, 4}, qmv_diag_gather_kernel<NW, SUP, NR, 4> \
+    }
+#define AQ_QMVDG3(NW, SUP, NR)                                                                                            \
+    {                                                                                                                     \
+        {"qmvd_b4_m1_r" #NR "_w" #NW "_d" #SUP "_g1_c3", 4, 1, NR, NW, SUP, 1, 3, 4}, qmv_diag_gather_kernel<NW, SUP, NR, 3> \
+    }
+#define AQ_QMVD8(NW, SUP, NR)                                                                                   \
+    {                                                                                                           \
+        {"qmvd_b4_m8_r" #NR "_w" #NW "_d" #SUP "_g0", 4, 8, NR, NW, SUP, 0, 0, 4}, qmv_diag_kernel<NW, SUP, NR, 2, 4> \
+    }
+#define AQ_QMVD83(NW, SUP, NR)                                                                                     \
+    {                                                                                                              \
+        {"qmvd_b4_m8_r" #NR "_w" #NW "_d" #SUP "_g0_c3", 4, 8, NR, NW, SUP, 0, 3, 4}, qmv_diag_kernel<NW, SUP, NR, 2, 3> \
     }
 static const QmvDiagEntry kQmvDiagTable[] = {
     AQ_QMVD(4, 1, 1), AQ_QMVD(4, 1, 2), AQ_QMVD(4, 1, 4), AQ_QMVD(2, 2, 2), AQ_QMVD(2, 1, 2), AQ_QMVD(8, 1, 1),
     AQ_QMVD(4, 2, 1), AQ_QMVD(2, 1, 4), AQ_QMVD(6, 1, 1), AQ_QMVD(10, 1, 1), AQ_QMVD(12, 1, 1),
     AQ_QMVD(14, 1, 1), AQ_QMVD(16, 1, 1), AQ_QMVD8(4, 1, 4), AQ_QMVD8(4, 1, 2), AQ_QMVD8(2, 1, 4),
     AQ_QMVDG(2, 1, 1), AQ_QMVDG(2, 1, 2), AQ_QMVDG(4, 1, 1), AQ_QMVDG(4, 1, 2), AQ_QMVDG(6, 1, 1), AQ_QMVDG(8, 1, 1),
+    AQ_QMVD3(4, 1, 1), AQ_QMVD3(4, 1, 2), AQ_QMVD3(4, 1, 4), AQ_QMVD3(2, 1, 2), AQ_QMVD3(2, 1, 4),
+    AQ_QMVD83(4, 1, 4), AQ_QMVD83(4, 1, 2), AQ_QMVD83(2, 1, 4), AQ_QMVDG3(2, 1, 2), AQ_QMVDG3(4, 1, 1),
 };
+
+static int cps_of(const QmvVariant& v) { return v.xmode ? v.xmode : 4; }
+// Steps of cps chunks of 256 codes that cover K (its last chunk may be a single half of 128 codes).
+static int steps_for(int K, int cps) { return ((K + kDiagChunk - 1) / kDiagChunk + cps - 1) / cps; }
+// Chunks per step for this K: three where the even number of wavefronts that four would need holds them too (the
+// heaviest wavefront then has three chunks instead of four).  A function of K alone, so that every launch form
+// splits a row the same way and computes the same bytes.
+static int cps_for(int K) {
+    const int chunks = (K + kDiagChunk - 1) / kDiagChunk;
+    const int nw4 = ((chunks + 3) / 4 + 1) & ~1;
+    return (nw4 <= 4 && (chunks + 2) / 3 <= nw4) ? 3 : 4;
+}
 
 int qmvd_variant_count() { return (int)(sizeof(kQmvDiagTable) / sizeof(kQmvDiagTable[0])); }
 const QmvVariant* qmvd_variant(int idx) {
@@ -470,7 +498,7 @@ bool qmvd_fits(const QmvArgs& a, int bits, int group_size, bool gather, int idx)
     if (!v || bits != 4 || group_size != 64 || gather != (v->gather != 0)) return false;
     if (gather && (a.M != 1 || a.routes < 1 || a.routes > 65535)) return false;
     if (a.M < 1 || a.M > v->m || a.K <= 0 || a.K % 128 != 0 || a.N < 1) return false;
-    if ((a.K + kDiagSuper - 1) / kDiagSuper > v->waves * v->depth) return false;
+    if (steps_for(a.K, cps_of(*v)) > v->waves * v->depth) return false;
     const uintptr_t al16 = reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.w);
     const uintptr_t al8 = reinterpret_cast<uintptr_t>(a.s) | reinterpret_cast<uintptr_t>(a.b);
     if ((al16 & 15) || (al8 & 7)) return false;
@@ -497,8 +525,9 @@ hipError_t qmvd_launch(int idx, const QmvArgs& a, hipStream_t stream) {
 // The variant the library picks for M rows and this K, or -1: one step of 1024 codes per wavefront; up to 4 steps,
 // more rows per workgroup the more activation rows there are to stage.
 int qmvd_pick(int M, int K, int N) {
-    if (M < 1 || M > 8 || K <= 0 || K % 128 != 0) return -1;
-    const int steps = (K + kDiagSuper - 1) / kDiagSuper;
+    if (M < 1 || M > 8 || K <= 1024 || K % 128 != 0) return -1;  // (up to 1024 codes: one wavefront per row set, not built)
+    const int cps = cps_for(K);
+    const int steps = steps_for(K, cps);
     const int cap = M <= 4 ? 4 : 8;
     int nw, nr;
     if (steps == 2) {
@@ -520,25 +549,26 @@ int qmvd_pick(int M, int K, int N) {
     if (cap == 8 && nw == 2) nr = 4;
     for (int i = 0; i < qmvd_variant_count(); i++) {
         const QmvVariant& v = kQmvDiagTable[i].v;
-        if (v.waves == nw && v.depth == 1 && v.rows == nr && v.m == cap && !v.gather) return i;
+        if (v.waves == nw && v.depth == 1 && v.rows == nr && v.m == cap && !v.gather && cps_of(v) == cps) return i;
     }
     return -1;
 }
 
 // act(gate . x) * (up . x) with the variant's (wavefronts, steps) split of K; a.w2 / a.s2 / a.b2 are the `up` matrix.
 struct QmvDiagPairEntry {
-    int nw, sup;
+    int nw, sup, cps;
     QmvDiagKernel fn, gather_fn;
 };
-#define AQ_QMVD_PAIR(NW, SUP) {NW, SUP, qmv_diag_pair_kernel<NW, SUP>, qmv_diag_gather_pair_kernel<NW, SUP>}
+#define AQ_QMVD_PAIR(NW, SUP, CPS) {NW, SUP, CPS, qmv_diag_pair_kernel<NW, SUP, CPS>, qmv_diag_gather_pair_kernel<NW, SUP, CPS>}
 static const QmvDiagPairEntry kQmvDiagPairTable[] = {
-    AQ_QMVD_PAIR(2, 1), AQ_QMVD_PAIR(4, 1), AQ_QMVD_PAIR(6, 1), AQ_QMVD_PAIR(8, 1),
+    AQ_QMVD_PAIR(2, 1, 4), AQ_QMVD_PAIR(4, 1, 4), AQ_QMVD_PAIR(6, 1, 4), AQ_QMVD_PAIR(8, 1, 4),
+    AQ_QMVD_PAIR(2, 1, 3), AQ_QMVD_PAIR(4, 1, 3),
 };
 static const QmvDiagPairEntry* find_pair(int idx) {
     const QmvVariant* v = qmvd_variant(idx);
     if (v)
         for (const QmvDiagPairEntry& e : kQmvDiagPairTable)
-            if (e.nw == v->waves && e.sup == v->depth) return &e;
+            if (e.nw == v->waves && e.sup == v->depth && e.cps == cps_of(*v)) return &e;
     return nullptr;
 }
 bool qmvd_pair_supported(int idx) { return find_pair(idx) != nullptr; }
@@ -560,28 +590,31 @@ hipError_t qmvd_pair_launch(int idx, const QmvArgs& a, bool gather, hipStream_t 
 
 // The gathered variant for this K (one activation row per route), or -1.
 int qmvd_pick_gather(int K) {
-    if (K <= 0 || K % 128 != 0) return -1;
-    const int steps = (K + kDiagSuper - 1) / kDiagSuper;
+    if (K <= 1024 || K % 128 != 0) return -1;
+    const int cps = cps_for(K);
+    const int steps = steps_for(K, cps);
     if (steps < 2 || steps > 8) return -1;
     const int nw = (steps + 1) & ~1;
     const int nr = nw == 2 ? 2 : 1;
     for (int i = 0; i < qmvd_variant_count(); i++) {
         const QmvVariant& v = kQmvDiagTable[i].v;
-        if (v.gather && v.waves == nw && v.depth == 1 && v.rows == nr) return i;
+        if (v.gather && v.waves == nw && v.depth == 1 && v.rows == nr && cps_of(v) == cps) return i;
     }
     return -1;
 }
 
 typedef void (*QmvDiagMultiKernel)(const QmvMultiArgs);
 struct QmvDiagMultiEntry {
-    int nw, sup, nr;
+    int nw, sup, nr, cps;
     QmvDiagMultiKernel fn;
 };
-#define AQ_QMVD_MULTI(NW, SUP, NR) {NW, SUP, NR, qmv_diag_multi_kernel<NW, SUP, NR>}
+#define AQ_QMVD_MULTI(NW, SUP, NR) {NW, SUP, NR, 4, qmv_diag_multi_kernel<NW, SUP, NR, 4>}
+#define AQ_QMVD_MULTI3(NW, SUP, NR) {NW, SUP, NR, 3, qmv_diag_multi_kernel<NW, SUP, NR, 3>}
 static const QmvDiagMultiEntry kQmvDiagMultiTable[] = {
     AQ_QMVD_MULTI(4, 1, 1), AQ_QMVD_MULTI(4, 1, 2), AQ_QMVD_MULTI(4, 1, 4), AQ_QMVD_MULTI(2, 1, 2), AQ_QMVD_MULTI(2, 1, 4),
     AQ_QMVD_MULTI(6, 1, 1), AQ_QMVD_MULTI(8, 1, 1), AQ_QMVD_MULTI(10, 1, 1), AQ_QMVD_MULTI(12, 1, 1), AQ_QMVD_MULTI(14, 1, 1),
-    AQ_QMVD_MULTI(16, 1, 1),
+    AQ_QMVD_MULTI(16, 1, 1), AQ_QMVD_MULTI3(4, 1, 1), AQ_QMVD_MULTI3(4, 1, 2), AQ_QMVD_MULTI3(4, 1, 4), AQ_QMVD_MULTI3(2, 1, 2),
+    AQ_QMVD_MULTI3(2, 1, 4),
 };
 
 // The multi-matrix launch of variant idx (the same arithmetic, so the same bytes, as one launch per matrix).
@@ -589,7 +622,7 @@ bool qmvd_multi_supported(int idx) {
     const QmvVariant* v = qmvd_variant(idx);
     if (!v) return false;
     for (const QmvDiagMultiEntry& e : kQmvDiagMultiTable)
-        if (e.nw == v->waves && e.sup == v->depth && e.nr == v->rows) return true;
+        if (e.nw == v->waves && e.sup == v->depth && e.nr == v->rows && e.cps == cps_of(*v)) return true;
     return false;
 }
 
@@ -598,7 +631,7 @@ hipError_t qmvd_multi_launch(int idx, QmvMultiArgs ma, hipStream_t stream) {
     const QmvDiagMultiEntry* e = nullptr;
     if (v)
         for (const QmvDiagMultiEntry& c : kQmvDiagMultiTable)
-            if (c.nw == v->waves && c.sup == v->depth && c.nr == v->rows) e = &c;
+            if (c.nw == v->waves && c.sup == v->depth && c.nr == v->rows && c.cps == cps_of(*v)) e = &c;
     if (!e || ma.count < 1 || ma.count > kQmvMultiMax) return hipErrorInvalidValue;
     const int wg_rows = kDiagRows * e->nr;
     int blocks = 0;
