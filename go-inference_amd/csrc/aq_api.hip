@@ -187,6 +187,15 @@ int launch_qmv_rows(aq_ctx* ctx, aq::QmvArgs a, int group_size, int bits, bool g
             return AQ_OK;
         }
     }
+    if (forced < 0 && !gather && group_size == 32) {
+        // 4-bit group-32 codes, up to 2 rows: the diagonal-MFMA kernels with two tokens x eight groups as A rows
+        const int di = aq::qmvd_pick_g32(M, a.K, a.N);
+        if (di >= 0 && aq::qmvd_fits(a, bits, group_size, false, di)) {
+            ctx->last_variant[0] = aq::qmvd_variant(di)->name;
+            AQ_HIP(aq::qmvd_launch(di, a, ctx->stream), "hipLaunchKernel");
+            return AQ_OK;
+        }
+    }
     if (forced < 0 && !gather) {
         // 4-bit group-64 codes: up to 8 rows at a K of 2..4 steps of 1024 codes, one row up to 16 steps: the diagonal-MFMA kernels
         const int di = aq::qmvd_pick(M, a.K, a.N);
@@ -780,7 +789,7 @@ int aq_qmv_gate_up(aq_ctx* ctx, const void* x, const void* gate_packed, const vo
         up.b = a.b2;
         if (di >= 0 && aq::qmvd_pair_supported(di) && aq::qmvd_fits(a, bits, group_size, false, di) &&
             aq::qmvd_fits(up, bits, group_size, false, di) &&
-            (size_t)M * K * 2 + (size_t)M * ((K + 255) / 256) * 48 + 64 + (size_t)2 * aq::qmvd_variant(di)->waves * 256 <= 96 * 1024) {
+            (size_t)M * K * 2 + (size_t)M * ((K + 255) / 256) * 48 + 128 + (size_t)2 * aq::qmvd_variant(di)->waves * 256 <= 96 * 1024) {
             std::lock_guard<std::mutex> lk(ctx->mu);
             ctx->last_variant[0] = "qmv_gate_up_diag";
             AQ_HIP(aq::qmvd_pair_launch(di, a, false, ctx->stream), "hipLaunchKernel");
@@ -1119,6 +1128,38 @@ int head_call(aq_ctx* ctx, const char* op, int fuse, const void* x, const void* 
         return fail(AQ_ERR_ARG, "%s: operand pointer is not element-aligned", op);
     if (fused) {
         std::lock_guard<std::mutex> lk(ctx->mu);
+        {
+            // the diagonal-MFMA kernel aq_qmv would pick for this projection, with the head epilogue
+            const int di = bits != 4 ? -1 : group_size == 32 ? aq::qmvd_pick_g32(1, K, N) : group_size == 64 ? aq::qmvd_pick(1, K, N) : -1;
+            aq::QmvArgs a{};
+            a.x = static_cast<const uint16_t*>(x);
+            a.w = static_cast<const uint32_t*>(packed);
+            a.s = static_cast<const uint16_t*>(scales);
+            a.b = static_cast<const uint16_t*>(biases);
+            a.y = out;
+            a.K = K;
+            a.N = N;
+            a.M = 1;
+            a.gs_shift = ilog2(group_size);
+            a.routes = 1;
+            a.suppress = suppress;
+            a.suppress_count = suppress_count;
+            if (di >= 0 && aq::qmvd_head_supported(di, fuse) && aq::qmvd_fits(a, bits, group_size, false, di)) {
+                const size_t slots = aq::qmvd_head_partials(di, N);
+                if (fuse == 3) {
+                    AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+                    if (int rc = aq::workspace_reserve(ctx->stream, &ctx->head_ws, slots * 8, fail)) return rc;
+                    a.partial = static_cast<unsigned long long*>(ctx->head_ws.ptr);
+                }
+                ctx->last_variant[0] = fuse == 3 ? "qmv_greedy_diag" : "qmv_scores_diag";
+                AQ_HIP(aq::qmvd_head_launch(di, fuse, a, ctx->stream), "hipLaunchKernel");
+                if (fuse == 3)
+                    AQ_HIP(aq::head_fold_launch(a.partial, (int)slots, static_cast<unsigned long long*>(ctx->head_fold),
+                                                reinterpret_cast<unsigned long long*>(out), ctx->stream),
+                           "hipLaunchKernel");
+                return AQ_OK;
+            }
+        }
         const int idx = pick_qmv_variant(ctx, bits, 1, false, N, K, 1);
         int rows = idx >= 0 ? aq::qmv_variant(idx)->rows : 1;
         while (rows > 1 && !aq::qmv_head_supported(bits, fuse, rows)) rows >>= 1;

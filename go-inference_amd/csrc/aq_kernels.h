@@ -85,7 +85,8 @@ struct QmvVariant {
     int kind;    // 0: VALU dot2 kernel (aq_qmv.hip), 1: MFMA kernel (aq_qmv_mfma.hip; m = most rows it takes),
                  // 2: block-MFMA kernel (aq_qmv_blk.hip; m = most rows, depth = K pieces per wavefront),
                  // 3: streaming dot2 kernel (aq_qmv_stream.hip; depth = rows in flight, xmode = slices per row)
-                 // 4: diagonal-MFMA kernel (aq_qmv_diag.hip; m = most rows, rows = rows per workgroup)
+                 // 4: diagonal-MFMA kernel (aq_qmv_diag.hip; m = most rows, rows = sets of 16 rows per workgroup,
+                 //    xmode = chunks per step when not 4), 5: the same for quantisation groups of 32 codes
 };
 
 int qmv_variant_count();
@@ -148,12 +149,22 @@ bool qmvd_fits(const QmvArgs& a, int bits, int group_size, bool gather, int idx)
 hipError_t qmvd_launch(int idx, const QmvArgs& a, hipStream_t stream);
 // The variant the library picks for M rows and this K, or -1 when another family takes the shape.
 int qmvd_pick(int M, int K, int N);
+// The same for quantisation groups of 32 codes (up to two rows, K a multiple of 256).
+int qmvd_pick_g32(int M, int K, int N);
 // y = act(gate . x) * (up . x) with variant idx's split of K (a.w2, a.s2, a.b2: the `up` matrix; a.act); the two
 // dot products are the bytes qmvd_launch computes for each matrix.
 bool qmvd_pair_supported(int idx);
 hipError_t qmvd_pair_launch(int idx, const QmvArgs& a, bool gather, hipStream_t stream);
 // The gathered variant (one activation row per route, grid.y = routes) for this K, or -1.
 int qmvd_pick_gather(int K);
+// lm_head epilogues on variant idx (fuse 3: best packed value per 16 rows into a.partial, qmvd_head_partials(idx, N)
+// slots, to be folded by head_fold_launch; fuse 4: packed scores into a.y).
+bool qmvd_head_supported(int idx, int fuse);
+size_t qmvd_head_partials(int idx, int N);
+hipError_t qmvd_head_launch(int idx, int fuse, const QmvArgs& a, hipStream_t stream);
+// Folds `count` partial maxima into best[0] (aq_qmv_head.hip).
+hipError_t head_fold_launch(const unsigned long long* partial, int count, unsigned long long* fold, unsigned long long* best,
+                            hipStream_t stream);
 bool qmvd_multi_supported(int idx);
 hipError_t qmvd_multi_launch(int idx, QmvMultiArgs ma, hipStream_t stream);
 

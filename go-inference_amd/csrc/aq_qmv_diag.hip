@@ -69,15 +69,16 @@ constexpr int kDiagRows = 16;      // weight rows per workgroup
 constexpr int kDiagChunk = 256;    // codes of a row per MFMA chain (four groups of 64)
 // A wavefront step is CPS chunks (a template parameter: 4, or 3 where that shares K out more evenly, e.g. the 11
 // chunks of K = 2816 as 3 + 3 + 3 + 2 over four wavefronts instead of 4 + 4 + 3 + none).
-constexpr int kDiagZeroBytes = 64;
+constexpr int kDiagZeroBytes = 128;
 #ifndef AQ_DIAG_WROWS
 #define AQ_DIAG_WROWS 1  // most activation rows a wavefront stages for itself (4 measured slower for every row count)
 #endif
 
 // LDS: activations in expansion order [M][K] bf16, the split group sums [M][chunks of 256 codes] x 48 B, 64 zero bytes,
 // the partial sums of the wavefronts [NW][sets of four activation rows][64] fp32.
-__host__ __device__ inline size_t qmvd_lds_bytes_for(int M, int K, int nw, int mt = 1) {
-    return (size_t)M * K * 2 + (size_t)M * ((K + kDiagChunk - 1) / kDiagChunk) * 48 + kDiagZeroBytes + (size_t)nw * mt * 64 * 4;
+__host__ __device__ inline size_t qmvd_lds_bytes_for(int M, int K, int nw, int mt = 1, bool g32 = false) {
+    return (size_t)M * K * 2 + (size_t)M * ((K + kDiagChunk - 1) / kDiagChunk) * (g32 ? 96 : 48) + kDiagZeroBytes +
+           (size_t)nw * mt * 64 * 4;
 }
 
 // NR sets of NW wavefronts (a set per 16 rows); each wavefront takes SUP steps of 1024 codes (steps wave,
@@ -88,8 +89,19 @@ __host__ __device__ inline size_t qmvd_lds_bytes_for(int M, int K, int nw, int m
 // eight more MFMAs per chunk).
 // GATHER: blockIdx.y is a route; the expert id and the activation row are read from a.rhs / a.lhs on the device
 // (kernels/moe/lthn_gather_qmv.metal:54-66 semantics), one activation row per route.
-template <int NW, int SUP, int NR, bool PAIR, int MT = 1, bool GATHER = false, int CPS = 4>
+// G32: quantisation groups of 32 codes.  A lane group's 32 codes are then one whole group: the 16 rows of A are
+// (token, group slot) for TWO tokens and the eight groups of a chunk, row (t, g) is non-zero in load L for lane
+// group j iff g == 4 L + j, D lands as lane (2 t + g / 4, n), register g % 4, and the two halves of a token's sum
+// meet at the end.  Scales and biases are 16 bytes per chunk and lane.  K is then a multiple of 256.
+// HEAD (lm_head, one activation row): 4 stores every row's packed (score, row) instead of the score, 3 keeps the
+// best packed value of the 16 rows in a.partial[set] for fold_best_kernel (aq_qmv_head.hip).
+template <int NW, int SUP, int NR, bool PAIR, int MT = 1, bool GATHER = false, int CPS = 4, bool G32 = false, int HEAD = 0>
 __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block) {
+    static_assert(HEAD == 0 || (!PAIR && !GATHER && MT == 1), "the head epilogues take one plain activation row");
+    static_assert(!G32 || MT == 1, "group 32: one set of two activation rows");
+    constexpr int TPS = G32 ? 2 : 4;      // activation rows per set
+    constexpr int A2B = G32 ? 96 : 48;    // bytes of split group sums per chunk and activation row
+    constexpr int SBB = G32 ? 16 : 8;     // bytes of scales (or biases) per chunk and weight row
     static_assert(!PAIR || NR == 2, "the pair kernel runs one set per matrix");
     static_assert(!GATHER || MT == 1, "a route has one activation row");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
@@ -99,14 +111,14 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     const int wave = wave_wg % NW;  // which steps of K
     const int rg = wave_wg / NW;    // which 16 rows of the workgroup's NR x 16
     const int K = a.K, N = a.N, M = GATHER ? 1 : a.M;
-    const int groups = K >> 6;
+    const int groups = K >> (G32 ? 5 : 6);
     const int halves = K >> 7;             // 128-code halves of a row (K % 128 == 0)
     const int chunks = (halves + 1) >> 1;  // the last chunk may be a single half
     static_assert(CPS >= 2 && CPS <= 4, "a step holds 2..4 chunks (one lane group per chunk for the scales)");
     const int supers = (chunks + CPS - 1) / CPS;  // the last step may hold fewer chunks
     const uint32_t xs_off = 0;
     const uint32_t a2_off = (uint32_t)M * K * 2;
-    const uint32_t zero_off = a2_off + (uint32_t)M * chunks * 48;
+    const uint32_t zero_off = a2_off + (uint32_t)M * chunks * A2B;
     const uint32_t red_off = zero_off + kDiagZeroBytes;
 
     // gather: the route's expert slab and activation row
@@ -144,8 +156,9 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
         // half row adds the other quad (DPP, no LDS round trips)
         sum += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sum), 0xB1, 0xF, 0xF, true));
         sum += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sum), 0x4E, 0xF, 0xF, true));
-        sum += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sum), 0x141, 0xF, 0xF, true));
-        if ((p & 7) == 0) {
+        if constexpr (!G32)
+            sum += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sum), 0x141, 0xF, 0xF, true));
+        if ((p & (G32 ? 3 : 7)) == 0) {
             const uint32_t u0 = __float_as_uint(sum) & 0xffff0000u;
             const float r1 = sum - __uint_as_float(u0);
             const uint32_t u1 = __float_as_uint(r1) & 0xffff0000u;
@@ -156,12 +169,13 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
             const uint32_t n2 = __float_as_uint(-128.0f * __uint_as_float(u2));
             // group g of token t: 12 bytes at [t][chunk g / 4][g % 4]
             const uint32_t t = (uint32_t)p / (uint32_t)ppt;
-            const uint32_t g = ((uint32_t)p - t * (uint32_t)ppt) >> 3;
-            uint32_t* e = reinterpret_cast<uint32_t*>(lds_raw + a2_off + (t * chunks + (g >> 2)) * 48 + (g & 3) * 12);
+            const uint32_t g = ((uint32_t)p - t * (uint32_t)ppt) >> (G32 ? 2 : 3);
+            uint32_t* e = G32 ? reinterpret_cast<uint32_t*>(lds_raw + a2_off + (t * chunks + (g >> 3)) * 96 + (g & 7) * 12)
+                              : reinterpret_cast<uint32_t*>(lds_raw + a2_off + (t * chunks + (g >> 2)) * 48 + (g & 3) * 12);
             e[0] = (u0 >> 16) | u1;  // (X0, X1)
             e[1] = (u2 >> 16) | n0;  // (X2, -128 X0)
             e[2] = (n1 >> 16) | n2;  // (-128 X1, -128 X2)
-            if ((halves & 1) && (int)g == groups - 1) {
+            if (!G32 && (halves & 1) && (int)g == groups - 1) {
                 // a last chunk of one half: its two missing groups must add nothing to the affine term
 #pragma unroll
                 for (int q = 3; q < 9; q++) e[q] = 0;
@@ -193,8 +207,8 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     // ---- per-lane constants ----
     const int n = lane & 15;   // weight row of the lane (B operand, D column)
     const int j = lane >> 4;   // lane group: which 16 bytes of a 64-byte row piece (B), token (D)
-    const int at = (lane & 15) >> 2;  // A operand: token of the lane's A row
-    const int ag = lane & 3;          // A operand: group slot of the lane's A row
+    const int at = G32 ? (lane & 15) >> 3 : (lane & 15) >> 2;  // A operand: token of the lane's A row
+    const int ag = G32 ? lane & 7 : lane & 3;                  // A operand: group slot of the lane's A row
     const int row0 = (PAIR ? block : block * NR + rg) * kDiagRows;
     int row = row0 + n;
     if (row >= N) row = N - 1;
@@ -206,7 +220,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     const gptr_t bg = uniform_ptr(reinterpret_cast<const char*>(other ? a.b2 : a.b) + srow * groups * 2);
     const uint32_t w_lane = (uint32_t)row * (uint32_t)(K >> 1) + (uint32_t)j * 16;  // bytes
     // scales and biases: lane group j holds the four groups of chunk j of the step
-    const uint32_t sb_lane = (uint32_t)row * (uint32_t)groups * 2 + (uint32_t)j * 8;  // bytes
+    const uint32_t sb_lane = (uint32_t)row * (uint32_t)groups * 2 + (uint32_t)j * SBB;  // bytes
 
     // A fragments: load L (0, 1) of a chunk holds groups 2L and 2L + 1; lane group j holds codes of group
     // 2L + (j >> 1).  The lane's A row (at, ag) is non-zero in load L iff ag == 2L + (j >> 1).
@@ -214,10 +228,10 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     uint32_t a_base0[MT], a_base1[MT], a_mul0[MT], a_mul1[MT], a_chunk0[MT], a_chunk1[MT], a2_base[MT], a2_mul[MT];
 #pragma unroll
     for (int tg = 0; tg < MT; tg++) {
-        const int token = tg * 4 + at;
+        const int token = tg * TPS + at;
         const bool tok = token < M;
-        const bool d0 = tok && ag == (j >> 1);
-        const bool d1 = tok && ag == 2 + (j >> 1);
+        const bool d0 = tok && ag == (G32 ? j : j >> 1);
+        const bool d1 = tok && ag == (G32 ? 4 + j : 2 + (j >> 1));
         const uint32_t x_lane = xs_off + (uint32_t)token * K * 2 + (uint32_t)j * 64;  // codes j*32.. of a 128-code load
         a_base0[tg] = d0 ? x_lane : zero_off;
         a_base1[tg] = d1 ? x_lane + 256 : zero_off;
@@ -226,8 +240,8 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
         a_chunk0[tg] = d0 ? 512 : 0;
         a_chunk1[tg] = d1 ? 512 : 0;
         const bool d2 = tok && ag == 0;
-        a2_base[tg] = d2 ? a2_off + ((uint32_t)token * chunks + j) * 48 : zero_off;
-        a2_mul[tg] = d2 ? CPS * 48 : 0;
+        a2_base[tg] = d2 ? a2_off + ((uint32_t)token * chunks + j) * A2B : zero_off;
+        a2_mul[tg] = d2 ? CPS * A2B : 0;
     }
     // the lane that holds the scales of chunk 0 of the step for this lane's row (ds_bpermute byte address)
     const int sc_addr = n * 4;
@@ -236,7 +250,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     const uint32_t magic = opaque_v(kMagic128);
 
     uint4 wq[SUP][CPS][2];
-    uint2 sq[SUP], bq[SUP];
+    uint4 sq[SUP], bq[SUP];  // (group 64: x and y only)
 #pragma unroll
     for (int u = 0; u < SUP; u++) {
         int sp = wave + u * NW;
@@ -253,10 +267,16 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
         // A last chunk of one half has two groups: its 8 bytes are read 4 bytes early (inside the row) and the
         // upper word, which holds the two groups, moves down.
         const bool halfl = (halves & 1) && j < CPS && CPS * sp + j == chunks - 1;
-        const uint32_t so = sb_lane + (uint32_t)sp * (CPS * 8) - (j < valid ? 0u : (uint32_t)j * 8) - (halfl ? 4u : 0u);
-        sq[u] = load_u64_at(sg, so);
-        bq[u] = load_u64_at(bg, so);
-        if (halves & 1) {
+        const uint32_t so = sb_lane + (uint32_t)sp * (CPS * SBB) - (j < valid ? 0u : (uint32_t)j * SBB) - (halfl ? 4u : 0u);
+        if constexpr (G32) {
+            sq[u] = load_u128_at(sg, so);
+            bq[u] = load_u128_at(bg, so);
+        } else {
+            const uint2 s2 = load_u64_at(sg, so), b2 = load_u64_at(bg, so);
+            sq[u] = make_uint4(s2.x, s2.y, 0, 0);
+            bq[u] = make_uint4(b2.x, b2.y, 0, 0);
+        }
+        if (!G32 && (halves & 1)) {
             sq[u].x = halfl ? sq[u].y : sq[u].x;
             bq[u].x = halfl ? bq[u].y : bq[u].x;
         }
@@ -287,27 +307,33 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
         const int sp = wave + u * NW;
         if (sp < supers) {
             const int valid = min(CPS, chunks - CPS * sp);
-            const uint2 sv = sq[u], bv = bq[u];
-            // affine term of the 16 groups of the step: 24 k-slots per lane, three MFMAs
+            const uint4 sv = sq[u], bv = bq[u];
+            // affine term of the groups of the step: six k-slots per group (b b b s s s), 24 (group 32: 48) per lane
             {
-                // (b0 b0 b0 s0 s0 s0 b1 b1 | b1 s1 s1 s1 b2 b2 b2 s2 | s2 s2 b3 b3 b3 s3 s3 s3)
                 const uint32_t lo2 = 0x01000100u, hi2 = 0x03020302u, lolo = 0x05040100u, hihi = 0x07060302u;
-                const uint32_t e0 = __builtin_amdgcn_perm(bv.x, bv.x, lo2), e1 = __builtin_amdgcn_perm(sv.x, bv.x, lolo);
-                const uint32_t e2 = __builtin_amdgcn_perm(sv.x, sv.x, lo2), e3 = __builtin_amdgcn_perm(bv.x, bv.x, hi2);
-                const uint32_t e4 = __builtin_amdgcn_perm(sv.x, bv.x, hihi), e5 = __builtin_amdgcn_perm(sv.x, sv.x, hi2);
-                const uint32_t e6 = __builtin_amdgcn_perm(bv.y, bv.y, lo2), e7 = __builtin_amdgcn_perm(sv.y, bv.y, lolo);
-                const uint32_t e8 = __builtin_amdgcn_perm(sv.y, sv.y, lo2), e9 = __builtin_amdgcn_perm(bv.y, bv.y, hi2);
-                const uint32_t e10 = __builtin_amdgcn_perm(sv.y, bv.y, hihi), e11 = __builtin_amdgcn_perm(sv.y, sv.y, hi2);
+                constexpr int NWORD = G32 ? 4 : 2;  // words of two groups each
+                const uint32_t sw[4] = {sv.x, sv.y, sv.z, sv.w}, bw[4] = {bv.x, bv.y, bv.z, bv.w};
+                uint32_t e[6 * NWORD];
+#pragma unroll
+                for (int w = 0; w < NWORD; w++) {
+                    // (b0 b0 | b0 s0 | s0 s0 | b1 b1 | b1 s1 | s1 s1) of the word's two groups
+                    e[6 * w + 0] = __builtin_amdgcn_perm(bw[w], bw[w], lo2);
+                    e[6 * w + 1] = __builtin_amdgcn_perm(sw[w], bw[w], lolo);
+                    e[6 * w + 2] = __builtin_amdgcn_perm(sw[w], sw[w], lo2);
+                    e[6 * w + 3] = __builtin_amdgcn_perm(bw[w], bw[w], hi2);
+                    e[6 * w + 4] = __builtin_amdgcn_perm(sw[w], bw[w], hihi);
+                    e[6 * w + 5] = __builtin_amdgcn_perm(sw[w], sw[w], hi2);
+                }
 #pragma unroll
                 for (int tg = 0; tg < MT; tg++) {
                     // (lane groups past the last chunk of the row contribute zeros)
                     const uint32_t a2_addr = j < valid ? a2_base[tg] + (uint32_t)sp * a2_mul[tg] : zero_off;
-                    const bf16x8_t a20 = *reinterpret_cast<const bf16x8_t*>(lds_raw + a2_addr);
-                    const bf16x8_t a21 = *reinterpret_cast<const bf16x8_t*>(lds_raw + a2_addr + 16);
-                    const bf16x8_t a22 = *reinterpret_cast<const bf16x8_t*>(lds_raw + a2_addr + 32);
-                    dsum[tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a20, as_bf16x8(e0, e1, e2, e3), dsum[tg], 0, 0, 0);
-                    dsum[tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a21, as_bf16x8(e4, e5, e6, e7), dsum[tg], 0, 0, 0);
-                    dsum[tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a22, as_bf16x8(e8, e9, e10, e11), dsum[tg], 0, 0, 0);
+#pragma unroll
+                    for (int q = 0; q < 6 * NWORD / 4; q++) {
+                        const bf16x8_t a2 = *reinterpret_cast<const bf16x8_t*>(lds_raw + a2_addr + q * 16);
+                        dsum[tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            a2, as_bf16x8(e[4 * q], e[4 * q + 1], e[4 * q + 2], e[4 * q + 3]), dsum[tg], 0, 0, 0);
+                    }
                 }
             }
             uint32_t a_addr0[MT], a_addr1[MT];
@@ -329,8 +355,15 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
                     }
                 }
                 // the four scales of chunk cc of this lane's row sit in lane group cc
-                const uint32_t sx = (uint32_t)__builtin_amdgcn_ds_bpermute(sc_addr + cc * 64, (int)sv.x);
-                const uint32_t sy = (uint32_t)__builtin_amdgcn_ds_bpermute(sc_addr + cc * 64, (int)sv.y);
+                uint32_t sx = (uint32_t)__builtin_amdgcn_ds_bpermute(sc_addr + cc * 64, (int)sv.x);
+                uint32_t sy = (uint32_t)__builtin_amdgcn_ds_bpermute(sc_addr + cc * 64, (int)sv.y);
+                if constexpr (G32) {
+                    // this lane's D registers are groups 4 (j & 1) .. + 3 of the chunk's eight
+                    const uint32_t sz = (uint32_t)__builtin_amdgcn_ds_bpermute(sc_addr + cc * 64, (int)sv.z);
+                    const uint32_t sw2 = (uint32_t)__builtin_amdgcn_ds_bpermute(sc_addr + cc * 64, (int)sv.w);
+                    sx = (j & 1) ? sz : sx;
+                    sy = (j & 1) ? sw2 : sy;
+                }
                 f32x4_t dq[MT];
 #pragma unroll
                 for (int tg = 0; tg < MT; tg++) dq[tg] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
@@ -378,13 +411,36 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
                 float up = red[(NW * MT + tg) * 64 + lane];
 #pragma unroll
                 for (int w2 = 1; w2 < NW; w2++) up += red[((NW + w2) * MT + tg) * 64 + lane];
+                static_assert(!G32, "the pair kernels are built for group 64");
                 total = fmul_unfused(act_value(a.act, total), up);
             }
             if constexpr (GATHER) {
                 if (!route_ok) total = 0.0f;
             }
-            const int t = tg * 4 + j, r = row0 + n;
-            if (t < M && r < N) {
+            if constexpr (G32) total += __shfl_xor(total, 16);  // the two halves of a token's groups
+            const int t = G32 ? (j >> 1) : tg * 4 + j, r = row0 + n;
+            if constexpr (HEAD != 0) {
+                // lanes 0..15 hold the scores of rows row0 .. row0 + 15 for the one activation row
+                unsigned long long packed = 0;
+                if (lane < 16 && r < N && isfinite(total) && !token_suppressed((uint32_t)r, a.suppress, a.suppress_count))
+                    packed = pack_score_index(total, (uint32_t)r);
+                if constexpr (HEAD == 4) {
+                    if (lane < 16 && r < N) reinterpret_cast<unsigned long long*>(a.y)[r] = packed;
+                } else {
+                    // maximum over the 16 lanes, 32 bits at a time (the halves travel together)
+                    uint32_t hi = (uint32_t)(packed >> 32), lo = (uint32_t)packed;
+#pragma unroll
+                    for (int d = 8; d >= 1; d >>= 1) {
+                        const uint32_t ohi = (uint32_t)__shfl_xor((int)hi, d), olo = (uint32_t)__shfl_xor((int)lo, d);
+                        const bool take = ohi > hi || (ohi == hi && olo > lo);
+                        hi = take ? ohi : hi;
+                        lo = take ? olo : lo;
+                    }
+                    if (lane == 0) a.partial[(size_t)block * NR + rg] = ((unsigned long long)hi << 32) | lo;
+                }
+                continue;
+            }
+            if (t < M && r < N && (!G32 || (j & 1) == 0)) {
                 const size_t o = (size_t)(GATHER ? y_row : t) * N + r;
                 if (a.out_f32) {
                     static_cast<float*>(a.y)[o] = total;
@@ -404,6 +460,18 @@ __global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_kernel(const QmvArgs a
 template <int NW, int SUP, int CPS>
 __global__ __launch_bounds__(2 * NW* kWave) void qmv_diag_pair_kernel(const QmvArgs a) {
     qmv_diag_body<NW, SUP, 2, true, 1, false, CPS>(a, (int)blockIdx.x);
+}
+
+// Quantisation groups of 32 codes, up to two activation rows.
+template <int NW, int SUP, int NR, int CPS>
+__global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_g32_kernel(const QmvArgs a) {
+    qmv_diag_body<NW, SUP, NR, false, 1, false, CPS, true>(a, (int)blockIdx.x);
+}
+
+// lm_head forms (one activation row): packed scores (4) or the best packed value per 16 rows (3).
+template <int NW, int SUP, int NR, int CPS, bool G32, int HEAD>
+__global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_head_kernel(const QmvArgs a) {
+    qmv_diag_body<NW, SUP, NR, false, 1, false, CPS, G32, HEAD>(a, (int)blockIdx.x);
 }
 
 // Gathered forms: grid.y = routes.
@@ -466,6 +534,15 @@ struct QmvDiagEntry {
     {                                                                                                              \
         {"qmvd_b4_m8_r" #NR "_w" #NW "_d" #SUP "_g0_c3", 4, 8, NR, NW, SUP, 0, 3, 4}, qmv_diag_kernel<NW, SUP, NR, 2, 3> \
     }
+// kind 5: quantisation groups of 32 codes
+#define AQ_QMVDS(NW, SUP, NR)                                                                                          \
+    {                                                                                                                  \
+        {"qmvd_b4_m2_r" #NR "_w" #NW "_d" #SUP "_g0_s32", 4, 2, NR, NW, SUP, 0, 0, 5}, qmv_diag_g32_kernel<NW, SUP, NR, 4> \
+    }
+#define AQ_QMVDS3(NW, SUP, NR)                                                                                            \
+    {                                                                                                                     \
+        {"qmvd_b4_m2_r" #NR "_w" #NW "_d" #SUP "_g0_s32_c3", 4, 2, NR, NW, SUP, 0, 3, 5}, qmv_diag_g32_kernel<NW, SUP, NR, 3> \
+    }
 static const QmvDiagEntry kQmvDiagTable[] = {
     AQ_QMVD(4, 1, 1), AQ_QMVD(4, 1, 2), AQ_QMVD(4, 1, 4), AQ_QMVD(2, 2, 2), AQ_QMVD(2, 1, 2), AQ_QMVD(8, 1, 1),
     AQ_QMVD(4, 2, 1), AQ_QMVD(2, 1, 4), AQ_QMVD(6, 1, 1), AQ_QMVD(10, 1, 1), AQ_QMVD(12, 1, 1),
@@ -473,9 +550,11 @@ static const QmvDiagEntry kQmvDiagTable[] = {
     AQ_QMVDG(2, 1, 1), AQ_QMVDG(2, 1, 2), AQ_QMVDG(4, 1, 1), AQ_QMVDG(4, 1, 2), AQ_QMVDG(6, 1, 1), AQ_QMVDG(8, 1, 1),
     AQ_QMVD3(4, 1, 1), AQ_QMVD3(4, 1, 2), AQ_QMVD3(4, 1, 4), AQ_QMVD3(2, 1, 2), AQ_QMVD3(2, 1, 4),
     AQ_QMVD83(4, 1, 4), AQ_QMVD83(4, 1, 2), AQ_QMVD83(2, 1, 4), AQ_QMVDG3(2, 1, 2), AQ_QMVDG3(4, 1, 1),
+    AQ_QMVDS(2, 1, 2), AQ_QMVDS(4, 1, 1), AQ_QMVDS(4, 1, 2), AQ_QMVDS(8, 1, 1), AQ_QMVDS3(2, 1, 2), AQ_QMVDS3(4, 1, 1),
 };
 
 static int cps_of(const QmvVariant& v) { return v.xmode ? v.xmode : 4; }
+static bool g32_of(const QmvVariant& v) { return v.kind == 5; }
 // Steps of cps chunks of 256 codes that cover K (its last chunk may be a single half of 128 codes).
 static int steps_for(int K, int cps) { return ((K + kDiagChunk - 1) / kDiagChunk + cps - 1) / cps; }
 // Chunks per step for this K: three where the even number of wavefronts that four would need holds them too (the
@@ -495,7 +574,9 @@ const QmvVariant* qmvd_variant(int idx) {
 
 bool qmvd_fits(const QmvArgs& a, int bits, int group_size, bool gather, int idx) {
     const QmvVariant* v = qmvd_variant(idx);
-    if (!v || bits != 4 || group_size != 64 || gather != (v->gather != 0)) return false;
+    if (!v || bits != 4 || group_size != (g32_of(*v) ? 32 : 64) || gather != (v->gather != 0)) return false;
+    if (g32_of(*v) && (a.K % kDiagChunk != 0 || ((reinterpret_cast<uintptr_t>(a.s) | reinterpret_cast<uintptr_t>(a.b)) & 15)))
+        return false;
     if (gather && (a.M != 1 || a.routes < 1 || a.routes > 65535)) return false;
     if (a.M < 1 || a.M > v->m || a.K <= 0 || a.K % 128 != 0 || a.N < 1) return false;
     if (steps_for(a.K, cps_of(*v)) > v->waves * v->depth) return false;
@@ -504,13 +585,13 @@ bool qmvd_fits(const QmvArgs& a, int bits, int group_size, bool gather, int idx)
     if ((al16 & 15) || (al8 & 7)) return false;
     // 32-bit byte offsets into the packed matrix
     if ((uint64_t)a.N * (uint64_t)(a.K / 2) >= (1ull << 32)) return false;
-    return qmvd_lds_bytes_for(a.M, a.K, v->waves * v->rows, (v->m + 3) / 4) <= 96 * 1024;
+    return qmvd_lds_bytes_for(a.M, a.K, v->waves * v->rows, (v->m + 3) / 4, g32_of(*v)) <= 96 * 1024;
 }
 
 hipError_t qmvd_launch(int idx, const QmvArgs& a, hipStream_t stream) {
     if (idx < 0 || idx >= qmvd_variant_count()) return hipErrorInvalidValue;
     const QmvDiagEntry& e = kQmvDiagTable[idx];
-    const size_t lds = qmvd_lds_bytes_for(a.M, a.K, e.v.waves * e.v.rows, (e.v.m + 3) / 4);
+    const size_t lds = qmvd_lds_bytes_for(a.M, a.K, e.v.waves * e.v.rows, (e.v.m + 3) / 4, g32_of(e.v));
     if (lds > 48 * 1024) {
         hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e.fn),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -549,7 +630,25 @@ int qmvd_pick(int M, int K, int N) {
     if (cap == 8 && nw == 2) nr = 4;
     for (int i = 0; i < qmvd_variant_count(); i++) {
         const QmvVariant& v = kQmvDiagTable[i].v;
-        if (v.waves == nw && v.depth == 1 && v.rows == nr && v.m == cap && !v.gather && cps_of(v) == cps) return i;
+        if (v.waves == nw && v.depth == 1 && v.rows == nr && v.m == cap && !v.gather && cps_of(v) == cps && !g32_of(v)) return i;
+    }
+    return -1;
+}
+
+// The group-32 variant for up to two rows and this K (a multiple of 256), or -1.
+int qmvd_pick_g32(int M, int K, int N) {
+    if (M < 1 || M > 2 || K <= 1024 || K % kDiagChunk != 0) return -1;
+    const int cps = cps_for(K);
+    const int steps = steps_for(K, cps);
+    if (steps > 8) return -1;
+    const int nw = (steps + 1) & ~1;
+    int nr = nw == 2 ? 2 : (nw == 4 && M == 2 && N >= 4096) ? 2 : 1;
+    for (int pass = 0; pass < 2; pass++) {
+        for (int i = 0; i < qmvd_variant_count(); i++) {
+            const QmvVariant& v = kQmvDiagTable[i].v;
+            if (g32_of(v) && v.waves == nw && v.depth == 1 && v.rows == nr && cps_of(v) == cps) return i;
+        }
+        nr = 1;
     }
     return -1;
 }
@@ -568,7 +667,7 @@ static const QmvDiagPairEntry* find_pair(int idx) {
     const QmvVariant* v = qmvd_variant(idx);
     if (v)
         for (const QmvDiagPairEntry& e : kQmvDiagPairTable)
-            if (e.nw == v->waves && e.sup == v->depth && e.cps == cps_of(*v)) return &e;
+            if (e.nw == v->waves && e.sup == v->depth && e.cps == cps_of(*v) && !g32_of(*v)) return &e;
     return nullptr;
 }
 bool qmvd_pair_supported(int idx) { return find_pair(idx) != nullptr; }
@@ -598,9 +697,51 @@ int qmvd_pick_gather(int K) {
     const int nr = nw == 2 ? 2 : 1;
     for (int i = 0; i < qmvd_variant_count(); i++) {
         const QmvVariant& v = kQmvDiagTable[i].v;
-        if (v.gather && v.waves == nw && v.depth == 1 && v.rows == nr && cps_of(v) == cps) return i;
+        if (v.gather && v.waves == nw && v.depth == 1 && v.rows == nr && cps_of(v) == cps && !g32_of(v)) return i;
     }
     return -1;
+}
+
+// lm_head epilogues on variant idx's split of K: fuse 4 writes packed scores to a.y, fuse 3 one partial maximum per
+// set of 16 rows into a.partial (qmvd_head_partials slots), which the caller folds.
+struct QmvDiagHeadEntry {
+    int nw, sup, nr, cps, g32, fuse;
+    QmvDiagKernel fn;
+};
+#define AQ_QMVD_HEAD(NW, NR, CPS, G32) \
+    {NW, 1, NR, CPS, G32, 3, qmv_diag_head_kernel<NW, 1, NR, CPS, (G32 != 0), 3>}, {NW, 1, NR, CPS, G32, 4, qmv_diag_head_kernel<NW, 1, NR, CPS, (G32 != 0), 4>}
+static const QmvDiagHeadEntry kQmvDiagHeadTable[] = {
+    AQ_QMVD_HEAD(2, 2, 3, 1), AQ_QMVD_HEAD(2, 2, 4, 1), AQ_QMVD_HEAD(4, 1, 4, 1), AQ_QMVD_HEAD(4, 1, 3, 1),
+    AQ_QMVD_HEAD(2, 2, 3, 0), AQ_QMVD_HEAD(2, 2, 4, 0), AQ_QMVD_HEAD(4, 1, 4, 0), AQ_QMVD_HEAD(4, 1, 3, 0),
+};
+static const QmvDiagHeadEntry* find_head(int idx, int fuse) {
+    const QmvVariant* v = qmvd_variant(idx);
+    if (v && !v->gather)
+        for (const QmvDiagHeadEntry& e : kQmvDiagHeadTable)
+            if (e.nw == v->waves && e.sup == v->depth && e.nr == v->rows && e.cps == cps_of(*v) &&
+                (e.g32 != 0) == g32_of(*v) && e.fuse == fuse)
+                return &e;
+    return nullptr;
+}
+bool qmvd_head_supported(int idx, int fuse) { return find_head(idx, fuse) != nullptr; }
+size_t qmvd_head_partials(int idx, int N) {
+    const QmvVariant* v = qmvd_variant(idx);
+    const int wg_rows = kDiagRows * (v ? v->rows : 1);
+    return (size_t)((N + wg_rows - 1) / wg_rows) * (v ? v->rows : 1);
+}
+hipError_t qmvd_head_launch(int idx, int fuse, const QmvArgs& a, hipStream_t stream) {
+    const QmvDiagHeadEntry* e = find_head(idx, fuse);
+    if (!e || a.M != 1 || (fuse == 3 && !a.partial)) return hipErrorInvalidValue;
+    const size_t lds = qmvd_lds_bytes_for(1, a.K, e->nw * e->nr, 1, e->g32 != 0);
+    if (lds > 48 * 1024) {
+        hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e->fn),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (rc != hipSuccess) return rc;
+    }
+    const int wg_rows = kDiagRows * e->nr;
+    hipLaunchKernelGGL(e->fn, dim3((unsigned)((a.N + wg_rows - 1) / wg_rows)), dim3((unsigned)(e->nw * e->nr * kWave)), lds,
+                       stream, a);
+    return hipGetLastError();
 }
 
 typedef void (*QmvDiagMultiKernel)(const QmvMultiArgs);
@@ -622,7 +763,7 @@ bool qmvd_multi_supported(int idx) {
     const QmvVariant* v = qmvd_variant(idx);
     if (!v) return false;
     for (const QmvDiagMultiEntry& e : kQmvDiagMultiTable)
-        if (e.nw == v->waves && e.sup == v->depth && e.nr == v->rows && e.cps == cps_of(*v)) return true;
+        if (e.nw == v->waves && e.sup == v->depth && e.nr == v->rows && e.cps == cps_of(*v) && !g32_of(*v)) return true;
     return false;
 }
 

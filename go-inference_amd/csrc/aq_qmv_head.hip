@@ -116,6 +116,12 @@ hipError_t qmv_head_launch(int bits, int fuse, int rows, const QmvArgs& a, hipSt
     return hipGetLastError();
 }
 
+hipError_t head_fold_launch(const unsigned long long* partial, int count, unsigned long long* fold, unsigned long long* best,
+                            hipStream_t stream) {
+    hipLaunchKernelGGL(fold_best_kernel, dim3(kHeadFoldGroups), dim3(256), 0, stream, partial, count, fold, best);
+    return hipGetLastError();
+}
+
 // grid.y = activation row; a workgroup folds its share of a row before touching the shared maximum
 __global__ __launch_bounds__(256) void pack_scores_kernel(const float* __restrict__ scores, int N, const int32_t* suppress,
                                                           int suppress_count, unsigned long long* best,

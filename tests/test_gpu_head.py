@@ -57,7 +57,8 @@ def _greedy(ctx, x, dw, M, K, N, gs, bits, suppress=None):
 @pytest.mark.parametrize("bits,gs,M,K,N,fused", [(4, 32, 1, 1536, 32768, True), (4, 64, 1, 4096, 20011, True),
                                                  (8, 64, 1, 1024, 4096, True), (4, 64, 1, 512, 37, True),
                                                  (6, 32, 1, 192, 301, False), (4, 64, 3, 512, 1000, False),
-                                                 (4, 64, 20, 1024, 515, False)])
+                                                 (4, 64, 20, 1024, 515, False), (4, 32, 1, 2048, 1000, True),
+                                                 (4, 64, 1, 2816, 777, True), (4, 32, 1, 4096, 50, True)])
 def test_greedy_and_scores_against_oracle(ctx, orc, bits, gs, M, K, N, fused):
     say("head", bits, gs, M, K, N)
     if 32 % bits == 0:
@@ -73,8 +74,10 @@ def test_greedy_and_scores_against_oracle(ctx, orc, bits, gs, M, K, N, fused):
     suppress = [int(np.argmax(ref[0])), 5, N - 1]
     for sup in (None, suppress):
         packed = _scores(ctx, x, dw, M, K, N, gs, bits, sup)
+        # 4-bit codes in groups of 32 or 64 with more than 1024 columns: the diagonal-MFMA kernels
+        diag = bits == 4 and K > 1024 and (K % 256 == 0 if gs == 32 else K % 128 == 0)
         if fused:
-            assert ctx.last_variant(0) == "qmv_scores_dot2"
+            assert ctx.last_variant(0) == ("qmv_scores_diag" if diag else "qmv_scores_dot2")
         toks, dev = _unpack_all(packed)
         live = packed != 0
         if sup is not None:
@@ -89,7 +92,7 @@ def test_greedy_and_scores_against_oracle(ctx, orc, bits, gs, M, K, N, fused):
         check_accumulators(dev, ref, "packed scores")
         best = _greedy(ctx, x, dw, M, K, N, gs, bits, sup)
         if fused:
-            assert ctx.last_variant(0) == "qmv_greedy_dot2"
+            assert ctx.last_variant(0) == ("qmv_greedy_diag" if diag else "qmv_greedy_dot2")
         for m in range(M):
             tok, sc = _unpack(best[m])
             want_tok, want_sc = orc.greedy_sample_suppress(dev[m], sup)

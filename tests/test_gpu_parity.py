@@ -351,31 +351,34 @@ def test_qmvd_every_variant(ctx, orc):
             steps = waves * int(name.split("_d")[1].split("_")[0])
             wg_waves = waves * int(name.split("_r")[1].split("_")[0])
             step = 768 if name.endswith("_c3") else 1024  # codes per wavefront step
+            gs = 32 if "_s32" in name else 64             # (group 32: K in whole chunks of 256 codes)
             for K in sorted({step * steps, step * max(1, steps - 1), step * steps - 256, step * (steps - 1) + 256,
                              step * steps - 128, step * (steps - 1) + 128}):
+                if gs == 32 and K % 256:
+                    continue
                 say("variant", idx, name, "K", K)
-                if K not in data:
-                    words, s, b = F.synthetic_affine(N, K, bits, 64, seed=530 + K // 128)
+                if (K, gs) not in data:
+                    words, s, b = F.synthetic_affine(N, K, bits, gs, seed=530 + K // 128)
                     x = F.synthetic_x(8, K, seed=630 + K // 128)
-                    data[K] = (DeviceAffine(ctx, words, s, b), x, F.reference_f64(x, words, s, b, bits, 64, K))
-                dw, x, ref = data[K]
+                    data[(K, gs)] = (DeviceAffine(ctx, words, s, b), x, F.reference_f64(x, words, s, b, bits, gs, K))
+                dw, x, ref = data[(K, gs)]
                 ctx.force_variant(0, idx)
-                for rows in ((1, 2, 3, 4) if m == 4 else (1, 4, 5, 7, 8)):
-                    if rows * K * 2 + rows * (K // 256) * 48 + 64 + wg_waves * (m // 4) * 256 > 96 * 1024:
+                for rows in ((1, 2) if m == 2 else (1, 2, 3, 4) if m == 4 else (1, 4, 5, 7, 8)):
+                    if rows * K * 2 + rows * ((K + 255) // 256) * (96 if gs == 32 else 48) + 128 + wg_waves * max(1, m // 4) * 256 > 96 * 1024:
                         # the activations of all rows and their group sums sit in LDS: beyond 96 KiB the variant refuses
                         with pytest.raises(aq_mi355.AqError) as ei:
-                            run_qmv(ctx, x[:rows], dw, rows, K, N, 64, bits, True)
+                            run_qmv(ctx, x[:rows], dw, rows, K, N, gs, bits, True)
                         assert ei.value.code == aq_mi355.AQ_ERR_ARG
                         continue
-                    acc = run_qmv(ctx, x[:rows], dw, rows, K, N, 64, bits, True)
+                    acc = run_qmv(ctx, x[:rows], dw, rows, K, N, gs, bits, True)
                     assert ctx.last_variant(0) == name
                     check_accumulators(acc, ref[:rows], "%s rows=%d" % (name, rows))
-                out = run_qmv(ctx, x[:2], dw, 2, K, N, 64, bits, False)
+                out = run_qmv(ctx, x[:2], dw, 2, K, N, gs, bits, False)
                 check_bf16_store(out, ref[:2], name)
-            dw, x, ref = data[step * steps]
+            dw, x, ref = data[(step * steps, gs)]
             for bad_k in (step * steps - 64, step * steps + 256):
                 with pytest.raises(aq_mi355.AqError) as ei:
-                    run_qmv(ctx, np.zeros((1, bad_k), np.uint16), dw, 1, bad_k, N, 64, bits, True)
+                    run_qmv(ctx, np.zeros((1, bad_k), np.uint16), dw, 1, bad_k, N, gs, bits, True)
                 assert ei.value.code == aq_mi355.AQ_ERR_ARG
     finally:
         ctx.force_variant(0, -1)
@@ -451,6 +454,17 @@ def test_qmvd_is_the_default_for_few_rows(ctx, orc):
         acc = run_qmv(ctx, x, dw, 1, K, 40, 64, 4, True)
         assert ctx.last_variant(0).startswith("qmvd_"), ctx.last_variant(0)
         check_accumulators(acc, F.reference_f64(x, words, s, b, 4, 64, K), "diag default K=%d" % K)
+        dw.free()
+    for K in (1536, 4096, 3072):  # group 32: up to two rows
+        words, s, b = F.synthetic_affine(70, K, 4, 32, seed=860 + K // 256)
+        x = F.synthetic_x(2, K, seed=870 + K // 256)
+        ref = F.reference_f64(x, words, s, b, 4, 32, K)
+        dw = DeviceAffine(ctx, words, s, b)
+        for rows in (1, 2):
+            say("default group 32", K, rows)
+            acc = run_qmv(ctx, x[:rows], dw, rows, K, 70, 32, 4, True)
+            assert ctx.last_variant(0).startswith("qmvd_") and "_s32" in ctx.last_variant(0), ctx.last_variant(0)
+            check_accumulators(acc, ref[:rows], "diag g32 K=%d rows=%d" % (K, rows))
         dw.free()
     for K, bits, rows in ((17408, 4, 1), (1024, 4, 1), (4096, 8, 1), (8192, 4, 2), (2880, 4, 1)):
         words, s, b = F.synthetic_affine(32, K, bits, 64, seed=830)
