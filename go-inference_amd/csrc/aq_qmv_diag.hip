@@ -1,4 +1,5 @@
-// affine_qmv for gfx950, M = 1..4 activation rows of 4-bit group-64 codes: the diagonal-MFMA kernel.
+// affine_qmv / gather_qmv for gfx950, 4-bit codes in groups of 64 (1..8 activation rows) or 32 (1..2): the
+// diagonal-MFMA kernels, with their multi-matrix, gate|up pair, gathered and lm_head forms.
 //
 // Same contract as the dot2 kernel (aq_qmv.hip): replaces rocm_mlx_q4_projection*
 // (go/engine/hip/kernels/quant/affine_projection.hipinc:3-266), semantics of MLX affine_qmv
