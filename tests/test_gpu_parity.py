@@ -476,6 +476,60 @@ def test_qmvd_is_the_default_for_few_rows(ctx, orc):
         dw.free()
 
 
+def test_qmvd_default_paths_random_shapes(ctx, orc):
+    """The library's own choice over seeded random shapes the diagonal-MFMA kernels take: K any multiple of 128 (group
+    32: 256) from 1152 to 16384, ragged N, 1..8 (group 32: 1..2) activation rows; plain, multi-matrix and fused gate|up
+    calls, each against the float64 reference, and the byte-identity contracts between them."""
+    import aq_mi355
+    rng = np.random.default_rng(20240607)
+    for case in range(28):
+        gs = 32 if case % 4 == 3 else 64
+        K = int(rng.integers(1152 // 128, 16384 // 128 + 1)) * 128
+        if gs == 32:
+            K = max(1280, K // 256 * 256)
+        if case % 7 == 0:
+            K = int(rng.choice([2816, 1408, 3584, 5120, 11008, 14336]))
+            gs = 64
+        M = int(rng.integers(1, 3 if gs == 32 else 9))
+        if K > 4096 and M > 1:
+            M = 1 if gs == 64 else M
+        N = int(rng.integers(1, 300))
+        say("random diag shape", case, "K", K, "N", N, "M", M, "group", gs)
+        words, s, b = F.synthetic_affine(N, K, 4, gs, seed=9000 + case)
+        x = F.synthetic_x(M, K, seed=9100 + case)
+        ref = F.reference_f64(x, words, s, b, 4, gs, K)
+        dw = DeviceAffine(ctx, words, s, b)
+        acc = run_qmv(ctx, x, dw, M, K, N, gs, 4, True)
+        name = ctx.last_variant(0)
+        if not (gs == 32 and K > 8192):
+            assert name.startswith("qmvd_"), (name, K, N, M, gs)
+        check_accumulators(acc, ref, "random shape %d (%s)" % (case, name))
+        out = run_qmv(ctx, x, dw, M, K, N, gs, 4, False)
+        assert np.array_equal(out, F.f32_to_bf16_bits(acc).reshape(M, N)), "bf16 store is not the RNE of the accumulator"
+        # every row on its own: the same bytes
+        if M > 1:
+            one = run_qmv(ctx, x[M - 1:M], dw, 1, K, N, gs, 4, True)
+            assert np.array_equal(one[0].view(np.uint32), acc[M - 1].view(np.uint32)), (K, N, M, gs)
+        if gs == 64 and M <= 4:
+            # two matrices in one launch, and the fused gate|up of the same two
+            w2, s2, b2 = F.synthetic_affine(N, K, 4, gs, seed=9200 + case)
+            dw2 = DeviceAffine(ctx, w2, s2, b2)
+            dx = ctx.to_device(x)
+            ys = [ctx.alloc(M * N * 4), ctx.alloc(M * N * 4)]
+            ctx.qmv_multi(dx, [dw.w, dw2.w], [dw.s, dw2.s], [dw.b, dw2.b], ys, [N, N], M, K, gs, 4, aq_mi355.AQ_OUT_F32)
+            ctx.sync()
+            m0 = ys[0].download(np.float32, M * N).reshape(M, N)
+            m1 = ys[1].download(np.float32, M * N).reshape(M, N)
+            assert np.array_equal(m0.view(np.uint32), acc.view(np.uint32)), ("multi member 0", K, N, M)
+            acc2 = run_qmv(ctx, x, dw2, M, K, N, gs, 4, True)
+            assert np.array_equal(m1.view(np.uint32), acc2.view(np.uint32)), ("multi member 1", K, N, M)
+            check_accumulators(acc2, F.reference_f64(x, w2, s2, b2, 4, gs, K), "random shape %d, second matrix" % case)
+            for t in ys + [dx]:
+                t.free()
+            dw2.free()
+        dw.free()
+
+
 def test_qmvb_gather_every_variant(ctx, orc):
     """Each gather-capable block-MFMA variant, forced, against the oracle (batched x, row_base slab
     offset)."""
