@@ -55,6 +55,15 @@ class DeviceLinear(ctypes.Structure):
                 ("bits", _i), ("experts", _i)]
 
 
+class GgufAffineLayout(ctypes.Structure):
+    """aq_gguf_affine_layout (include/aq_mi355.h)."""
+    _fields_ = [("bits", _i), ("group_size", _i), ("packed_cols", _c.c_int64), ("groups", _c.c_int64),
+                ("src_bytes", _c.c_uint64), ("packed_bytes", _c.c_uint64), ("scales_bytes", _c.c_uint64)]
+
+
+GGUF_F32, GGUF_Q4_0, GGUF_Q4_1, GGUF_Q8_0, GGUF_Q4_K, GGUF_Q5_K, GGUF_Q6_K = 0, 2, 3, 8, 12, 13, 14
+
+
 # name -> (restype, argtypes); every symbol include/*.h declares
 PROTOTYPES = {
     "aq_version": (_cp, []),
@@ -101,6 +110,8 @@ PROTOTYPES = {
     "aq_upload_fused_gate_up": (_i, [_vp, _c.POINTER(HostLinear), _c.POINTER(HostLinear), _c.POINTER(DeviceLinear)]),
     "aq_free_device_linear": (_i, [_vp, _c.POINTER(DeviceLinear)]),
     "aq_dequant_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _c.c_int64, _i, _i, _i]),
+    "aq_gguf_affine_layout_of": (_i, [_i, _c.c_int64, _c.c_int64, _c.POINTER(GgufAffineLayout)]),
+    "aq_gguf_to_affine": (_i, [_vp, _i, _vp, _c.c_uint64, _c.c_int64, _c.c_int64, _vp, _vp, _vp]),
     "aq_matvec_host": (_i, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _i, _i, _i, _i, _vp, _sz]),
     "aq_proj_quant_matmul_host": (_i, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _i, _i, _i, _i, _i]),
     "aq_variant_count": (_i, [_i]),
@@ -364,6 +375,11 @@ class Context:
         self._check(self.lib.aq_dequant_f32(self.handle, _ptr(w), _ptr(s), _ptr(b), _ptr(out), N, K, group_size,
                                             bits))
 
+    def gguf_to_affine(self, gguf_type, src, src_bytes, rows, cols, packed, scales, biases):
+        """GGUF blocks at `src` (device) -> packed / scales / biases (device), sized by gguf_affine_layout()."""
+        self._check(self.lib.aq_gguf_to_affine(self.handle, gguf_type, _ptr(src), src_bytes, rows, cols, _ptr(packed),
+                                               _ptr(scales), _ptr(biases)))
+
     def force_variant(self, op, variant):
         self._check(self.lib.aq_force_variant(self.handle, op, variant))
 
@@ -439,6 +455,17 @@ class SafetensorsFile:
         if rc != AQ_OK:
             raise AqError(rc, self.lib.aqh_last_error().decode())
         return out
+
+
+def gguf_affine_layout(gguf_type, rows, cols):
+    """What a GGUF tensor of this type and shape repacks to (no device needed); raises AqError as the Go
+    repack returns errors."""
+    lib = load()
+    lay = GgufAffineLayout()
+    rc = lib.aq_gguf_affine_layout_of(gguf_type, rows, cols, ctypes.byref(lay))
+    if rc != AQ_OK:
+        raise AqError(rc, lib.aq_last_error().decode())
+    return lay
 
 
 def pack_best(score, token):

@@ -1380,6 +1380,44 @@ int aq_dequant_f32(aq_ctx* ctx, const void* packed, const void* scales, const vo
     return AQ_OK;
 }
 
+int aq_gguf_affine_layout_of(int gguf_type, int64_t rows, int64_t cols, aq_gguf_affine_layout* out) {
+    if (!out) return fail(AQ_ERR_ARG, "aq_gguf_affine_layout_of: out is null");
+    aq::GgufFormat f;
+    if (!aq::gguf_format(gguf_type, &f))
+        return fail(AQ_ERR_UNSUPPORTED, "aq_gguf_affine_layout_of: tensor must be GGUF affine-compatible (type %d)", gguf_type);
+    if (rows <= 0 || cols <= 0 || cols % f.block_cols != 0)
+        return fail(AQ_ERR_SHAPE, "aq_gguf_affine_layout_of: tensor shape must align to %d-column blocks", f.block_cols);
+    if (rows > (int64_t)0x7fffffff * 32 / cols * 256)
+        return fail(AQ_ERR_UNSUPPORTED, "aq_gguf_affine_layout_of: tensor too large");
+    out->bits = f.bits;
+    out->group_size = f.group_size;
+    out->packed_cols = cols * f.bits / 32;
+    out->groups = cols / f.group_size;
+    out->src_bytes = (uint64_t)rows * (uint64_t)(cols / f.block_cols) * (uint64_t)f.block_bytes;
+    out->packed_bytes = (uint64_t)rows * (uint64_t)out->packed_cols * 4;
+    out->scales_bytes = (uint64_t)rows * (uint64_t)out->groups * 2;
+    return AQ_OK;
+}
+
+int aq_gguf_to_affine(aq_ctx* ctx, int gguf_type, const void* src, uint64_t src_bytes, int64_t rows, int64_t cols,
+                      void* packed, void* scales, void* biases) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_gguf_to_affine: ctx is null");
+    aq_gguf_affine_layout lay;
+    if (int rc = aq_gguf_affine_layout_of(gguf_type, rows, cols, &lay)) return rc;
+    if (src_bytes != lay.src_bytes)
+        return fail(AQ_ERR_SHAPE, "aq_gguf_to_affine: tensor byte count %llu does not match dimensions (%llu)",
+                    (unsigned long long)src_bytes, (unsigned long long)lay.src_bytes);
+    if (!src || !packed || !scales || !biases) return fail(AQ_ERR_ARG, "aq_gguf_to_affine: null operand");
+    if (!aligned(packed, 16) || !aligned(scales, 2) || !aligned(biases, 2) || (gguf_type == aq::kGgufF32 && !aligned(src, 4)))
+        return fail(AQ_ERR_ARG, "aq_gguf_to_affine: packed must be 16-byte, scales/biases 2-byte, F32 input 4-byte aligned");
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    AQ_HIP(aq::gguf_repack_launch(gguf_type, static_cast<const uint8_t*>(src), static_cast<uint32_t*>(packed),
+                                  static_cast<uint16_t*>(scales), static_cast<uint16_t*>(biases), rows * (cols / 32),
+                                  ctx->stream),
+           "hipLaunchKernel");
+    return AQ_OK;
+}
+
 int aq_matvec_host(aq_ctx* ctx, const uint8_t* x, size_t x_len, const uint8_t* packed, size_t packed_len,
                    const uint8_t* scales, size_t scales_len, const uint8_t* biases, size_t biases_len, int out_dim,
                    int in_dim, int group_size, int bits, uint8_t* out, size_t out_len) {

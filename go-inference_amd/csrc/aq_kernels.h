@@ -223,4 +223,15 @@ hipError_t qmv_generic_launch(const QmvArgs& a, int bits, int group_size, bool g
 hipError_t dequant_launch(const uint32_t* w, const uint16_t* s, const uint16_t* b, float* out, int64_t N, int K,
                           int group_size, int bits, hipStream_t stream);
 
+// GGUF block formats -> affine layout (aq_gguf.hip).  Type ids are GGUF's own
+// (go/engine/hip/hip_gguf_affine_adapter.go:19-25, :56).
+constexpr int kGgufF32 = 0, kGgufQ4_0 = 2, kGgufQ4_1 = 3, kGgufQ8_0 = 8, kGgufQ4_K = 12, kGgufQ5_K = 13, kGgufQ6_K = 14;
+struct GgufFormat {
+    int block_cols, block_bytes, bits, group_size;
+};
+bool gguf_format(int type, GgufFormat* f);
+// spans = rows * cols / 32.  w 16-byte aligned, s and b 2-byte aligned, src 4-byte aligned for F32.
+hipError_t gguf_repack_launch(int type, const uint8_t* src, uint32_t* w, uint16_t* s, uint16_t* b, int64_t spans,
+                              hipStream_t stream);
+
 }  // namespace aq

@@ -288,6 +288,29 @@ int aq_upload_fused_gate_up(aq_ctx *ctx, const struct aqh_linear *gate, const st
 
 int aq_free_device_linear(aq_ctx *ctx, aq_device_linear *lin);
 
+/* GGUF block tensors -> affine tensors on the device, for checkpoints that ship Q4_0 / Q4_1 / Q8_0 / Q4_K / Q5_K /
+ * Q6_K blocks (or F32, quantised to eight bits in groups of 32) instead of MLX-affine triples.  Replaces the
+ * host round trip of synthesizeGemma4GGUFAffineTensor (go/engine/hip/hip_gguf_affine_adapter.go:199-218: device
+ * -> host copy, hipRepackGGUFKQuantToAffine :321-341 on the CPU, three uploads) with one kernel over the tensor
+ * where it lies; the three outputs are bit-identical to that function's payload (Weights / Scales / Biases,
+ * :61-71): Q4_0 -> 4 bits, group 32, bias -8*d; Q4_1 -> 4 bits, group 32; Q8_0 -> 8 bits, group 32, codes
+ * q + 128, bias -128*d; Q4_K -> 4 bits, group 32, scale d*sc, bias -dmin*m; Q5_K -> 6-bit fields holding
+ * five-bit codes, group 32; Q6_K -> 6 bits, group 16, bias -32*scale; F32 -> min/max quantiser.
+ * gguf_type is GGUF's tensor type id (F32 0, Q4_0 2, Q4_1 3, Q8_0 8, Q4_K 12, Q5_K 13, Q6_K 14).  rows and
+ * cols are the tensor's (GGUF lists the dimensions as [cols, rows]); stacked expert tensors pass experts * rows.
+ * aq_gguf_affine_layout_of needs no device: it tells the caller what to allocate.
+ * Errors as the reference raises them: another type AQ_ERR_UNSUPPORTED; cols not a whole number of blocks (32,
+ * or 256 for the K formats) or non-positive dims AQ_ERR_SHAPE; src_bytes != rows * blocks * block bytes
+ * AQ_ERR_SHAPE.  packed must be 16-byte aligned, F32 input 4-byte aligned.  Stream-ordered, may be captured. */
+typedef struct aq_gguf_affine_layout {
+    int bits, group_size;
+    int64_t packed_cols, groups;                   /* uint32 words per row, groups per row */
+    uint64_t src_bytes, packed_bytes, scales_bytes; /* scales_bytes is also the size of biases */
+} aq_gguf_affine_layout;
+int aq_gguf_affine_layout_of(int gguf_type, int64_t rows, int64_t cols, aq_gguf_affine_layout *out);
+int aq_gguf_to_affine(aq_ctx *ctx, int gguf_type, const void *src, uint64_t src_bytes, int64_t rows, int64_t cols,
+                      void *packed, void *scales, void *biases);
+
 /* mlxaffine.DequantizeTensor on device (go/model/quant/mlxaffine/mlxaffine.go:178-208):
  * out_f32[N,K] = scale*code + bias, bit-exact with the CPU path. */
 int aq_dequant_f32(aq_ctx *ctx, const void *packed, const void *scales, const void *biases, float *out_f32, int64_t N,

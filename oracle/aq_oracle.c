@@ -595,6 +595,229 @@ int orc_greedy_sample_suppress(const float *logits, int n, const int32_t *suppre
     return ORC_OK;
 }
 
+/* ---- GGUF blocks -> affine layout (go/engine/hip/hip_gguf_affine_adapter.go) ---- */
+
+/* hip_projection_reference.go:240-261 */
+float orc_gguf_f16_to_f32(uint16_t value) {
+    uint32_t sign = (uint32_t)(value & 0x8000) << 16;
+    int exponent = (value >> 10) & 0x1f;
+    uint32_t fraction = value & 0x03ff;
+    uint32_t bits;
+    if (exponent == 0) {
+        if (fraction == 0) {
+            bits = sign;
+        } else {
+            exponent = -14;
+            while ((fraction & 0x0400) == 0) {
+                fraction <<= 1;
+                exponent--;
+            }
+            fraction &= 0x03ff;
+            bits = sign | (uint32_t)(exponent + 127) << 23 | fraction << 13;
+        }
+    } else if (exponent == 0x1f) {
+        bits = sign | 0x7f800000u | fraction << 13;
+    } else {
+        bits = sign | (uint32_t)(exponent - 15 + 127) << 23 | fraction << 13;
+    }
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+/* hip_bf16_portable.go:19-23: round to nearest even on the bit pattern, NaN payloads included */
+uint16_t orc_gguf_f32_to_bf16(float v) {
+    uint32_t bits;
+    memcpy(&bits, &v, 4);
+    bits += 0x7fff + ((bits >> 16) & 1);
+    return (uint16_t)(bits >> 16);
+}
+
+static uint16_t gguf_le16(const uint8_t *p) { return (uint16_t)(p[0] | p[1] << 8); }
+static void gguf_put16(uint8_t *p, uint16_t v) {
+    p[0] = (uint8_t)v;
+    p[1] = (uint8_t)(v >> 8);
+}
+
+/* hip_gguf_affine_adapter.go:843-857 (weights start zeroed; a code may straddle two words) */
+static void gguf_put_code(uint8_t *weights, int64_t row_word_base, int64_t col, int bits, uint32_t value) {
+    int64_t bit_off = col * bits;
+    int64_t word = row_word_base + bit_off / 32;
+    unsigned shift = (unsigned)(bit_off % 32);
+    uint32_t mask = (1u << bits) - 1;
+    uint32_t w;
+    memcpy(&w, weights + word * 4, 4);
+    w |= (value & mask) << shift;
+    memcpy(weights + word * 4, &w, 4);
+    if (shift + (unsigned)bits > 32) {
+        memcpy(&w, weights + word * 4 + 4, 4);
+        w |= (value & mask) >> (32 - shift);
+        memcpy(weights + word * 4 + 4, &w, 4);
+    }
+}
+
+/* :793-799 */
+static void gguf_k_scale_min(const uint8_t *s, int group, uint8_t *scale, uint8_t *min) {
+    if (group < 4) {
+        *scale = s[group] & 63;
+        *min = s[group + 4] & 63;
+    } else {
+        *scale = (uint8_t)((s[group + 4] & 0x0f) | ((s[group - 4] >> 6) << 4));
+        *min = (uint8_t)((s[group + 4] >> 4) | ((s[group] >> 6) << 4));
+    }
+}
+
+/* :801-820 */
+static uint8_t gguf_q5k_code(const uint8_t *block, int group, int lane) {
+    int il = group / 2, high = group % 2 == 1, ir = lane / 2, sub = lane % 2;
+    uint8_t value = block[48 + 32 * il + 2 * ir + sub];
+    if (high) value >>= 4;
+    value &= 0x0f;
+    uint8_t mask = (uint8_t)(1u << (2 * il));
+    if (high) mask <<= 1;
+    if (block[16 + 2 * ir + sub] & mask) value += 16;
+    return value & 0x1f;
+}
+
+/* :822-841 */
+static uint8_t gguf_q6k_code(const uint8_t *block, int group, int lane) {
+    int ip = group / 8, local = group % 8;
+    int lane_off = local % 2 == 1 ? 16 : 0;
+    int quartile = local / 2;
+    int ql_index = ip * 64 + lane_off + lane;
+    if (quartile == 1 || quartile == 3) ql_index += 32;
+    uint8_t ql = block[ql_index];
+    if (quartile >= 2) ql >>= 4;
+    int qh_index = 128 + ip * 32 + lane_off + lane;
+    return (uint8_t)((ql & 0x0f) | (((block[qh_index] >> (quartile * 2)) & 0x03) << 4));
+}
+
+static int gguf_format(int type, int *block_cols, int *block_bytes, int *bits, int *group) {
+    switch (type) {
+        case 0: *block_cols = 32, *block_bytes = 128, *bits = 8, *group = 32; return 1;  /* F32, :650-720 */
+        case 2: *block_cols = 32, *block_bytes = 18, *bits = 4, *group = 32; return 1;   /* Q4_0, :27-30 */
+        case 3: *block_cols = 32, *block_bytes = 20, *bits = 4, *group = 32; return 1;   /* Q4_1, :31-34 */
+        case 8: *block_cols = 32, *block_bytes = 34, *bits = 8, *group = 32; return 1;   /* Q8_0, :52-54 */
+        case 12: *block_cols = 256, *block_bytes = 144, *bits = 4, *group = 32; return 1; /* Q4_K, :37-41 */
+        case 13: *block_cols = 256, *block_bytes = 176, *bits = 6, *group = 32; return 1; /* Q5_K, :42-46 */
+        case 14: *block_cols = 256, *block_bytes = 210, *bits = 6, *group = 16; return 1; /* Q6_K, :47-51 */
+        default: return 0;
+    }
+}
+
+int orc_gguf_affine_layout(int type, int64_t rows, int64_t cols, int *bits, int *group_size, int64_t *packed_cols,
+                           int64_t *groups, uint64_t *src_bytes) {
+    int bc, bb, b, g;
+    if (!gguf_format(type, &bc, &bb, &b, &g)) return ORC_ERR_BITS;
+    if (rows <= 0 || cols <= 0 || cols % bc != 0) return ORC_ERR_DIMS;
+    *bits = b;
+    *group_size = g;
+    *packed_cols = cols * b / 32;
+    *groups = cols / g;
+    *src_bytes = (uint64_t)rows * (uint64_t)(cols / bc) * (uint64_t)bb;
+    return ORC_OK;
+}
+
+int orc_gguf_to_affine(int type, int64_t rows, int64_t cols, const uint8_t *data, uint64_t data_len, uint8_t *weights,
+                       uint8_t *scales, uint8_t *biases) {
+    int bits, gs;
+    int64_t packed_cols, groups;
+    uint64_t want;
+    int rc = orc_gguf_affine_layout(type, rows, cols, &bits, &gs, &packed_cols, &groups, &want);
+    if (rc != ORC_OK) return rc;
+    if (data_len != want) return ORC_ERR_SIZE;
+    memset(weights, 0, (size_t)(rows * packed_cols * 4));
+    for (int64_t row = 0; row < rows; row++) {
+        if (type == 0) { /* :677-718 */
+            for (int64_t group = 0; group < groups; group++) {
+                float values[32], lo = 0, hi = 0;
+                for (int lane = 0; lane < 32; lane++) {
+                    float v;
+                    memcpy(&v, data + ((size_t)row * cols + group * 32 + lane) * 4, 4);
+                    if (isnan(v) || isinf(v)) v = 0;
+                    values[lane] = v;
+                    if (lane == 0 || v < lo) lo = v;
+                    if (lane == 0 || v > hi) hi = v;
+                }
+                float scale = (hi - lo) / 255;
+                if (scale == 0) scale = 1;
+                gguf_put16(scales + (row * groups + group) * 2, orc_gguf_f32_to_bf16(scale));
+                gguf_put16(biases + (row * groups + group) * 2, orc_gguf_f32_to_bf16(lo));
+                for (int lane = 0; lane < 32; lane++) {
+                    uint32_t q = 0;
+                    if (hi != lo) {
+                        float quotient = (values[lane] - lo) / scale;
+                        q = (uint32_t)round((double)quotient);
+                        if (q > 255) q = 255;
+                    }
+                    gguf_put_code(weights, row * packed_cols, group * 32 + lane, 8, q);
+                }
+            }
+            continue;
+        }
+        if (type == 2 || type == 3 || type == 8) {
+            int bb = type == 2 ? 18 : type == 3 ? 20 : 34;
+            int64_t blocks = cols / 32;
+            for (int64_t bi = 0; bi < blocks; bi++) {
+                const uint8_t *block = data + (size_t)(row * blocks + bi) * bb;
+                float scale = orc_gguf_f16_to_f32(gguf_le16(block));
+                float bias = type == 2 ? -8 * scale : type == 3 ? orc_gguf_f16_to_f32(gguf_le16(block + 2)) : -128 * scale;
+                gguf_put16(scales + (row * groups + bi) * 2, orc_gguf_f32_to_bf16(scale));
+                gguf_put16(biases + (row * groups + bi) * 2, orc_gguf_f32_to_bf16(bias));
+                for (int lane = 0; lane < 32; lane++) {
+                    uint32_t value;
+                    if (type == 8) {
+                        value = (uint32_t)((int)(int8_t)block[2 + lane] + 128); /* :631 */
+                    } else {
+                        uint8_t packed = block[(type == 2 ? 2 : 4) + lane % 16]; /* :374-378, :432-436 */
+                        value = lane >= 16 ? packed >> 4 : packed & 0x0f;
+                    }
+                    gguf_put_code(weights, row * packed_cols, bi * 32 + lane, bits, value);
+                }
+            }
+            continue;
+        }
+        int bb = type == 12 ? 144 : type == 13 ? 176 : 210;
+        int64_t blocks = cols / 256;
+        for (int64_t bi = 0; bi < blocks; bi++) {
+            const uint8_t *block = data + (size_t)(row * blocks + bi) * bb;
+            if (type == 14) { /* :774-791 */
+                float d = orc_gguf_f16_to_f32(gguf_le16(block + 208));
+                for (int group = 0; group < 16; group++) {
+                    float scale = d * (float)(int8_t)block[192 + group];
+                    int64_t gi = row * groups + bi * 16 + group;
+                    gguf_put16(scales + gi * 2, orc_gguf_f32_to_bf16(scale));
+                    gguf_put16(biases + gi * 2, orc_gguf_f32_to_bf16(-32 * scale));
+                    for (int lane = 0; lane < 16; lane++)
+                        gguf_put_code(weights, row * packed_cols, bi * 256 + group * 16 + lane, 6,
+                                      gguf_q6k_code(block, group, lane));
+                }
+                continue;
+            }
+            float d = orc_gguf_f16_to_f32(gguf_le16(block));
+            float dmin = orc_gguf_f16_to_f32(gguf_le16(block + 2));
+            for (int group = 0; group < 8; group++) { /* :722-751, :753-772 */
+                uint8_t sc, mn;
+                gguf_k_scale_min(block + 4, group, &sc, &mn);
+                int64_t gi = row * groups + bi * 8 + group;
+                gguf_put16(scales + gi * 2, orc_gguf_f32_to_bf16(d * (float)sc));
+                gguf_put16(biases + gi * 2, orc_gguf_f32_to_bf16(-dmin * (float)mn));
+                for (int lane = 0; lane < 32; lane++) {
+                    uint32_t value;
+                    if (type == 12) {
+                        uint8_t q = block[16 + (group / 2) * 32 + lane]; /* word w, lane l: qs[pair*32 + w*8 + l] */
+                        value = group % 2 == 1 ? q >> 4 : q & 0x0f;
+                    } else {
+                        value = gguf_q5k_code(block, group, lane);
+                    }
+                    gguf_put_code(weights, row * packed_cols, bi * 256 + group * 32 + lane, bits, value);
+                }
+            }
+        }
+    }
+    return ORC_OK;
+}
+
 int orc_max_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

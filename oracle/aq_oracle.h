@@ -160,6 +160,23 @@ int orc_unpack_greedy_best(uint64_t packed, float softcap, int vocab_size, int *
 int orc_greedy_sample_suppress(const float *logits, int n, const int32_t *suppress, int suppress_count, int *index,
                                float *value);
 
+/* GGUF block formats -> the affine layout, the synthesis the HIP engine's loader runs on the host
+ * (hipRepackGGUFKQuantToAffine, go/engine/hip/hip_gguf_affine_adapter.go:321-341): Q4_0 (:342-397), Q4_1
+ * (:399-455), Q4_K (:457-502, block :722-751), Q5_K (:504-549, block :753-772, codes :801-820, six-bit fields),
+ * Q6_K (:551-596, block :774-791, codes :822-841, groups of 16), Q8_0 (:598-648), F32 quantised to eight bits
+ * (:650-720); the 6-bit scale/min unpack :793-799; code placement hipPutAffinePackedValue :843-857; half to
+ * float hipFloat16ToFloat32, go/engine/hip/hip_projection_reference.go:240-261; float to bf16 WITHOUT a NaN case,
+ * hipFloat32ToBFloat16, go/engine/hip/hip_bf16_portable.go:19-23.  `type` is the GGUF tensor type id (F32 0,
+ * Q4_0 2, Q4_1 3, Q8_0 8, Q4_K 12, Q5_K 13, Q6_K 14; :19-25, :56).  ORC_ERR_BITS for another type, ORC_ERR_DIMS
+ * when cols is not a whole number of blocks, ORC_ERR_SIZE when data_len is not rows * blocks * block bytes.
+ * The layout query fills bits, group size, words per row and groups per row. */
+int orc_gguf_affine_layout(int type, int64_t rows, int64_t cols, int *bits, int *group_size, int64_t *packed_cols,
+                           int64_t *groups, uint64_t *src_bytes);
+int orc_gguf_to_affine(int type, int64_t rows, int64_t cols, const uint8_t *data, uint64_t data_len, uint8_t *weights,
+                       uint8_t *scales, uint8_t *biases);
+uint16_t orc_gguf_f32_to_bf16(float v);
+float orc_gguf_f16_to_f32(uint16_t h);
+
 /* Number of hardware threads OpenMP would use (for reporting). */
 int orc_max_threads(void);
 

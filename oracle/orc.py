@@ -236,5 +236,45 @@ def greedy_sample_suppress(logits_f32, suppress=None):
     return idx.value, val.value
 
 
+GGUF_F32, GGUF_Q4_0, GGUF_Q4_1, GGUF_Q8_0, GGUF_Q4_K, GGUF_Q5_K, GGUF_Q6_K = 0, 2, 3, 8, 12, 13, 14
+
+
+def gguf_affine_layout(gguf_type, rows, cols):
+    """(bits, group_size, packed_cols, groups, src_bytes) of the affine tensors a GGUF tensor repacks to."""
+    bits, gs = ctypes.c_int(), ctypes.c_int()
+    pc, groups, src = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_uint64()
+    fn = lib().orc_gguf_affine_layout
+    fn.argtypes = [ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int),
+                   ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_uint64)]
+    _check(fn(gguf_type, rows, cols, bits, gs, pc, groups, src))
+    return bits.value, gs.value, pc.value, groups.value, src.value
+
+
+def gguf_to_affine(gguf_type, rows, cols, data):
+    """GGUF block bytes -> (packed uint32 [rows, packed_cols], scales uint16 [rows, groups], biases uint16)."""
+    data = _u8(data)
+    bits, gs, pc, groups, _ = gguf_affine_layout(gguf_type, rows, cols)
+    w = np.zeros((rows, pc), np.uint32)
+    s = np.zeros((rows, groups), np.uint16)
+    b = np.zeros((rows, groups), np.uint16)
+    fn = lib().orc_gguf_to_affine
+    fn.argtypes = [ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p,
+                   ctypes.c_void_p, ctypes.c_void_p]
+    _check(fn(gguf_type, rows, cols, _p(data), data.size, _p(w), _p(s), _p(b)))
+    return w, s, b
+
+
+def gguf_f32_to_bf16(v):
+    fn = lib().orc_gguf_f32_to_bf16
+    fn.argtypes, fn.restype = [ctypes.c_float], ctypes.c_uint16
+    return int(fn(v))
+
+
+def gguf_f16_to_f32(h):
+    fn = lib().orc_gguf_f16_to_f32
+    fn.argtypes, fn.restype = [ctypes.c_uint16], ctypes.c_float
+    return float(fn(h))
+
+
 def max_threads():
     return int(lib().orc_max_threads())
