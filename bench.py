@@ -588,6 +588,30 @@ def main():
         sf.close()
         os.unlink(ckpt)
 
+    # ---- extra: GGUF block tensors -> affine tensors on the device (load-time synthesis) -------------------
+    gguf = None
+    if not args.no_extras:
+        GR, GC = 262144, 1536             # the lm_head's shape: larger than the Infinity Cache in every format
+        gguf = {"rows": GR, "cols": GC, "formats": {},
+                "note": "aq_gguf_to_affine on a 262144 x 1536 tensor resident in HBM (random block bytes); bytes = blocks "
+                        "read + packed/scales/biases written; the reference does this on the host between two copies"}
+        for gname, gtype in (("Q4_0", 2), ("Q8_0", 8), ("Q4_K", 12), ("Q5_K", 13), ("Q6_K", 14)):
+            lay = aq_mi355.gguf_affine_layout(gtype, GR, GC)
+            blocks = np.tile(np.random.default_rng(F.BASE_SEED + 70).integers(0, 256, lay.src_bytes // 256, dtype=np.uint8), 256)
+            gsrc = ctx.to_device(blocks)
+            gw_, gs2, gb2 = ctx.alloc(lay.packed_bytes), ctx.alloc(lay.scales_bytes), ctx.alloc(lay.scales_bytes)
+            ctx.gguf_to_affine(gtype, gsrc, lay.src_bytes, GR, GC, gw_, gs2, gb2)
+            ctx.sync()
+            ctx.timer_start()
+            for _ in range(5):
+                ctx.gguf_to_affine(gtype, gsrc, lay.src_bytes, GR, GC, gw_, gs2, gb2)
+            g_us = ctx.timer_stop() * 1e3 / 5
+            moved = lay.src_bytes + lay.packed_bytes + 2 * lay.scales_bytes
+            gguf["formats"][gname] = {"us": round(g_us, 1), "bytes": int(moved), "GBps": round(moved / g_us / 1e3, 1),
+                                      "bits": lay.bits, "group": lay.group_size}
+            for t in (gsrc, gw_, gs2, gb2):
+                t.free()
+
     # ---- CPU baseline: the reference's CPU path (oracle port of matNTQuantHost), bounded sample ----
     cpu = None
     if not args.no_cpu:
@@ -650,6 +674,7 @@ def main():
         "mlp_fused": mlp,
         "lm_head": head,
         "loader": loader,
+        "gguf_repack": gguf,
     }
     print(json.dumps(out))
     ctx.close()

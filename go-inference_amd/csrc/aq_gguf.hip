@@ -52,16 +52,22 @@ __device__ __forceinline__ uint16_t bf16_bits_no_nan_case(float v) {
     return (uint16_t)(bits >> 16);
 }
 
-template <bool A2>
+// Block fields sit at odd offsets (18-, 34- and 210-byte blocks): the loads are written as copies of unknown
+// alignment and the compiler picks the widest access the target allows for them.
 __device__ __forceinline__ uint32_t rd16(const uint8_t* p) {
-    if constexpr (A2) return *reinterpret_cast<const uint16_t*>(p);
-    return (uint32_t)p[0] | (uint32_t)p[1] << 8;
+    uint16_t v;
+    __builtin_memcpy(&v, p, 2);
+    return v;
 }
-
-template <bool A2>
+__device__ __forceinline__ uint32_t rd32(const uint8_t* p) {
+    uint32_t v;
+    __builtin_memcpy(&v, p, 4);
+    return v;
+}
 __device__ __forceinline__ uint64_t rd64(const uint8_t* p) {
-    return (uint64_t)rd16<A2>(p) | (uint64_t)rd16<A2>(p + 2) << 16 | (uint64_t)rd16<A2>(p + 4) << 32 |
-           (uint64_t)rd16<A2>(p + 6) << 48;
+    uint64_t v;
+    __builtin_memcpy(&v, p, 8);
+    return v;
 }
 
 // The low nibbles of eight bytes -> one word, byte i's nibble at bits [4i, 4i+4).
@@ -87,19 +93,19 @@ __device__ __forceinline__ void store_sixes(uint32_t* w, uint64_t t0, uint64_t t
     out[2] = make_uint2((uint32_t)(t2 >> 32) | (uint32_t)t3 << 16, (uint32_t)(t3 >> 16));
 }
 
-// The 6-bit (scale, min) pair of group g in a K-quant block's 12 packed bytes
-// (hipGGUFQ4KScaleMin, hip_gguf_affine_adapter.go:793-799).
-__device__ __forceinline__ void k_scale_min(const uint8_t* s, int g, uint32_t* scale, uint32_t* min) {
-    if (g < 4) {
-        *scale = s[g] & 63u;
-        *min = s[g + 4] & 63u;
-    } else {
-        *scale = (s[g + 4] & 0x0fu) | ((uint32_t)(s[g - 4] >> 6) << 4);
-        *min = (uint32_t)(s[g + 4] >> 4) | ((uint32_t)(s[g] >> 6) << 4);
-    }
+// The 6-bit (scale, min) pair of group g from a K-quant block's 12 packed bytes, given as three words
+// (hipGGUFQ4KScaleMin, hip_gguf_affine_adapter.go:793-799): groups 0..3 use the low six bits of bytes g and g+4;
+// groups 4..7 a nibble of byte g+4 with the top two bits of byte g-4 (scale) or of byte g (min).  No branch:
+// with l = g % 4 the three bytes involved are l, l+4 and l+8 either way.
+__device__ __forceinline__ void k_scale_min(uint32_t w0, uint32_t w1, uint32_t w2, int g, uint32_t* scale,
+                                            uint32_t* min) {
+    const int sh = 8 * (g & 3);
+    const uint32_t a = (w0 >> sh) & 0xffu, c = (w1 >> sh) & 0xffu, e = (w2 >> sh) & 0xffu;
+    *scale = g < 4 ? (a & 63u) : ((e & 0x0fu) | ((a >> 6) << 4));
+    *min = g < 4 ? (c & 63u) : ((e >> 4) | ((c >> 6) << 4));
 }
 
-template <int TYPE, bool A2>
+template <int TYPE>
 __global__ __launch_bounds__(kSpanThreads) void gguf_repack_kernel(const uint8_t* __restrict__ src,
                                                                    uint32_t* __restrict__ w, uint16_t* __restrict__ s,
                                                                    uint16_t* __restrict__ b, int64_t spans) {
@@ -108,9 +114,9 @@ __global__ __launch_bounds__(kSpanThreads) void gguf_repack_kernel(const uint8_t
     if constexpr (TYPE == kGgufQ4_0 || TYPE == kGgufQ4_1) {
         constexpr int kHeader = TYPE == kGgufQ4_0 ? 2 : 4;
         const uint8_t* blk = src + span * (kHeader + 16);
-        const float d = half_bits_to_f32(rd16<A2>(blk));
-        const float bias = TYPE == kGgufQ4_0 ? -8.0f * d : half_bits_to_f32(rd16<A2>(blk + 2));
-        const uint64_t lo = rd64<A2>(blk + kHeader), hi = rd64<A2>(blk + kHeader + 8);
+        const float d = half_bits_to_f32(rd16(blk));
+        const float bias = TYPE == kGgufQ4_0 ? -8.0f * d : half_bits_to_f32(rd16(blk + 2));
+        const uint64_t lo = rd64(blk + kHeader), hi = rd64(blk + kHeader + 8);
         // lanes 0..15 are the low nibbles of the 16 bytes, lanes 16..31 their high nibbles
         *reinterpret_cast<uint4*>(w + span * 4) =
             make_uint4(squeeze_nibbles(lo), squeeze_nibbles(hi), squeeze_nibbles(lo >> 4), squeeze_nibbles(hi >> 4));
@@ -118,11 +124,10 @@ __global__ __launch_bounds__(kSpanThreads) void gguf_repack_kernel(const uint8_t
         b[span] = bf16_bits_no_nan_case(bias);
     } else if constexpr (TYPE == kGgufQ8_0) {
         const uint8_t* blk = src + span * 34;
-        const float d = half_bits_to_f32(rd16<A2>(blk));
+        const float d = half_bits_to_f32(rd16(blk));
         uint32_t word[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i)  // int8 + 128 = the byte with its top bit flipped
-            word[i] = (rd16<A2>(blk + 2 + 4 * i) | rd16<A2>(blk + 4 + 4 * i) << 16) ^ 0x80808080u;
+        for (int i = 0; i < 8; ++i) word[i] = rd32(blk + 2 + 4 * i) ^ 0x80808080u;  // int8 + 128: top bit flipped
         uint4* out = reinterpret_cast<uint4*>(w + span * 8);
         out[0] = make_uint4(word[0], word[1], word[2], word[3]);
         out[1] = make_uint4(word[4], word[5], word[6], word[7]);
@@ -132,9 +137,10 @@ __global__ __launch_bounds__(kSpanThreads) void gguf_repack_kernel(const uint8_t
         constexpr int kBlockBytes = TYPE == kGgufQ4_K ? 144 : 176;
         const uint8_t* blk = src + (span >> 3) * kBlockBytes;
         const int g = (int)(span & 7);
-        const float d = half_bits_to_f32(rd16<A2>(blk)), dmin = half_bits_to_f32(rd16<A2>(blk + 2));
+        const uint32_t head = rd32(blk);
+        const float d = half_bits_to_f32(head & 0xffffu), dmin = half_bits_to_f32(head >> 16);
         uint32_t sc, mn;
-        k_scale_min(blk + 4, g, &sc, &mn);
+        k_scale_min(rd32(blk + 4), rd32(blk + 8), rd32(blk + 12), g, &sc, &mn);
         s[span] = bf16_bits_no_nan_case(d * (float)sc);
         b[span] = bf16_bits_no_nan_case(-dmin * (float)mn);
         const int pair = g >> 1, nib_shift = (g & 1) * 4;
@@ -142,7 +148,7 @@ __global__ __launch_bounds__(kSpanThreads) void gguf_repack_kernel(const uint8_t
             const uint8_t* qs = blk + 16 + pair * 32;
             uint32_t word[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) word[i] = squeeze_nibbles(rd64<A2>(qs + 8 * i) >> nib_shift);
+            for (int i = 0; i < 4; ++i) word[i] = squeeze_nibbles(rd64(qs + 8 * i) >> nib_shift);
             *reinterpret_cast<uint4*>(w + span * 4) = make_uint4(word[0], word[1], word[2], word[3]);
         } else {
             const uint8_t* qh = blk + 16;
@@ -150,8 +156,8 @@ __global__ __launch_bounds__(kSpanThreads) void gguf_repack_kernel(const uint8_t
             uint64_t t[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {  // code = nibble + 16 * (bit 2*pair + (g & 1) of qh[lane])
-                const uint64_t nib = (rd64<A2>(qs + 8 * i) >> nib_shift) & 0x0f0f0f0f0f0f0f0fULL;
-                const uint64_t top = (rd64<A2>(qh + 8 * i) >> (2 * pair + (g & 1))) & 0x0101010101010101ULL;
+                const uint64_t nib = (rd64(qs + 8 * i) >> nib_shift) & 0x0f0f0f0f0f0f0f0fULL;
+                const uint64_t top = (rd64(qh + 8 * i) >> (2 * pair + (g & 1))) & 0x0101010101010101ULL;
                 t[i] = squeeze_sixes(nib | top << 4);
             }
             store_sixes(w + span * 6, t[0], t[1], t[2], t[3]);
@@ -161,8 +167,8 @@ __global__ __launch_bounds__(kSpanThreads) void gguf_repack_kernel(const uint8_t
         // offsets 0 and 16, i.e. 32 consecutive bytes of ql and of qh (hipGGUFQ6KQuant, :822-841)
         const uint8_t* blk = src + (span >> 3) * 210;
         const int p = (int)(span & 7), ip = p >> 2, q = p & 3;
-        const float d = half_bits_to_f32(rd16<A2>(blk + 208));
-        const uint32_t two = rd16<A2>(blk + 192 + 2 * p);
+        const float d = half_bits_to_f32(rd16(blk + 208));
+        const uint32_t two = rd16(blk + 192 + 2 * p);
         const float s0 = d * (float)(int)(int8_t)(two & 0xff), s1 = d * (float)(int)(int8_t)(two >> 8);
         s[2 * span] = bf16_bits_no_nan_case(s0);
         s[2 * span + 1] = bf16_bits_no_nan_case(s1);
@@ -173,8 +179,8 @@ __global__ __launch_bounds__(kSpanThreads) void gguf_repack_kernel(const uint8_t
         uint64_t t[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const uint64_t nib = (rd64<A2>(ql + 8 * i) >> ((q & 2) * 2)) & 0x0f0f0f0f0f0f0f0fULL;
-            const uint64_t top = (rd64<A2>(qh + 8 * i) >> (2 * q)) & 0x0303030303030303ULL;
+            const uint64_t nib = (rd64(ql + 8 * i) >> ((q & 2) * 2)) & 0x0f0f0f0f0f0f0f0fULL;
+            const uint64_t top = (rd64(qh + 8 * i) >> (2 * q)) & 0x0303030303030303ULL;
             t[i] = squeeze_sixes(nib | top << 4);
         }
         store_sixes(w + span * 6, t[0], t[1], t[2], t[3]);
@@ -218,10 +224,7 @@ __global__ __launch_bounds__(kSpanThreads) void gguf_repack_kernel(const uint8_t
 template <int TYPE>
 hipError_t launch_type(const uint8_t* src, uint32_t* w, uint16_t* s, uint16_t* b, int64_t spans, hipStream_t stream) {
     const dim3 grid((unsigned)((spans + kSpanThreads - 1) / kSpanThreads)), block(kSpanThreads);
-    if ((reinterpret_cast<uintptr_t>(src) & 1) == 0)
-        hipLaunchKernelGGL((gguf_repack_kernel<TYPE, true>), grid, block, 0, stream, src, w, s, b, spans);
-    else
-        hipLaunchKernelGGL((gguf_repack_kernel<TYPE, false>), grid, block, 0, stream, src, w, s, b, spans);
+    hipLaunchKernelGGL((gguf_repack_kernel<TYPE>), grid, block, 0, stream, src, w, s, b, spans);
     return hipGetLastError();
 }
 
