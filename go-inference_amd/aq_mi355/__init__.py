@@ -110,6 +110,7 @@ PROTOTYPES = {
     "aq_upload_fused_gate_up": (_i, [_vp, _c.POINTER(HostLinear), _c.POINTER(HostLinear), _c.POINTER(DeviceLinear)]),
     "aq_free_device_linear": (_i, [_vp, _c.POINTER(DeviceLinear)]),
     "aq_dequant_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _c.c_int64, _i, _i, _i]),
+    "aq_packed_topk_sample": (_i, [_vp, _vp, _i, _c.c_float, _c.c_float, _c.c_float, _c.c_double, _vp]),
     "aq_gguf_affine_layout_of": (_i, [_i, _c.c_int64, _c.c_int64, _c.POINTER(GgufAffineLayout)]),
     "aq_gguf_to_affine": (_i, [_vp, _i, _vp, _c.c_uint64, _c.c_int64, _c.c_int64, _vp, _vp, _vp]),
     "aq_matvec_host": (_i, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _i, _i, _i, _i, _vp, _sz]),
@@ -374,6 +375,9 @@ class Context:
     def dequant_f32(self, w, s, b, out, N, K, group_size=64, bits=4):
         self._check(self.lib.aq_dequant_f32(self.handle, _ptr(w), _ptr(s), _ptr(b), _ptr(out), N, K, group_size,
                                             bits))
+
+    def packed_topk_sample(self, top, top_k, temperature, top_p, softcap, draw, out):
+        self._check(self.lib.aq_packed_topk_sample(self.handle, _ptr(top), top_k, temperature, top_p, softcap, draw, _ptr(out)))
 
     def gguf_to_affine(self, gguf_type, src, src_bytes, rows, cols, packed, scales, biases):
         """GGUF blocks at `src` (device) -> packed / scales / biases (device), sized by gguf_affine_layout()."""

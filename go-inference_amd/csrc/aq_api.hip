@@ -1252,6 +1252,28 @@ int aq_packed_topk(aq_ctx* ctx, const uint64_t* scores, int64_t count, int top_k
     return AQ_OK;
 }
 
+int aq_packed_topk_sample(aq_ctx* ctx, const uint64_t* top, int top_k, float temperature, float top_p, float softcap,
+                          double draw, uint64_t* out) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_packed_topk_sample: ctx is null");
+    if (top_k <= 0) return fail(AQ_ERR_SHAPE, "aq_packed_topk_sample: top-k must be positive");
+    if (top_k > aq::kSampleTopKMax)
+        return fail(AQ_ERR_UNSUPPORTED, "aq_packed_topk_sample: top-k is at most %d", aq::kSampleTopKMax);
+    if (!top || !out) return fail(AQ_ERR_ARG, "aq_packed_topk_sample: null operand");
+    if (!aligned(top, 8) || !aligned(out, 8)) return fail(AQ_ERR_ARG, "aq_packed_topk_sample: operand pointer is not 8-byte aligned");
+    // rocm_valid_packed_topk_sample_args, kernels/sampling/topk_validate.hipinc:53-77
+    if (!(temperature >= 0.0f) || !std::isfinite(temperature))
+        return fail(AQ_ERR_ARG, "aq_packed_topk_sample: temperature must be non-negative and finite");
+    if (!(top_p >= 0.0f) || !(top_p <= 1.0f)) return fail(AQ_ERR_ARG, "aq_packed_topk_sample: top-p must be in [0, 1]");
+    if (!(softcap >= 0.0f) || !std::isfinite(softcap))
+        return fail(AQ_ERR_ARG, "aq_packed_topk_sample: softcap must be non-negative and finite");
+    if (!std::isfinite(draw)) return fail(AQ_ERR_ARG, "aq_packed_topk_sample: draw must be finite");
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    AQ_HIP(aq::packed_topk_sample_launch(reinterpret_cast<const unsigned long long*>(top), top_k, temperature, top_p, softcap,
+                                         draw, reinterpret_cast<unsigned long long*>(out), ctx->stream),
+           "hipLaunchKernel");
+    return AQ_OK;
+}
+
 uint64_t aq_pack_best(float score, int token) {
     return ((uint64_t)ordered_key_host(score) << 32) | (uint64_t)(~(uint32_t)token);
 }

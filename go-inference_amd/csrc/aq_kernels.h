@@ -223,6 +223,11 @@ hipError_t qmv_generic_launch(const QmvArgs& a, int bits, int group_size, bool g
 hipError_t dequant_launch(const uint32_t* w, const uint16_t* s, const uint16_t* b, float* out, int64_t N, int K,
                           int group_size, int bits, hipStream_t stream);
 
+// Temperature / top-p sampling over a descending packed list of at most kSampleTopKMax entries (aq_qmv_head.hip).
+constexpr int kSampleTopKMax = 128;
+hipError_t packed_topk_sample_launch(const unsigned long long* in, int top_k, float temperature, float top_p, float softcap,
+                                     double draw, unsigned long long* out, hipStream_t stream);
+
 // GGUF block formats -> affine layout (aq_gguf.hip).  Type ids are GGUF's own
 // (go/engine/hip/hip_gguf_affine_adapter.go:19-25, :56).
 constexpr int kGgufF32 = 0, kGgufQ4_0 = 2, kGgufQ4_1 = 3, kGgufQ8_0 = 8, kGgufQ4_K = 12, kGgufQ5_K = 13, kGgufQ6_K = 14;

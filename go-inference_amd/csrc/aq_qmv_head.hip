@@ -257,4 +257,107 @@ hipError_t packed_topk_launch(const unsigned long long* in, int64_t count, int t
     }
 }
 
+// Temperature / top-p sampling over the packed top-k list (rocm_packed_topk_sample,
+// go/engine/hip/kernels/sampling/topk.hipinc:86-191; score decode and softcap kernels/common/numeric.hipinc:95-110).
+// The reference runs the whole thing on one thread and evaluates exp() of every candidate in each of its four
+// passes; here each of up to 128 threads evaluates its candidate's weight once (tanh and exp in double are the
+// cost) and thread 0 then walks the list, adding in list order as the reference does, so every sum rounds the
+// same way.  out[0] = 0 when nothing can be sampled.
+constexpr int kSampleMax = 128;
+
+__device__ __forceinline__ double sample_score(unsigned long long packed, double softcap) {
+    const uint32_t key = (uint32_t)(packed >> 32);
+    const double score = (double)__uint_as_float((key & 0x80000000u) ? key ^ 0x80000000u : ~key);
+    return softcap > 0.0 ? tanh(score / softcap) * softcap : score;
+}
+
+__global__ __launch_bounds__(kSampleMax) void packed_topk_sample_kernel(const unsigned long long* __restrict__ in,
+                                                                        int top_k, float raw_temperature, float raw_top_p,
+                                                                        float softcap_f, double draw,
+                                                                        unsigned long long* __restrict__ out) {
+    __shared__ unsigned long long vals[kSampleMax];
+    __shared__ double wts[kSampleMax];
+    const int t = threadIdx.x;
+    vals[t] = t < top_k ? in[t] : 0ull;
+    __syncthreads();
+    int first_valid = top_k;  // the same scan on every thread: the branches below are uniform
+    for (int i = 0; i < top_k; ++i)
+        if (vals[i] != 0ull) {
+            first_valid = i;
+            break;
+        }
+    unsigned long long result = 0ull;
+    bool sample = false;
+    double temperature = 1.0, top_p = 1.0;
+    if (first_valid < top_k) {
+        if (raw_temperature <= 0.0f && raw_top_p <= 0.0f) {
+            result = vals[first_valid];  // greedy
+        } else {
+            temperature = raw_temperature == 0.0f ? 1.0 : (double)raw_temperature;
+            top_p = raw_top_p == 0.0f ? 1.0 : (double)raw_top_p;
+            sample = temperature > 0.0 && top_p > 0.0 && top_p <= 1.0;
+        }
+    }
+    if (!sample) {
+        if (t == 0) out[0] = result;
+        return;
+    }
+    const double softcap = (double)softcap_f;
+    const double max_value = sample_score(vals[first_valid], softcap) / temperature;
+    wts[t] = (t >= first_valid && t < top_k && vals[t] != 0ull)
+                 ? exp(sample_score(vals[t], softcap) / temperature - max_value)
+                 : 0.0;
+    __syncthreads();
+    if (t != 0) return;
+    out[0] = 0ull;
+    double total = 0.0;
+    for (int i = first_valid; i < top_k; ++i) {
+        if (vals[i] == 0ull) continue;
+        if (!isfinite(wts[i])) return;
+        total += wts[i];
+    }
+    if (!(total > 0.0) || !isfinite(total)) return;
+    int limit = top_k;
+    if (top_p < 1.0) {
+        double cumulative = 0.0;
+        for (int i = first_valid; i < top_k; ++i) {
+            if (vals[i] == 0ull) continue;
+            cumulative += wts[i];
+            if (cumulative / total >= top_p) {
+                limit = i + 1;
+                break;
+            }
+        }
+    }
+    double selected_total = 0.0;
+    unsigned long long fallback = vals[first_valid];
+    for (int i = first_valid; i < limit; ++i) {
+        if (vals[i] == 0ull) continue;
+        fallback = vals[i];
+        selected_total += wts[i];
+    }
+    if (!(selected_total > 0.0) || !isfinite(selected_total)) return;
+    if (draw < 0.0) draw = 0.0;
+    if (draw >= 1.0) draw = 0x1.fffffffffffffp-1;  // the double below 1
+    const double target = draw * selected_total;
+    double cumulative = 0.0;
+    for (int i = first_valid; i < limit; ++i) {
+        if (vals[i] == 0ull) continue;
+        cumulative += wts[i];
+        if (target <= cumulative) {
+            out[0] = vals[i];
+            return;
+        }
+    }
+    out[0] = fallback;
+}
+
+hipError_t packed_topk_sample_launch(const unsigned long long* in, int top_k, float temperature, float top_p, float softcap,
+                                     double draw, unsigned long long* out, hipStream_t stream) {
+    if (top_k <= 0 || top_k > kSampleMax) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(packed_topk_sample_kernel, dim3(1), dim3(kSampleMax), 0, stream, in, top_k, temperature, top_p, softcap,
+                       draw, out);
+    return hipGetLastError();
+}
+
 }  // namespace aq

@@ -257,6 +257,20 @@ int aq_qmv_scores(aq_ctx *ctx, const void *x, const void *packed, const void *sc
  * applied chunk by chunk until one chunk is left; scratch comes from the context's workspace. */
 int aq_packed_topk(aq_ctx *ctx, const uint64_t *scores, int64_t count, int top_k, uint64_t *out);
 
+/* Temperature / top-p sampling over the list aq_packed_topk wrote (descending packed values, zeros = no candidate),
+ * the device sampler rocm_packed_topk_sample (go/engine/hip/kernels/sampling/topk.hipinc:86-191, launched by
+ * hipRunPackedTopKSampleKernel, go/engine/hip/hip_projection_launch.go:4538): weights exp(score / temperature -
+ * max) in double over the soft-capped scores (softcap 0 = none), the nucleus cut at cumulative / total >= top_p,
+ * then the candidate whose cumulative weight first reaches draw * (sum of the kept weights); `draw` in [0, 1) comes
+ * from the caller's generator, so a run is reproducible.  temperature <= 0 and top_p <= 0 together select the first
+ * candidate (greedy); a zero of either alone stands for 1.  out[0] (device) receives the chosen packed value, to
+ * be read with aq_unpack_best; 0 when nothing can be sampled.  Argument rules of topk_validate.hipinc:53-77:
+ * top_k 1..128 (AQ_ERR_SHAPE / AQ_ERR_UNSUPPORTED), temperature >= 0 finite, top_p in [0, 1], softcap >= 0
+ * finite, draw finite (AQ_ERR_ARG).  Sums run in list order as in the reference; exp and tanh are the device
+ * library's double-precision ones.  Stream-ordered, may be captured. */
+int aq_packed_topk_sample(aq_ctx *ctx, const uint64_t *top, int top_k, float temperature, float top_p, float softcap,
+                          double draw, uint64_t *out);
+
 /* Host-side codec of the packed values: hipPackGreedyBest / hipUnpackGreedyBest
  * (go/engine/hip/hip_projection_launch.go:2393-2416).  Unpacking rejects packed == 0 ("did not produce a
  * result"), a token outside [0, vocab_size) and a negative or non-finite softcap; softcap > 0 returns

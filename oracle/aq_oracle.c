@@ -818,6 +818,172 @@ int orc_gguf_to_affine(int type, int64_t rows, int64_t cols, const uint8_t *data
     return ORC_OK;
 }
 
+/* ---- temperature / top-p sampling over the packed top-k ---- */
+
+/* kernels/common/numeric.hipinc:95-110 */
+static double sample_score(uint64_t packed, double softcap) {
+    uint32_t key = (uint32_t)(packed >> 32);
+    uint32_t bits = (key & 0x80000000u) ? key ^ 0x80000000u : ~key;
+    float f;
+    memcpy(&f, &bits, 4);
+    double score = (double)f;
+    return softcap > 0.0 ? tanh(score / softcap) * softcap : score;
+}
+
+/* kernels/sampling/topk.hipinc:86-191 */
+int orc_packed_topk_sample(const uint64_t *input, int top_k, float raw_temperature, float raw_top_p, float softcap_f,
+                           double draw, uint64_t *out) {
+    if (top_k <= 0 || top_k > 128) return ORC_ERR_DIMS;
+    if (!(raw_temperature >= 0.0f) || !isfinite(raw_temperature) || !(raw_top_p >= 0.0f) || !(raw_top_p <= 1.0f) ||
+        !(softcap_f >= 0.0f) || !isfinite(softcap_f) || !isfinite(draw))
+        return ORC_ERR_SIZE;
+    *out = 0;
+    int first_valid = top_k;
+    for (int i = 0; i < top_k; i++)
+        if (input[i] != 0) {
+            first_valid = i;
+            break;
+        }
+    if (first_valid >= top_k) return ORC_OK;
+    if (raw_temperature <= 0.0f && raw_top_p <= 0.0f) {
+        *out = input[first_valid];
+        return ORC_OK;
+    }
+    const double temperature = raw_temperature == 0.0f ? 1.0 : (double)raw_temperature;
+    const double top_p = raw_top_p == 0.0f ? 1.0 : (double)raw_top_p;
+    if (!(temperature > 0.0) || !(top_p > 0.0 && top_p <= 1.0)) return ORC_OK;
+    const double softcap = (double)softcap_f;
+    const double max_value = sample_score(input[first_valid], softcap) / temperature;
+    double total = 0.0;
+    for (int i = first_valid; i < top_k; i++) {
+        if (input[i] == 0) continue;
+        double weight = exp(sample_score(input[i], softcap) / temperature - max_value);
+        if (!isfinite(weight)) return ORC_OK;
+        total += weight;
+    }
+    if (!(total > 0.0) || !isfinite(total)) return ORC_OK;
+    int limit = top_k;
+    if (top_p < 1.0) {
+        double cumulative = 0.0;
+        for (int i = first_valid; i < top_k; i++) {
+            if (input[i] == 0) continue;
+            cumulative += exp(sample_score(input[i], softcap) / temperature - max_value);
+            if (cumulative / total >= top_p) {
+                limit = i + 1;
+                break;
+            }
+        }
+    }
+    double selected_total = 0.0;
+    uint64_t fallback = input[first_valid];
+    for (int i = first_valid; i < limit; i++) {
+        if (input[i] == 0) continue;
+        fallback = input[i];
+        selected_total += exp(sample_score(input[i], softcap) / temperature - max_value);
+    }
+    if (!(selected_total > 0.0) || !isfinite(selected_total)) return ORC_OK;
+    if (draw < 0.0) draw = 0.0;
+    if (draw >= 1.0) draw = nextafter(1.0, 0.0);
+    const double target = draw * selected_total;
+    double cumulative = 0.0;
+    for (int i = first_valid; i < limit; i++) {
+        if (input[i] == 0) continue;
+        cumulative += exp(sample_score(input[i], softcap) / temperature - max_value);
+        if (target <= cumulative) {
+            *out = input[i];
+            return ORC_OK;
+        }
+    }
+    *out = fallback;
+    return ORC_OK;
+}
+
+/* hip_gemma4_q4_layer.go:3166-3178 */
+int orc_softcap_logits(float *logits, int n, float softcap) {
+    if (softcap < 0 || isnan(softcap) || isinf(softcap)) return ORC_ERR_SIZE;
+    if (softcap == 0) return ORC_OK;
+    for (int i = 0; i < n; i++) logits[i] = (float)tanh((double)(logits[i] / softcap)) * softcap;
+    return ORC_OK;
+}
+
+typedef struct {
+    int index;
+    float value;
+} host_candidate;
+
+/* hip_transformer_reference.go:502-506: score descending, token id ascending */
+static int host_candidate_cmp(const void *a, const void *b) {
+    const host_candidate *x = a, *y = b;
+    if (x->value > y->value) return -1;
+    if (x->value < y->value) return 1;
+    return x->index < y->index ? -1 : x->index > y->index;
+}
+
+/* hip_tiny_model.go:2763-2879 (no suppression list, history or min-p) */
+int orc_host_sample(const float *logits, int n, float temperature, int top_k, float top_p, double draw, int *token,
+                    float *score) {
+    if (n <= 0) return ORC_ERR_DIMS;
+    if (temperature <= 0 && top_k <= 0 && top_p <= 0) return orc_greedy_sample_suppress(logits, n, NULL, 0, token, score);
+    if (temperature == 0) temperature = 1;
+    if (temperature <= 0 || isnan(temperature) || isinf(temperature)) return ORC_ERR_SIZE;
+    if (top_p == 0) top_p = 1;
+    if (top_p <= 0 || top_p > 1 || isnan(top_p)) return ORC_ERR_SIZE;
+    host_candidate *cand = malloc((size_t)n * sizeof *cand);
+    int count = 0;
+    for (int i = 0; i < n; i++)
+        if (!isnan(logits[i]) && !isinf(logits[i])) cand[count++] = (host_candidate){i, logits[i]};
+    if (count == 0) {
+        free(cand);
+        return ORC_ERR_INDEX;
+    }
+    qsort(cand, (size_t)count, sizeof *cand, host_candidate_cmp);
+    if (top_k < 0 || top_k > n) {
+        free(cand);
+        return ORC_ERR_DIMS;
+    }
+    if (top_k == 0 || top_k > count) top_k = count;
+    double *weights = malloc((size_t)top_k * sizeof *weights);
+    double max_value = (double)cand[0].value / (double)temperature, total = 0.0;
+    for (int i = 0; i < top_k; i++) {
+        weights[i] = exp((double)cand[i].value / (double)temperature - max_value);
+        total += weights[i];
+    }
+    int rc = ORC_OK;
+    if (total <= 0 || isnan(total) || isinf(total)) {
+        rc = ORC_ERR_SIZE;
+    } else {
+        int limit = top_k;
+        if (top_p < 1) {
+            double cumulative = 0.0;
+            for (int i = 0; i < top_k; i++) {
+                cumulative += weights[i];
+                if (cumulative / total >= (double)top_p) {
+                    limit = i + 1;
+                    break;
+                }
+            }
+        }
+        double selected_total = 0.0;
+        for (int i = 0; i < limit; i++) selected_total += weights[i];
+        if (draw < 0) draw = 0;
+        if (draw >= 1) draw = nextafter(1.0, 0.0);
+        double target = draw * selected_total, cumulative = 0.0;
+        int pick = limit - 1;
+        for (int i = 0; i < limit; i++) {
+            cumulative += weights[i];
+            if (target <= cumulative) {
+                pick = i;
+                break;
+            }
+        }
+        *token = cand[pick].index;
+        *score = cand[pick].value;
+    }
+    free(weights);
+    free(cand);
+    return rc;
+}
+
 int orc_max_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

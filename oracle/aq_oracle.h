@@ -177,6 +177,26 @@ int orc_gguf_to_affine(int type, int64_t rows, int64_t cols, const uint8_t *data
 uint16_t orc_gguf_f32_to_bf16(float v);
 float orc_gguf_f16_to_f32(uint16_t h);
 
+/* rocm_packed_topk_sample, go/engine/hip/kernels/sampling/topk.hipinc:86-191 (argument rules
+ * topk_validate.hipinc:53-77, score decode + softcap kernels/common/numeric.hipinc:95-110): temperature / top-p
+ * sampling over a descending list of packed (score, token) values (zeros = no candidate), every sum in double and
+ * in list order, `draw` in [0,1) chosen by the caller.  *out = 0 when nothing can be sampled (no candidate, a
+ * non-finite weight).  temperature <= 0 and top_p <= 0 together mean greedy (the first candidate); a zero of
+ * either alone means 1.  ORC_ERR_DIMS for top_k outside 1..128, ORC_ERR_SIZE for temperature / top_p / softcap /
+ * draw outside their ranges. */
+int orc_packed_topk_sample(const uint64_t *input, int top_k, float temperature, float top_p, float softcap, double draw,
+                           uint64_t *out);
+
+/* The host sampler the reference checks that kernel against (hipGemma4Q4HostSampleResult,
+ * go/engine/hip/hip_tiny_model.go:2763-2879, without suppression, repeat penalty and min-p; candidate order
+ * hip_transformer_reference.go:502-506: score descending, token ascending) over full logits, which the caller
+ * softcaps first as hipGemma4Q4SoftcapLogits does (hip_gemma4_q4_layer.go:3166-3178: orc_softcap_logits).
+ * ORC_ERR_DIMS without logits or top_k outside 0..n, ORC_ERR_SIZE for a bad temperature / top-p, ORC_ERR_INDEX
+ * when no logit is finite. */
+int orc_host_sample(const float *logits, int n, float temperature, int top_k, float top_p, double draw, int *token,
+                    float *score);
+int orc_softcap_logits(float *logits, int n, float softcap);
+
 /* Number of hardware threads OpenMP would use (for reporting). */
 int orc_max_threads(void);
 

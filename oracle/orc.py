@@ -276,5 +276,35 @@ def gguf_f16_to_f32(h):
     return float(fn(h))
 
 
+def packed_topk_sample(packed_u64, temperature, top_p, softcap, draw):
+    """rocm_packed_topk_sample over a descending packed list; returns the chosen packed value (0 = none)."""
+    packed = np.ascontiguousarray(packed_u64, dtype=np.uint64)
+    out = ctypes.c_uint64(0)
+    fn = lib().orc_packed_topk_sample
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_double,
+                   ctypes.POINTER(ctypes.c_uint64)]
+    _check(fn(_p(packed), packed.size, temperature, top_p, softcap, draw, ctypes.byref(out)))
+    return int(out.value)
+
+
+def softcap_logits(logits_f32, softcap):
+    out = np.array(logits_f32, dtype=np.float32)
+    fn = lib().orc_softcap_logits
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_float]
+    _check(fn(_p(out), out.size, softcap))
+    return out
+
+
+def host_sample(logits_f32, temperature, top_k, top_p, draw):
+    """hipGemma4Q4HostSampleResult over (already softcapped) logits -> (token, score)."""
+    logits = np.ascontiguousarray(logits_f32, dtype=np.float32)
+    tok, sc = ctypes.c_int(0), ctypes.c_float(0)
+    fn = lib().orc_host_sample
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_double,
+                   ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_float)]
+    _check(fn(_p(logits), logits.size, temperature, top_k, top_p, draw, ctypes.byref(tok), ctypes.byref(sc)))
+    return tok.value, float(sc.value)
+
+
 def max_threads():
     return int(lib().orc_max_threads())

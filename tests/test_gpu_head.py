@@ -188,3 +188,68 @@ def test_head_top_k_pipeline_and_errors(ctx, orc):
     for t in (dx, dsc, dtop, buf, best):
         t.free()
     dw.free()
+
+
+def _sample(ctx, top, temperature, top_p, softcap, draw):
+    dtop, dout = ctx.to_device(np.ascontiguousarray(top, np.uint64)), ctx.to_device(np.full(1, 0xDEAD, np.uint64))
+    ctx.packed_topk_sample(dtop, len(top), temperature, top_p, softcap, draw, dout)
+    ctx.sync()
+    got = int(_u64(dout, 1)[0])
+    dtop.free()
+    dout.free()
+    return got
+
+
+def test_packed_topk_sample_against_oracle(ctx, orc):
+    """The device sampler picks the oracle's candidate: the scenario of the reference's hardware test (through the
+    device top-k, against the host sampler over soft-capped logits too), then random lists with holes, every
+    temperature / top-p mode and out-of-range draws."""
+    import aq_mi355
+    say("packed topk sample")
+    V = 262144
+    logits = np.full(V, -100, np.float32)
+    for rank in range(64):
+        logits[200000 + rank * 17] = 60 - rank / 2
+    packed = np.array([aq_mi355.pack_best(float(v), t) for t, v in enumerate(logits)], dtype=np.uint64)
+    host = orc.softcap_logits(logits, 30)
+    din = ctx.to_device(packed)
+    for k in (40, 64):
+        dtop, dout = ctx.alloc(k * 8), ctx.alloc(8)
+        ctx.packed_topk(din, V, k, dtop)
+        for top_p in (1.0, 0.95):
+            for draw in (0, 0.1, 0.5, 0.9, 0.999999):
+                ctx.packed_topk_sample(dtop, k, 1.0, top_p, 30.0, draw, dout)
+                ctx.sync()
+                got = int(_u64(dout, 1)[0])
+                assert got == orc.packed_topk_sample(_u64(dtop, k), 1.0, top_p, 30.0, draw), (k, top_p, draw)
+                assert _unpack(got)[0] == orc.host_sample(host, 1.0, k, top_p, draw)[0], (k, top_p, draw)
+        dtop.free()
+        dout.free()
+    din.free()
+    rng = np.random.default_rng(77)
+    for case in range(60):
+        k = int(rng.integers(1, 129))
+        scores = np.sort(rng.normal(0, 3, k).astype(np.float32))[::-1]
+        top = np.array([aq_mi355.pack_best(float(s), int(t)) for s, t in zip(scores, rng.permutation(100000)[:k])], np.uint64)
+        top[rng.random(k) < 0.15] = 0
+        temperature = float(rng.choice([0.0, 0.3, 1.0, 2.5]))
+        top_p = float(rng.choice([0.0, 0.5, 0.9, 1.0]))
+        softcap = float(rng.choice([0.0, 2.0, 30.0]))
+        for draw in (-0.5, 0.0, float(rng.random()), float(rng.random()), 0.999999999, 1.0, 3.0):
+            want = orc.packed_topk_sample(top, temperature, top_p, softcap, draw)
+            assert _sample(ctx, top, temperature, top_p, softcap, draw) == want, (case, k, temperature, top_p, softcap, draw)
+    assert _sample(ctx, np.zeros(5, np.uint64), 1.0, 1.0, 0.0, 0.5) == 0
+    huge = np.array([aq_mi355.pack_best(3e38, 1), aq_mi355.pack_best(-3e38, 2)], np.uint64)     # weight 1 and exp(-inf) = 0
+    assert _sample(ctx, huge, 1e-3, 1.0, 0.0, 0.999) == orc.packed_topk_sample(huge, 1e-3, 1.0, 0.0, 0.999) == int(huge[0])
+    buf = ctx.alloc(1024)
+    for call, code in [(lambda: ctx.packed_topk_sample(buf, 0, 1.0, 1.0, 0.0, 0.5, buf), aq_mi355.AQ_ERR_SHAPE),
+                       (lambda: ctx.packed_topk_sample(buf, 129, 1.0, 1.0, 0.0, 0.5, buf), aq_mi355.AQ_ERR_UNSUPPORTED),
+                       (lambda: ctx.packed_topk_sample(None, 4, 1.0, 1.0, 0.0, 0.5, buf), aq_mi355.AQ_ERR_ARG),
+                       (lambda: ctx.packed_topk_sample(buf, 4, -1.0, 1.0, 0.0, 0.5, buf), aq_mi355.AQ_ERR_ARG),
+                       (lambda: ctx.packed_topk_sample(buf, 4, 1.0, 1.5, 0.0, 0.5, buf), aq_mi355.AQ_ERR_ARG),
+                       (lambda: ctx.packed_topk_sample(buf, 4, 1.0, 1.0, float("inf"), 0.5, buf), aq_mi355.AQ_ERR_ARG),
+                       (lambda: ctx.packed_topk_sample(buf, 4, 1.0, 1.0, 0.0, float("nan"), buf), aq_mi355.AQ_ERR_ARG)]:
+        with pytest.raises(aq_mi355.AqError) as e:
+            call()
+        assert e.value.code == code
+    buf.free()
