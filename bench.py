@@ -534,11 +534,18 @@ def main():
             ctx.packed_topk(h_scores, HN, 40, h_top)
 
         us_topk = head_time(topk40)
+
+        def sample40(t):
+            topk40(t)
+            ctx.packed_topk_sample(h_top, 40, 0.8, 0.95, 30.0, 0.37, h_best)
+
+        us_sample = head_time(sample40)
         head = {"N": HN, "K": HK, "group": HG, "bits": BITS, "weight_bytes": head_bytes,
                 "logits": {"us": round(us_logits, 2), "GBps": round((head_bytes + HN * 2) / us_logits / 1e3, 1), "kernel": k_logits},
                 "greedy_fused": {"us": round(us_greedy, 2), "GBps": round(head_bytes / us_greedy / 1e3, 1),
                                  "pct_of_hbm_peak": round(head_bytes / us_greedy / 1e3 / HBM_PEAK_GBPS * 100, 2)},
                 "scores_then_top40": {"us": round(us_topk, 2), "GBps": round((head_bytes + HN * 8) / us_topk / 1e3, 1)},
+                "scores_top40_sample": {"us": round(us_sample, 2), "sampler_us": round(us_sample - us_topk, 2)},
                 "note": "lm_head 262144 x 1536, 4-bit group 32 (251 MB), two copies alternated; greedy_fused = aq_qmv_greedy "
                         "(8 bytes out); scores_then_top40 = aq_qmv_scores + aq_packed_topk"}
         for t in pool[0] + pool[1] + (hx, h_logits, h_best, h_scores, h_top):
