@@ -261,8 +261,8 @@ hipError_t packed_topk_launch(const unsigned long long* in, int64_t count, int t
 // go/engine/hip/kernels/sampling/topk.hipinc:86-191; score decode and softcap kernels/common/numeric.hipinc:95-110).
 // The reference runs the whole thing on one thread and evaluates exp() of every candidate in each of its four
 // passes; here each of up to 128 threads evaluates its candidate's weight once (tanh and exp in double are the
-// cost) and thread 0 then walks the list, adding in list order as the reference does, so every sum rounds the
-// same way.  out[0] = 0 when nothing can be sampled.
+// cost), thread 0 adds them once in list order, as the reference does, so every sum rounds the same way, and the
+// threads compare against that running sum side by side.  out[0] = 0 when nothing can be sampled.
 constexpr int kSampleMax = 128;
 
 __device__ __forceinline__ double sample_score(unsigned long long packed, double softcap) {
@@ -277,8 +277,17 @@ __global__ __launch_bounds__(kSampleMax) void packed_topk_sample_kernel(const un
                                                                         unsigned long long* __restrict__ out) {
     __shared__ unsigned long long vals[kSampleMax];
     __shared__ double wts[kSampleMax];
+    __shared__ double prefix[kSampleMax];
+    __shared__ double total_s;
+    __shared__ int bad, limit_s, kept_s, pick_s;
     const int t = threadIdx.x;
     vals[t] = t < top_k ? in[t] : 0ull;
+    if (t == 0) {
+        bad = 0;
+        limit_s = top_k;
+        kept_s = 0;
+        pick_s = kSampleMax;
+    }
     __syncthreads();
     int first_valid = top_k;  // the same scan on every thread: the branches below are uniform
     for (int i = 0; i < top_k; ++i)
@@ -307,49 +316,44 @@ __global__ __launch_bounds__(kSampleMax) void packed_topk_sample_kernel(const un
     wts[t] = (t >= first_valid && t < top_k && vals[t] != 0ull)
                  ? exp(sample_score(vals[t], softcap) / temperature - max_value)
                  : 0.0;
+    const bool valid = t >= first_valid && t < top_k && vals[t] != 0ull;
+    if (valid && !isfinite(wts[t])) bad = 1;  // any non-finite weight: nothing is sampled
     __syncthreads();
-    if (t != 0) return;
-    out[0] = 0ull;
-    double total = 0.0;
-    for (int i = first_valid; i < top_k; ++i) {
-        if (vals[i] == 0ull) continue;
-        if (!isfinite(wts[i])) return;
-        total += wts[i];
-    }
-    if (!(total > 0.0) || !isfinite(total)) return;
-    int limit = top_k;
-    if (top_p < 1.0) {
-        double cumulative = 0.0;
-        for (int i = first_valid; i < top_k; ++i) {
-            if (vals[i] == 0ull) continue;
-            cumulative += wts[i];
-            if (cumulative / total >= top_p) {
-                limit = i + 1;
-                break;
-            }
+    // The reference's four passes all add the same weights in the same order from 0.0: its total, its nucleus
+    // cumulative, its selected total and its draw cumulative are entries of ONE running sum.  Thread 0 forms that
+    // sum once; the comparisons against it are independent and every thread does its own.
+    if (t == 0) {
+        double run = 0.0;  // holes carry weight 0.0, and x + 0.0 is x: no branch in the chain of adds
+#pragma unroll 8
+        for (int i = 0; i < top_k; ++i) {
+            run += wts[i];
+            prefix[i] = run;
         }
+        total_s = run;
     }
-    double selected_total = 0.0;
-    unsigned long long fallback = vals[first_valid];
-    for (int i = first_valid; i < limit; ++i) {
-        if (vals[i] == 0ull) continue;
-        fallback = vals[i];
-        selected_total += wts[i];
+    __syncthreads();
+    const double total = total_s;
+    if (bad || !(total > 0.0) || !isfinite(total)) {
+        if (t == 0) out[0] = 0ull;
+        return;
     }
-    if (!(selected_total > 0.0) || !isfinite(selected_total)) return;
+    if (top_p < 1.0 && valid && prefix[t] / total >= top_p) atomicMin(&limit_s, t + 1);
+    __syncthreads();
+    const int limit = limit_s;
+    if (valid && t < limit) atomicMax(&kept_s, t);  // the last candidate inside the nucleus
+    __syncthreads();
+    const int kept = kept_s;
+    const double selected_total = prefix[kept];
+    if (!(selected_total > 0.0) || !isfinite(selected_total)) {
+        if (t == 0) out[0] = 0ull;
+        return;
+    }
     if (draw < 0.0) draw = 0.0;
     if (draw >= 1.0) draw = 0x1.fffffffffffffp-1;  // the double below 1
     const double target = draw * selected_total;
-    double cumulative = 0.0;
-    for (int i = first_valid; i < limit; ++i) {
-        if (vals[i] == 0ull) continue;
-        cumulative += wts[i];
-        if (target <= cumulative) {
-            out[0] = vals[i];
-            return;
-        }
-    }
-    out[0] = fallback;
+    if (valid && t < limit && target <= prefix[t]) atomicMin(&pick_s, t);
+    __syncthreads();
+    if (t == 0) out[0] = vals[pick_s < kSampleMax ? pick_s : kept];
 }
 
 hipError_t packed_topk_sample_launch(const unsigned long long* in, int top_k, float temperature, float top_p, float softcap,
