@@ -20,7 +20,7 @@ def _repack(ctx, gguf_type, rows, cols, data, offset=0):
     ctx._check(ctx.lib.aq_h2d(ctx.handle, src.ptr + offset, data.ctypes.data, data.nbytes))
     w, s, b = ctx.alloc(lay.packed_bytes), ctx.alloc(lay.scales_bytes), ctx.alloc(lay.scales_bytes)
     for t in (w, s, b):                      # stale contents must not survive
-        ctx._check(ctx.lib.aq_h2d(ctx.handle, t.ptr, np.full(t.nbytes, 0xA5, np.uint8).ctypes.data, t.nbytes))
+        t.upload(np.full(t.nbytes, 0xA5, np.uint8))
     ctx.gguf_to_affine(gguf_type, src.ptr + offset, data.nbytes, rows, cols, w, s, b)
     ctx.sync()
     out = (w.download(np.uint32).reshape(rows, lay.packed_cols), s.download(np.uint16).reshape(rows, lay.groups),
@@ -119,4 +119,43 @@ def test_repack_captured_and_errors(ctx, orc):
             call()
         assert e.value.code == code
     for t in (src, w, s, b):
+        t.free()
+
+
+@pytest.mark.parametrize("gguf_type", [G.Q4_K, G.Q6_K])
+def test_repack_full_size_projection_tensor(ctx, orc, gguf_type):
+    """The gate projection's shape (14336 x 4096), bit for bit against the oracle."""
+    rows, cols = 14336, 4096
+    say("gguf repack full size", G.NAMES[gguf_type], rows, cols)
+    data = G.random_blocks(gguf_type, rows, cols, seed=F.BASE_SEED + 360 + gguf_type)
+    (w, s, b), _ = _repack(ctx, gguf_type, rows, cols, data)
+    ow, os_, ob = orc.gguf_to_affine(gguf_type, rows, cols, data)
+    assert np.array_equal(w, ow) and np.array_equal(s, os_) and np.array_equal(b, ob)
+
+
+def test_gguf_lm_head_to_greedy_token(ctx, orc):
+    """A Q4_0 vocabulary projection as a GGUF file ships it -> device repack -> aq_qmv_greedy (group 32: the
+    diagonal-MFMA head kernel) -> the token ggml's dequantisation of the same blocks makes the winner."""
+    import aq_mi355
+    rows, cols = 32768, 1536
+    say("gguf lm_head greedy", rows, cols)
+    data = G.random_blocks(G.Q4_0, rows, cols, seed=F.BASE_SEED + 370, exact=True)
+    lay = aq_mi355.gguf_affine_layout(G.Q4_0, rows, cols)
+    src = ctx.to_device(data)
+    w, s, b = ctx.alloc(lay.packed_bytes), ctx.alloc(lay.scales_bytes), ctx.alloc(lay.scales_bytes)
+    ctx.gguf_to_affine(G.Q4_0, src, data.nbytes, rows, cols, w, s, b)
+    x = F.synthetic_x(1, cols, seed=F.BASE_SEED + 371)
+    dx, best, scores = ctx.to_device(x), ctx.alloc(8), ctx.alloc(rows * 8)
+    ctx.qmv_greedy(dx, w, s, b, best, 1, cols, rows, lay.group_size, lay.bits)
+    assert ctx.last_variant(0) == "qmv_greedy_diag"
+    ctx.qmv_scores(dx, w, s, b, scores, 1, cols, rows, lay.group_size, lay.bits)
+    ctx.sync()
+    packed = scores.download(np.uint64, rows)
+    got = int(best.download(np.uint64, 1)[0])
+    assert got == int(packed.max())
+    tok, score = aq_mi355.unpack_best(got)
+    ref = F.bf16_bits_to_f32(x).astype(np.float64).reshape(cols) @ G.ggml_dequant(G.Q4_0, rows, cols, data).T
+    norm = np.abs(ref).max()
+    assert abs(score - ref[tok]) <= 2e-3 * norm and ref[tok] >= ref.max() - 4e-3 * norm
+    for t in (src, w, s, b, dx, best, scores):
         t.free()
