@@ -159,3 +159,39 @@ def test_gguf_lm_head_to_greedy_token(ctx, orc):
     assert abs(score - ref[tok]) <= 2e-3 * norm and ref[tok] >= ref.max() - 4e-3 * norm
     for t in (src, w, s, b, dx, best, scores):
         t.free()
+
+
+@pytest.mark.parametrize("gguf_type", [G.Q4_K, G.Q6_K, G.Q8_0])
+def test_gguf_expert_stack_to_gather(ctx, orc, gguf_type):
+    """A stacked expert tensor [E, rows, cols] of GGUF blocks (as *_exps.weight ships) -> one repack over E * rows rows
+    -> aq_gather_qmv with the expert ids on the device, against ggml's dequantisation of the chosen experts' rows."""
+    import aq_mi355
+    E, rows, cols, routes, x_rows = 6, 96, 1024, 9, 3
+    say("gguf experts gather", G.NAMES[gguf_type], E, rows, cols)
+    data = G.random_blocks(gguf_type, E * rows, cols, seed=F.BASE_SEED + 380 + gguf_type, exact=True)
+    lay = aq_mi355.gguf_affine_layout(gguf_type, E * rows, cols)
+    src = ctx.to_device(data)
+    w, s, b = ctx.alloc(lay.packed_bytes), ctx.alloc(lay.scales_bytes), ctx.alloc(lay.scales_bytes)
+    ctx.gguf_to_affine(gguf_type, src, data.nbytes, E * rows, cols, w, s, b)
+    rng = np.random.default_rng(9)
+    rhs = rng.integers(0, E, routes).astype(np.int32)
+    lhs = rng.integers(0, x_rows, routes).astype(np.int32)
+    x = F.synthetic_x(x_rows, cols, seed=F.BASE_SEED + 381)
+    dx, dl, dr = ctx.to_device(x), ctx.to_device(lhs), ctx.to_device(rhs)
+    out_dim, row_base = 64, 32
+    dy = ctx.alloc(routes * out_dim * 4)
+    ctx.gather_qmv(dx, w, s, b, dl, dr, dy, routes, x_rows, cols, out_dim, E, rows, row_base, lay.group_size, lay.bits,
+                   aq_mi355.AQ_OUT_F32)
+    ctx.sync()
+    got = dy.download(np.float32, routes * out_dim).reshape(routes, out_dim).astype(np.float64)
+    weights = G.ggml_dequant(gguf_type, E * rows, cols, data).reshape(E, rows, cols)
+    xf = F.bf16_bits_to_f32(x).astype(np.float64).reshape(x_rows, cols)
+    ref = np.stack([weights[rhs[z], row_base:row_base + out_dim] @ xf[lhs[z]] for z in range(routes)])
+    norm = max(1.0, np.abs(weights).max())
+    check_accumulators(got / norm, ref / norm, G.NAMES[gguf_type])
+    # and against the oracle's gather over the oracle's repack of the same blocks
+    ow, os_, ob = orc.gguf_to_affine(gguf_type, E * rows, cols, data)
+    ref64, _ = orc.gather_qmv(x, x_rows, ow, os_, ob, lhs, rhs, routes, E, rows, row_base, out_dim, cols, lay.group_size, lay.bits)
+    check_accumulators(got / norm, np.asarray(ref64, np.float64).reshape(routes, out_dim) / norm, G.NAMES[gguf_type] + " oracle")
+    for t in (src, w, s, b, dx, dl, dr, dy):
+        t.free()
