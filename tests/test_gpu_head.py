@@ -253,3 +253,41 @@ def test_packed_topk_sample_against_oracle(ctx, orc):
             call()
         assert e.value.code == code
     buf.free()
+
+
+def test_sampling_pipeline_captured(ctx, orc):
+    """scores -> top-k -> sampler recorded into one graph (after an eager call has sized the scratch) and replayed with
+    eager work in between: every replay gives the eager token, which is the oracle's choice over the device's list."""
+    say("sampling pipeline captured")
+    K, N, gs, bits, k = 1536, 32768, 32, 4, 40
+    words, s, b = F.synthetic_affine(N, K, bits, gs, seed=F.BASE_SEED + 106)
+    dw = DeviceAffine(ctx, words, s, b)
+    xs = [ctx.to_device(F.synthetic_x(1, K, seed=F.BASE_SEED + 107 + i)) for i in range(2)]
+    dsc, dtop, dbest, dx = ctx.alloc(N * 8), ctx.alloc(k * 8), ctx.alloc(8), ctx.alloc(K * 2)
+
+    def pipeline():
+        ctx.qmv_scores(dx, dw.w, dw.s, dw.b, dsc, 1, K, N, gs, bits)
+        ctx.packed_topk(dsc, N, k, dtop)
+        ctx.packed_topk_sample(dtop, k, 0.9, 0.9, 30.0, 0.61, dbest)
+
+    want = []
+    for x in xs:                                   # eager, per input
+        ctx._check(ctx.lib.aq_d2d(ctx.handle, dx.ptr, x.ptr, K * 2))
+        pipeline()
+        ctx.sync()
+        got = int(_u64(dbest, 1)[0])
+        assert got == orc.packed_topk_sample(_u64(dtop, k), 0.9, 0.9, 30.0, 0.61) and got != 0
+        want.append(got)
+    ctx.capture_begin()
+    pipeline()
+    graph = ctx.capture_end()
+    for i in range(4):
+        ctx._check(ctx.lib.aq_d2d(ctx.handle, dx.ptr, xs[i % 2].ptr, K * 2))
+        ctx.fill_zero(dbest)
+        ctx.graph_launch(graph)
+        ctx.sync()
+        assert int(_u64(dbest, 1)[0]) == want[i % 2], i
+    ctx.graph_destroy(graph)
+    for t in xs + [dsc, dtop, dbest, dx]:
+        t.free()
+    dw.free()
