@@ -265,7 +265,7 @@ int launch_qmv_rows(aq_ctx* ctx, aq::QmvArgs a, int group_size, int bits, bool g
     }
     const bool fast = dot2_eligible(a.K, group_size, bits, a.x, a.w, (size_t)(M < 4 ? M : 4) * a.K * 2);
     if (!fast) {
-        ctx->last_variant[0] = "qmv_generic";
+        ctx->last_variant[0] = aq::qmv_six_eligible(a, bits, group_size) ? "qmv_six" : "qmv_generic";
         AQ_HIP(aq::qmv_generic_launch(a, bits, group_size, gather, ctx->stream), "hipLaunchKernel");
         return AQ_OK;
     }

@@ -217,6 +217,8 @@ hipError_t moe_combine_launch(const MoeCombineArgs& a, hipStream_t stream);
 
 // Any-width (2..8 bit, codes may straddle words), any-group fallback.
 hipError_t qmv_generic_launch(const QmvArgs& a, int bits, int group_size, bool gather, hipStream_t stream);
+// Six-bit codes in groups of 16 or 32 with K a multiple of 16 take a kernel of their own inside that launch.
+bool qmv_six_eligible(const QmvArgs& a, int bits, int group_size);
 
 // fp32 dequantisation of a whole tensor, bits in {1,2,4,8} (word-clean widths)
 // or {3,5,6} through the straddling path.

@@ -173,8 +173,105 @@ __global__ __launch_bounds__(256) void qmv_generic_kernel(const QmvArgs a, int b
     }
 }
 
+// Six-bit codes in groups of 16 or 32 (the layouts GGUF Q6_K and Q5_K tensors repack to): one wavefront per row as
+// above, but a lane takes 16 codes = three whole words at a time (a wavefront reads 768 contiguous bytes of codes per
+// step), decodes them with shifts of one 64-bit and one 32-bit piece, and uses the group form of the sum,
+// scale * sum(code * x) + bias * sum(x), with one scale and bias per lane and step (16 codes never straddle a group).
+template <int GS>
+__global__ __launch_bounds__(256) void qmv_six_kernel(const QmvArgs a, int gather) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int row = blockIdx.x * 4 + wave;
+    const int K = a.K, N = a.N;
+    if (row >= N) return;
+    const int64_t words = (int64_t)K * 6 / 32;
+    const int gpr = K / GS;
+    const uint32_t* wbase = a.w;
+    const uint16_t* sbase = a.s;
+    const uint16_t* bbase = a.b;
+    const uint16_t* xbase = a.x;
+    int64_t yoff = 0;
+    int m_count = a.M;
+    bool ok = true;
+    if (gather) {
+        const int z = blockIdx.y;
+        const int e = a.rhs[z];
+        int xr = a.lhs ? a.lhs[z] : 0;
+        ok = (unsigned)e < (unsigned)a.num_experts && (unsigned)xr < (unsigned)a.x_rows;
+        const int64_t row0 = ok ? ((int64_t)e * a.expert_rows + a.row_base) : 0;
+        if (!ok) xr = 0;
+        wbase += row0 * words;
+        sbase += row0 * gpr;
+        bbase += row0 * gpr;
+        xbase += (int64_t)xr * K;
+        yoff = (int64_t)z * N;
+        m_count = 1;
+    }
+    const uint32_t* wr = wbase + (int64_t)row * words;
+    const uint16_t* sr = sbase + (int64_t)row * gpr;
+    const uint16_t* br = bbase + (int64_t)row * gpr;
+    for (int m0 = 0; m0 < m_count; m0 += 4) {
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int k0 = lane * 16; k0 < K; k0 += kWave * 16) {
+            const uint32_t* wp = wr + (k0 >> 4) * 3;
+            const uint32_t w0 = wp[0], w1 = wp[1], w2 = wp[2];
+            const float scale = bf16_bits_to_f32(sr[k0 / GS]), bias = bf16_bits_to_f32(br[k0 / GS]);
+            const uint64_t lo = (uint64_t)w0 | (uint64_t)w1 << 32;
+            float c[16];
+#pragma unroll
+            for (int i = 0; i < 10; i++) c[i] = (float)(uint32_t)((lo >> (6 * i)) & 63u);
+            c[10] = (float)((uint32_t)(lo >> 60) | ((w2 & 3u) << 4));
+#pragma unroll
+            for (int i = 0; i < 5; i++) c[11 + i] = (float)((w2 >> (2 + 6 * i)) & 63u);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                if (m0 + j < m_count) {
+                    const uint4* xp = reinterpret_cast<const uint4*>(xbase + (int64_t)(m0 + j) * K + k0);
+                    const uint4 x0 = xp[0], x1 = xp[1];
+                    const uint32_t xw[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+                    float dot = 0.f, xs = 0.f;
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        const float xa = __uint_as_float(xw[i] << 16), xb = __uint_as_float(xw[i] & 0xffff0000u);
+                        dot = __fmaf_rn(c[2 * i], xa, dot);
+                        dot = __fmaf_rn(c[2 * i + 1], xb, dot);
+                        xs += xa + xb;
+                    }
+                    acc[j] += scale * dot + bias * xs;
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            float tot = wave_sum(acc[j]);
+            if (!ok) tot = 0.0f;
+            if (lane == 0 && m0 + j < m_count) {
+                const int64_t o = yoff + (int64_t)(m0 + j) * N + row;
+                if (a.out_f32) {
+                    reinterpret_cast<float*>(a.y)[o] = tot;
+                } else {
+                    reinterpret_cast<uint16_t*>(a.y)[o] = f32_to_bf16_bits(tot);
+                }
+            }
+        }
+    }
+}
+
+bool qmv_six_eligible(const QmvArgs& a, int bits, int group_size) {
+    return bits == 6 && (group_size == 16 || group_size == 32) && a.K % 16 == 0 &&
+           (reinterpret_cast<uintptr_t>(a.x) & 15) == 0 && (reinterpret_cast<uintptr_t>(a.w) & 3) == 0 &&
+           (reinterpret_cast<uintptr_t>(a.s) & 1) == 0 && (reinterpret_cast<uintptr_t>(a.b) & 1) == 0;
+}
+
 hipError_t qmv_generic_launch(const QmvArgs& a, int bits, int group_size, bool gather, hipStream_t stream) {
     dim3 grid((unsigned)((a.N + 3) / 4), gather ? (unsigned)a.routes : 1u, 1u);
+    if (qmv_six_eligible(a, bits, group_size)) {
+        if (group_size == 16)
+            hipLaunchKernelGGL(qmv_six_kernel<16>, grid, dim3(256), 0, stream, a, gather ? 1 : 0);
+        else
+            hipLaunchKernelGGL(qmv_six_kernel<32>, grid, dim3(256), 0, stream, a, gather ? 1 : 0);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(qmv_generic_kernel, grid, dim3(256), 0, stream, a, bits, group_size, gather ? 1 : 0);
     return hipGetLastError();
 }
