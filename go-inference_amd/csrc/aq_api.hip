@@ -474,6 +474,9 @@ int aq_capture_end(aq_ctx* ctx, aq_graph** out) {
     std::lock_guard<std::mutex> lk(ctx->mu);
     hipGraph_t g = nullptr;
     AQ_HIP(hipStreamEndCapture(ctx->stream, &g), "hipStreamEndCapture");
+    // the context workspaces whose addresses the captured kernels carry, and the generation they were captured under
+    bool uses_ws = false, uses_head_ws = false;
+    uint64_t ws_generation = 0, head_ws_generation = 0;
     aq_graph* ag = new (std::nothrow) aq_graph();
     if (!ag) {
         (void)hipGraphDestroy(g);
@@ -481,6 +484,7 @@ int aq_capture_end(aq_ctx* ctx, aq_graph** out) {
     }
     ag->graph = g;
     hipError_t rc = hipGraphInstantiate(&ag->exec, g, nullptr, nullptr, 0);
+    ctx->ws.touched = ctx->head_ws.touched = false;
     if (rc != hipSuccess) {
         aq_graph_destroy(ag);
         return hip_fail(rc, "hipGraphInstantiate");
@@ -496,6 +500,10 @@ int aq_graph_launch(aq_ctx* ctx, aq_graph* graph) {
     return AQ_OK;
 }
 
+    ag->uses_ws = ctx->ws.touched;
+    ag->uses_head_ws = ctx->head_ws.touched;
+    ag->ws_generation = ctx->ws.generation;
+    ag->head_ws_generation = ctx->head_ws.generation;
 void aq_graph_destroy(aq_graph* graph) {
     if (!graph) return;
     if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
@@ -508,6 +516,12 @@ int aq_qmv(aq_ctx* ctx, const void* x, const void* packed, const void* scales, c
     if (!ctx) return fail(AQ_ERR_ARG, "aq_qmv: ctx is null");
     if (M < 0 || K < 0 || N < 0) return fail(AQ_ERR_SHAPE, "aq_qmv: M, K, N must be non-negative");
     if (M == 0 || N == 0 || K == 0) return AQ_OK;
+    if ((graph->uses_ws && graph->ws_generation != ctx->ws.generation) ||
+        (graph->uses_head_ws && graph->head_ws_generation != ctx->head_ws.generation))
+        return fail(AQ_ERR_UNSUPPORTED,
+                    "aq_graph_launch: the context's workspace was reallocated after this graph was captured (a later call "
+                    "needed more room); the graph's kernels still point at the freed block: capture it again, and reserve "
+                    "the largest workspace first (aq_reserve_workspace / aq_reserve_workspace_bytes)");
     if (int rc = check_geometry("aq_qmv", K, group_size, bits)) return rc;
     if (!x || !packed || !scales || !biases || !y) return fail(AQ_ERR_ARG, "aq_qmv: null operand");
     if (!aligned(x, 2) || !aligned(packed, 4) || !aligned(scales, 2) || !aligned(biases, 2) || !aligned(y, 2))

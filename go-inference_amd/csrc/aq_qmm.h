@@ -74,9 +74,14 @@ const QmmVariant* qmmh_variant(int idx);
 hipError_t qmmh_launch(int idx, const QmmArgs& a, void* workspace, hipStream_t stream);
 
 // Scratch memory a context lends to the matmul path; grown on demand, never while a capture is open.
+// `generation` counts reallocations: a captured graph has the block's address in its kernel arguments and is
+// only valid while the generation it was captured under stands.  `touched` is set by every reserve call, so
+// that the owner can tell whether a capture used the block.
 struct Workspace {
     void* ptr = nullptr;
     size_t bytes = 0;
+    uint64_t generation = 0;
+    bool touched = false;
 };
 
 int qmm_variant_count();

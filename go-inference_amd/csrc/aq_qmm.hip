@@ -391,6 +391,7 @@ static int find_qmm(int bits, int mb, int nb, int wm, int wn) {
 // Makes ws hold at least `need` bytes.  Growing frees the old block, so everything queued on the stream
 // is drained first; a stream that is being captured cannot be drained.
 static int grow_workspace(Workspace* ws, size_t need, hipStream_t stream, FailFn fail) {
+    ws->touched = true;
     if (ws->bytes >= need) return AQ_OK;
     hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
     if (stream != nullptr && hipStreamIsCapturing(stream, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone)
@@ -402,6 +403,7 @@ static int grow_workspace(Workspace* ws, size_t need, hipStream_t stream, FailFn
     if (ws->ptr) (void)hipFree(ws->ptr);
     ws->ptr = nullptr;
     ws->bytes = 0;
+    ws->generation++;  // graphs captured over the old block must not run again
     const size_t want = need + need / 4;  // headroom: prompts grow a little from call to call
     rc = hipMalloc(&ws->ptr, want);
     if (rc != hipSuccess) return fail(AQ_ERR_NOMEM, "aq_qmm: cannot allocate a %zu-byte workspace (HIP %d)", want, (int)rc);

@@ -88,7 +88,12 @@ int aq_timer_stop(aq_ctx *ctx, float *elapsed_ms); /* records, waits, reports */
  * launch batch (hipLaunchKernelContext batching, go/engine/hip/hip_launch.go:240-273,
  * cgoHIPDriver.LaunchKernelBatch go/engine/hip/hip_driver_cgo.go:1137-1190).  Only the
  * kernel entry points (aq_qmv*, aq_qmm, aq_gather_qmv*, aq_act_mul, aq_moe_*, aq_dequant_f32, aq_fill_zero, aq_d2d)
- * may be called while capturing; the pointers they were given must stay valid for replays. */
+ * may be called while capturing; the pointers they were given must stay valid for replays.
+ * Calls that go through the context's workspace (aq_qmm, aq_qmv with many rows, aq_packed_topk, aq_qmv_greedy,
+ * the unfused fallbacks) record the workspace's address: the workspace cannot grow during a capture (the call
+ * fails with a message), and when a later call makes it grow, every graph captured over the old block is
+ * refused by aq_graph_launch with AQ_ERR_UNSUPPORTED - reserve the largest workspace first
+ * (aq_reserve_workspace / aq_reserve_workspace_bytes), or capture again. */
 typedef struct aq_graph aq_graph;
 int aq_capture_begin(aq_ctx *ctx);
 int aq_capture_end(aq_ctx *ctx, aq_graph **out);
@@ -240,7 +245,9 @@ int aq_moe_combine(aq_ctx *ctx, const void *route_rows, const float *weights, vo
  * row qualified.  best is device uint64[M]; the call clears it itself.  Replaces
  * rocm_mlx_q4_projection_greedy / _greedy_batch (go/engine/hip/kernels/quant/affine_projection_fused.hipinc:190-410):
  * for M == 1 and 4/8-bit codes 8 bytes leave the kernel instead of N logits; other shapes run the projection
- * into the context's workspace and reduce it there. */
+ * into the context's workspace and reduce it there.  Greedy calls on one context share one set of partial
+ * maxima and fold tickets: they must be ordered with each other on the stream (no greedy call, direct or
+ * inside a replayed graph, may overlap another one of the same context). */
 int aq_qmv_greedy(aq_ctx *ctx, const void *x, const void *packed, const void *scales, const void *biases,
                   const int32_t *suppress, int suppress_count, uint64_t *best, int M, int K, int N, int group_size,
                   int bits);

@@ -291,3 +291,51 @@ def test_sampling_pipeline_captured(ctx, orc):
     for t in xs + [dsc, dtop, dbest, dx]:
         t.free()
     dw.free()
+
+
+def test_graph_is_refused_once_the_workspace_has_moved(orc):
+    """A captured graph carries the address of the context's workspace.  When a later call makes the workspace
+    grow (the old block is freed), launching that graph must be refused, not run; a graph that never touched the
+    workspace still launches."""
+    import aq_mi355
+    say("graph vs workspace growth")
+    c = aq_mi355.Context(0)
+    try:
+        K, N, k = 1024, 4096, 8
+        words, s, b = F.synthetic_affine(N, K, 4, 64, seed=F.BASE_SEED + 120)
+        dw = DeviceAffine(c, words, s, b)
+        dx = c.to_device(F.synthetic_x(1, K, seed=F.BASE_SEED + 121))
+        dsc, dtop, dy = c.alloc(N * 8), c.alloc(k * 8), c.alloc(N * 2)
+        c.qmv_scores(dx, dw.w, dw.s, dw.b, dsc, 1, K, N, 64, 4)
+        c.packed_topk(dsc, N, k, dtop)          # eager: sizes the workspace
+        c.sync()
+        want = _u64(dtop, k).copy()
+        c.capture_begin()
+        c.packed_topk(dsc, N, k, dtop)
+        with_ws = c.capture_end()
+        c.capture_begin()
+        c.qmv(dx, dw.w, dw.s, dw.b, dy, 1, K, N, 64, 4)
+        without_ws = c.capture_end()
+        c.graph_launch(with_ws)
+        c.sync()
+        assert np.array_equal(_u64(dtop, k), want)
+        c.reserve_workspace_bytes(64 << 20)      # the workspace moves
+        with pytest.raises(aq_mi355.AqError) as e:
+            c.graph_launch(with_ws)
+        assert e.value.code == aq_mi355.AQ_ERR_UNSUPPORTED and "workspace" in str(e.value)
+        c.graph_launch(without_ws)               # no workspace inside: still fine
+        c.sync()
+        c.capture_begin()                        # captured again over the new block: runs
+        c.packed_topk(dsc, N, k, dtop)
+        again = c.capture_end()
+        c.fill_zero(dtop)
+        c.graph_launch(again)
+        c.sync()
+        assert np.array_equal(_u64(dtop, k), want)
+        for g in (with_ws, without_ws, again):
+            c.graph_destroy(g)
+        for t in (dx, dsc, dtop, dy):
+            t.free()
+        dw.free()
+    finally:
+        c.close()
