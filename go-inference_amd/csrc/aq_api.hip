@@ -54,6 +54,15 @@ bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) &
 
 }  // namespace
 
+// Scratch of aq_qmv_greedy_static, the entry point that allocates nothing: the packed best of every 16 rows
+// (or of every wavefront) of the projection, then the fold's tickets and slots.  Every GPU the library runs on
+// holds its own copy until the process ends; host code uses the address hipGetSymbolAddress returns for the
+// current device (kept in the context), never the array's name.
+constexpr size_t kStaticPartialBytes = (size_t)2 << 20;
+constexpr size_t kStaticScratchBytes = kStaticPartialBytes + 1024;
+static_assert(aq::kHeadFoldBytes <= 1024, "the fold area sits behind the partials");
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 struct aq_ctx {
     int device = 0;
     hipStream_t own_stream = nullptr;
@@ -66,6 +75,7 @@ struct aq_ctx {
     aq::Workspace ws;       // scratch of the matmul path and of the unfused fallbacks (aq_qmm.h)
     aq::Workspace head_ws;         // per-wavefront maxima of aq_qmv_greedy; sized at creation for common vocabularies
     void* head_fold = nullptr;     // aq_qmv_greedy's fold tickets and slots (aq::kHeadFoldBytes, kept zeroed by the kernel)
+    unsigned char* static_scratch = nullptr;  // this device's copy of `scratch` (hipGetSymbolAddress at creation)
     char name[256] = {0};
 };
 
@@ -344,6 +354,12 @@ int aq_create(int device, aq_ctx** out) {
         aq_destroy(ctx);
         return hip_fail(rc, "hipStreamCreate");
     }
+    // the device is current (hipSetDevice above): this is its own copy of the array
+    rc = hipGetSymbolAddress(reinterpret_cast<void**>(&ctx->static_scratch), HIP_SYMBOL(scratch));
+    if (rc != hipSuccess || !ctx->static_scratch) {
+        aq_destroy(ctx);
+        return hip_fail(rc != hipSuccess ? rc : hipErrorInvalidSymbol, "hipGetSymbolAddress");
+    }
     ctx->stream = ctx->own_stream;
     *out = ctx;
     return AQ_OK;
@@ -458,6 +474,9 @@ int aq_timer_stop(aq_ctx* ctx, float* elapsed_ms) {
 struct aq_graph {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
+    // the context workspaces whose addresses the captured kernels carry, and the generation they were captured under
+    bool uses_ws = false, uses_head_ws = false;
+    uint64_t ws_generation = 0, head_ws_generation = 0;
 };
 
 int aq_capture_begin(aq_ctx* ctx) {
@@ -465,6 +484,7 @@ int aq_capture_begin(aq_ctx* ctx) {
     std::lock_guard<std::mutex> lk(ctx->mu);
     if (ctx->stream == nullptr) return fail(AQ_ERR_UNSUPPORTED, "aq_capture_begin: the legacy default stream cannot be captured");
     AQ_HIP(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
+    ctx->ws.touched = ctx->head_ws.touched = false;
     return AQ_OK;
 }
 
@@ -474,17 +494,17 @@ int aq_capture_end(aq_ctx* ctx, aq_graph** out) {
     std::lock_guard<std::mutex> lk(ctx->mu);
     hipGraph_t g = nullptr;
     AQ_HIP(hipStreamEndCapture(ctx->stream, &g), "hipStreamEndCapture");
-    // the context workspaces whose addresses the captured kernels carry, and the generation they were captured under
-    bool uses_ws = false, uses_head_ws = false;
-    uint64_t ws_generation = 0, head_ws_generation = 0;
     aq_graph* ag = new (std::nothrow) aq_graph();
     if (!ag) {
         (void)hipGraphDestroy(g);
         return fail(AQ_ERR_NOMEM, "aq_capture_end: out of host memory");
     }
     ag->graph = g;
+    ag->uses_ws = ctx->ws.touched;
+    ag->uses_head_ws = ctx->head_ws.touched;
+    ag->ws_generation = ctx->ws.generation;
+    ag->head_ws_generation = ctx->head_ws.generation;
     hipError_t rc = hipGraphInstantiate(&ag->exec, g, nullptr, nullptr, 0);
-    ctx->ws.touched = ctx->head_ws.touched = false;
     if (rc != hipSuccess) {
         aq_graph_destroy(ag);
         return hip_fail(rc, "hipGraphInstantiate");
@@ -496,14 +516,16 @@ int aq_capture_end(aq_ctx* ctx, aq_graph** out) {
 int aq_graph_launch(aq_ctx* ctx, aq_graph* graph) {
     if (!ctx || !graph || !graph->exec) return fail(AQ_ERR_ARG, "aq_graph_launch: bad argument");
     std::lock_guard<std::mutex> lk(ctx->mu);
+    if ((graph->uses_ws && graph->ws_generation != ctx->ws.generation) ||
+        (graph->uses_head_ws && graph->head_ws_generation != ctx->head_ws.generation))
+        return fail(AQ_ERR_UNSUPPORTED,
+                    "aq_graph_launch: the context's workspace was reallocated after this graph was captured (a later call "
+                    "needed more room); the graph's kernels still point at the freed block: capture it again, and reserve "
+                    "the largest workspace first (aq_reserve_workspace / aq_reserve_workspace_bytes)");
     AQ_HIP(hipGraphLaunch(graph->exec, ctx->stream), "hipGraphLaunch");
     return AQ_OK;
 }
 
-    ag->uses_ws = ctx->ws.touched;
-    ag->uses_head_ws = ctx->head_ws.touched;
-    ag->ws_generation = ctx->ws.generation;
-    ag->head_ws_generation = ctx->head_ws.generation;
 void aq_graph_destroy(aq_graph* graph) {
     if (!graph) return;
     if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
@@ -516,12 +538,6 @@ int aq_qmv(aq_ctx* ctx, const void* x, const void* packed, const void* scales, c
     if (!ctx) return fail(AQ_ERR_ARG, "aq_qmv: ctx is null");
     if (M < 0 || K < 0 || N < 0) return fail(AQ_ERR_SHAPE, "aq_qmv: M, K, N must be non-negative");
     if (M == 0 || N == 0 || K == 0) return AQ_OK;
-    if ((graph->uses_ws && graph->ws_generation != ctx->ws.generation) ||
-        (graph->uses_head_ws && graph->head_ws_generation != ctx->head_ws.generation))
-        return fail(AQ_ERR_UNSUPPORTED,
-                    "aq_graph_launch: the context's workspace was reallocated after this graph was captured (a later call "
-                    "needed more room); the graph's kernels still point at the freed block: capture it again, and reserve "
-                    "the largest workspace first (aq_reserve_workspace / aq_reserve_workspace_bytes)");
     if (int rc = check_geometry("aq_qmv", K, group_size, bits)) return rc;
     if (!x || !packed || !scales || !biases || !y) return fail(AQ_ERR_ARG, "aq_qmv: null operand");
     if (!aligned(x, 2) || !aligned(packed, 4) || !aligned(scales, 2) || !aligned(biases, 2) || !aligned(y, 2))
@@ -1116,10 +1132,27 @@ int aq_moe_combine(aq_ctx* ctx, const void* route_rows, const float* weights, vo
 
 namespace {
 
+// The static scratch array of the context's device as (partial maxima, fold area) for `slots` maxima; the fold
+// area's tickets must start at zero whatever an earlier call left there, so they are cleared by a fill kernel
+// ahead of the projection on the same stream (a kernel, not a memset node: the call may be under capture).
+int static_head_scratch(aq_ctx* ctx, const char* op, size_t slots, unsigned long long** partial, unsigned long long** fold) {
+    if (slots * 8 > kStaticPartialBytes)
+        return fail(AQ_ERR_SIZE, "%s: %zu partial maxima need %zu bytes, the static scratch holds %zu; use aq_qmv_greedy", op,
+                    slots, slots * 8, kStaticPartialBytes);
+    if (!ctx->static_scratch) return fail(AQ_ERR_NODEVICE, "%s: the device's scratch array was not resolved", op);
+    *partial = reinterpret_cast<unsigned long long*>(ctx->static_scratch);
+    *fold = reinterpret_cast<unsigned long long*>(ctx->static_scratch + kStaticPartialBytes);
+    AQ_HIP(aq::fill_zero_launch(*fold, aq::kHeadFoldBytes, ctx->stream), "hipLaunchKernel");
+    return AQ_OK;
+}
+
 // Shared front of aq_qmv_greedy / aq_qmv_scores.  fuse 3: best[M]; fuse 4: scores[M, N].
+// no_alloc (fuse 3 only): the partial maxima and the fold area live in the device's static scratch array instead of
+// the context's workspaces, and a shape the fused kernels do not take is refused instead of going through scratch
+// that would have to be allocated.
 int head_call(aq_ctx* ctx, const char* op, int fuse, const void* x, const void* packed, const void* scales,
               const void* biases, const int32_t* suppress, int suppress_count, uint64_t* out, int M, int K, int N,
-              int group_size, int bits) {
+              int group_size, int bits, bool no_alloc = false) {
     if (!ctx) return fail(AQ_ERR_ARG, "%s: ctx is null", op);
     if (M < 0 || K < 0 || N < 0 || suppress_count < 0) return fail(AQ_ERR_SHAPE, "%s: M, K, N, suppress_count must be non-negative", op);
     if (M == 0) return AQ_OK;
@@ -1129,6 +1162,10 @@ int head_call(aq_ctx* ctx, const char* op, int fuse, const void* x, const void* 
     if (suppress && !aligned(suppress, 4)) return fail(AQ_ERR_ARG, "%s: operand pointer is not element-aligned", op);
     const bool fused = M == 1 && N > 0 && K > 0 && ctx->forced[0] < 0 && (bits == 4 || bits == 8) && x && packed &&
                        dot2_eligible(K, group_size, bits, x, packed, (size_t)K * 2);
+    if (no_alloc && !fused && M > 0 && N > 0 && K > 0)
+        return fail(AQ_ERR_UNSUPPORTED,
+                    "%s: takes one activation row of 4- or 8-bit codes with 16-byte aligned rows (the fused kernels); "
+                    "other shapes need scratch memory: use aq_qmv_greedy", op);
     if (fuse == 3 && !fused) {
         // the unfused reduction accumulates with atomics and starts from "no result"
         std::lock_guard<std::mutex> lk(ctx->mu);
@@ -1160,7 +1197,10 @@ int head_call(aq_ctx* ctx, const char* op, int fuse, const void* x, const void* 
             a.suppress_count = suppress_count;
             if (di >= 0 && aq::qmvd_head_supported(di, fuse) && aq::qmvd_fits(a, bits, group_size, false, di)) {
                 const size_t slots = aq::qmvd_head_partials(di, N);
-                if (fuse == 3) {
+                unsigned long long* fold = static_cast<unsigned long long*>(ctx->head_fold);
+                if (fuse == 3 && no_alloc) {
+                    if (int rc = static_head_scratch(ctx, op, slots, &a.partial, &fold)) return rc;
+                } else if (fuse == 3) {
                     AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
                     if (int rc = aq::workspace_reserve(ctx->stream, &ctx->head_ws, slots * 8, fail)) return rc;
                     a.partial = static_cast<unsigned long long*>(ctx->head_ws.ptr);
@@ -1168,8 +1208,8 @@ int head_call(aq_ctx* ctx, const char* op, int fuse, const void* x, const void* 
                 ctx->last_variant[0] = fuse == 3 ? "qmv_greedy_diag" : "qmv_scores_diag";
                 AQ_HIP(aq::qmvd_head_launch(di, fuse, a, ctx->stream), "hipLaunchKernel");
                 if (fuse == 3)
-                    AQ_HIP(aq::head_fold_launch(a.partial, (int)slots, static_cast<unsigned long long*>(ctx->head_fold),
-                                                reinterpret_cast<unsigned long long*>(out), ctx->stream),
+                    AQ_HIP(aq::head_fold_launch(a.partial, (int)slots, fold, reinterpret_cast<unsigned long long*>(out),
+                                                ctx->stream),
                            "hipLaunchKernel");
                 return AQ_OK;
             }
@@ -1178,9 +1218,14 @@ int head_call(aq_ctx* ctx, const char* op, int fuse, const void* x, const void* 
         int rows = idx >= 0 ? aq::qmv_variant(idx)->rows : 1;
         while (rows > 1 && !aq::qmv_head_supported(bits, fuse, rows)) rows >>= 1;
         if (!aq::qmv_head_supported(bits, fuse, rows)) return fail(AQ_ERR_UNSUPPORTED, "%s: no kernel for bits=%d", op, bits);
-        if (fuse == 3) {
+        unsigned long long* partial = nullptr;
+        unsigned long long* fold = static_cast<unsigned long long*>(ctx->head_fold);
+        if (fuse == 3 && no_alloc) {
+            if (int rc = static_head_scratch(ctx, op, aq::qmv_head_partials(N, rows), &partial, &fold)) return rc;
+        } else if (fuse == 3) {
             AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
             if (int rc = aq::workspace_reserve(ctx->stream, &ctx->head_ws, aq::qmv_head_partials(N, rows) * 8, fail)) return rc;
+            partial = static_cast<unsigned long long*>(ctx->head_ws.ptr);
         }
         {
             aq::QmvArgs a{};
@@ -1196,8 +1241,8 @@ int head_call(aq_ctx* ctx, const char* op, int fuse, const void* x, const void* 
             a.routes = 1;
             a.suppress = suppress;
             a.suppress_count = suppress_count;
-            a.partial = static_cast<unsigned long long*>(ctx->head_ws.ptr);
-            a.fold = static_cast<unsigned long long*>(ctx->head_fold);
+            a.partial = partial;
+            a.fold = fold;
             ctx->last_variant[0] = fuse == 3 ? "qmv_greedy_dot2" : "qmv_scores_dot2";
             AQ_HIP(aq::qmv_head_launch(bits, fuse, rows, a, ctx->stream), "hipLaunchKernel");
             return AQ_OK;
@@ -1233,6 +1278,12 @@ int aq_qmv_greedy(aq_ctx* ctx, const void* x, const void* packed, const void* sc
                   int bits) {
     return head_call(ctx, "aq_qmv_greedy", 3, x, packed, scales, biases, suppress, suppress_count, best, M, K, N,
                      group_size, bits);
+}
+
+int aq_qmv_greedy_static(aq_ctx* ctx, const void* x, const void* packed, const void* scales, const void* biases,
+                         const int32_t* suppress, int suppress_count, uint64_t* best, int K, int N, int group_size, int bits) {
+    return head_call(ctx, "aq_qmv_greedy_static", 3, x, packed, scales, biases, suppress, suppress_count, best, 1, K, N,
+                     group_size, bits, true);
 }
 
 int aq_qmv_scores(aq_ctx* ctx, const void* x, const void* packed, const void* scales, const void* biases,

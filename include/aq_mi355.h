@@ -252,6 +252,20 @@ int aq_qmv_greedy(aq_ctx *ctx, const void *x, const void *packed, const void *sc
                   const int32_t *suppress, int suppress_count, uint64_t *best, int M, int K, int N, int group_size,
                   int bits);
 
+/* aq_qmv_greedy for one activation row with NO allocation of any kind (no hipMalloc / hipFree, no workspace
+ * growth): it has no counterpart in the reference and exists for callers that cannot allocate - code under
+ * HIP graph capture, tight serving loops, harnesses that forbid it.  The partial maxima and the fold tickets
+ * live in a static device array of 2 MiB + 1 KiB that every GPU the library has a context on holds until the
+ * process ends.  Limits: M == 1; 4- or 8-bit codes whose rows are 16-byte aligned (the shapes the fused
+ * kernels take, anything else returns AQ_ERR_UNSUPPORTED); at most 262144 partial maxima (one per 16 rows for
+ * 4-bit group-32/64 codes with K > 1024, else one per 1..4 rows), i.e. vocabularies of up to 4 M rows on the
+ * fast path and at least 262144 rows otherwise: beyond that AQ_ERR_SIZE.  best[0] is bit-identical to
+ * aq_qmv_greedy's.  All calls on one GPU share that GPU's array (also across contexts): calls that overlap on
+ * one GPU race; order them on one stream. */
+int aq_qmv_greedy_static(aq_ctx *ctx, const void *x, const void *packed, const void *scales, const void *biases,
+                         const int32_t *suppress, int suppress_count, uint64_t *best, int K, int N, int group_size,
+                         int bits);
+
 /* The same projection storing every row's packed (score, row): scores is device uint64[M, N]; suppressed or
  * non-finite rows hold 0.  rocm_mlx_q4_projection_scores (affine_projection_fused.hipinc:411-446), the input
  * of top-k sampling. */
