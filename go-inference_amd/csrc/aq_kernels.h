@@ -87,6 +87,7 @@ struct QmvVariant {
                  // 3: streaming dot2 kernel (aq_qmv_stream.hip; depth = rows in flight, xmode = slices per row)
                  // 4: diagonal-MFMA kernel (aq_qmv_diag.hip; m = most rows, rows = sets of 16 rows per workgroup,
                  //    xmode = chunks per step when not 4), 5: the same for quantisation groups of 32 codes
+                 // 6: token-tile MFMA kernel (aq_qmv_tok.hip; m = most rows, rows = sets of 32 weight rows per wavefront)
 };
 
 int qmv_variant_count();
@@ -167,6 +168,14 @@ hipError_t head_fold_launch(const unsigned long long* partial, int count, unsign
                             hipStream_t stream);
 bool qmvd_multi_supported(int idx);
 hipError_t qmvd_multi_launch(int idx, QmvMultiArgs ma, hipStream_t stream);
+
+// Token-tile MFMA matvec kernels (aq_qmv_tok.hip; 4-bit group-64 codes, up to 32 activation rows as the rows of a
+// 32x32x16 MFMA, K a multiple of 256; one launch, no scratch memory).  kind 6 in QmvVariant.
+int qmvt_variant_count();
+const QmvVariant* qmvt_variant(int idx);
+bool qmvt_fits(const QmvArgs& a, int bits, int group_size, int idx);
+hipError_t qmvt_launch(int idx, const QmvArgs& a, hipStream_t stream);
+int qmvt_pick(int M, int K, int N, int cu_count);
 
 // lm_head kernels (aq_qmv_head.hip), one activation row: the projection with its epilogue replaced by
 //   fuse 3: best[0] = max over rows of pack(score, row): every wavefront stores its own maximum into

@@ -141,6 +141,8 @@ def _parse_variant(name):
         return "stream", parts["b"], 1, parts["g"]
     if name.startswith("qmvd_"):
         return "diag", parts["b"], parts["m"], parts["g"]
+    if name.startswith("qmvt_"):
+        return "tok", parts["b"], parts["m"], 0
     return "dot2", parts["b"], parts["m"], parts["g"]
 
 
@@ -159,7 +161,7 @@ def test_qmv_every_variant(ctx, orc):
     try:
         for idx, name in enumerate(names):
             fam, bits, m, gather = _parse_variant(name)
-            if gather or fam in ("blk", "stream", "diag"):
+            if gather or fam in ("blk", "stream", "diag", "tok"):
                 continue  # covered by test_gather_every_variant / test_qmvb_every_variant / test_qmvs_every_variant / test_qmvd_every_variant
             say("variant", idx, name)
             if bits not in data:
@@ -202,7 +204,7 @@ def test_gather_every_variant(ctx, orc):
     try:
         for idx, name in enumerate(names):
             fam, bits, m, gather = _parse_variant(name)
-            if not gather or fam in ("blk", "stream", "diag"):
+            if not gather or fam in ("blk", "stream", "diag", "tok"):
                 continue
             say("gather variant", idx, name)
             fx = F.gather_fixture(out_dim, in_dim, 64, bits, E, expert_rows, True, routes)
@@ -815,7 +817,7 @@ def test_few_rows_k_shared_over_workgroups(ctx, orc, fn, M, K, N, bits):
     say("few rows, split K", fn, M, K, N, bits)
     acc, ref, (words, s, b, x) = _qmv_case(ctx, orc, M, K, N, bits, 64, 4000 + M + K, fn=fn)
     say("  ran on", ctx.last_variant(0), ctx.last_variant(1))
-    if M > 16 and fn == "qmv":
+    if M > 32 and fn == "qmv":
         assert ctx.last_variant(1).startswith("qmm"), ctx.last_variant(1)
     dw = DeviceAffine(ctx, words, s, b)
     again = run_qmv(ctx, x, dw, M, K, N, 64, bits, True, fn)
@@ -824,7 +826,7 @@ def test_few_rows_k_shared_over_workgroups(ctx, orc, fn, M, K, N, bits):
 
 
 def test_few_rows_call_in_a_graph_after_reserving_workspace(orc):
-    """A call with 32 rows keeps fp32 partial tiles in the context's workspace.  On a fresh context the workspace
+    """A matmul call with 32 rows keeps fp32 partial tiles in the context's workspace.  On a fresh context the workspace
     cannot grow while a capture is open: the call is refused with an error, not mangled; after
     aq_reserve_workspace_bytes the same call is captured and every replay equals the eager result."""
     import aq_mi355
@@ -839,14 +841,14 @@ def test_few_rows_call_in_a_graph_after_reserving_workspace(orc):
         dx, dy = fresh.to_device(x), fresh.alloc(M * N * 4)
         fresh.capture_begin()
         with pytest.raises(aq_mi355.AqError):
-            fresh.qmv(dx, dw.w, dw.s, dw.b, dy, M, K, N, 64, 4, aq_mi355.AQ_OUT_F32)
+            fresh.qmm(dx, dw.w, dw.s, dw.b, dy, M, K, N, 64, 4, aq_mi355.AQ_OUT_F32)
         try:
             fresh.graph_destroy(fresh.capture_end())
         except aq_mi355.AqError:
             pass
         fresh.reserve_workspace_bytes(64 << 20)
         fresh.capture_begin()
-        fresh.qmv(dx, dw.w, dw.s, dw.b, dy, M, K, N, 64, 4, aq_mi355.AQ_OUT_F32)
+        fresh.qmm(dx, dw.w, dw.s, dw.b, dy, M, K, N, 64, 4, aq_mi355.AQ_OUT_F32)
         graph = fresh.capture_end()
         first = None
         for i in range(3):
@@ -859,7 +861,7 @@ def test_few_rows_call_in_a_graph_after_reserving_workspace(orc):
                 first = got
             assert np.array_equal(got.view(np.uint32), first.view(np.uint32)), i
         fresh.graph_destroy(graph)
-        fresh.qmv(dx, dw.w, dw.s, dw.b, dy, M, K, N, 64, 4, aq_mi355.AQ_OUT_F32)
+        fresh.qmm(dx, dw.w, dw.s, dw.b, dy, M, K, N, 64, 4, aq_mi355.AQ_OUT_F32)
         fresh.sync()
         assert np.array_equal(dy.download(np.float32, M * N).view(np.uint32), first.view(np.uint32))
         dw.free()
