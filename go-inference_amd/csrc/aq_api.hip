@@ -138,7 +138,7 @@ int pick_qmv_variant(const aq_ctx* ctx, int bits, int m, bool gather, int N, int
 // variants, then the block-MFMA variants, then the streaming dot2 variants, then the diagonal-MFMA variants.
 int qmv_total_variants() {
     return aq::qmv_variant_count() + aq::qmvx_variant_count() + aq::qmvb_variant_count() + aq::qmvs_variant_count() +
-           aq::qmvd_variant_count() + aq::qmvt_variant_count();
+           aq::qmvd_variant_count() + aq::qmvt_variant_count() + aq::qmvd8_variant_count();
 }
 const aq::QmvVariant* qmv_any_variant(int idx) {
     const int nd = aq::qmv_variant_count();
@@ -151,7 +151,9 @@ const aq::QmvVariant* qmv_any_variant(int idx) {
     if (idx < nd + nx + nb + ns) return aq::qmvs_variant(idx - nd - nx - nb);
     const int ndg = aq::qmvd_variant_count();
     if (idx < nd + nx + nb + ns + ndg) return aq::qmvd_variant(idx - nd - nx - nb - ns);
-    return aq::qmvt_variant(idx - nd - nx - nb - ns - ndg);
+    const int nt = aq::qmvt_variant_count();
+    if (idx < nd + nx + nb + ns + ndg + nt) return aq::qmvt_variant(idx - nd - nx - nb - ns - ndg);
+    return aq::qmvd8_variant(idx - nd - nx - nb - ns - ndg - nt);
 }
 
 constexpr size_t kMaxLds = 160 * 1024;
@@ -180,6 +182,16 @@ int launch_qmv_rows(aq_ctx* ctx, aq::QmvArgs a, int group_size, int bits, bool g
     int forced = ctx->forced[0];
     const int nbk = aq::qmvb_variant_count();
     const int nst = aq::qmvs_variant_count();
+    if (forced >= nd + nx + nbk + nst + aq::qmvd_variant_count() + aq::qmvt_variant_count()) {
+        // 8-bit MFMA family, forced
+        const int ei = forced - nd - nx - nbk - nst - aq::qmvd_variant_count() - aq::qmvt_variant_count();
+        if (gather || !aq::qmvd8_fits(a, bits, group_size, ei))
+            return fail(AQ_ERR_ARG, "aq_qmv: forced variant %d does not fit bits=%d gather=%d rows=%d K=%d N=%d", forced,
+                        bits, (int)gather, M, a.K, a.N);
+        ctx->last_variant[0] = aq::qmvd8_variant(ei)->name;
+        AQ_HIP(aq::qmvd8_launch(ei, a, ctx->stream), "hipLaunchKernel");
+        return AQ_OK;
+    }
     if (forced >= nd + nx + nbk + nst + aq::qmvd_variant_count()) {
         // token-tile MFMA family, forced: the whole call in one launch
         const int ti = forced - nd - nx - nbk - nst - aq::qmvd_variant_count();
@@ -206,6 +218,16 @@ int launch_qmv_rows(aq_ctx* ctx, aq::QmvArgs a, int group_size, int bits, bool g
         if (di >= 0 && aq::qmvd_fits(a, bits, group_size, true, di)) {
             ctx->last_variant[0] = aq::qmvd_variant(di)->name;
             AQ_HIP(aq::qmvd_launch(di, a, ctx->stream), "hipLaunchKernel");
+            return AQ_OK;
+        }
+    }
+    if (forced < 0 && !gather && bits == 8 && group_size == 64 && M > 4) {
+        // 8-bit group-64 codes, 5..16 rows: the 8-bit MFMA kernels (up to 4 rows the block-MFMA kernels below measure
+        // the same or faster: 14.3 / 15.3 us against 14.1 / 17.0 us for 1 / 4 rows at 4096 x 14336)
+        const int ei = aq::qmvd8_pick(M, a.K, a.N);
+        if (ei >= 0 && aq::qmvd8_fits(a, bits, group_size, ei)) {
+            ctx->last_variant[0] = aq::qmvd8_variant(ei)->name;
+            AQ_HIP(aq::qmvd8_launch(ei, a, ctx->stream), "hipLaunchKernel");
             return AQ_OK;
         }
     }
@@ -573,6 +595,11 @@ int aq_qmv(aq_ctx* ctx, const void* x, const void* packed, const void* scales, c
         // (up to 8 rows of 4-bit codes at a K of 2..4 steps of 1024: the diagonal-MFMA kernels, one launch)
         const int di = aq::qmvd_pick(M, K, N);
         if (di >= 0 && aq::qmvd_fits(a, bits, group_size, false, di)) return launch_qmv_rows(ctx, a, group_size, bits, false);
+        // 8-bit group-64 codes up to 16 rows: one launch of the 8-bit MFMA kernels
+        if (bits == 8 && group_size == 64) {
+            const int ei = aq::qmvd8_pick(M, K, N);
+            if (ei >= 0 && aq::qmvd8_fits(a, bits, group_size, ei)) return launch_qmv_rows(ctx, a, group_size, bits, false);
+        }
         // 9..32 rows of 4-bit group-64 codes: the token-tile MFMA kernels, one launch, no workspace
         if (M > 8 && M <= 32) {
             const int ti = aq::qmvt_pick(M, K, N, ctx->cu_count);

@@ -490,7 +490,14 @@ int qmm_dispatch(hipStream_t stream, Workspace* ws, int cu_count, int forced, co
         // scale * (code - 8) as fp16 (half the vector instructions per MFMA, no fp32 work on the accumulators;
         // measured 10 % faster at 2048 x 14336)
         if (bits == 4 && (int64_t)((M + 255) / 256) * ((N + 127) / 128) >= 2 * (cu_count > 0 ? cu_count : 256)) {
-            const int half = find_qmmt_named("qmmh_b4_mb4_nb2_wm2_wn2_s2c");
+            int half = find_qmmt_named("qmmh_b4_mb4_nb2_wm2_wn2_s2c");
+            // at least one 256 x 256 tile per CU: eight wavefronts on a tile that feeds twice the MFMAs per byte of x
+            // copied into LDS, three stages (the copies of x were at two thirds of what a CU takes in; measured
+            // 0.305 -> 0.277 ms at 2048 x 14336 x 4096)
+            if ((int64_t)((M + 255) / 256) * ((N + 255) / 256) >= (cu_count > 0 ? cu_count : 256)) {
+                const int wide = find_qmmt_named("qmmh_b4_mb4_nb2_wm2_wn4");
+                if (wide >= 0) half = wide;
+            }
             if (half >= 0) tile_idx = half;
         }
     }

@@ -722,6 +722,10 @@ static const QmmHalfEntry kQmmHalfTable[] = {
     AQ_QMMH_S(4, 2, 2, 2, 2, 2, false, true, "_s2c"),
     AQ_QMMH(2, 2, 2, 2, 3, 2, false, ""),            // 128 x 128 with 64 x 64 wavefront tiles
     AQ_QMMH(2, 2, 2, 2, 3, 2, true, "_p"),           // ... with the hand-pipelined loop
+    AQ_QMMH_S(4, 2, 2, 4, 2, 2, false, true, "_s2c"),  // 256 x 256, eight wavefronts: an A tile feeds twice the MFMAs
+    AQ_QMMH(4, 2, 2, 4, 2, 2, false, "_s2"),
+    AQ_QMMH(4, 2, 2, 4, 3, 2, false, ""),              // ... three stages (120 KiB)
+    AQ_QMMH_S(4, 2, 1, 8, 2, 2, false, true, "_s2c"),  // 128 x 512, eight wavefronts
 };
 
 int qmmh_variant_count() { return (int)(sizeof(kQmmHalfTable) / sizeof(kQmmHalfTable[0])); }

@@ -143,6 +143,8 @@ def _parse_variant(name):
         return "diag", parts["b"], parts["m"], parts["g"]
     if name.startswith("qmvt_"):
         return "tok", parts["b"], parts["m"], 0
+    if name.startswith("qmvd8_"):
+        return "d8", parts["b"], parts["m"], 0
     return "dot2", parts["b"], parts["m"], parts["g"]
 
 
@@ -161,7 +163,7 @@ def test_qmv_every_variant(ctx, orc):
     try:
         for idx, name in enumerate(names):
             fam, bits, m, gather = _parse_variant(name)
-            if gather or fam in ("blk", "stream", "diag", "tok"):
+            if gather or fam in ("blk", "stream", "diag", "tok", "d8"):
                 continue  # covered by test_gather_every_variant / test_qmvb_every_variant / test_qmvs_every_variant / test_qmvd_every_variant
             say("variant", idx, name)
             if bits not in data:
@@ -204,7 +206,7 @@ def test_gather_every_variant(ctx, orc):
     try:
         for idx, name in enumerate(names):
             fam, bits, m, gather = _parse_variant(name)
-            if not gather or fam in ("blk", "stream", "diag", "tok"):
+            if not gather or fam in ("blk", "stream", "diag", "tok", "d8"):
                 continue
             say("gather variant", idx, name)
             fx = F.gather_fixture(out_dim, in_dim, 64, bits, E, expert_rows, True, routes)
