@@ -50,16 +50,23 @@ def pmc_summary(root):
         print("%-90s %-12s n=%-4d mean=%.6g" % (k[:90], c, len(v), sum(v) / len(v)))
 
 
-def traffic_from_profiles(name="qmv_dominant_traffic.md"):
-    """Bytes per launch of a kernel as recorded in profiles/ (from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
-    passes, scaled by the kernels of known traffic in the same passes)."""
+def traffic_from_profiles(name, kernel):
+    """(bytes per launch, note) of a kernel as recorded in profiles/ (from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
+    passes, scaled by the kernels of known traffic in the same passes).  The record names the kernel variant it was
+    taken on; when that is not the variant that ran here the figure is withheld, with the reason."""
     import re
     path = os.path.join(ROOT, "profiles", name)
     try:
-        m = re.search(r"traffic_bytes_per_launch:\s*([0-9]+)", open(path).read())
-        return int(m.group(1)) if m else None
+        text = open(path).read()
     except OSError:
-        return None
+        return None, "profiles/%s is missing" % name
+    m = re.search(r"traffic_bytes_per_launch:\s*([0-9]+)", text)
+    k = re.search(r"traffic_kernel:\s*(\S+)", text)
+    if not m or not k:
+        return None, "profiles/%s holds no traffic_bytes_per_launch / traffic_kernel record" % name
+    if k.group(1) != kernel:
+        return None, "profiles/%s was taken on %s, this run used %s" % (name, k.group(1), kernel)
+    return int(m.group(1)), "rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE on %s (profiles/%s)" % (kernel, name)
 
 
 def run_probe(which, variant=None):
@@ -90,6 +97,35 @@ def run_probe(which, variant=None):
         for i in range(200 * ncopy):  # long enough for the clocks to settle: the first few hundred launches run slower
             ww, ss, bb = pool[i % ncopy]
             ctx.qmv(x, ww, ss, bb, y, 1, K, N, GROUP, BITS)
+    elif which in ("rows16", "rows32"):
+        # cfg 2: 16 / 32 rows of x against the same tensor
+        M = int(which[4:])
+        x = ctx.to_device(F.synthetic_x(M, K, seed=F.BASE_SEED + 1100 + M))
+        y = ctx.alloc(M * N * 2)
+        for i in range(60 * ncopy):
+            ww, ss, bb = pool[i % ncopy]
+            ctx.qmv(x, ww, ss, bb, y, M, K, N, GROUP, BITS)
+    elif which == "read_floor":
+        for i in range(200 * ncopy):
+            ww, ss, bb = pool[i % ncopy]
+            ctx.probe_read(ww, ss, bb, K, N, 0)
+    elif which == "gather":
+        # cfg 4: the fused gate|up gather and the down gather, 128 experts, 8 tokens x top-8
+        E, TOK, TOPK, DM, DFF = 128, 8, 8, 2816, 1408
+        routes = TOK * TOPK
+        rng = np.random.Generator(np.random.PCG64(F.BASE_SEED + 77))
+        rhs = np.concatenate([rng.permutation(E)[:TOPK] for _ in range(TOK)]).astype(np.int32)
+        gu = tuple(ctx.to_device(t) for t in F.synthetic_affine(E * 2 * DFF, DM, BITS, GROUP, seed=F.BASE_SEED + 40))
+        dd = tuple(ctx.to_device(t) for t in F.synthetic_affine(E * DM, DFF, BITS, GROUP, seed=F.BASE_SEED + 41))
+        xt = ctx.to_device(F.synthetic_x(TOK, DM, seed=F.BASE_SEED + 1200))
+        d_rhs = ctx.to_device(rhs)
+        d_tok = ctx.to_device(np.repeat(np.arange(TOK, dtype=np.int32), TOPK))
+        d_route = ctx.to_device(np.arange(routes, dtype=np.int32))
+        yh, yd = ctx.alloc(routes * DFF * 2), ctx.alloc(routes * DM * 2)
+        for i in range(300):
+            ctx.gather_qmv_gate_up(xt, gu[0], gu[1], gu[2], d_tok, d_rhs, yh, routes, TOK, DM, DFF, E, 2 * DFF, 0, DFF, GROUP,
+                                   BITS, aq_mi355.AQ_ACT_GELU_TANH)
+            ctx.gather_qmv(yh, dd[0], dd[1], dd[2], d_route, d_rhs, yd, routes, routes, DFF, DM, E, DM, 0, GROUP, BITS)
     else:
         M = 2048
         x = ctx.to_device(F.synthetic_x(M, K, seed=F.BASE_SEED + 1003))
@@ -103,7 +139,7 @@ def run_probe(which, variant=None):
     ctx.sync()
     print(json.dumps({"probe": which, "fill_zero_bytes_written": 256 << 20,
                       "dequant_bytes_read": w.nbytes + s.nbytes + b.nbytes, "dequant_bytes_written": N * K * 4,
-                      "kernel": ctx.last_variant(0 if which == "dominant" else 1)}))
+                      "kernel": ctx.last_variant(1 if which == "qmm" else 0)}))
     ctx.close()
 
 
@@ -118,7 +154,7 @@ def main():
                          "does not survive stream capture; its per-dispatch durations are what such a run is for)")
     ap.add_argument("--no-qmm", action="store_true", help="skip the prefill qmm extra")
     ap.add_argument("--no-extras", action="store_true", help="skip the small-M and MoE gather extras")
-    ap.add_argument("--probe", choices=["dominant", "qmm"], help="run only the named kernel a few times, preceded by two "
+    ap.add_argument("--probe", choices=["dominant", "qmm", "rows16", "rows32", "read_floor", "gather"], help="run only the named kernel a few times, preceded by two "
                     "kernels of known traffic (a 256 MiB zero fill, a dequantisation of the gate tensor): the workload "
                     "of the rocprofv3 --pmc passes behind roofline.traffic")
     ap.add_argument("--variant", help="with --probe qmm: force this kernel variant (a name aq_variant_name lists)")
@@ -143,6 +179,8 @@ def main():
 
     ctx = aq_mi355.Context(0)
     dev_name = ctx.device_name()
+    if dev_name.startswith(" ("):  # the driver reports no marketing name on some boxes
+        dev_name = "AMD Instinct MI355X" + dev_name
 
     # ---- synthetic layer, resident in HBM; copies made device-to-device -------------------------
     layer_bytes = sum(qmv_bytes(K, N) for _, K, N in LAYER)
@@ -279,6 +317,17 @@ def main():
     dom_gbps = dom_bytes / (dom_us * 1e-6) / 1e9
     # cached (same tensor every launch), reported separately
     dom_cached_us = replay_ms(lambda i: dom_launch(0), reps) * 1e3
+    # read floor: the same tensors, rotation and load instructions with the arithmetic, the activations and the store
+    # removed (mode 0: the matvec's own access shape; mode 1: contiguous 1 KiB per instruction)
+    floor_us = {}
+    for mode in (0, 1):
+        def floor_launch(i, mode=mode):
+            w, s, b = dom[i % len(dom)]
+            ctx.probe_read(w, s, b, 4096, 14336, mode)
+        for i in range(24):
+            floor_launch(i)
+        ctx.sync()
+        floor_us[mode] = replay_ms(floor_launch, reps) * 1e3
 
     per_shape = {}
     for name, K, N in LAYER:
@@ -324,10 +373,10 @@ def main():
         q_ms = ctx.timer_stop() / n
         flops = 2.0 * M * N * K
         tf = flops / (q_ms * 1e-3) / 1e12
+        q_traffic, q_note = traffic_from_profiles("qmm_cfg3_traffic.md", ctx.last_variant(1))
         qmm = {"M": M, "K": K, "N": N, "ms": round(q_ms, 4), "TFLOPs": round(tf, 1), "kernel": ctx.last_variant(1),
                "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                            "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
-                            "traffic": traffic_from_profiles("qmm_cfg3_traffic.md")}}
+                            "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": q_traffic, "traffic_note": q_note}}
         # the same call on the other kernel family: bare codes as bf16 operands and one fp32 FMA per output element
         # and 64-code block (the default is the family whose MFMA operand carries scale * (code - 8) as fp16)
         other = "qmmt_b4_mb2_nb2_wm2_wn2"
@@ -346,6 +395,30 @@ def main():
             ctx.force_variant(1, -1)
             qmm["bf16_code_variant"] = {"kernel": other, "ms": round(o_ms, 4),
                                            "TFLOPs": round(flops / (o_ms * 1e-3) / 1e12, 1)}
+        # the 8-bit variant of the same call (codes 0..255, bias = -128 * scale): the bf16-code tile kernels
+        w8q = F.synthetic_affine(N, K, 8, GROUP, seed=F.BASE_SEED + 31)
+        pool8 = [tuple(ctx.to_device(t) for t in w8q)]
+        for c in range(1, 6):
+            dst = tuple(ctx.alloc(t.nbytes) for t in pool8[0])
+            for d, t in zip(dst, pool8[0]):
+                ctx._check(ctx.lib.aq_d2d(ctx.handle, d.ptr, t.ptr, t.nbytes))
+            pool8.append(dst)
+        for i in range(24):
+            w, s, b = pool8[i % len(pool8)]
+            ctx.qmm(xm, w, s, b, ym, M, K, N, GROUP, 8)
+        ctx.sync()
+        ctx.timer_start()
+        for i in range(n):
+            w, s, b = pool8[i % len(pool8)]
+            ctx.qmm(xm, w, s, b, ym, M, K, N, GROUP, 8)
+        q8_ms = ctx.timer_stop() / n
+        tf8 = flops / (q8_ms * 1e-3) / 1e12
+        qmm["b8"] = {"ms": round(q8_ms, 4), "TFLOPs": round(tf8, 1), "kernel": ctx.last_variant(1),
+                     "roofline": {"bound": "mfma", "achieved": round(tf8, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                  "frac": round(tf8 / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None}}
+        for t in pool8:
+            for d in t:
+                d.free()
         xm.free()
         ym.free()
 
@@ -540,12 +613,14 @@ def main():
             ctx.packed_topk_sample(h_top, 40, 0.8, 0.95, 30.0, 0.37, h_best)
 
         us_sample = head_time(sample40)
+        # the sampler kernel on its own list of 40 (the list the last call left)
+        us_sampler = head_time(lambda t: ctx.packed_topk_sample(h_top, 40, 0.8, 0.95, 30.0, 0.37, h_best), n=200)
         head = {"N": HN, "K": HK, "group": HG, "bits": BITS, "weight_bytes": head_bytes,
                 "logits": {"us": round(us_logits, 2), "GBps": round((head_bytes + HN * 2) / us_logits / 1e3, 1), "kernel": k_logits},
                 "greedy_fused": {"us": round(us_greedy, 2), "GBps": round(head_bytes / us_greedy / 1e3, 1),
                                  "pct_of_hbm_peak": round(head_bytes / us_greedy / 1e3 / HBM_PEAK_GBPS * 100, 2)},
                 "scores_then_top40": {"us": round(us_topk, 2), "GBps": round((head_bytes + HN * 8) / us_topk / 1e3, 1)},
-                "scores_top40_sample": {"us": round(us_sample, 2), "sampler_us": round(us_sample - us_topk, 2)},
+                "scores_top40_sample": {"us": round(us_sample, 2), "sampler_alone_us": round(us_sampler, 2)},
                 "note": "lm_head 262144 x 1536, 4-bit group 32 (251 MB), two copies alternated; greedy_fused = aq_qmv_greedy "
                         "(8 bytes out); scores_then_top40 = aq_qmv_scores + aq_packed_topk"}
         for t in pool[0] + pool[1] + (hx, h_logits, h_best, h_scores, h_top):
@@ -626,7 +701,10 @@ def main():
         name, K, N = LAYER[4]
         w, s, b = host[name]
         xf = F.bf16_bits_to_f32(F.synthetic_x(1, K, seed=F.BASE_SEED + 1000)).reshape(1, K)
-        threads = max(1, min(16, orc.max_threads(), os.cpu_count() or 1))
+        # every core this job may use: the box hands a one-GPU job 16 and says so through OMP_NUM_THREADS, whatever the
+        # host's core count; without that variable, all cores
+        share = int(os.environ.get("OMP_NUM_THREADS", "0") or 0)
+        threads = max(1, min(orc.max_threads(), share if share > 0 else (os.cpu_count() or 1)))
         rows1 = 1024
         t0 = time.perf_counter()
         orc.matnt_quant_host(xf, w[:rows1], s[:rows1], b[:rows1], 1, K, rows1, GROUP, BITS, threads=1)
@@ -639,9 +717,12 @@ def main():
         tn = (time.perf_counter() - t0) / reps_cpu
         cpu = {"value": round(qmv_bytes(K, N) / tn / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
                "sample": "oracle port of attn.matNTQuantHost (fp32 row dequant + f64 dot), gate projection K=4096 N=14336 M=1, "
-                         "%d full passes on %d OpenMP threads (%.2f ms/pass); single thread on %d rows: %.3f GB/s"
-                         % (reps_cpu, threads, tn * 1e3, rows1, qmv_bytes(K, rows1) / t1 / 1e9)}
+                         "%d full passes on %d OpenMP threads (%.2f ms/pass; the host shows %d cores, OMP_NUM_THREADS=%s); "
+                         "single thread on %d rows: %.3f GB/s"
+                         % (reps_cpu, threads, tn * 1e3, os.cpu_count() or 0, os.environ.get("OMP_NUM_THREADS", "unset"), rows1,
+                            qmv_bytes(K, rows1) / t1 / 1e9)}
 
+    dom_traffic, dom_traffic_note = traffic_from_profiles("qmv_dominant_traffic.md", variants["gate"])
     out = {
         "metric": "4-bit affine qmv HBM GB/s at M=1 (one decoder layer's quantized GEMVs)",
         "value": round(value, 1),
@@ -670,9 +751,14 @@ def main():
         "host_wall_ms_per_step": round(t_host * 1e3 / args.steps, 5),
         "roofline": {"bound": "hbm", "kernel": variants["gate"], "shape": "qmv M=1 K=4096 N=14336 4-bit g64",
                      "achieved": round(dom_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(dom_gbps / HBM_PEAK_GBPS, 4), "traffic": traffic_from_profiles(),
+                     "frac": round(dom_gbps / HBM_PEAK_GBPS, 4), "traffic": dom_traffic, "traffic_note": dom_traffic_note,
                      "bytes_per_launch": dom_bytes, "us_per_launch": round(dom_us, 3),
-                     "us_per_launch_cached": round(dom_cached_us, 3)},
+                     "us_per_launch_cached": round(dom_cached_us, 3),
+                     "read_floor": {"us_same_access_shape": round(floor_us[0], 3), "us_contiguous": round(floor_us[1], 3),
+                                    "frac_of_read_floor": round(floor_us[0] / dom_us, 4),
+                                    "note": "aq_probe_read over the same tensors in the same rotation and graph: the "
+                                            "matvec's load instructions (codes, scales, biases) with no activations, "
+                                            "arithmetic or store; frac_of_read_floor = that time / the matvec's"}},
         "cpu_baseline": cpu,
         "per_shape": per_shape,
         "qmm": qmm,

@@ -567,6 +567,18 @@ void aq_graph_destroy(aq_graph* graph) {
     delete graph;
 }
 
+int aq_probe_read(aq_ctx* ctx, const void* packed, const void* scales, const void* biases, int K, int N, int mode) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_probe_read: ctx is null");
+    if (K <= 0 || N <= 0 || K % 1024 != 0) return fail(AQ_ERR_SHAPE, "aq_probe_read: K must be a positive multiple of 1024, N positive");
+    if (mode != 0 && mode != 1) return fail(AQ_ERR_ARG, "aq_probe_read: mode is 0 or 1");
+    if (!packed || !scales || !biases) return fail(AQ_ERR_ARG, "aq_probe_read: null operand");
+    if (!aligned(packed, 16) || !aligned(scales, 8) || !aligned(biases, 8))
+        return fail(AQ_ERR_ARG, "aq_probe_read: packed must be 16-byte, scales and biases 8-byte aligned");
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    AQ_HIP(aq::read_probe_launch(packed, scales, biases, N, K / 2, K / 32, mode, nullptr, ctx->stream), "hipLaunchKernel");
+    return AQ_OK;
+}
+
 int aq_qmv(aq_ctx* ctx, const void* x, const void* packed, const void* scales, const void* biases, void* y, int M,
            int K, int N, int group_size, int bits, unsigned flags) {
     if (!ctx) return fail(AQ_ERR_ARG, "aq_qmv: ctx is null");

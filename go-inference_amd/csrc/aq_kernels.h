@@ -238,6 +238,11 @@ hipError_t qmv_generic_launch(const QmvArgs& a, int bits, int group_size, bool g
 // Six-bit codes in groups of 16 or 32 with K a multiple of 16 take a kernel of their own inside that launch.
 bool qmv_six_eligible(const QmvArgs& a, int bits, int group_size);
 
+// Measurement aid (aq_misc.hip): reads the codes, scales and biases of a 4-bit group-64 tensor once with no arithmetic,
+// in the access shape of the diagonal-MFMA matvec (mode 0) or as contiguous 1 KiB pieces (mode 1).
+hipError_t read_probe_launch(const void* w, const void* s, const void* b, int64_t rows, int row_bytes, int sb_bytes, int mode,
+                             uint32_t* out, hipStream_t stream);
+
 // fp32 dequantisation of a whole tensor, bits in {1,2,4,8} (word-clean widths)
 // or {3,5,6} through the straddling path.
 hipError_t dequant_launch(const uint32_t* w, const uint16_t* s, const uint16_t* b, float* out, int64_t N, int K,

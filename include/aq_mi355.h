@@ -100,6 +100,13 @@ int aq_capture_end(aq_ctx *ctx, aq_graph **out);
 int aq_graph_launch(aq_ctx *ctx, aq_graph *graph);
 void aq_graph_destroy(aq_graph *graph);
 
+/* Measurement aid with no counterpart in the reference: streams the packed codes, scales and biases of a 4-bit
+ * group-64 tensor [N, K] through the same load instructions the single-row matvec issues (mode 0: 64 contiguous
+ * bytes of each of 16 rows per instruction; mode 1: contiguous 1 KiB pieces) and does nothing with them.  Its time
+ * is the floor any matvec over that tensor can reach on this device: the benchmark reports the matvec beside it.
+ * K a multiple of 1024.  Stream-ordered; writes nothing. */
+int aq_probe_read(aq_ctx *ctx, const void *packed, const void *scales, const void *biases, int K, int N, int mode);
+
 /* affine_qmv: y[M,N] = x[M,K] . dequant(w[N,K])^T, all operands device-resident.
  * Stands in for rocm_mlx_q4_projection / _batch launches
  * (go/engine/hip/hip_projection_launch.go:1306-1406, 2671-2720, 4907-5287) with the bf16
