@@ -134,198 +134,95 @@ int pick_qmv_variant(const aq_ctx* ctx, int bits, int m, bool gather, int N, int
     return best;
 }
 
-// One index space over the matvec kernel families: dot2 variants first, then the 32x32 MFMA
-// variants, then the block-MFMA variants, then the streaming dot2 variants, then the diagonal-MFMA variants.
+// ---- the matvec kernel families and the one table that chooses among them ---------------------------------------
+
+// Families with variants of their own.  aq_variant_name(0, i) and aq_force_variant(ctx, 0, i) index the
+// concatenation of their tables, in this order.
+enum { kFamDot2, kFamBlk, kFamDiag, kFamTok, kFamD8, kFamCount };
+// Two more take part in the selection: the tile kernels of the matmul path (their variants are those of op 1)
+// and the kernel that takes any geometry.
+enum { kFamTiles = kFamCount, kFamTilesLarge, kFamGeneric };
+
+struct QmvFamily {
+    int (*count)();
+    const aq::QmvVariant* (*variant)(int);
+};
+const QmvFamily kQmvFamilies[kFamCount] = {
+    {aq::qmv_variant_count, aq::qmv_variant},      // VALU dot2 kernels (aq_qmv.hip)
+    {aq::qmvb_variant_count, aq::qmvb_variant},    // block-MFMA kernels (aq_qmv_blk.hip)
+    {aq::qmvd_variant_count, aq::qmvd_variant},    // diagonal-MFMA kernels (aq_qmv_diag.hip)
+    {aq::qmvt_variant_count, aq::qmvt_variant},    // token-tile MFMA kernels (aq_qmv_tok.hip)
+    {aq::qmvd8_variant_count, aq::qmvd8_variant},  // 8-bit MFMA kernels (aq_qmv_d8.hip)
+};
+
 int qmv_total_variants() {
-    return aq::qmv_variant_count() + aq::qmvx_variant_count() + aq::qmvb_variant_count() + aq::qmvs_variant_count() +
-           aq::qmvd_variant_count() + aq::qmvt_variant_count() + aq::qmvd8_variant_count();
+    int n = 0;
+    for (const QmvFamily& f : kQmvFamilies) n += f.count();
+    return n;
+}
+// Family and index inside it of entry idx of the concatenated table.
+bool qmv_locate(int idx, int* family, int* local) {
+    if (idx < 0) return false;
+    for (int f = 0; f < kFamCount; f++) {
+        const int n = kQmvFamilies[f].count();
+        if (idx < n) {
+            *family = f;
+            *local = idx;
+            return true;
+        }
+        idx -= n;
+    }
+    return false;
 }
 const aq::QmvVariant* qmv_any_variant(int idx) {
-    const int nd = aq::qmv_variant_count();
-    const int nx = aq::qmvx_variant_count();
-    if (idx < nd) return aq::qmv_variant(idx);
-    if (idx < nd + nx) return aq::qmvx_variant(idx - nd);
-    const int nb = aq::qmvb_variant_count();
-    if (idx < nd + nx + nb) return aq::qmvb_variant(idx - nd - nx);
-    const int ns = aq::qmvs_variant_count();
-    if (idx < nd + nx + nb + ns) return aq::qmvs_variant(idx - nd - nx - nb);
-    const int ndg = aq::qmvd_variant_count();
-    if (idx < nd + nx + nb + ns + ndg) return aq::qmvd_variant(idx - nd - nx - nb - ns);
-    const int nt = aq::qmvt_variant_count();
-    if (idx < nd + nx + nb + ns + ndg + nt) return aq::qmvt_variant(idx - nd - nx - nb - ns - ndg);
-    return aq::qmvd8_variant(idx - nd - nx - nb - ns - ndg - nt);
+    int f, i;
+    return qmv_locate(idx, &f, &i) ? kQmvFamilies[f].variant(i) : nullptr;
 }
 
-constexpr size_t kMaxLds = 160 * 1024;
-constexpr bool kStreamDefault = false;
+// Which family runs an unforced call.  The first rule whose key matches the call and whose family accepts the shape
+// runs it; the key holds what the families differ in at first sight (code width, group size, rows of x, dense or
+// gathered), and each family's own pick / fits / plan function narrows K, N and operand alignment and passes the call
+// on when the shape is not its to run.  The last rule of each kind accepts everything.
+struct QmvRule {
+    int bits;        // 0: any
+    int group_size;  // 0: any
+    int gather;      // 1: gathered calls (one row of x per route), 0: dense calls
+    int m_lo, m_hi;  // rows of x in the call
+    int family;
+};
+const QmvRule kQmvRules[] = {
+    // bits group gather rows         family
+    {4, 64, 1, 1, 1, kFamDiag},             // K a multiple of 128 in 2..8 steps of 1024 codes
+    {0, 0, 1, 1, 1, kFamDot2},              // 4 / 8 bit, groups of 32 / 64 / 128, 16-byte chunks inside one group
+    {0, 0, 1, 1, 1, kFamGeneric},
+    {4, 64, 0, 1, 8, kFamDiag},             // one row up to 16 steps of 1024 codes, up to 8 rows at 2..4 steps
+    {4, 32, 0, 1, 2, kFamDiag},             // groups of 32: two tokens x eight groups as MFMA rows
+    {8, 64, 0, 5, 16, kFamD8},              // (up to 4 rows the block-MFMA kernels measure the same or faster)
+    {4, 64, 0, 9, 32, kFamTok},             // K a multiple of 256: one launch, weights streamed once, no scratch
+    {0, 0, 0, 9, 64, kFamTilesLarge},       // 16 Mi codes and more: the 16-row block-MFMA kernel is bound by its 4x4x4 MFMAs
+    {0, 0, 0, 2, 16, kFamBlk},              // the whole call in one launch of up to 16 rows (4 where K is long)
+    {8, 0, 0, 1, 1, kFamBlk},               // (a single row of 4-bit codes is faster on the dot2 kernels)
+    {0, 0, 0, 5, INT32_MAX, kFamTiles},     // K shared out over workgroups for few rows; any geometry
+    {0, 0, 0, 1, 4, kFamDot2},
+    {0, 0, 0, 1, 4, kFamGeneric},
+};
 
-bool mfma_eligible(const aq::QmvArgs& a, int group_size, int bits) {
-    if (bits != 4 && bits != 8) return false;
-    // scales are staged as pairs of consecutive groups: group size 64 and an even group count
-    if (group_size != 64 || a.K % 128 != 0 || a.M > 32) return false;
-    return aligned(a.x, 16) && aligned(a.w, 16) && aligned(a.s, 4) && aligned(a.b, 4);
-}
+constexpr int kPass = INT32_MIN;  // a family's answer when the shape is not its to run
 
-int find_qmvx(int bits, int mr_max_m, int ks, bool gather) {
-    for (int i = 0; i < aq::qmvx_variant_count(); i++) {
-        const aq::QmvVariant* v = aq::qmvx_variant(i);
-        if (v->bits == bits && v->m == mr_max_m && v->waves == ks && (v->gather != 0) == gather) return i;
-    }
-    return -1;
-}
-
-int launch_qmv_rows(aq_ctx* ctx, aq::QmvArgs a, int group_size, int bits, bool gather) {
+int run_dot2(aq_ctx* ctx, const aq::QmvArgs& a, int group_size, int bits, bool gather, int forced) {
     const int M = a.M;
-    a.gs_shift = is_pow2(group_size) ? ilog2(group_size) : 0;
-    const int nd = aq::qmv_variant_count();
-    const int nx = aq::qmvx_variant_count();
-    int forced = ctx->forced[0];
-    const int nbk = aq::qmvb_variant_count();
-    const int nst = aq::qmvs_variant_count();
-    if (forced >= nd + nx + nbk + nst + aq::qmvd_variant_count() + aq::qmvt_variant_count()) {
-        // 8-bit MFMA family, forced
-        const int ei = forced - nd - nx - nbk - nst - aq::qmvd_variant_count() - aq::qmvt_variant_count();
-        if (gather || !aq::qmvd8_fits(a, bits, group_size, ei))
-            return fail(AQ_ERR_ARG, "aq_qmv: forced variant %d does not fit bits=%d gather=%d rows=%d K=%d N=%d", forced,
-                        bits, (int)gather, M, a.K, a.N);
-        ctx->last_variant[0] = aq::qmvd8_variant(ei)->name;
-        AQ_HIP(aq::qmvd8_launch(ei, a, ctx->stream), "hipLaunchKernel");
-        return AQ_OK;
-    }
-    if (forced >= nd + nx + nbk + nst + aq::qmvd_variant_count()) {
-        // token-tile MFMA family, forced: the whole call in one launch
-        const int ti = forced - nd - nx - nbk - nst - aq::qmvd_variant_count();
-        if (gather || !aq::qmvt_fits(a, bits, group_size, ti))
-            return fail(AQ_ERR_ARG, "aq_qmv: forced variant %d does not fit bits=%d gather=%d rows=%d K=%d N=%d", forced,
-                        bits, (int)gather, M, a.K, a.N);
-        ctx->last_variant[0] = aq::qmvt_variant(ti)->name;
-        AQ_HIP(aq::qmvt_launch(ti, a, ctx->stream), "hipLaunchKernel");
-        return AQ_OK;
-    }
-    if (forced >= nd + nx + nbk + nst) {
-        // diagonal-MFMA family, forced
-        const int di = forced - nd - nx - nbk - nst;
-        if (!aq::qmvd_fits(a, bits, group_size, gather, di))
-            return fail(AQ_ERR_ARG, "aq_qmv: forced variant %d does not fit bits=%d gather=%d rows=%d K=%d N=%d", forced,
-                        bits, (int)gather, M, a.K, a.N);
-        ctx->last_variant[0] = aq::qmvd_variant(di)->name;
-        AQ_HIP(aq::qmvd_launch(di, a, ctx->stream), "hipLaunchKernel");
-        return AQ_OK;
-    }
-    if (forced < 0 && gather) {
-        // 4-bit group-64 codes, K a multiple of 128 in 2..8 steps of 1024: the gathered diagonal-MFMA kernels
-        const int di = aq::qmvd_pick_gather(a.K);
-        if (di >= 0 && aq::qmvd_fits(a, bits, group_size, true, di)) {
-            ctx->last_variant[0] = aq::qmvd_variant(di)->name;
-            AQ_HIP(aq::qmvd_launch(di, a, ctx->stream), "hipLaunchKernel");
-            return AQ_OK;
-        }
-    }
-    if (forced < 0 && !gather && bits == 8 && group_size == 64 && M > 4) {
-        // 8-bit group-64 codes, 5..16 rows: the 8-bit MFMA kernels (up to 4 rows the block-MFMA kernels below measure
-        // the same or faster: 14.3 / 15.3 us against 14.1 / 17.0 us for 1 / 4 rows at 4096 x 14336)
-        const int ei = aq::qmvd8_pick(M, a.K, a.N);
-        if (ei >= 0 && aq::qmvd8_fits(a, bits, group_size, ei)) {
-            ctx->last_variant[0] = aq::qmvd8_variant(ei)->name;
-            AQ_HIP(aq::qmvd8_launch(ei, a, ctx->stream), "hipLaunchKernel");
-            return AQ_OK;
-        }
-    }
-    if (forced < 0 && !gather && group_size == 32) {
-        // 4-bit group-32 codes, up to 2 rows: the diagonal-MFMA kernels with two tokens x eight groups as A rows
-        const int di = aq::qmvd_pick_g32(M, a.K, a.N);
-        if (di >= 0 && aq::qmvd_fits(a, bits, group_size, false, di)) {
-            ctx->last_variant[0] = aq::qmvd_variant(di)->name;
-            AQ_HIP(aq::qmvd_launch(di, a, ctx->stream), "hipLaunchKernel");
-            return AQ_OK;
-        }
-    }
-    if (forced < 0 && !gather) {
-        // 4-bit group-64 codes: up to 8 rows at a K of 2..4 steps of 1024 codes, one row up to 16 steps: the diagonal-MFMA kernels
-        const int di = aq::qmvd_pick(M, a.K, a.N);
-        if (di >= 0 && aq::qmvd_fits(a, bits, group_size, gather, di)) {
-            ctx->last_variant[0] = aq::qmvd_variant(di)->name;
-            AQ_HIP(aq::qmvd_launch(di, a, ctx->stream), "hipLaunchKernel");
-            return AQ_OK;
-        }
-    }
-    if (forced >= nd + nx + nbk || (forced < 0 && M == 1 && kStreamDefault)) {
-        // streaming dot2 family: forced, or the default for one activation row wherever K fits it
-        aq::StreamPlan plan;
-        if (aq::qmvs_plan(a, bits, group_size, gather, ctx->cu_count, forced < 0 ? -1 : forced - nd - nx - nbk, &plan)) {
-            ctx->last_variant[0] = aq::qmvs_variant(plan.idx)->name;
-            AQ_HIP(aq::qmvs_launch(plan, a, ctx->stream), "hipLaunchKernel");
-            return AQ_OK;
-        }
-        if (forced >= 0)
-            return fail(AQ_ERR_ARG, "aq_qmv: forced variant %d does not fit bits=%d gather=%d rows=%d K=%d N=%d", forced,
-                        bits, (int)gather, M, a.K, a.N);
-    }
-    if ((forced >= nd + nx && forced < nd + nx + nbk) || (forced < 0 && (M >= 2 || (bits == 8 && !gather)))) {
-        // block-MFMA family: forced, or the default for 2 and more activation rows (and for a single row
-        // of 8-bit codes) wherever the shape fits it; a single row of 4-bit codes is faster on the dot2 kernels.  Rows beyond what one launch of the
-        // family takes for this K go in further launches.
-        const size_t esize = a.out_f32 ? 4 : 2;
-        const int blk_forced = forced < 0 ? -1 : forced - nd - nx;
-        // rows the family takes in one launch for this shape: all that are left, else 16, else 4
-        auto plan_rows = [&](aq::QmvArgs& c, int rows_left, aq::BlkPlan* plan) {
-            for (int rows : {rows_left, 16, 4}) {
-                if (rows > rows_left || (rows != rows_left && forced >= 0)) continue;  // forced: whole or not at all
-                c.M = rows;
-                if (aq::qmvb_plan(c, bits, group_size, gather, ctx->cu_count, blk_forced, plan)) return rows;
-            }
-            return 0;
-        };
-        bool ok = true;
-        for (int m0 = 0; m0 < M;) {
-            aq::QmvArgs c = a;
-            c.x = a.x + (size_t)m0 * a.K;
-            c.y = static_cast<char*>(a.y) + (size_t)m0 * a.N * esize;
-            aq::BlkPlan plan;
-            const int rows = plan_rows(c, M - m0, &plan);
-            if (rows == 0) {
-                ok = false;
-                break;
-            }
-            ctx->last_variant[0] = aq::qmvb_variant(plan.idx)->name;
-            AQ_HIP(aq::qmvb_launch(plan, c, ctx->stream), "hipLaunchKernel");
-            m0 += rows;
-        }
-        if (ok) return AQ_OK;
-        if (forced >= 0)
-            return fail(AQ_ERR_ARG, "aq_qmv: forced variant %d does not fit bits=%d gather=%d rows=%d K=%d N=%d", forced,
-                        bits, (int)gather, M, a.K, a.N);
-    }
-    if (forced >= nd) {
-        // a forced MFMA variant: the whole call in one launch
-        const aq::QmvVariant* v = aq::qmvx_variant(forced - nd);
-        if (!v || v->bits != bits || (v->gather != 0) != gather || M > v->m || !mfma_eligible(a, group_size, bits) ||
-            aq::qmvx_lds_bytes(forced - nd, a) > kMaxLds)
-            return fail(AQ_ERR_ARG, "aq_qmv: forced variant %d does not fit bits=%d gather=%d rows=%d K=%d", forced, bits,
-                        (int)gather, M, a.K);
-        ctx->last_variant[0] = v->name;
-        AQ_HIP(aq::qmvx_launch(forced - nd, a, ctx->stream), "hipLaunchKernel");
-        return AQ_OK;
-    }
-    const bool fast = dot2_eligible(a.K, group_size, bits, a.x, a.w, (size_t)(M < 4 ? M : 4) * a.K * 2);
-    if (!fast) {
-        ctx->last_variant[0] = aq::qmv_six_eligible(a, bits, group_size) ? "qmv_six" : "qmv_generic";
-        AQ_HIP(aq::qmv_generic_launch(a, bits, group_size, gather, ctx->stream), "hipLaunchKernel");
-        return AQ_OK;
-    }
+    if (!dot2_eligible(a.K, group_size, bits, a.x, a.w, (size_t)(M < 4 ? M : 4) * a.K * 2)) return kPass;
     const size_t esize = a.out_f32 ? 4 : 2;
     for (int m0 = 0; m0 < M;) {
         int m = M - m0 < 4 ? M - m0 : 4;
         int idx = forced;
         if (idx >= 0) {
             const aq::QmvVariant* v = aq::qmv_variant(idx);
-            if (!v || v->bits != bits || (v->gather != 0) != gather || v->m > M - m0)
-                return fail(AQ_ERR_ARG, "aq_qmv: forced variant %d does not fit bits=%d gather=%d rows=%d", idx, bits,
-                            (int)gather, M - m0);
+            if (!v || v->bits != bits || (v->gather != 0) != gather || v->m > M - m0) return kPass;
             m = v->m;
         } else {
             idx = pick_qmv_variant(ctx, bits, m, gather, a.N, a.K, a.routes);
-            if (idx < 0) return fail(AQ_ERR_UNSUPPORTED, "aq_qmv: no kernel variant for bits=%d m=%d", bits, m);
+            if (idx < 0) return kPass;
         }
         aq::QmvArgs c = a;
         c.M = m;
@@ -336,6 +233,90 @@ int launch_qmv_rows(aq_ctx* ctx, aq::QmvArgs a, int group_size, int bits, bool g
         m0 += m;
     }
     return AQ_OK;
+}
+
+int run_blk(aq_ctx* ctx, const aq::QmvArgs& a, int group_size, int bits, bool gather, int forced) {
+    aq::BlkPlan plan;
+    if (!aq::qmvb_plan(a, bits, group_size, gather, ctx->cu_count, forced, &plan)) return kPass;
+    ctx->last_variant[0] = aq::qmvb_variant(plan.idx)->name;
+    AQ_HIP(aq::qmvb_launch(plan, a, ctx->stream), "hipLaunchKernel");
+    return AQ_OK;
+}
+
+int run_diag(aq_ctx* ctx, const aq::QmvArgs& a, int group_size, int bits, bool gather, int forced) {
+    const int di = forced >= 0        ? forced
+                   : gather           ? aq::qmvd_pick_gather(a.K)
+                   : group_size == 32 ? aq::qmvd_pick_g32(a.M, a.K, a.N)
+                                      : aq::qmvd_pick(a.M, a.K, a.N);
+    if (di < 0 || !aq::qmvd_fits(a, bits, group_size, gather, di)) return kPass;
+    ctx->last_variant[0] = aq::qmvd_variant(di)->name;
+    AQ_HIP(aq::qmvd_launch(di, a, ctx->stream), "hipLaunchKernel");
+    return AQ_OK;
+}
+
+int run_tok(aq_ctx* ctx, const aq::QmvArgs& a, int group_size, int bits, bool gather, int forced) {
+    const int ti = forced >= 0 ? forced : aq::qmvt_pick(a.M, a.K, a.N, ctx->cu_count);
+    if (gather || ti < 0 || !aq::qmvt_fits(a, bits, group_size, ti)) return kPass;
+    ctx->last_variant[0] = aq::qmvt_variant(ti)->name;
+    AQ_HIP(aq::qmvt_launch(ti, a, ctx->stream), "hipLaunchKernel");
+    return AQ_OK;
+}
+
+int run_d8(aq_ctx* ctx, const aq::QmvArgs& a, int group_size, int bits, bool gather, int forced) {
+    const int ei = forced >= 0 ? forced : aq::qmvd8_pick(a.M, a.K, a.N);
+    if (gather || ei < 0 || !aq::qmvd8_fits(a, bits, group_size, ei)) return kPass;
+    ctx->last_variant[0] = aq::qmvd8_variant(ei)->name;
+    AQ_HIP(aq::qmvd8_launch(ei, a, ctx->stream), "hipLaunchKernel");
+    return AQ_OK;
+}
+
+int run_tiles(aq_ctx* ctx, const aq::QmvArgs& a, int group_size, int bits, bool large_only) {
+    if (large_only && ((a.K / 64) % 4 != 0 || (int64_t)a.N * a.K < (int64_t)16 << 20)) return kPass;
+    const int rc = aq::qmm_dispatch(ctx->stream, &ctx->ws, ctx->cu_count, ctx->forced[1], &ctx->last_variant[1], a.x, a.w,
+                                    a.s, a.b, a.y, a.M, a.K, a.N, group_size, bits, a.out_f32 != 0, fail);
+    if (rc == AQ_OK) ctx->last_variant[0] = ctx->last_variant[1];  // the kernel this matvec call ran
+    return rc;
+}
+
+int run_generic(aq_ctx* ctx, const aq::QmvArgs& a, int group_size, int bits, bool gather) {
+    ctx->last_variant[0] = aq::qmv_six_eligible(a, bits, group_size) ? "qmv_six" : "qmv_generic";
+    AQ_HIP(aq::qmv_generic_launch(a, bits, group_size, gather, ctx->stream), "hipLaunchKernel");
+    return AQ_OK;
+}
+
+int run_family(int family, aq_ctx* ctx, const aq::QmvArgs& a, int group_size, int bits, bool gather, int forced) {
+    switch (family) {
+        case kFamDot2: return run_dot2(ctx, a, group_size, bits, gather, forced);
+        case kFamBlk: return run_blk(ctx, a, group_size, bits, gather, forced);
+        case kFamDiag: return run_diag(ctx, a, group_size, bits, gather, forced);
+        case kFamTok: return run_tok(ctx, a, group_size, bits, gather, forced);
+        case kFamD8: return run_d8(ctx, a, group_size, bits, gather, forced);
+        case kFamTiles: return run_tiles(ctx, a, group_size, bits, false);
+        case kFamTilesLarge: return run_tiles(ctx, a, group_size, bits, true);
+        default: return run_generic(ctx, a, group_size, bits, gather);
+    }
+}
+
+// One matvec call, dense (a.M rows of x) or gathered (one row per route): the forced variant, or the rule table.
+int launch_qmv_rows(aq_ctx* ctx, aq::QmvArgs a, int group_size, int bits, bool gather) {
+    a.gs_shift = is_pow2(group_size) ? ilog2(group_size) : 0;
+    const int forced = ctx->forced[0];
+    if (forced >= 0) {
+        int family = 0, local = 0;
+        const int rc = qmv_locate(forced, &family, &local) ? run_family(family, ctx, a, group_size, bits, gather, local) : kPass;
+        if (rc == kPass)
+            return fail(AQ_ERR_ARG, "aq_qmv: forced variant %d does not fit bits=%d group=%d gather=%d rows=%d K=%d N=%d",
+                        forced, bits, group_size, (int)gather, a.M, a.K, a.N);
+        return rc;
+    }
+    for (const QmvRule& r : kQmvRules) {
+        if ((r.bits && r.bits != bits) || (r.group_size && r.group_size != group_size) || (r.gather != 0) != gather ||
+            a.M < r.m_lo || a.M > r.m_hi)
+            continue;
+        const int rc = run_family(r.family, ctx, a, group_size, bits, gather, -1);
+        if (rc != kPass) return rc;
+    }
+    return fail(AQ_ERR_UNSUPPORTED, "aq_qmv: no kernel for bits=%d group=%d rows=%d K=%d N=%d", bits, group_size, a.M, a.K, a.N);
 }
 
 }  // namespace
@@ -600,47 +581,6 @@ int aq_qmv(aq_ctx* ctx, const void* x, const void* packed, const void* scales, c
     a.M = M;
     a.out_f32 = (flags & AQ_OUT_F32) ? 1 : 0;
     a.routes = 1;
-    if (M > aq::kQmvMaxRows && ctx->forced[0] < 0) {
-        // More rows than the dot2 kernels take.  The block-MFMA family streams the weights once per launch of
-        // up to 16 rows (4 where K is long); when the call fits one such launch it is the fastest up to 8 rows.
-        // Beyond that the matmul tiles with K shared out over workgroups read the weights once for all rows.
-        // (up to 8 rows of 4-bit codes at a K of 2..4 steps of 1024: the diagonal-MFMA kernels, one launch)
-        const int di = aq::qmvd_pick(M, K, N);
-        if (di >= 0 && aq::qmvd_fits(a, bits, group_size, false, di)) return launch_qmv_rows(ctx, a, group_size, bits, false);
-        // 8-bit group-64 codes up to 16 rows: one launch of the 8-bit MFMA kernels
-        if (bits == 8 && group_size == 64) {
-            const int ei = aq::qmvd8_pick(M, K, N);
-            if (ei >= 0 && aq::qmvd8_fits(a, bits, group_size, ei)) return launch_qmv_rows(ctx, a, group_size, bits, false);
-        }
-        // 9..32 rows of 4-bit group-64 codes: the token-tile MFMA kernels, one launch, no workspace
-        if (M > 8 && M <= 32) {
-            const int ti = aq::qmvt_pick(M, K, N, ctx->cu_count);
-            if (ti >= 0 && aq::qmvt_fits(a, bits, group_size, ti)) {
-                ctx->last_variant[0] = aq::qmvt_variant(ti)->name;
-                AQ_HIP(aq::qmvt_launch(ti, a, ctx->stream), "hipLaunchKernel");
-                return AQ_OK;
-            }
-        }
-        aq::BlkPlan plan;
-        aq::QmvArgs probe = a;
-        int rows_per_launch = 0;
-        for (int rows : {16, 4}) {
-            probe.M = M < rows ? M : rows;
-            if (aq::qmvb_plan(probe, bits, group_size, false, ctx->cu_count, -1, &plan)) {
-                rows_per_launch = rows;
-                break;
-            }
-        }
-        // (9..16 rows of a large matrix: the 16-row block-MFMA kernel is bound by its 4x4x4 MFMAs, the tiles are not)
-        const bool tiles_win = M > 8 && M <= 64 && (K / 64) % 4 == 0 && (int64_t)N * K >= (int64_t)16 << 20;
-        if (rows_per_launch == 0 || M > 64 || M > rows_per_launch || tiles_win) {
-            const int rc = aq::qmm_dispatch(ctx->stream, &ctx->ws, ctx->cu_count, ctx->forced[1], &ctx->last_variant[1], x,
-                                            packed, scales, biases, y, M, K, N, group_size, bits,
-                                            (flags & AQ_OUT_F32) != 0, fail);
-            if (rc == AQ_OK) ctx->last_variant[0] = ctx->last_variant[1];  // the kernel this aq_qmv call ran
-            return rc;
-        }
-    }
     return launch_qmv_rows(ctx, a, group_size, bits, false);
 }
 
@@ -743,6 +683,23 @@ int aq_qmm(aq_ctx* ctx, const void* x, const void* packed, const void* scales, c
     if (!aligned(x, 2) || !aligned(packed, 4) || !aligned(scales, 2) || !aligned(biases, 2) || !aligned(y, 2))
         return fail(AQ_ERR_ARG, "aq_qmm: operand pointer is not element-aligned");
     std::lock_guard<std::mutex> lk(ctx->mu);
+    if (M <= aq::kQmvMaxRows && ctx->forced[1] < 0) {
+        // a matmul of up to four rows is a matvec: the matvec selection runs it (no pass over x, no workspace)
+        aq::QmvArgs a{};
+        a.x = static_cast<const uint16_t*>(x);
+        a.w = static_cast<const uint32_t*>(packed);
+        a.s = static_cast<const uint16_t*>(scales);
+        a.b = static_cast<const uint16_t*>(biases);
+        a.y = y;
+        a.K = K;
+        a.N = N;
+        a.M = M;
+        a.out_f32 = (flags & AQ_OUT_F32) ? 1 : 0;
+        a.routes = 1;
+        const int rc = launch_qmv_rows(ctx, a, group_size, bits, false);
+        if (rc == AQ_OK) ctx->last_variant[1] = ctx->last_variant[0];
+        return rc;
+    }
     return aq::qmm_dispatch(ctx->stream, &ctx->ws, ctx->cu_count, ctx->forced[1], &ctx->last_variant[1], x, packed, scales,
                             biases, y, M, K, N, group_size, bits, (flags & AQ_OUT_F32) != 0, fail);
 }
@@ -1652,7 +1609,7 @@ int aq_proj_quant_matmul_host(aq_ctx* ctx, float* out, const float* x, size_t x_
 
 int aq_variant_count(int op) {
     if (op == 0) return qmv_total_variants();
-    if (op == 1) return aq::qmm_variant_count() + aq::qmmt_variant_count();
+    if (op == 1) return aq::qmmt_variant_count();
     return 0;
 }
 
@@ -1662,9 +1619,7 @@ const char* aq_variant_name(int op, int variant) {
         return v ? v->name : "";
     }
     if (op == 1) {
-        const int nd = aq::qmm_variant_count();
-        if (variant < nd) return aq::qmm_variant_name(variant);
-        const aq::QmmVariant* v = aq::qmmt_variant(variant - nd);
+        const aq::QmmVariant* v = aq::qmmt_variant(variant);
         return v ? v->name : "";
     }
     return "";

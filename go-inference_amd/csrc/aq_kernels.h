@@ -82,9 +82,8 @@ struct QmvVariant {
     int depth;   // K slices in flight per wavefront
     int gather;  // 1: reads rhs/lhs on device, grid.y = routes
     int xmode;   // 0: x staged through LDS, 1: every lane reads its x chunk from global
-    int kind;    // 0: VALU dot2 kernel (aq_qmv.hip), 1: MFMA kernel (aq_qmv_mfma.hip; m = most rows it takes),
+    int kind;    // 0: VALU dot2 kernel (aq_qmv.hip),
                  // 2: block-MFMA kernel (aq_qmv_blk.hip; m = most rows, depth = K pieces per wavefront),
-                 // 3: streaming dot2 kernel (aq_qmv_stream.hip; depth = rows in flight, xmode = slices per row)
                  // 4: diagonal-MFMA kernel (aq_qmv_diag.hip; m = most rows, rows = sets of 16 rows per workgroup,
                  //    xmode = chunks per step when not 4), 5: the same for quantisation groups of 32 codes
                  // 6: token-tile MFMA kernel (aq_qmv_tok.hip; m = most rows, rows = sets of 32 weight rows per wavefront)
@@ -98,12 +97,6 @@ const QmvVariant* qmv_variant(int idx);
 hipError_t qmv_launch(int idx, const QmvArgs& a, hipStream_t stream);
 // LDS bytes variant idx needs for these args (x staging).
 size_t qmv_lds_bytes(int idx, const QmvArgs& a);
-
-// MFMA matvec kernels (M <= 32), same argument block.
-int qmvx_variant_count();
-const QmvVariant* qmvx_variant(int idx);
-hipError_t qmvx_launch(int idx, const QmvArgs& a, hipStream_t stream);
-size_t qmvx_lds_bytes(int idx, const QmvArgs& a);
 
 // Block-MFMA matvec kernels (aq_qmv_blk.hip; M <= 16, persistent workgroups that split K among their
 // wavefronts).  A launch needs a plan: which kernel, how many wavefronts and workgroups, LDS bytes.
@@ -131,18 +124,6 @@ const QmvVariant* qmvb_variant(int idx);
 // forced_idx < 0: choose the variant; otherwise plan for exactly that one.
 bool qmvb_plan(const QmvArgs& a, int bits, int group_size, bool gather, int cu_count, int forced_idx, BlkPlan* out);
 hipError_t qmvb_launch(const BlkPlan& p, const QmvArgs& a, hipStream_t stream);
-
-// Streaming dot2 kernels (aq_qmv_stream.hip; one activation row, K = 1, 2, 4 or 7 slices of 64 chunks,
-// long-lived wavefronts with the activations in registers).
-struct StreamPlan {
-    int idx;   // variant
-    int nwg;   // workgroups (4 wavefronts each) along x
-    bool sbw;  // scales and biases of a row fit one dword load
-};
-int qmvs_variant_count();
-const QmvVariant* qmvs_variant(int idx);
-bool qmvs_plan(const QmvArgs& a, int bits, int group_size, bool gather, int cu_count, int forced_idx, StreamPlan* out);
-hipError_t qmvs_launch(const StreamPlan& p, const QmvArgs& a, hipStream_t stream);
 
 // Diagonal-MFMA matvec kernels (aq_qmv_diag.hip; 4-bit group-64 codes, M <= 8, K a multiple of 256 in 2..16 steps of 1024).
 int qmvd_variant_count();

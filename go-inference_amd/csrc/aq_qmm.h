@@ -1,12 +1,11 @@
-// MFMA matmul path (affine_qmm and the M > 4 rows of affine_qmv).
+// MFMA matmul path (affine_qmm and the many-row calls of affine_qmv).
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
 namespace aq {
 
-// Largest M the dot2 matvec kernels take in one pass; above it aq_qmv hands
-// the call to the MFMA kernels.
+// Largest M the dot2 matvec kernels take in one pass; a matmul call of up to this many rows runs as a matvec.
 constexpr int kQmvMaxRows = 4;
 
 struct QmmArgs {
@@ -51,10 +50,6 @@ int qmmt_variant_count();
 const QmmVariant* qmmt_variant(int idx);
 // Device bytes the tile kernels need beside their operands for an M x K activation matrix.
 size_t qmmt_workspace_bytes(int M, int K);
-// Variants named *_q move scales, biases and block sums through LDS as well; they take group size 64,
-// K a multiple of 512 and 16-byte aligned scale / bias arrays.
-bool qmmt_quad_staging_ok(const QmmArgs& a);
-bool qmmt_variant_stages_quads(int idx);
 // Pass over x + tile kernel `idx`; `workspace` holds at least qmmt_workspace_bytes(M, K).
 hipError_t qmmt_launch(int idx, const QmmArgs& a, void* workspace, hipStream_t stream);
 // The same with K shared out over ksplit workgroups per tile and a second kernel that adds the partial
@@ -84,10 +79,6 @@ struct Workspace {
     bool touched = false;
 };
 
-int qmm_variant_count();
-const char* qmm_variant_name(int idx);
-const QmmVariant* qmm_variant(int idx);
-hipError_t qmm_launch(int idx, const QmmArgs& a, hipStream_t stream);
 hipError_t fill_zero_launch(void* p, size_t bytes, hipStream_t stream);
 
 typedef int (*FailFn)(int code, const char* fmt, ...);
@@ -104,9 +95,9 @@ size_t qmm_scratch_bytes(int M, int K, int N);
 // Sizes ws for activations of M x K ahead of time (not during capture).
 int qmm_reserve(hipStream_t stream, Workspace* ws, int M, int K, FailFn fail);
 
-// Validated-shape dispatch used by aq_qmm and by aq_qmv for M > kQmvMaxRows.
+// Validated-shape dispatch used by aq_qmm and by aq_qmv for calls the matvec families pass on.
 // Returns an AQ_* / hipError_t code through `fail`.
-// `forced` indexes the direct-load variants first, then the tile variants.
+// `forced` indexes the tile variants (qmmt_variant), or is negative.
 int qmm_dispatch(hipStream_t stream, Workspace* ws, int cu_count, int forced, const char** last_variant, const void* x,
                  const void* packed, const void* scales, const void* biases, void* y, int M, int K, int N,
                  int group_size, int bits, bool out_f32, FailFn fail);

@@ -149,9 +149,9 @@ __global__ __launch_bounds__(256) void qmmh_prep_kernel(const uint16_t* __restri
 // ---- main kernel ----------------------------------------------------------------------------
 // OCC: wavefronts per SIMD the register budget is cut for (2: 256 registers, 1: 512, the accumulators then live in
 // the accumulation half of the register file).
-// PIPE: the MFMA steps of a block are software-pipelined by hand (see the loop); otherwise the compiler schedules a
-// block at a time.
-template <int MB, int NB, int WM, int WN, int STAGES, int OCC, bool PIPE, bool SPREAD>
+// SPREAD: the copies of the block requested in an iteration are issued a few at a time in front of every row block's
+// MFMAs instead of together at the top.
+template <int MB, int NB, int WM, int WN, int STAGES, int OCC, bool SPREAD>
 __global__ __launch_bounds__(WM* WN* kWave, OCC) void qmmh_kernel(const QmmTileArgs a) {
     static_assert(STAGES == 2 || STAGES == 3 || STAGES == 4, "LDS stages");
     constexpr int AHEAD = STAGES - 1;  // iteration g requests block g + AHEAD
@@ -247,12 +247,10 @@ __global__ __launch_bounds__(WM* WN* kWave, OCC) void qmmh_kernel(const QmmTileA
     const uint32_t mask_s = opaque_s(kMaskH);
     const uint32_t magic_v = opaque_v(kMagicH);
     // the first blocks are on their way while the prologue scans the scale rows
-    if constexpr (!PIPE) {
 #pragma unroll
-        for (int d = 0; d < AHEAD; d++) {
-            issue_a(d < K / 64 ? d : K / 64 - 1, d);
-            issue_b(d < K / 64 ? d : K / 64 - 1, d);
-        }
+    for (int d = 0; d < AHEAD; d++) {
+        issue_a(d < K / 64 ? d : K / 64 - 1, d);
+        issue_b(d < K / 64 ? d : K / 64 - 1, d);
     }
 
     // this lane's weight rows (one per column block), and the power of two that brings the row's largest scale
@@ -368,7 +366,6 @@ __global__ __launch_bounds__(WM* WN* kWave, OCC) void qmmh_kernel(const QmmTileA
         }
     };
 
-    if constexpr (!PIPE) {
     // One 64-code block per iteration; Q = g & 3 is static so that everything indexed by it stays in fixed
     // registers.  Iteration g requests block g + AHEAD.  Past the end of K the last block is requested again.
     //
@@ -486,142 +483,6 @@ __global__ __launch_bounds__(WM* WN* kWave, OCC) void qmmh_kernel(const QmmTileA
         if (g + 2 < G) iteration(std::integral_constant<int, 2>{}, g + 2);
         if (g + 3 < G) iteration(std::integral_constant<int, 3>{}, g + 3);
     }
-    } else {
-    // One 64-code block = four MFMA steps of 16 codes; Q = g & 3 is static so that everything indexed by it
-    // stays in fixed registers.  The steps are software-pipelined across blocks: while step t is multiplied, the
-    // A fragments of step t+1 are read from LDS and its codes expanded, into the other half of two small
-    // buffers.  The wait for block g+1's copies and the block's one barrier sit in front of step 3, so that step
-    // 3's MFMAs cover the first LDS reads of block g+1; every read of block g has returned by then (the wait
-    // includes the LDS counter), which is what lets the next iteration's copies overwrite its stage.
-    // Iteration g requests block g + AHEAD (at Q = 1 first the next quad's scales, biases and sums, with
-    // ordinary loads: the wait in front of step 3 counts the copies issued behind them).  The compiler cannot
-    // count the copies, so wherever it first uses a loaded register it drains them all; it is made to do so in
-    // iteration Q = 2 right behind the wait, where the only copies in flight are a whole block old.
-    // Past the end of K the last block is requested again.
-    const int glast = G - 1;
-    int sa = 0;  // LDS stage that holds block g
-    f16x8_t afr[2][MB];
-    f16x8_t bfr[2][NB];
-    uint4 cw[NB];
-    f16x2_t s2[NB], m24[NB];
-    auto word_of = [](const uint4& v, int t) { return t == 0 ? v.x : t == 1 ? v.y : t == 2 ? v.z : v.w; };
-    // this lane's codes of a stage: row (wave_n * NB + nb) * 32 + j, words 4h .. 4h+3; its A fragments
-    auto read_block_head = [&](int stage) {
-        const uint8_t* bb = bbuf + stage * B_STAGE + ((wave_n * NB) * 32 + j) * 32 + h * 16;
-        const uint8_t* ab = abuf + stage * A_STAGE + (wave_m * MB) * 4096 + lane * 16;
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) cw[nb] = *reinterpret_cast<const uint4*>(bb + nb * 32 * 32);
-#pragma unroll
-        for (int mb = 0; mb < MB; mb++) afr[0][mb] = *reinterpret_cast<const f16x8_t*>(ab + (mb * 4) * 1024);
-    };
-    // the block's scale, brought into fp16 range (8 significant bits: exact), -24 times it (10 bits), and the
-    // codes of step 0
-    auto start_block = [&](int q) {
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) {
-            const float sv = __uint_as_float(quad_hi(s_cur[nb], q)) * col_up[nb];
-            const float mv = sv * -24.0f;
-            s2[nb] = f16x2_t{(_Float16)sv, (_Float16)sv};
-            m24[nb] = f16x2_t{(_Float16)mv, (_Float16)mv};
-            bfr[0][nb] = __builtin_bit_cast(f16x8_t, expand_word(cw[nb].x, mask_s, magic_v, s2[nb], m24[nb]));
-        }
-    };
-    auto iteration = [&](auto q_tag, int g) {
-        constexpr int Q = decltype(q_tag)::value;
-        const bool more = g + 1 < G;
-        if constexpr (Q == 1) {
-            const int nq = (g >> 2) + 1 < G4 ? (g >> 2) + 1 : G4 - 1;
-            load_quad(a.s, nq, s_nxt);
-            load_quad(a.b, g >> 2, b_cur);
-            load_xs(g >> 2);
-        }
-        {
-            const int g2 = g + AHEAD < G ? g + AHEAD : glast;
-            const int st2 = sa == 0 ? STAGES - 1 : sa - 1;  // stage (sa + AHEAD) % STAGES: read last in iteration g-1
-            issue_a(g2, st2);
-            issue_b(g2, st2);
-        }
-        const uint8_t* ab = abuf + sa * A_STAGE + (wave_m * MB) * 4096 + lane * 16;
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-            if (t < 3) {
-#pragma unroll
-                for (int mb = 0; mb < MB; mb++)
-                    afr[(t + 1) & 1][mb] = *reinterpret_cast<const f16x8_t*>(ab + (mb * 4 + t + 1) * 1024);
-#pragma unroll
-                for (int nb = 0; nb < NB; nb++)
-                    bfr[(t + 1) & 1][nb] =
-                        __builtin_bit_cast(f16x8_t, expand_word(word_of(cw[nb], t + 1), mask_s, magic_v, s2[nb], m24[nb]));
-            } else {
-                // block g+1 has landed once at most the copies of the AHEAD-1 newest blocks are outstanding.  A
-                // bare s_barrier on purpose: __syncthreads() carries a workgroup fence, for which the compiler
-                // drains ALL outstanding copies into LDS.
-                asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((AHEAD - 1) * GROUP_OPS) : "memory");
-                __builtin_amdgcn_s_barrier();
-                asm volatile("" ::: "memory");
-                if constexpr (Q == 2) {
-#pragma unroll
-                    for (int nb = 0; nb < NB; nb++)
-                        asm volatile("" : "+v"(s_nxt[nb].x), "+v"(s_nxt[nb].y), "+v"(b_cur[nb].x), "+v"(b_cur[nb].y));
-#pragma unroll
-                    for (int mb = 0; mb < MB; mb++)
-                        asm volatile("" : "+v"(xs_cur[mb].x), "+v"(xs_cur[mb].y), "+v"(xs_cur[mb].z), "+v"(xs_cur[mb].w));
-                }
-                sa = sa == STAGES - 1 ? 0 : sa + 1;
-                read_block_head(sa);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-                for (int nb = 0; nb < NB; nb++)
-                    out[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[t & 1][mb], bfr[t & 1][nb], out[mb][nb], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-
-        if (Q == 3 || !more) {
-            if (Q < 2) {  // K ends inside a quad before its biases and sums were asked for
-                load_quad(a.b, g >> 2, b_cur);
-                load_xs(g >> 2);
-            }
-            affine(q_tag);
-        }
-        if constexpr (Q == 3) {
-#pragma unroll
-            for (int nb = 0; nb < NB; nb++) s_cur[nb] = s_nxt[nb];
-        }
-        start_block((Q + 1) & 3);  // past the end of K: values nobody uses
-    };
-
-    // the first quad and blocks 0 .. AHEAD-1 are requested up front
-    load_quad(a.s, 0, s_cur);
-#pragma unroll
-    for (int d = 0; d < AHEAD; d++) {
-        issue_a(d < G ? d : glast, d);
-        issue_b(d < G ? d : glast, d);
-    }
-    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((AHEAD - 1) * GROUP_OPS) : "memory");  // block 0 has landed
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    read_block_head(0);
-    start_block(0);
-#pragma unroll
-    for (int nb = 0; nb < NB; nb++) {
-        s_nxt[nb] = s_cur[nb];
-        b_cur[nb] = make_uint2(0u, 0u);
-    }
-#pragma unroll
-    for (int mb = 0; mb < MB; mb++) xs_cur[mb] = make_uint4(0u, 0u, 0u, 0u);
-
-    for (int g = 0; g < G; g += 4) {
-        iteration(std::integral_constant<int, 0>{}, g);
-        if (g + 1 < G) iteration(std::integral_constant<int, 1>{}, g + 1);
-        if (g + 2 < G) iteration(std::integral_constant<int, 2>{}, g + 2);
-        if (g + 3 < G) iteration(std::integral_constant<int, 3>{}, g + 3);
-    }
-
-    }  // PIPE
-
     // the copies requested past the end of K must not outlive the wavefront's use of LDS
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
@@ -708,24 +569,15 @@ struct QmmHalfEntry {
     int lds_bytes;
 };
 
-#define AQ_QMMH_S(MB, NB, WM, WN, ST, OCC, PIPE, SPREAD, SUFFIX)                                             \
-    {                                                                                                       \
-        {"qmmh_b4_mb" #MB "_nb" #NB "_wm" #WM "_wn" #WN SUFFIX, 4, MB, NB, WM, WN},                         \
-            qmmh_kernel<MB, NB, WM, WN, ST, OCC, PIPE, SPREAD>, ST*((WM * MB * 4096) + (WN * NB * 32 * 32)) \
+#define AQ_QMMH(MB, NB, WM, WN, ST, OCC, SPREAD, SUFFIX)                                               \
+    {                                                                                                 \
+        {"qmmh_b4_mb" #MB "_nb" #NB "_wm" #WM "_wn" #WN SUFFIX, 4, MB, NB, WM, WN},                   \
+            qmmh_kernel<MB, NB, WM, WN, ST, OCC, SPREAD>, ST*((WM * MB * 4096) + (WN * NB * 32 * 32)) \
     }
-#define AQ_QMMH(MB, NB, WM, WN, ST, OCC, PIPE, SUFFIX) AQ_QMMH_S(MB, NB, WM, WN, ST, OCC, PIPE, false, SUFFIX)
 
 static const QmmHalfEntry kQmmHalfTable[] = {
-    AQ_QMMH(4, 2, 1, 4, 3, 2, false, ""),            // 128 x 256 workgroup tiles, 72 KiB of LDS: two workgroups a CU
-    AQ_QMMH_S(4, 2, 1, 4, 3, 2, false, true, "_c"),  // the same with the copies spread over the iteration
-    AQ_QMMH(4, 2, 2, 2, 2, 2, false, "_s2"),         // 256 x 128, two stages: every LDS address a constant
-    AQ_QMMH_S(4, 2, 2, 2, 2, 2, false, true, "_s2c"),
-    AQ_QMMH(2, 2, 2, 2, 3, 2, false, ""),            // 128 x 128 with 64 x 64 wavefront tiles
-    AQ_QMMH(2, 2, 2, 2, 3, 2, true, "_p"),           // ... with the hand-pipelined loop
-    AQ_QMMH_S(4, 2, 2, 4, 2, 2, false, true, "_s2c"),  // 256 x 256, eight wavefronts: an A tile feeds twice the MFMAs
-    AQ_QMMH(4, 2, 2, 4, 2, 2, false, "_s2"),
-    AQ_QMMH(4, 2, 2, 4, 3, 2, false, ""),              // ... three stages (120 KiB)
-    AQ_QMMH_S(4, 2, 1, 8, 2, 2, false, true, "_s2c"),  // 128 x 512, eight wavefronts
+    AQ_QMMH(4, 2, 2, 2, 2, 2, true, "_s2c"),  // 256 x 128, four wavefronts, two stages (every LDS address a constant)
+    AQ_QMMH(4, 2, 2, 4, 3, 2, false, ""),     // 256 x 256, eight wavefronts, three stages (120 KiB): an A tile feeds twice the MFMAs
 };
 
 int qmmh_variant_count() { return (int)(sizeof(kQmmHalfTable) / sizeof(kQmmHalfTable[0])); }

@@ -112,20 +112,11 @@ __global__ __launch_bounds__(256) void qmm_prep_kernel(const uint16_t* __restric
 
 // ---- main kernel ----------------------------------------------------------------------------
 // Wavefront tiles of at most 64 x 64 keep under 256 registers, so two wavefronts share a SIMD.
-// SBL: scales, biases and block sums also travel global -> LDS by copy instructions (then the loop holds no
-// load the compiler has to wait for: it cannot count the copies, so any wait of its own drains them all).
-// Needs group size 64, K a multiple of 512 and 16-byte aligned scale / bias rows.
-// PIPE: the packed codes get a fourth LDS stage and are requested three blocks ahead, so that block g+1's codes
-// are in LDS while block g is multiplied: they are read and expanded in the shadow of block g's MFMAs instead
-// of in front of block g+1's.  The output tiles of a wavefront are walked column block by column block, a
-// tile's fp32 scaling follows the next tile's MFMAs in program order, and the expanded codes of a column
-// block are overwritten with the next block's as soon as its last tile has been issued.
-template <int BITS, int MB, int NB, int WM, int WN, int STAGES, bool SBL, bool PIPE>
+template <int BITS, int MB, int NB, int WM, int WN, int STAGES>
 __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTileArgs a) {
     static_assert(STAGES == 3 || STAGES == 4, "LDS stages");
-    static_assert(!PIPE || STAGES == 3, "the pipelined loop keeps three stages of A and four of B");
     constexpr int AHEAD = STAGES - 1;  // iteration g requests block g + AHEAD
-    constexpr int BST = PIPE ? 4 : STAGES;  // LDS stages of packed codes
+    constexpr int BST = STAGES;  // LDS stages of packed codes
     constexpr int BM = WM * MB * 32;
     constexpr int BN = WN * NB * 32;
     constexpr int NWAVE = WM * WN;
@@ -148,15 +139,6 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
     extern __shared__ __align__(16) uint8_t lds[];
     uint8_t* const abuf = lds;                     // [STAGES][A_STAGE]
     uint8_t* const bbuf = lds + STAGES * A_STAGE;  // [BST][B_STAGE]
-    // SBL: one quad ahead of (hi, lo) sums per tile row, and 16 bytes (eight blocks) of scales and of biases
-    // per tile column
-    uint8_t* const xsq = bbuf + BST * B_STAGE;  // [BM][16]
-    uint8_t* const sq = xsq + BM * 16;             // [BN][16]
-    uint8_t* const bq = sq + BN * 16;              // [BN][16]
-    constexpr int SB_SLOTS = BM / 64 + 2 * (BN / 64);           // 1 KiB copies per quad and workgroup
-    constexpr int SBE = SBL ? (SB_SLOTS + NWAVE - 1) / NWAVE : 0;  // per wavefront (spare slots repeat one)
-    static_assert(!SBL || (BM % 64 == 0 && BN % 64 == 0), "quad staging moves 64 rows per copy");
-
     // tile of this workgroup: workgroups are dealt to the 8 XCDs round-robin, so every 8th one
     // shares an L2; give each XCD a contiguous run of tiles in row-band-major order
     // With K split (a.ksplit > 1) every tile is computed by ksplit workgroups, each over a.gsplit blocks of K,
@@ -221,42 +203,6 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
 #pragma unroll
         for (int i = 0; i < WPT; i++)
             copy16_to_lds(wtile + (int64_t)g * WPB, woff[i], lds_offset(dst + (i * NWAVE + wave) * 1024));
-    };
-    // SBL: slot e of this wavefront: which array, which 64 rows
-    const uint8_t* sb_src[SBE > 0 ? SBE : 1];
-    uint32_t sb_off[SBE > 0 ? SBE : 1];
-    uint32_t sb_dst[SBE > 0 ? SBE : 1];
-    bool sb_is_xs[SBE > 0 ? SBE : 1];
-    if constexpr (SBL) {
-#pragma unroll
-        for (int e = 0; e < SBE; e++) {
-            const int slot = (wave * SBE + e) % SB_SLOTS;
-            if (slot < BM / 64) {
-                int row = m0 + slot * 64 + lane;
-                row = row < a.mblks * 32 ? row : a.mblks * 32 - 1;
-                sb_src[e] = reinterpret_cast<const uint8_t*>(a.xs);
-                sb_off[e] = (uint32_t)row * (uint32_t)G4 * 16u;
-                sb_dst[e] = lds_offset(xsq + slot * 1024);
-                sb_is_xs[e] = true;
-            } else {
-                const int t = slot - BM / 64;
-                const bool bias = t >= BN / 64;
-                const int n = min(n0 + (bias ? t - BN / 64 : t) * 64 + lane, N - 1);
-                sb_src[e] = reinterpret_cast<const uint8_t*>(bias ? a.b : a.s);
-                sb_off[e] = (uint32_t)n * (uint32_t)sb_per_row * 2u;
-                sb_dst[e] = lds_offset((bias ? bq : sq) + (bias ? t - BN / 64 : t) * 1024);
-                sb_is_xs[e] = false;
-            }
-        }
-    }
-    // requests quad `quad` (clamped to the last one) into the staging rows
-    auto issue_quad = [&](int quad) {
-        if constexpr (SBL) {
-            const int nq = quad < G4 ? quad : G4 - 1;
-#pragma unroll
-            for (int e = 0; e < SBE; e++)
-                copy16_to_lds(sb_src[e] + (sb_is_xs[e] ? nq * 16 : (nq >> 1) * 16), sb_off[e], sb_dst[e]);
-        }
     };
     const uint32_t mask_s = opaque_s(kMask16);
     const uint32_t magic_v = opaque_v(kMagic16);
@@ -336,20 +282,7 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
     auto iteration = [&](auto q_tag, int g) {
         constexpr int Q = decltype(q_tag)::value;
         const bool more = g + 1 < G;
-        if constexpr (Q == 0 && SBL) {
-            // the quad's scales, biases and sums landed in LDS two blocks ago (the first quad: before the loop)
-            const int half = ((g >> 2) & 1) * 8;
-#pragma unroll
-            for (int nb = 0; nb < NB; nb++) {
-                const int col = (wave_n * NB + nb) * 32 + j;
-                s_cur[nb] = *reinterpret_cast<const uint2*>(sq + col * 16 + half);
-                b_cur[nb] = *reinterpret_cast<const uint2*>(bq + col * 16 + half);
-            }
-#pragma unroll
-            for (int mb = 0; mb < MB; mb++)
-                xs_cur[mb] = *reinterpret_cast<const uint4*>(xsq + ((wave_m * MB + mb) * 32 + j) * 16);
-        }
-        if constexpr (Q == 0 && !SBL) {
+        if constexpr (Q == 0) {
             // the quad's scales, biases and sums were requested three blocks ago (the first quad: before
             // the loop).  Taken over here, before this iteration's copies are issued: the compiler waits
             // for every request it cannot count before the first use of a loaded register.
@@ -361,8 +294,7 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
 #pragma unroll
             for (int mb = 0; mb < MB; mb++) xs_cur[mb] = xs_nxt[mb];
         }
-        if constexpr (Q == 1 && SBL) issue_quad((g >> 2) + 1);  // every wavefront read the staging rows in the block before
-        if constexpr (Q == 1 && !SBL) {
+        if constexpr (Q == 1) {
             // ordinary loads first: the wait at the end of the iteration counts the copies behind them
             const int nq = (g >> 2) + 1 < G4 ? (g >> 2) + 1 : G4 - 1;
             load_quad(nq, s_nxt, b_nxt);
@@ -447,225 +379,14 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
         // Block g+1 has landed once at most the copies of the AHEAD-1 newest blocks are outstanding;
         // this iteration's LDS reads have returned.  A bare s_barrier on purpose: __syncthreads() carries
         // a workgroup fence, for which the compiler drains ALL outstanding copies into LDS.
-        // (the quad copies of block Q == 1 stay countable as long as they are among the AHEAD-1 newest groups)
-        constexpr int QUAD_OPS = (SBL && Q >= 1 && Q <= AHEAD - 1) ? SBE : 0;
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((AHEAD - 1) * GROUP_OPS + QUAD_OPS) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((AHEAD - 1) * GROUP_OPS) : "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
     };
-
-    // ---- pipelined loop (PIPE) ----
-    // An iteration is MB*NB*4 slots of { one MFMA, a quarter of the previous tile's fp32 scaling, half a
-    // packed word's expansion }, kept in that order by scheduling barriers: the vector work of a slot issues
-    // while its MFMA runs and the next MFMA of the chain waits for it anyway.  Tiles go column block by
-    // column block; while column block nb is multiplied, the codes of column block nb-1 (of the NEXT block of
-    // K; for nb = 0: of the last column block of THIS block, read one iteration ago) are expanded in place.
-    static_assert(!PIPE || (MB * NB) % 2 == 0, "two accumulator buffers alternate across iterations");
-    constexpr int CWN = BITS == 4 ? 1 : 2;  // 16-byte reads that hold a lane's codes of one block and column block
-    uint32_t bw[NB][4][4];                  // expanded codes: [column block][MFMA step][dword]
-    uint4 carried[CWN];                     // packed codes of the last column block, one block ahead
-    f32x16_t p[2];
-    float sc_prev = 0.0f;
-    auto read_codes = [&](int stage, int nb, uint4 (&cw)[CWN]) {
-        const uint8_t* bb = bbuf + stage * B_STAGE + ((wave_n * NB + nb) * 32 + j) * (WPB * 4) + h * (WPB * 2);
-#pragma unroll
-        for (int c = 0; c < CWN; c++) cw[c] = *reinterpret_cast<const uint4*>(bb + c * 16);
-    };
-    // dwords 2*half and 2*half+1 of MFMA step t
-    auto expand_half = [&](const uint4 (&cw)[CWN], int t, int half, uint32_t (&dst)[4]) {
-        if constexpr (BITS == 4) {
-            const uint32_t w = t == 0 ? cw[0].x : t == 1 ? cw[0].y : t == 2 ? cw[0].z : cw[0].w;
-            if (half == 0) {
-                dst[0] = and_or(w << 3, mask_s, magic_v);
-                dst[1] = and_or(w >> 1, mask_s, magic_v);
-            } else {
-                dst[2] = and_or(w >> 5, mask_s, magic_v);
-                dst[3] = and_or(w >> 9, mask_s, magic_v);
-            }
-        } else {
-            const uint4& c = cw[t >> 1];
-            const uint32_t w = (t & 1) ? (half ? c.w : c.z) : (half ? c.y : c.x);
-            uint32_t two[2];
-            unpack8_word(w, two);
-            dst[2 * half] = two[0];
-            dst[2 * half + 1] = two[1];
-        }
-    };
-    auto pipe_iteration = [&](auto q_tag, int g) {
-        constexpr int Q = decltype(q_tag)::value;  // = g & 3 = the B stage that holds block g
-        const bool more = g + 1 < G;
-        if constexpr (Q == 0 && SBL) {
-            const int half = ((g >> 2) & 1) * 8;
-#pragma unroll
-            for (int nb = 0; nb < NB; nb++) {
-                const int col = (wave_n * NB + nb) * 32 + j;
-                s_cur[nb] = *reinterpret_cast<const uint2*>(sq + col * 16 + half);
-                b_cur[nb] = *reinterpret_cast<const uint2*>(bq + col * 16 + half);
-            }
-#pragma unroll
-            for (int mb = 0; mb < MB; mb++)
-                xs_cur[mb] = *reinterpret_cast<const uint4*>(xsq + ((wave_m * MB + mb) * 32 + j) * 16);
-        }
-        if constexpr (Q == 0 && !SBL) {
-#pragma unroll
-            for (int nb = 0; nb < NB; nb++) {
-                s_cur[nb] = s_nxt[nb];
-                b_cur[nb] = b_nxt[nb];
-            }
-#pragma unroll
-            for (int mb = 0; mb < MB; mb++) xs_cur[mb] = xs_nxt[mb];
-        }
-        if constexpr (Q == 1 && SBL) issue_quad((g >> 2) + 1);
-        if constexpr (Q == 1 && !SBL) {
-            const int nq = (g >> 2) + 1 < G4 ? (g >> 2) + 1 : G4 - 1;
-            load_quad(nq, s_nxt, b_nxt);
-            load_xs(nq, xs_nxt);
-        }
-        issue_a(g + 2 < G ? g + 2 : glast, sa == 0 ? 2 : sa - 1);
-        issue_b(g + 3 < G ? g + 3 : glast, (Q + 3) & 3);
-
-        const uint8_t* ab = abuf + sa * A_STAGE + (wave_m * MB) * 4096 + lane * 16;
-        bf16x8_t afrag[MB][4];
-#pragma unroll
-        for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-            for (int t = 0; t < 4; t++) afrag[mb][t] = *reinterpret_cast<const bf16x8_t*>(ab + (mb * 4 + t) * 1024);
-        // block g+1's codes have been in LDS since the end of the previous iteration
-        uint4 cwn[NB][CWN];
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) read_codes((Q + 1) & 3, nb, cwn[nb]);
-        float sc[NB];
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) sc[nb] = __uint_as_float(quad_hi(s_cur[nb], Q));
-        __builtin_amdgcn_sched_barrier(0);
-
-        constexpr int T = MB * NB;
-#pragma unroll
-        for (int i = 0; i < T; i++) {
-            const int nb = i / MB, mb = i % MB;
-            // the tile whose scaling rides along: the one before (the first tile: the last of the previous block)
-            const int pi = (i + T - 1) % T;
-            const int pn = pi / MB, pm = pi % MB;
-            const float psc = i == 0 ? sc_prev : sc[pn];
-            f32x16_t acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int t = 0; t < 4; t++) {
-                const uint4 bq4 = {bw[nb][t][0], bw[nb][t][1], bw[nb][t][2], bw[nb][t][3]};
-                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag[mb][t], __builtin_bit_cast(bf16x8_t, bq4), acc, 0, 0, 0);
-#pragma unroll
-                for (int r = 4 * t; r < 4 * t + 4; r++) out[pm][pn][r] = __fmaf_rn(psc, p[pi & 1][r], out[pm][pn][r]);
-                // column block nb's tiles give 4 * MB slots to the 8 half words of the column block before it
-                constexpr int HALVES_PER_SLOT = MB >= 2 ? 1 : 2;
-                const int slot = mb * 4 + t;
-                const int tgt = (nb + NB - 1) % NB;
-#pragma unroll
-                for (int e = 0; e < HALVES_PER_SLOT; e++) {
-                    const int hw = slot * HALVES_PER_SLOT + e;  // 0 .. 7 (more slots than half words when MB > 2)
-                    if (hw < 8) {
-                        if (nb == 0) {
-                            expand_half(carried, hw >> 1, hw & 1, bw[tgt][hw >> 1]);
-                        } else {
-                            expand_half(cwn[tgt], hw >> 1, hw & 1, bw[tgt][hw >> 1]);
-                        }
-                    }
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            p[i & 1] = acc;
-        }
-        sc_prev = sc[NB - 1];
-#pragma unroll
-        for (int c = 0; c < CWN; c++) carried[c] = cwn[NB - 1][c];
-
-        if (Q == 3 || !more) {
-            bf16x8_t bbf[NB];
-#pragma unroll
-            for (int nb = 0; nb < NB; nb++) {
-                uint32_t v[4];
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    if (q <= Q) {
-                        const uint32_t neg = __float_as_uint(__uint_as_float(quad_hi(s_cur[nb], q)) * -OFFSET) >> 16;
-                        const uint32_t bia = quad_hi(b_cur[nb], q) >> 16;
-                        v[q] = dup16(h ? neg : bia);
-                    } else {
-                        v[q] = 0u;
-                    }
-                }
-                const uint4 u = {v[0], v[1], v[2], v[3]};
-                bbf[nb] = __builtin_bit_cast(bf16x8_t, u);
-            }
-#pragma unroll
-            for (int mb = 0; mb < MB; mb++) {
-                const bf16x8_t aa = __builtin_bit_cast(bf16x8_t, xs_cur[mb]);
-#pragma unroll
-                for (int nb = 0; nb < NB; nb++)
-                    out[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aa, bbf[nb], out[mb][nb], 0, 0, 0);
-            }
-        }
-        sa = sa == 2 ? 0 : sa + 1;
-        // A of block g+1 and the codes of block g+2 were requested one iteration ago: they have landed once
-        // at most this iteration's own copies are outstanding
-        constexpr int QUAD_OPS = (SBL && Q == 1) ? SBE : 0;
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(GROUP_OPS + QUAD_OPS) : "memory");
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-    };
-
-    if constexpr (PIPE) {
-        if constexpr (SBL) {
-            issue_quad(gb >> 2);
-        } else {
-            load_quad(gb >> 2, s_nxt, b_nxt);
-            load_xs(gb >> 2, xs_nxt);
-        }
-        // oldest first: what iteration 0 needs (A 0, codes 0 and 1), then one iteration's worth (A 1, codes 2)
-        issue_a(gb, 0);
-        issue_b(gb, 0);
-        issue_b(gb + 1 < G ? gb + 1 : glast, 1);
-        issue_a(gb + 1 < G ? gb + 1 : glast, 1);
-        issue_b(gb + 2 < G ? gb + 2 : glast, 2);
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(GROUP_OPS) : "memory");
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-        // block 0: every column block but the last is expanded here, the last one rides in `carried`
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) {
-            uint4 cw0[CWN];
-            read_codes(0, nb, cw0);
-            if (nb == NB - 1) {
-#pragma unroll
-                for (int c = 0; c < CWN; c++) carried[c] = cw0[c];
-            } else {
-#pragma unroll
-                for (int hw = 0; hw < 8; hw++) expand_half(cw0, hw >> 1, hw & 1, bw[nb][hw >> 1]);
-            }
-        }
-#pragma unroll
-        for (int r = 0; r < 16; r++) p[0][r] = p[1][r] = 0.0f;
-        for (int g = gb; g < G; g += 4) {
-            pipe_iteration(std::integral_constant<int, 0>{}, g);
-            if (g + 1 < G) pipe_iteration(std::integral_constant<int, 1>{}, g + 1);
-            if (g + 2 < G) pipe_iteration(std::integral_constant<int, 2>{}, g + 2);
-            if (g + 3 < G) pipe_iteration(std::integral_constant<int, 3>{}, g + 3);
-        }
-        // the last tile of the last block is still unscaled
-        {
-            constexpr int T = MB * NB;
-#pragma unroll
-            for (int r = 0; r < 16; r++)
-                out[(T - 1) % MB][(T - 1) / MB][r] = __fmaf_rn(sc_prev, p[(T - 1) & 1][r], out[(T - 1) % MB][(T - 1) / MB][r]);
-        }
-    }
 
     // the first quad and blocks 0 .. AHEAD-1 are requested up front
-    if constexpr (!PIPE) {
-    if constexpr (SBL) {
-        issue_quad(gb >> 2);
-    } else {
-        load_quad(gb >> 2, s_nxt, b_nxt);
-        load_xs(gb >> 2, xs_nxt);
-    }
+    load_quad(gb >> 2, s_nxt, b_nxt);
+    load_xs(gb >> 2, xs_nxt);
 #pragma unroll
     for (int d = 0; d < AHEAD; d++) {
         issue_a(gb + d < G ? gb + d : glast, d);
@@ -681,7 +402,6 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
         if (g + 2 < G) iteration(std::integral_constant<int, 2>{}, g + 2);
         if (g + 3 < G) iteration(std::integral_constant<int, 3>{}, g + 3);
     }
-    }  // !PIPE
 
     // the copies requested past the end of K must not outlive the wavefront's use of LDS
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -757,26 +477,17 @@ struct QmmTileEntry {
     QmmVariant v;
     QmmTileKernel fn;
     int lds_bytes;
-    bool sbl;  // stages scales, biases and sums through LDS: needs qmmt_quad_staging_ok()
 };
 
-#define AQ_QMMT_P(BITS, MB, NB, WM, WN, ST, SBL, PIPE, SUFFIX)                                            \
-    {                                                                                                    \
-        {"qmmt_b" #BITS "_mb" #MB "_nb" #NB "_wm" #WM "_wn" #WN SUFFIX, BITS, MB, NB, WM, WN},           \
-            qmm_tile_kernel<BITS, MB, NB, WM, WN, ST, SBL, PIPE>,                                        \
-            ST * (WM * MB * 4096) + (PIPE ? 4 : ST) * (WN * NB * 32 * (BITS == 4 ? 32 : 64)) +           \
-                (SBL ? (WM * MB * 32 + 2 * WN * NB * 32) * 16 : 0),                                      \
-            SBL                                                                                          \
+#define AQ_QMMT(BITS, MB, NB, WM, WN, ST)                                                          \
+    {                                                                                             \
+        {"qmmt_b" #BITS "_mb" #MB "_nb" #NB "_wm" #WM "_wn" #WN, BITS, MB, NB, WM, WN},           \
+            qmm_tile_kernel<BITS, MB, NB, WM, WN, ST>,                                            \
+            ST * (WM * MB * 4096) + ST * (WN * NB * 32 * (BITS == 4 ? 32 : 64))                   \
     }
-#define AQ_QMMT_S(BITS, MB, NB, WM, WN, ST, SBL, SUFFIX) AQ_QMMT_P(BITS, MB, NB, WM, WN, ST, SBL, false, SUFFIX)
-#define AQ_QMMT(BITS, MB, NB, WM, WN) AQ_QMMT_S(BITS, MB, NB, WM, WN, 3, false, "")
-#define AQ_QMMT_SET(BITS)                                                                        \
-    AQ_QMMT(BITS, 4, 2, 2, 2), AQ_QMMT(BITS, 4, 2, 1, 2), AQ_QMMT(BITS, 2, 2, 2, 2),             \
-        AQ_QMMT(BITS, 2, 2, 1, 2), AQ_QMMT(BITS, 4, 2, 1, 4),         \
-        AQ_QMMT(BITS, 2, 2, 2, 4), AQ_QMMT(BITS, 1, 2, 1, 4), AQ_QMMT_S(BITS, 2, 2, 2, 2, 4, false, "_s4"), \
-        AQ_QMMT_S(BITS, 2, 2, 1, 4, 4, false, "_s4"), AQ_QMMT_S(BITS, 2, 2, 1, 4, 3, false, ""),       \
-        AQ_QMMT_S(BITS, 2, 2, 2, 2, 3, true, "_q"), AQ_QMMT_S(BITS, 2, 2, 1, 4, 3, true, "_q"),         \
-        AQ_QMMT_P(BITS, 2, 2, 2, 2, 3, false, true, "_p"), AQ_QMMT_P(BITS, 2, 2, 2, 2, 3, true, true, "_pq")
+// 128 x 128 workgroup tiles for prefill sizes (8 bit, and 4-bit calls too small for the fp16-operand kernels);
+// 32 x 256 and 64 x 256 for calls of fewer than 64 rows whose K the few-rows kernels do not take
+#define AQ_QMMT_SET(BITS) AQ_QMMT(BITS, 2, 2, 2, 2, 3), AQ_QMMT(BITS, 1, 2, 1, 4, 3), AQ_QMMT(BITS, 2, 2, 1, 4, 3)
 
 static const QmmTileEntry kQmmTileTable[] = {AQ_QMMT_SET(4), AQ_QMMT_SET(8)};
 
@@ -795,11 +506,6 @@ size_t qmmt_workspace_bytes(int M, int K) {
     const size_t g4 = ((size_t)K / 64 + 3) / 4;
     return mblks * 32 * (size_t)K * 2 + mblks * 32 * g4 * 16 + mblks * 32 * 4;
 }
-
-bool qmmt_quad_staging_ok(const QmmArgs& q) {
-    return q.gs_blocks == 1 && q.K % 512 == 0 && ((reinterpret_cast<uintptr_t>(q.s) | reinterpret_cast<uintptr_t>(q.b)) & 15) == 0;
-}
-bool qmmt_variant_stages_quads(int idx) { return idx >= 0 && idx < tile_variants() && kQmmTileTable[idx].sbl; }
 
 // Adds the ksplit partial tiles [ksplit][M*N] in split order and stores bf16 or fp32.
 __global__ __launch_bounds__(256) void qmm_splitk_reduce_kernel(const float* __restrict__ partial, int ksplit, int64_t mn,
@@ -831,7 +537,6 @@ hipError_t qmmt_launch_splitk(int idx, const QmmArgs& q, void* workspace, int ks
     static const QmmTileEntry kNone{};
     const QmmTileEntry& e = few < 0 ? kQmmTileTable[idx] : kNone;
     const QmmVariant& v = few < 0 ? e.v : *qmmf_variant(few);
-    if (e.sbl && !qmmt_quad_staging_ok(q)) return hipErrorInvalidValue;
     if (ksplit < 1 || (ksplit > 1 && (q.K / 64) % (4 * ksplit) != 0)) return hipErrorInvalidValue;
     const int mblks = (q.M + 31) / 32;
     uint16_t* xf = static_cast<uint16_t*>(workspace);

@@ -43,7 +43,7 @@ def test_variant_tables(aqlib):
     m = aq_mi355.variant_names(aq_mi355.OP_QMM)
     assert len(q) == len(set(q)) and len(m) == len(set(m)) and q and m
     assert any(n.startswith("qmv_b4_m1_") and "_g1_" in n for n in q)
-    assert any(n.startswith("qmm_b8_") for n in m)
+    assert any(n.startswith("qmmt_b8_") for n in m) and any(n.startswith("qmmh_b4_") for n in m)
 
 
 def test_backend_quant_registry(aqlib):

@@ -133,12 +133,8 @@ def test_qmv_other_widths_generic_kernel(ctx, orc, bits, gs, K, N, M):
 def _parse_variant(name):
     """-> (family, bits, rows it runs in one launch, gather)"""
     parts = dict((p.rstrip("0123456789"), int(p[len(p.rstrip("0123456789")):])) for p in name.split("_")[1:])
-    if name.startswith("qmvx_"):
-        return "mfma", parts["b"], {1: 1, 4: 8, 8: 16, 16: 32}[parts["mr"]], parts["g"]
     if name.startswith("qmvb_"):
         return "blk", parts["b"], parts["m"], parts["g"]
-    if name.startswith("qmvs_"):
-        return "stream", parts["b"], 1, parts["g"]
     if name.startswith("qmvd_"):
         return "diag", parts["b"], parts["m"], parts["g"]
     if name.startswith("qmvt_"):
@@ -154,8 +150,7 @@ def _blk_pieces(name):
 
 
 def test_qmv_every_variant(ctx, orc):
-    """Each tuned matvec kernel variant (dot2 and MFMA), forced, on a shape with a masked K tail
-    (K = 44 group blocks) and ragged N."""
+    """Each dot2 matvec kernel variant, forced, on a shape with a masked K tail (K = 44 group blocks) and ragged N."""
     import aq_mi355
     K, N = 2816, 150
     names = aq_mi355.variant_names(0)
@@ -163,8 +158,8 @@ def test_qmv_every_variant(ctx, orc):
     try:
         for idx, name in enumerate(names):
             fam, bits, m, gather = _parse_variant(name)
-            if gather or fam in ("blk", "stream", "diag", "tok", "d8"):
-                continue  # covered by test_gather_every_variant / test_qmvb_every_variant / test_qmvs_every_variant / test_qmvd_every_variant
+            if gather or fam != "dot2":
+                continue  # covered by test_gather_every_variant and the other families' own tests
             say("variant", idx, name)
             if bits not in data:
                 words, s, b = F.synthetic_affine(N, K, bits, 64, seed=500 + bits)
@@ -172,26 +167,9 @@ def test_qmv_every_variant(ctx, orc):
                 data[bits] = (DeviceAffine(ctx, words, s, b), x, F.reference_f64(x, words, s, b, bits, 64, K))
             dw, x, ref = data[bits]
             ctx.force_variant(0, idx)
-            if fam == "dot2":
-                acc = run_qmv(ctx, x[:m], dw, m, K, N, 64, bits, True)
-                assert ctx.last_variant(0) == name
-                check_accumulators(acc, ref[:m], name)
-                continue
-            # the MFMA kernels keep all of x in LDS next to their weight tiles: a row count that
-            # does not fit is refused with AQ_ERR_ARG, so walk down until one fits
-            rows, done = m, 0
-            while rows >= 1 and done < 2:
-                try:
-                    acc = run_qmv(ctx, x[:rows], dw, rows, K, N, 64, bits, True)
-                except aq_mi355.AqError as e:
-                    assert e.code == aq_mi355.AQ_ERR_ARG
-                    rows -= 3
-                    continue
-                assert ctx.last_variant(0) == name
-                check_accumulators(acc, ref[:rows], "%s rows=%d" % (name, rows))
-                done += 1
-                rows -= 3
-            assert done >= 1, name
+            acc = run_qmv(ctx, x[:m], dw, m, K, N, 64, bits, True)
+            assert ctx.last_variant(0) == name
+            check_accumulators(acc, ref[:m], name)
     finally:
         ctx.force_variant(0, -1)
     for dw, _, _ in data.values():
@@ -206,7 +184,7 @@ def test_gather_every_variant(ctx, orc):
     try:
         for idx, name in enumerate(names):
             fam, bits, m, gather = _parse_variant(name)
-            if not gather or fam in ("blk", "stream", "diag", "tok", "d8"):
+            if not gather or fam != "dot2":
                 continue
             say("gather variant", idx, name)
             fx = F.gather_fixture(out_dim, in_dim, 64, bits, E, expert_rows, True, routes)
@@ -293,53 +271,6 @@ def test_qmv_block_family_many_batches(ctx, orc):
     assert ctx.last_variant(0).startswith("qmvb_"), ctx.last_variant(0)
     check_accumulators(acc, ref, "many batches")
     dw.free()
-
-
-def test_qmvs_every_variant(ctx, orc):
-    """Each streaming dot2 variant, forced: K = its number of 64-chunk slices, rows that do not divide
-    among the wavefronts, plain and gathered (batched x, row_base slab offset)."""
-    import aq_mi355
-    names = aq_mi355.variant_names(0)
-    N = 2 * 4096 + 37
-    E, routes, out_dim, expert_rows, row_base = 4, 5, 75, 128, 32
-    data = {}
-    try:
-        for idx, name in enumerate(names):
-            fam, bits, m, gather = _parse_variant(name)
-            if fam != "stream":
-                continue
-            ns = int(name.split("_ns")[1].split("_")[0])
-            K = ns * (2048 if bits == 4 else 1024)
-            say("variant", idx, name, "K", K)
-            ctx.force_variant(0, idx)
-            if not gather:
-                if (bits, K) not in data:
-                    words, s, b = F.synthetic_affine(N, K, bits, 64, seed=520 + bits + ns)
-                    x = F.synthetic_x(1, K, seed=620 + bits + ns)
-                    data[(bits, K)] = (DeviceAffine(ctx, words, s, b), x, F.reference_f64(x, words, s, b, bits, 64, K))
-                dw, x, ref = data[(bits, K)]
-                acc = run_qmv(ctx, x, dw, 1, K, N, 64, bits, True)
-                assert ctx.last_variant(0) == name
-                check_accumulators(acc, ref, name)
-                out = run_qmv(ctx, x, dw, 1, K, N, 64, bits, False)
-                check_bf16_store(out, ref, name)
-                with pytest.raises(aq_mi355.AqError) as ei:
-                    run_qmv(ctx, x[:, :K - 64], dw, 1, K - 64, N, 64, bits, True)
-                assert ei.value.code == aq_mi355.AQ_ERR_ARG
-            else:
-                fx = F.gather_fixture(out_dim, K, 64, bits, E, expert_rows, True, routes)
-                _, s, b = F.synthetic_affine(E * expert_rows, K, bits, 64, seed=40 + bits)
-                fx["scales"], fx["biases"] = s, b
-                ref64, _ = orc.gather_qmv(fx["x"], fx["x_rows"], fx["packed"], s, b, fx["lhs"], fx["rhs"], routes, E,
-                                          expert_rows, row_base, out_dim, K, 64, bits)
-                acc, dwg = _gather_run(ctx, fx, routes, E, expert_rows, row_base, out_dim, K, 64, bits, True)
-                assert ctx.last_variant(0) == name
-                check_accumulators(acc, ref64, name)
-                dwg.free()
-    finally:
-        ctx.force_variant(0, -1)
-    for dw, _, _ in data.values():
-        dw.free()
 
 
 def test_qmvd_every_variant(ctx, orc):

@@ -1,0 +1,67 @@
+"""The kernel the library picks for a call, per (bits, group size, rows of x, K): one case per rule of the selection
+table in csrc/aq_api.hip, each also checked against the float64 reference, so that a rule that sends a shape to a
+family that cannot take it shows up as a wrong result and not only as a wrong name."""
+import numpy as np
+import pytest
+
+import fixtures as F
+from gpu_util import DeviceAffine, check_accumulators, run_qmv, say
+
+pytestmark = pytest.mark.gpu
+
+N = 520  # ragged against every family's rows per workgroup (16, 32, 64, 128, 256)
+
+# bits, group, rows, K, the kernel-name prefixes the rule may answer with
+CASES = [
+    (4, 64, 1, 4096, ("qmvd_",)),                    # diagonal MFMA: one row, K up to 16 steps of 1024
+    (4, 64, 1, 14336, ("qmvd_",)),
+    (4, 64, 8, 4096, ("qmvd_",)),                    # ... up to 8 rows at 2..4 steps
+    (4, 32, 2, 1536, ("qmvd_",)),                    # groups of 32
+    (8, 64, 8, 4096, ("qmvd8_",)),                   # 8-bit MFMA: 5..16 rows
+    (8, 64, 16, 4096, ("qmvd8_",)),
+    (4, 64, 9, 4096, ("qmvt_",)),                    # token tile: 9..32 rows, K a multiple of 256
+    (4, 64, 32, 4096, ("qmvt_",)),
+    (8, 64, 1, 4096, ("qmvb_",)),                    # block MFMA: one row of 8-bit codes
+    (8, 64, 4, 4096, ("qmvb_",)),                    # ... and 2..4 rows
+    (4, 64, 8, 14336, ("qmvb_", "qmmf_", "qmmt_")),  # 5..8 rows at a K the diagonal kernels take for one row only
+    (4, 128, 1, 4096, ("qmv_b4_",)),                 # dot2: groups of 128
+    (4, 64, 1, 2880, ("qmv_b4_",)),                  # dot2: K = 45 groups
+    (4, 64, 3, 2880, ("qmvb_", "qmv_b4_")),
+    (3, 64, 2, 512, ("qmv_generic",)),               # any width
+    (6, 32, 1, 512, ("qmv_six",)),
+    (4, 64, 48, 4096, ("qmmf_",)),                   # 33..64 rows, K a multiple of 256: K shared out over workgroups
+    (8, 64, 24, 4096, ("qmmf_",)),                   # 8 bit beyond 16 rows
+    (4, 64, 20, 320, ("qmmt_b4_mb1_nb2_wm1_wn4",)),  # fewer than 64 rows, K no multiple of 256: 32 x 256 tiles
+    (4, 64, 40, 320, ("qmmt_b4_mb2_nb2_wm1_wn4",)),  # ... 64 x 256 tiles
+    (8, 64, 70, 320, ("qmmt_b8_mb2_nb2_wm2_wn2",)),  # 64 rows and more: 128 x 128 tiles
+    (4, 64, 20, 4096 + 64, ("qmvb_", "qmmt_")),
+]
+
+
+@pytest.mark.parametrize("bits,gs,M,K,prefixes", CASES)
+def test_selected_family(ctx, bits, gs, M, K, prefixes):
+    say("selection", bits, gs, M, K)
+    words, s, b = F.synthetic_affine(N, K, bits, gs, seed=900 + bits + M)
+    x = F.synthetic_x(M, K, seed=950 + M)
+    ref = F.reference_f64(x, words, s, b, bits, gs, K)
+    dw = DeviceAffine(ctx, words, s, b)
+    acc = run_qmv(ctx, x, dw, M, K, N, gs, bits, True)
+    name = ctx.last_variant(0)
+    assert name.startswith(prefixes), (name, prefixes)
+    check_accumulators(acc, ref, name)
+    dw.free()
+
+
+@pytest.mark.parametrize("M", [1, 3, 4])
+def test_matmul_of_few_rows_runs_as_matvec(ctx, M):
+    """aq_qmm with up to four rows of x takes the matvec selection: same kernel, same bytes as aq_qmv."""
+    K = 4096
+    words, s, b = F.synthetic_affine(N, K, 4, 64, seed=990)
+    x = F.synthetic_x(M, K, seed=991)
+    dw = DeviceAffine(ctx, words, s, b)
+    via_qmv = run_qmv(ctx, x, dw, M, K, N, 64, 4, True)
+    name = ctx.last_variant(0)
+    via_qmm = run_qmv(ctx, x, dw, M, K, N, 64, 4, True, fn="qmm")
+    assert ctx.last_variant(1) == name and name.startswith("qmvd_")
+    assert np.array_equal(via_qmv.view(np.uint32), via_qmm.view(np.uint32))
+    dw.free()
