@@ -451,7 +451,7 @@ class SafetensorsFile:
         dtype = ctypes.create_string_buffer(16)
         shape = (_c.c_int64 * 8)()
         rank, data, n = _i(0), _vp(), _sz(0)
-        rc = self.lib.aqh_safetensors_tensor(self.handle, name.encode(), dtype, shape, ctypes.byref(rank), ctypes.byref(data),
+        rc = self.lib.aqh_safetensors_tensor(self.handle, name if isinstance(name, bytes) else name.encode(), dtype, shape, ctypes.byref(rank), ctypes.byref(data),
                                              ctypes.byref(n))
         if rc != AQ_OK:
             raise AqError(rc, self.lib.aqh_last_error().decode())

@@ -96,12 +96,8 @@ struct Parser {
                 case 'u': {
                     uint32_t cp;
                     if (!hex4(&cp)) return false;
-                    if (cp >= 0xD800 && cp < 0xDC00 && end - p >= 6 && p[0] == '\\' && p[1] == 'u') {
-                        p += 2;
-                        uint32_t lo;
-                        if (!hex4(&lo)) return false;
-                        cp = 0x10000 + ((cp - 0xD800) << 10) + (lo - 0xDC00);
-                    }
+                    // every \uXXXX escape becomes the UTF-8 form of its own 16-bit value, surrogate halves included
+                    // (header_parse.go:262-292 does not pair them): tensor names keep the reference's bytes
                     utf8(out, cp);
                     break;
                 }
@@ -269,8 +265,12 @@ model::Error File::Parse(const uint8_t* data, size_t len) {
             t.Len = (size_t)(endo - begin);
             if (const size_t eb = dtype_bytes(t.Dtype)) {
                 uint64_t elements = 1;
-                for (int d : t.Shape) elements *= (uint64_t)d;
-                if (elements * eb != t.Len) return bad("tensor byte length does not match dtype and shape: " + name);
+                bool fits = true;  // the product of the dimensions, as long as it can still describe t.Len bytes
+                for (int d : t.Shape) {
+                    if (d != 0 && elements > (uint64_t)payload_len / (uint64_t)d) fits = false;
+                    elements *= (uint64_t)d;
+                }
+                if (!fits || elements * eb != t.Len) return bad("tensor byte length does not match dtype and shape: " + name);
             }
             Tensors[name] = std::move(t);
         } while (ps.eat(','));

@@ -136,7 +136,7 @@ def test_one_bit_pack_is_widened_and_written_back(tmp_path, orc):
 
 
 @pytest.mark.parametrize("case", ["short", "header_size", "not_json", "missing_field", "offsets_reversed", "offsets_outside",
-                                  "length_mismatch", "negative_offset", "no_file"])
+                                  "length_mismatch", "negative_offset", "shape_product_wraps", "no_file"])
 def test_malformed_files_are_rejected(tmp_path, case):
     import aq_mi355
     path = str(tmp_path / (case + ".safetensors"))
@@ -161,6 +161,8 @@ def test_malformed_files_are_rejected(tmp_path, case):
         emit({"t": {**good, "dtype": "U32"}})
     elif case == "negative_offset":
         emit({"t": {**good, "data_offsets": [-1, 3]}})
+    elif case == "shape_product_wraps":     # 2^16 * 2^16 * 2^16 * 2^16 * 4 wraps to 4 in 64 bits
+        emit({"t": {**good, "shape": [65536, 65536, 65536, 65536, 4]}})
     with pytest.raises(aq_mi355.AqError):
         aq_mi355.SafetensorsFile(path)
     if case == "no_file":
@@ -168,6 +170,10 @@ def test_malformed_files_are_rejected(tmp_path, case):
     emit({"t": good})                       # the same framing with a sound header loads
     f = aq_mi355.SafetensorsFile(path)
     assert f.tensor("t")[2].tolist() == [1, 2, 3, 4]
+    f.close()
+    emit(b'{"a\\ud83d\\ude00": {"dtype": "U8", "shape": [4], "data_offsets": [0, 4]}}')
+    f = aq_mi355.SafetensorsFile(path)      # escapes decode one by one, as in the reference: two three-byte sequences
+    assert f.tensor(b"a\xed\xa0\xbd\xed\xb8\x80")[2].tolist() == [1, 2, 3, 4]
     with pytest.raises(aq_mi355.AqError) as e:
         f.tensor("absent")
     assert e.value.code == aq_mi355.AQ_ERR_INDEX
