@@ -195,10 +195,13 @@ const QmvRule kQmvRules[] = {
     {4, 64, 1, 1, 1, kFamDiag},             // K a multiple of 128 in 2..8 steps of 1024 codes
     {0, 0, 1, 1, 1, kFamDot2},              // 4 / 8 bit, groups of 32 / 64 / 128, 16-byte chunks inside one group
     {0, 0, 1, 1, 1, kFamGeneric},
-    {4, 64, 0, 1, 8, kFamDiag},             // one row up to 16 steps of 1024 codes, up to 8 rows at 2..4 steps
+    {4, 64, 0, 1, 8, kFamDiag},             // one row up to 16 steps of 1024 codes, up to 8 rows at 2..4 steps: every row
+                                            // of such a call has the bytes of a call with that row alone
     {4, 32, 0, 1, 2, kFamDiag},             // groups of 32: two tokens x eight groups as MFMA rows
     {8, 64, 0, 5, 16, kFamD8},              // (up to 4 rows the block-MFMA kernels measure the same or faster)
-    {4, 64, 0, 9, 32, kFamTok},             // K a multiple of 256: one launch, weights streamed once, no scratch
+    {4, 64, 0, 5, 32, kFamTok},             // K a multiple of 256: one launch, weights streamed once, no scratch
+                                            // (5..8 rows: only where the diagonal kernels passed; they measure 11.2 us
+                                            // against 14.4 us at 8 rows of 4096 x 14336, but not row by row the same bytes)
     {0, 0, 0, 9, 64, kFamTilesLarge},       // 16 Mi codes and more: the 16-row block-MFMA kernel is bound by its 4x4x4 MFMAs
     {0, 0, 0, 2, 16, kFamBlk},              // the whole call in one launch of up to 16 rows (4 where K is long)
     {8, 0, 0, 1, 1, kFamBlk},               // (a single row of 4-bit codes is faster on the dot2 kernels)

@@ -58,6 +58,8 @@ __device__ __forceinline__ bf16x8_t as_bf16x8(uint32_t a, uint32_t b, uint32_t c
 
 constexpr int kTokRows = 32;  // weight rows per set (the N side of the MFMA)
 constexpr int kTokMax = 32;   // activation rows per launch (the M side)
+// 8-byte pieces of scales (and of biases) a thread of the 16-token form stages at most: K up to 16384 with 16 wavefronts
+__host__ __device__ constexpr int tok16_stage_pieces(int nw) { return nw >= 16 ? 4 : 8; }
 
 }  // namespace
 
@@ -321,18 +323,318 @@ __global__ __launch_bounds__(NW* kWave) void qmv_tok_kernel(const QmvArgs a) {
     }
 }
 
+
+// ---- up to 16 rows of x: 16x16x32 MFMAs, sixteen wavefronts that share K ---------------------------------------------
+//
+// v_mfma_f32_16x16x32_bf16 with the tokens as the 16 rows of A and 16 weight rows as the columns of B.  A workgroup of
+// NW wavefronts owns RS sets of 16 weight rows; wavefront w takes the runs of 256 codes w, w + NW, ... of all of them.
+//   * A load instruction covers whole 128-byte lines (a run of 256 codes) of 8 rows; two DPP moves per register pair
+//     bring two such loads into the shape "lane (n = lane % 16, p = lane / 16) holds bytes 16 p .. 16 p + 15 of a
+//     64-byte block of row n".  The MFMA wants from lane (n, q) the eight codes 8 q .. 8 q + 7 of a run of 32, i.e. word
+//     q of four consecutive words: the four registers are transposed across the four 16-lane blocks (four lane swaps
+//     per 16 bytes), after which register i of a block of 128 codes is the B operand of its step i (codes 32 i ..
+//     32 i + 31), expanded with one v_and_or_b32 per pair of codes.
+//   * x is read a whole 128-byte line of each of 8 tokens per instruction: lanes i = lane % 16 < 8 take the first 64
+//     bytes of token i (an even step), lanes i >= 8 the second 64 bytes of token i - 8 (the odd step behind it); a
+//     second instruction does the same for tokens 8..15, and two DPP moves per register pair put the halves where the
+//     A operands want them.  Inside the 16 bytes the values are permuted into the order the expansion leaves the codes
+//     in.  Every wavefront reads just the runs it multiplies.  (Requests are what this kernel pays for at the L1: with
+//     64 bytes of 16 tokens per instruction, and every wavefront fetching its own 8 bytes of each row's scales and
+//     biases, x and the scales each cost as much time as the weights.)
+//   * scales and biases of the workgroup's rows are fetched once, whole rows by all threads together, and handed round
+//     in LDS.
+//   * two steps make a quantisation group: acc += scale * D, four FMAs per lane, group and set of rows.
+//   * the affine term is one MFMA per run and set of rows: lane block q carries group q of the run, A = the three-way
+//     bf16 split of the group's sum of x (and -128 times it), B = (b b b s s s 0 0); the sums of x come from v_dot2
+//     per lane and a 4 x 4 transpose-add over the lane blocks, which leaves group q's total in block q.
+//   * the wavefronts' partial sums meet in LDS; with sixteen wavefronts of at most 128 registers a SIMD holds four, whose
+//     loads, lane swaps, expansions and MFMAs overlap.
+// Token t of an M-row call equals token t of any other call on the same variant, bit for bit.
+template <int NW, int RS, int QW, int RING>
+__global__ __launch_bounds__(NW* kWave) void qmv_tok16_kernel(const QmvArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    constexpr int ROWS = RS * 16;   // weight rows per workgroup
+    constexpr int TSTRIDE = ROWS;   // floats between tokens in the LDS partials
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15;
+    const int q = lane >> 4;
+    const int K = a.K, N = a.N, M = a.M;
+    const int groups = K >> 6;
+    const int quads = K >> 8;
+    const int row0 = (int)blockIdx.x * ROWS;
+
+    const gptr_t wg = uniform_ptr(a.w), sg = uniform_ptr(a.s), bg = uniform_ptr(a.b), xg = uniform_ptr(a.x);
+    // weights: lane (i, q) of load `ab` reads row (i % 8) + 8 ab of a set, bytes 64 (i / 8) + 16 q of the run's 128: an
+    // instruction covers whole 128-byte lines of 8 rows
+    uint32_t w_lane[RS][2];
+#pragma unroll
+    for (int rs = 0; rs < RS; rs++)
+#pragma unroll
+        for (int ab = 0; ab < 2; ab++) {
+            const int row = min(row0 + rs * 16 + (n & 7) + 8 * ab, N - 1);  // past N: a valid row, never stored
+            w_lane[rs][ab] = (uint32_t)row * (uint32_t)(K >> 1) + (uint32_t)(n >> 3) * 64u + (uint32_t)q * 16u;
+        }
+    // x: lane (i, q) of load `ab` reads token (i % 8) + 8 ab, bytes 64 (i / 8) + 16 q of a 128-byte step pair
+    uint32_t x_lane[2];
+#pragma unroll
+    for (int ab = 0; ab < 2; ab++)
+        x_lane[ab] = (uint32_t)min((n & 7) + 8 * ab, M - 1) * (uint32_t)K * 2u + (uint32_t)(n >> 3) * 64u + (uint32_t)q * 16u;
+
+    const uint32_t mask = opaque_s(kNibbleMask);
+    const uint32_t magic = opaque_v(kMagic128);
+    const uint32_t ones = 0x3f803f80u;
+    // picks element q of four bf16 values in two registers, twice
+    const uint32_t sel_q = 0x01000100u + 0x02020202u * (uint32_t)q;
+
+    auto transpose = [](uint32_t& s0, uint32_t& s1, uint32_t& s2, uint32_t& s3) {
+        const auto p = __builtin_amdgcn_permlane16_swap(s0, s1, false, false);
+        const auto r = __builtin_amdgcn_permlane16_swap(s2, s3, false, false);
+        const auto e = __builtin_amdgcn_permlane32_swap(p[0], r[0], false, false);
+        const auto o = __builtin_amdgcn_permlane32_swap(p[1], r[1], false, false);
+        s0 = e[0];
+        s1 = o[0];
+        s2 = e[1];
+        s3 = o[1];
+    };
+
+    f32x4_t acc[RS];
+#pragma unroll
+    for (int rs = 0; rs < RS; rs++) acc[rs] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+    uint4* const sbq = reinterpret_cast<uint4*>(lds_raw);
+    const int sb_pitch = quads + 1;
+
+    // Scales and biases of the workgroup's rows: fetched once by all threads together, whole rows (every wavefront
+    // fetching its own 8 bytes per row and run cost as much time as the weights), into LDS as (s0 s1, s2 s3, b0 b1,
+    // b2 b3) per row and run; rows are a run apart plus 16 bytes, so that the 16 rows a wavefront reads at once fall into
+    // different banks.  The loads go out first, the first pass's x and weights behind them, and only then are they stored.
+    constexpr int NT = NW * kWave;
+    constexpr int PRE = tok16_stage_pieces(NW);
+    const int pieces = ROWS * quads;
+    uint2 sv[PRE], bv[PRE];
+#pragma unroll
+    for (int i = 0; i < PRE; i++) {
+        const int p = tid + i * NT;
+        if (p < pieces) {
+            const int r = p / quads, c = p - r * quads;
+            const uint32_t at = (uint32_t)min(row0 + r, N - 1) * (uint32_t)groups * 2u + (uint32_t)c * 8u;
+            sv[i] = load_u64_at(sg, at);
+            bv[i] = load_u64_at(bg, at);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // A pass: QW runs of this wavefront (NW runs apart), their A operands in registers, and the RS sets of rows streamed
+    // past them one set at a time through a ring of RING register slots.  Loads return in the order they were issued, and
+    // requests that are out at the same time come back in the order the memory likes, not in the order they are needed:
+    // a set is therefore requested only RING sets ahead of its use, which keeps HBM busy during the arithmetic without
+    // making the first set wait for the last.
+    uint4 ring[RING][QW][2];
+    auto issue_set = [&](auto slot_tag, int rs_dyn, const int (&qds)[QW]) {
+        constexpr int SL = decltype(slot_tag)::value;
+#pragma unroll
+        for (int j = 0; j < QW; j++)
+#pragma unroll
+            for (int ab = 0; ab < 2; ab++) {
+                uint32_t base = 0;
+#pragma unroll
+                for (int rs = 0; rs < RS; rs++) base = rs == rs_dyn ? w_lane[rs][ab] : base;
+                ring[SL][j][ab] = load_u128_at(wg, base + (uint32_t)qds[j] * 128u);
+            }
+    };
+    bool staged = false;
+    for (int qbase = wave; qbase < quads; qbase += NW * QW) {
+        int qds[QW];   // clamped: a run past the end of K is loaded from the last run and not used
+        bool live[QW];
+#pragma unroll
+        for (int j = 0; j < QW; j++) {
+            live[j] = qbase + j * NW < quads;
+            qds[j] = live[j] ? qbase + j * NW : qbase;
+        }
+        uint4 xa[QW][4], xb[QW][4];
+#pragma unroll
+        for (int j = 0; j < QW; j++)
+#pragma unroll
+            for (int sp = 0; sp < 4; sp++) {
+                xa[j][sp] = load_u128_at(xg, x_lane[0] + (uint32_t)qds[j] * 512u + (uint32_t)sp * 128u);
+                xb[j][sp] = load_u128_at(xg, x_lane[1] + (uint32_t)qds[j] * 512u + (uint32_t)sp * 128u);
+            }
+        __builtin_amdgcn_sched_barrier(0);
+        issue_set(std::integral_constant<int, 0>{}, 0, qds);
+        if constexpr (RING > 1 && RS > 1) issue_set(std::integral_constant<int, 1 % RING>{}, 1, qds);
+        if constexpr (RING > 2 && RS > 2) issue_set(std::integral_constant<int, 2 % RING>{}, 2, qds);
+        __builtin_amdgcn_sched_barrier(0);
+        if (!staged) {
+#pragma unroll
+            for (int i = 0; i < PRE; i++) {
+                const int p = tid + i * NT;
+                if (p < pieces) {
+                    const int r = p / quads, c = p - r * quads;
+                    sbq[r * sb_pitch + c] = make_uint4(sv[i].x, sv[i].y, bv[i].x, bv[i].y);
+                }
+            }
+            __syncthreads();
+            staged = true;
+        }
+
+        // A operands of the pass's runs, and per run the three-way split of the lane block's group sum of x
+        bf16x8_t af[QW][8], a2[QW];
+#pragma unroll
+        for (int j = 0; j < QW; j++) {
+            float ps[4];
+#pragma unroll
+            for (int st = 0; st < 8; st++) {
+                // even step: lanes i >= 8 take tokens 8..15 from the second load's lanes i - 8; odd step: lanes i < 8 take
+                // tokens 0..7 from the first load's lanes i + 8
+                const uint4 va = xa[j][st >> 1], vb = xb[j][st >> 1];
+                uint4 v;
+                if ((st & 1) == 0) {
+                    v.x = __builtin_amdgcn_update_dpp(va.x, vb.x, 0x118, 0xf, 0xc, false);
+                    v.y = __builtin_amdgcn_update_dpp(va.y, vb.y, 0x118, 0xf, 0xc, false);
+                    v.z = __builtin_amdgcn_update_dpp(va.z, vb.z, 0x118, 0xf, 0xc, false);
+                    v.w = __builtin_amdgcn_update_dpp(va.w, vb.w, 0x118, 0xf, 0xc, false);
+                } else {
+                    v.x = __builtin_amdgcn_update_dpp(vb.x, va.x, 0x108, 0xf, 0x3, false);
+                    v.y = __builtin_amdgcn_update_dpp(vb.y, va.y, 0x108, 0xf, 0x3, false);
+                    v.z = __builtin_amdgcn_update_dpp(vb.z, va.z, 0x108, 0xf, 0x3, false);
+                    v.w = __builtin_amdgcn_update_dpp(vb.w, va.w, 0x108, 0xf, 0x3, false);
+                }
+                af[j][st] = as_bf16x8(__builtin_amdgcn_perm(v.z, v.x, 0x05040100u), __builtin_amdgcn_perm(v.z, v.x, 0x07060302u),
+                                      __builtin_amdgcn_perm(v.w, v.y, 0x05040100u), __builtin_amdgcn_perm(v.w, v.y, 0x07060302u));
+                float hs = (st & 1) ? ps[st >> 1] : 0.0f;
+                hs = dot2_bf16(v.x, ones, hs);
+                hs = dot2_bf16(v.y, ones, hs);
+                hs = dot2_bf16(v.z, ones, hs);
+                hs = dot2_bf16(v.w, ones, hs);
+                ps[st >> 1] = hs;
+            }
+            // block q of register g holds lane block q's share of group g; transposed, the four registers of block q are
+            // the four shares of group q
+            uint32_t t0 = __float_as_uint(ps[0]), t1 = __float_as_uint(ps[1]), t2 = __float_as_uint(ps[2]), t3 = __float_as_uint(ps[3]);
+            transpose(t0, t1, t2, t3);
+            float X = (__uint_as_float(t0) + __uint_as_float(t1)) + (__uint_as_float(t2) + __uint_as_float(t3));
+            if (!live[j]) X = 0.0f;
+            const uint32_t u0 = __float_as_uint(X) & 0xffff0000u;
+            const float r1 = X - __uint_as_float(u0);
+            const uint32_t u1 = __float_as_uint(r1) & 0xffff0000u;
+            const float r2 = r1 - __uint_as_float(u1);
+            const uint32_t u2 = __float_as_uint(r2) & 0xffff0000u;
+            const uint32_t m0 = __float_as_uint(-128.0f * __uint_as_float(u0));
+            const uint32_t m1 = __float_as_uint(-128.0f * __uint_as_float(u1));
+            const uint32_t m2 = __float_as_uint(-128.0f * __uint_as_float(u2));
+            a2[j] = as_bf16x8((u0 >> 16) | u1, (u2 >> 16) | m0, (m1 >> 16) | m2, 0u);
+        }
+
+        auto run_set = [&](auto rs_tag) {
+            constexpr int rs = decltype(rs_tag)::value;
+            constexpr int SL = rs % RING;
+#pragma unroll
+            for (int j = 0; j < QW; j++) {
+                // first 64 bytes of all 16 rows (lanes i >= 8 from the second load's lanes i - 8), second 64 bytes (lanes
+                // i < 8 from the first load's lanes i + 8): as for x
+                const uint4 la = ring[SL][j][0], lb = ring[SL][j][1];
+                uint32_t f0 = __builtin_amdgcn_update_dpp(la.x, lb.x, 0x118, 0xf, 0xc, false);
+                uint32_t f1 = __builtin_amdgcn_update_dpp(la.y, lb.y, 0x118, 0xf, 0xc, false);
+                uint32_t f2 = __builtin_amdgcn_update_dpp(la.z, lb.z, 0x118, 0xf, 0xc, false);
+                uint32_t f3 = __builtin_amdgcn_update_dpp(la.w, lb.w, 0x118, 0xf, 0xc, false);
+                uint32_t g0 = __builtin_amdgcn_update_dpp(lb.x, la.x, 0x108, 0xf, 0x3, false);
+                uint32_t g1 = __builtin_amdgcn_update_dpp(lb.y, la.y, 0x108, 0xf, 0x3, false);
+                uint32_t g2 = __builtin_amdgcn_update_dpp(lb.z, la.z, 0x108, 0xf, 0x3, false);
+                uint32_t g3 = __builtin_amdgcn_update_dpp(lb.w, la.w, 0x108, 0xf, 0x3, false);
+                transpose(f0, f1, f2, f3);
+                transpose(g0, g1, g2, g3);
+                const uint32_t ww[8] = {f0, f1, f2, f3, g0, g1, g2, g3};
+                const uint4 sbv = sbq[(rs * 16 + n) * sb_pitch + qds[j]];
+                f32x4_t part = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    f32x4_t d = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                    for (int half = 0; half < 2; half++) {
+                        uint32_t e[4];
+                        unpack4_word(ww[2 * g + half], mask, magic, e);
+                        d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[j][2 * g + half], as_bf16x8(e[0], e[1], e[2], e[3]), d, 0, 0, 0);
+                    }
+                    const uint32_t sw = g < 2 ? sbv.x : sbv.y;
+                    const float sc = (g & 1) ? __uint_as_float(sw & 0xffff0000u) : __uint_as_float(sw << 16);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) part[r] = __builtin_fmaf(sc, d[r], part[r]);
+                }
+                const uint32_t bb = __builtin_amdgcn_perm(sbv.w, sbv.z, sel_q);
+                const uint32_t ss = __builtin_amdgcn_perm(sbv.y, sbv.x, sel_q);
+                const bf16x8_t b2 = as_bf16x8(bb, __builtin_amdgcn_perm(ss, bb, 0x05040100u), ss, 0u);
+                part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2[j], b2, part, 0, 0, 0);
+                // a run past the end of K (x and weights of the last run were loaded in its place) adds nothing
+                if (live[j]) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) acc[rs][r] += part[r];
+                }
+            }
+            if constexpr (rs + RING < RS) {
+                __builtin_amdgcn_sched_barrier(0);
+                issue_set(std::integral_constant<int, SL>{}, rs + RING, qds);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        run_set(std::integral_constant<int, 0>{});
+        if constexpr (RS > 1) run_set(std::integral_constant<int, 1>{});
+        if constexpr (RS > 2) run_set(std::integral_constant<int, 2>{});
+        if constexpr (RS > 3) run_set(std::integral_constant<int, 3>{});
+        static_assert(RS <= 4, "sets of rows per workgroup");
+    }
+    if (!staged) __syncthreads();  // a wavefront without a run of its own
+
+    // ---- the wavefronts' partial sums meet in LDS: red[wave][token][row]; thread (token, row) adds them in wave order ----
+    // (behind the staged scales and biases: a wavefront may get here while another still reads those)
+    float* red = reinterpret_cast<float*>(lds_raw + (size_t)ROWS * sb_pitch * 16);
+    // D layout of the 16x16 MFMA: lane (n, q), register r -> token 4 q + r, weight row n
+#pragma unroll
+    for (int rs = 0; rs < RS; rs++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) red[(wave * 16 + 4 * q + r) * TSTRIDE + rs * 16 + n] = acc[rs][r];
+    __syncthreads();
+    for (int o = tid; o < 16 * ROWS; o += NW * kWave) {
+        const int t = o / ROWS, rl = o - t * ROWS;
+        float total = red[t * TSTRIDE + rl];
+#pragma unroll
+        for (int p = 1; p < NW; p++) total += red[(p * 16 + t) * TSTRIDE + rl];
+        const int row = row0 + rl;
+        if (t < M && row < N) {
+            const size_t at = (size_t)t * N + row;
+            if (a.out_f32) {
+                static_cast<float*>(a.y)[at] = total;
+            } else {
+                static_cast<uint16_t*>(a.y)[at] = f32_to_bf16_bits(total);
+            }
+        }
+    }
+}
+
 // ---- variant table --------------------------------------------------------
 
 typedef void (*QmvTokKernel)(const QmvArgs);
 struct QmvTokEntry {
-    QmvVariant v;  // m = most activation rows, rows = sets of 32 weight rows per wavefront, waves = wavefronts that share K
+    QmvVariant v;  // m = most activation rows, rows = sets of weight rows per wavefront, waves = wavefronts that share K
+                   // (16-token form: depth = sets of rows in flight, xmode = runs of 256 codes a wavefront holds per pass)
     QmvTokKernel fn;
+    int wg_rows;  // weight rows per workgroup
+    int lds;      // bytes
 };
 #define AQ_QMVT(NW, R)                                                                               \
     {                                                                                                \
-        {"qmvt_b4_m32_r" #R "_w" #NW, 4, kTokMax, R, NW, 4, 0, 0, 6}, qmv_tok_kernel<NW, R>          \
+        {"qmvt_b4_m32_r" #R "_w" #NW, 4, kTokMax, R, NW, 4, 0, 0, 6}, qmv_tok_kernel<NW, R>,         \
+            kTokRows * R, NW * R * 16 * 64 * 4                                                       \
     }
-static const QmvTokEntry kQmvTokTable[] = {AQ_QMVT(8, 2), AQ_QMVT(8, 1), AQ_QMVT(4, 1), AQ_QMVT(4, 2)};
+#define AQ_QMVT16(NW, RS, QW, RING)                                                                       \
+    {                                                                                                     \
+        {"qmvt_b4_m16_r" #RS "_w" #NW "_q" #QW "_d" #RING, 4, 16, RS, NW, RING, 0, QW, 6},                 \
+            qmv_tok16_kernel<NW, RS, QW, RING>, 16 * RS, NW * 16 * (16 * RS) * 4                          \
+    }
+static const QmvTokEntry kQmvTokTable[] = {AQ_QMVT(8, 2), AQ_QMVT(8, 1), AQ_QMVT(4, 1), AQ_QMVT(4, 2),
+                                           AQ_QMVT16(8, 4, 1, 2), AQ_QMVT16(8, 2, 1, 2), AQ_QMVT16(8, 1, 1, 1),
+                                           AQ_QMVT16(16, 4, 1, 3), AQ_QMVT16(8, 4, 2, 2)};
 
 int qmvt_variant_count() { return (int)(sizeof(kQmvTokTable) / sizeof(kQmvTokTable[0])); }
 const QmvVariant* qmvt_variant(int idx) {
@@ -349,19 +651,24 @@ bool qmvt_fits(const QmvArgs& a, int bits, int group_size, int idx) {
     if ((al16 & 15) || (al8 & 7)) return false;
     // 32-bit byte offsets into the packed matrix and into x
     if ((uint64_t)a.N * (uint64_t)(a.K / 2) >= (1ull << 32)) return false;
+    // the 16-token form keeps its rows' scales and biases in LDS next to the partial sums
+    if (v->m == 16 && ((size_t)kQmvTokTable[idx].lds + (size_t)kQmvTokTable[idx].wg_rows * (a.K / 256 + 1) * 16 > 160 * 1024 ||
+                       kQmvTokTable[idx].wg_rows * (a.K / 256) > tok16_stage_pieces(v->waves) * v->waves * kWave))
+        return false;
     return true;
 }
 
 hipError_t qmvt_launch(int idx, const QmvArgs& a, hipStream_t stream) {
     if (idx < 0 || idx >= qmvt_variant_count()) return hipErrorInvalidValue;
     const QmvTokEntry& e = kQmvTokTable[idx];
-    const size_t lds = (size_t)e.v.waves * e.v.rows * 16 * 64 * 4;
+    // the 16-token form also stages 16 bytes of scales and biases per row and run of 256 codes (rows a run apart plus 16 bytes)
+    const size_t lds = (size_t)e.lds + (e.v.m == 16 ? (size_t)e.wg_rows * (a.K / 256 + 1) * 16 : 0);
     if (lds > 48 * 1024) {
         hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e.fn), hipFuncAttributeMaxDynamicSharedMemorySize,
                                             (int)lds);
         if (rc != hipSuccess) return rc;
     }
-    const int wg_rows = kTokRows * e.v.rows;
+    const int wg_rows = e.wg_rows;
     hipLaunchKernelGGL(e.fn, dim3((unsigned)((a.N + wg_rows - 1) / wg_rows)), dim3((unsigned)(e.v.waves * kWave)), lds, stream, a);
     return hipGetLastError();
 }
@@ -371,12 +678,21 @@ hipError_t qmvt_launch(int idx, const QmvArgs& a, hipStream_t stream) {
 int qmvt_pick(int M, int K, int N, int cu_count) {
     if (M < 1 || M > kTokMax || K < 256 || K % 256 != 0) return -1;
     const int quads = K / 256;
-    const int nw = quads >= 8 ? 8 : 4;
     const int cus = cu_count > 0 ? cu_count : 256;
+    if (M <= 16 && K <= 16384) {
+        // the 16-token form: eight wavefronts, one run each per pass; as many sets of 16 rows per workgroup (fewer reads
+        // of x) as still leave three quarters of the CUs a workgroup
+        const int rs = (N + 63) / 64 >= (cus * 3) / 4 ? 4 : (N + 31) / 32 >= (cus * 3) / 4 ? 2 : 1;
+        for (int i = 0; i < qmvt_variant_count(); i++) {
+            const QmvVariant& v = kQmvTokTable[i].v;
+            if (v.m == 16 && v.waves == 8 && v.rows == rs && v.xmode == 1) return i;
+        }
+    }
+    const int nw = quads >= 8 ? 8 : 4;
     const int r = (N + 63) / 64 >= (cus * 3) / 4 ? 2 : 1;
     for (int i = 0; i < qmvt_variant_count(); i++) {
         const QmvVariant& v = kQmvTokTable[i].v;
-        if (v.waves == nw && v.rows == r) return i;
+        if (v.m == kTokMax && v.waves == nw && v.rows == r) return i;
     }
     return -1;
 }

@@ -16,14 +16,18 @@ CASES = [
     (4, 64, 1, 4096, ("qmvd_",)),                    # diagonal MFMA: one row, K up to 16 steps of 1024
     (4, 64, 1, 14336, ("qmvd_",)),
     (4, 64, 8, 4096, ("qmvd_",)),                    # ... up to 8 rows at 2..4 steps
+    (4, 64, 8, 4096 - 128, ("qmvd_",)),
+    (4, 64, 16, 14336, ("qmvt_b4_m16_",)),           # token tile, 16-token form: 9..16 rows, K a multiple of 256
     (4, 32, 2, 1536, ("qmvd_",)),                    # groups of 32
     (8, 64, 8, 4096, ("qmvd8_",)),                   # 8-bit MFMA: 5..16 rows
     (8, 64, 16, 4096, ("qmvd8_",)),
-    (4, 64, 9, 4096, ("qmvt_",)),                    # token tile: 9..32 rows, K a multiple of 256
-    (4, 64, 32, 4096, ("qmvt_",)),
+    (4, 64, 9, 4096, ("qmvt_b4_m16_",)),
+    (4, 64, 17, 4096, ("qmvt_b4_m32_",)),            # token tile, 32-token form: 17..32 rows
+    (4, 64, 32, 4096, ("qmvt_b4_m32_",)),
     (8, 64, 1, 4096, ("qmvb_",)),                    # block MFMA: one row of 8-bit codes
     (8, 64, 4, 4096, ("qmvb_",)),                    # ... and 2..4 rows
-    (4, 64, 8, 14336, ("qmvb_", "qmmf_", "qmmt_")),  # 5..8 rows at a K the diagonal kernels take for one row only
+    (4, 64, 8, 14336, ("qmvt_b4_m16_",)),            # 5..8 rows at a K the diagonal kernels take for one row only
+    (4, 64, 8, 14336 + 128, ("qmvb_", "qmmf_", "qmmt_")),
     (4, 128, 1, 4096, ("qmv_b4_",)),                 # dot2: groups of 128
     (4, 64, 1, 2880, ("qmv_b4_",)),                  # dot2: K = 45 groups
     (4, 64, 3, 2880, ("qmvb_", "qmv_b4_")),
