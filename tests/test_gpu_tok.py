@@ -1,4 +1,4 @@
-"""The token-tile MFMA matvec kernels (5..32 rows of x as the rows of a 32x32x16 MFMA, one launch, no scratch):
+"""The token-tile MFMA matvec kernels (5..32 rows of x as the rows of 16x16x32 MFMAs, one launch, no scratch):
 the M-row contract of go/engine/metal/qmv_rows.go:14-60 and rocm_mlx_q4_projection_batch*
 (go/engine/hip/kernels/quant/affine_projection_tuned.hipinc:292-472) beyond eight rows."""
 import numpy as np
@@ -16,9 +16,10 @@ def _tok_variants():
 
 
 def test_tok_every_variant(ctx, orc):
-    """Each variant forced: 1..32 rows, K of one run of four groups up to several per wavefront (an idle wavefront, a
-    ragged split), N that ends inside a set of 32 rows; fp32 accumulators and bf16 stores; token t of an M-row call is
-    bit-identical to token t of any other row count; 33 rows, a K that is no multiple of 256, 8-bit codes are refused."""
+    """Each variant forced: 1..32 rows (16 for the one-set forms), K of one run of four groups up to several per
+    wavefront (an idle wavefront, a ragged split), N that ends inside a set of 16 rows; fp32 accumulators and bf16
+    stores; token t of an M-row call is bit-identical to token t of any other row count; 33 rows, a K that is no multiple
+    of 256, a K beyond 16384, 8-bit codes are refused."""
     import aq_mi355
     N = 150
     try:
@@ -30,7 +31,7 @@ def test_tok_every_variant(ctx, orc):
             for idx, name in _tok_variants():
                 ctx.force_variant(0, idx)
                 full = None
-                most = int(name.split("_m")[1].split("_")[0])  # rows of x the variant takes: 32, or 16 for the 16x16 MFMA form
+                most = int(name.split("_m")[1].split("_")[0])  # rows of x the variant takes: 16, or 32 for the two-set forms
                 for rows in [r for r in (most, 1, 5, 9, 16, 17, 31) if r <= most]:
                     say("tok variant", name, "K", K, "rows", rows)
                     acc = run_qmv(ctx, x[:rows], dw, rows, K, N, 64, 4, True)
@@ -44,11 +45,11 @@ def test_tok_every_variant(ctx, orc):
                 check_bf16_store(out, ref[:some], name)
                 assert np.array_equal(out, F.f32_to_bf16_bits(full[:some]).reshape(some, N))
             dw.free()
-        idx, name = _tok_variants()[0]
+        idx, name = [v for v in _tok_variants() if "_m32_" in v[1]][0]
         ctx.force_variant(0, idx)
-        words, s, b = F.synthetic_affine(40, 1024, 4, 64, seed=1700)
+        words, s, b = F.synthetic_affine(40, 16640, 4, 64, seed=1700)
         dw = DeviceAffine(ctx, words, s, b)
-        for rows, K, bits in ((33, 1024, 4), (4, 1152, 4), (4, 1024, 8)):
+        for rows, K, bits in ((33, 1024, 4), (4, 1152, 4), (4, 1024, 8), (4, 16640, 4)):
             with pytest.raises(aq_mi355.AqError) as ei:
                 run_qmv(ctx, np.zeros((rows, K), np.uint16), dw, rows, K, 40, 64, bits, True)
             assert ei.value.code == aq_mi355.AQ_ERR_ARG, (rows, K, bits)
