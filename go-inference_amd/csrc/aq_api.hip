@@ -138,7 +138,7 @@ int pick_qmv_variant(const aq_ctx* ctx, int bits, int m, bool gather, int N, int
 
 // Families with variants of their own.  aq_variant_name(0, i) and aq_force_variant(ctx, 0, i) index the
 // concatenation of their tables, in this order.
-enum { kFamDot2, kFamBlk, kFamDiag, kFamTok, kFamD8, kFamCount };
+enum { kFamDot2, kFamBlk, kFamDiag, kFamTok, kFamCount };
 // Two more take part in the selection: the tile kernels of the matmul path (their variants are those of op 1)
 // and the kernel that takes any geometry.
 enum { kFamTiles = kFamCount, kFamTilesLarge, kFamGeneric };
@@ -152,7 +152,6 @@ const QmvFamily kQmvFamilies[kFamCount] = {
     {aq::qmvb_variant_count, aq::qmvb_variant},    // block-MFMA kernels (aq_qmv_blk.hip)
     {aq::qmvd_variant_count, aq::qmvd_variant},    // diagonal-MFMA kernels (aq_qmv_diag.hip)
     {aq::qmvt_variant_count, aq::qmvt_variant},    // token-tile MFMA kernels (aq_qmv_tok.hip)
-    {aq::qmvd8_variant_count, aq::qmvd8_variant},  // 8-bit MFMA kernels (aq_qmv_d8.hip)
 };
 
 int qmv_total_variants() {
@@ -198,8 +197,10 @@ const QmvRule kQmvRules[] = {
     {4, 64, 0, 1, 8, kFamDiag},             // one row up to 16 steps of 1024 codes, up to 8 rows at 2..4 steps: every row
                                             // of such a call has the bytes of a call with that row alone
     {4, 32, 0, 1, 2, kFamDiag},             // groups of 32: two tokens x eight groups as MFMA rows
-    {8, 64, 0, 5, 16, kFamD8},              // (up to 4 rows the block-MFMA kernels measure the same or faster)
-    {4, 64, 0, 5, 32, kFamTok},             // K a multiple of 256: one launch, weights streamed once, no scratch
+    {8, 64, 0, 5, 16, kFamTok},             // K a multiple of 256 up to 16384: one launch, weights streamed once, no scratch
+                                            // (up to 4 rows the block-MFMA kernels stay: 14.2 / 15.9 against 14.9 / 14.8 us for
+                                            // 1 / 4 rows of 4096 x 14336, and their rows have the bytes of single-row calls)
+    {4, 64, 0, 5, 32, kFamTok},             // the same for 4-bit codes, up to 32 rows
                                             // (5..8 rows: only where the diagonal kernels passed; they measure 11.2 us
                                             // against 14.4 us at 8 rows of 4096 x 14336, but not row by row the same bytes)
     {0, 0, 0, 9, 64, kFamTilesLarge},       // 16 Mi codes and more: the 16-row block-MFMA kernel is bound by its 4x4x4 MFMAs
@@ -258,18 +259,10 @@ int run_diag(aq_ctx* ctx, const aq::QmvArgs& a, int group_size, int bits, bool g
 }
 
 int run_tok(aq_ctx* ctx, const aq::QmvArgs& a, int group_size, int bits, bool gather, int forced) {
-    const int ti = forced >= 0 ? forced : aq::qmvt_pick(a.M, a.K, a.N, ctx->cu_count);
+    const int ti = forced >= 0 ? forced : aq::qmvt_pick(bits, a.M, a.K, a.N, ctx->cu_count);
     if (gather || ti < 0 || !aq::qmvt_fits(a, bits, group_size, ti)) return kPass;
     ctx->last_variant[0] = aq::qmvt_variant(ti)->name;
     AQ_HIP(aq::qmvt_launch(ti, a, ctx->stream), "hipLaunchKernel");
-    return AQ_OK;
-}
-
-int run_d8(aq_ctx* ctx, const aq::QmvArgs& a, int group_size, int bits, bool gather, int forced) {
-    const int ei = forced >= 0 ? forced : aq::qmvd8_pick(a.M, a.K, a.N);
-    if (gather || ei < 0 || !aq::qmvd8_fits(a, bits, group_size, ei)) return kPass;
-    ctx->last_variant[0] = aq::qmvd8_variant(ei)->name;
-    AQ_HIP(aq::qmvd8_launch(ei, a, ctx->stream), "hipLaunchKernel");
     return AQ_OK;
 }
 
@@ -293,7 +286,6 @@ int run_family(int family, aq_ctx* ctx, const aq::QmvArgs& a, int group_size, in
         case kFamBlk: return run_blk(ctx, a, group_size, bits, gather, forced);
         case kFamDiag: return run_diag(ctx, a, group_size, bits, gather, forced);
         case kFamTok: return run_tok(ctx, a, group_size, bits, gather, forced);
-        case kFamD8: return run_d8(ctx, a, group_size, bits, gather, forced);
         case kFamTiles: return run_tiles(ctx, a, group_size, bits, false);
         case kFamTilesLarge: return run_tiles(ctx, a, group_size, bits, true);
         default: return run_generic(ctx, a, group_size, bits, gather);

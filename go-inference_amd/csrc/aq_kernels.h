@@ -86,8 +86,7 @@ struct QmvVariant {
                  // 2: block-MFMA kernel (aq_qmv_blk.hip; m = most rows, depth = K pieces per wavefront),
                  // 4: diagonal-MFMA kernel (aq_qmv_diag.hip; m = most rows, rows = sets of 16 rows per workgroup,
                  //    xmode = chunks per step when not 4), 5: the same for quantisation groups of 32 codes
-                 // 6: token-tile MFMA kernel (aq_qmv_tok.hip; m = most rows, rows = sets of 32 weight rows per wavefront)
-                 // 7: 8-bit MFMA kernel (aq_qmv_d8.hip; m = most rows, rows = sets of 16 rows per workgroup)
+                 // 6: token-tile MFMA kernel (aq_qmv_tok.hip; m = most rows, rows = sets of 16 weight rows per workgroup)
 };
 
 int qmv_variant_count();
@@ -151,21 +150,13 @@ hipError_t head_fold_launch(const unsigned long long* partial, int count, unsign
 bool qmvd_multi_supported(int idx);
 hipError_t qmvd_multi_launch(int idx, QmvMultiArgs ma, hipStream_t stream);
 
-// Token-tile MFMA matvec kernels (aq_qmv_tok.hip; 4-bit group-64 codes, up to 32 activation rows as the rows of a
-// 32x32x16 MFMA, K a multiple of 256; one launch, no scratch memory).  kind 6 in QmvVariant.
+// Token-tile MFMA matvec kernels (aq_qmv_tok.hip; group-64 codes, 4 bit up to 32 and 8 bit up to 16 activation rows as
+// the rows of 16x16x32 MFMAs, K a multiple of 256 up to 16384; one launch, no scratch memory).  kind 6 in QmvVariant.
 int qmvt_variant_count();
 const QmvVariant* qmvt_variant(int idx);
 bool qmvt_fits(const QmvArgs& a, int bits, int group_size, int idx);
 hipError_t qmvt_launch(int idx, const QmvArgs& a, hipStream_t stream);
-int qmvt_pick(int M, int K, int N, int cu_count);
-
-// MFMA matvec kernels for 8-bit codes (aq_qmv_d8.hip; group 64, up to 16 rows of x as the rows of a 16x16x32 MFMA, K a
-// multiple of 256 up to 16384).  kind 7 in QmvVariant.
-int qmvd8_variant_count();
-const QmvVariant* qmvd8_variant(int idx);
-bool qmvd8_fits(const QmvArgs& a, int bits, int group_size, int idx);
-hipError_t qmvd8_launch(int idx, const QmvArgs& a, hipStream_t stream);
-int qmvd8_pick(int M, int K, int N);
+int qmvt_pick(int bits, int M, int K, int N, int cu_count);
 
 // lm_head kernels (aq_qmv_head.hip), one activation row: the projection with its epilogue replaced by
 //   fuse 3: best[0] = max over rows of pack(score, row): every wavefront stores its own maximum into

@@ -1,5 +1,5 @@
-// affine_qmv for 5..32 rows of x on gfx950 (batched / speculative-verify decode), 4-bit codes in groups of 64:
-// one launch, the weights streamed exactly once, no pass over x beforehand and no partial tiles in memory.
+// affine_qmv for 5..32 rows of x on gfx950 (batched / speculative-verify decode), 4-bit (8-bit: up to 16 rows) codes in
+// groups of 64: one launch, the weights streamed exactly once, no pass over x beforehand and no partial tiles in memory.
 //
 // Same contract as the other matvec kernels: replaces rocm_mlx_q4_projection_batch*
 // (go/engine/hip/kernels/quant/affine_projection_tuned.hipinc:292-472, 16 rows x 16 tokens in one launch) and the
@@ -67,8 +67,15 @@ __host__ __device__ constexpr int tok16_stage_pieces(int nw) { return nw >= 16 ?
 //   * a wavefront keeps the A operands of its runs in registers and streams the sets of rows past them, RING sets in
 //     flight (see the loop); the wavefronts' partial sums meet in LDS.
 // Token t of an M-row call equals token t of any other call on the same variant, bit for bit.
-template <int NW, int RS, int QW, int RING, int TS>
+// 8-bit codes (BITS = 8): a run of 256 codes is two lines per row, four loads per set of rows; the 64 bytes a
+// 16-lane-block row holds after the DPP moves are one quantisation group, lane (n, p) has its codes 16 p .. 16 p + 15, and
+// the two halves of those are the B operands of the group's two steps as they lie (no transpose: which codes share a
+// step is free as long as x follows, and x is loaded to follow: lane (t, p) takes x[64 g + 16 p + 8 i ..] for step i);
+// codes become bf16 by v_cvt_f32_ubyte + v_perm (exact), in their natural order; the affine term is bias * sum(x) alone.
+template <int BITS, int NW, int RS, int QW, int RING, int TS>
 __global__ __launch_bounds__(NW* kWave) void qmv_tok16_kernel(const QmvArgs a) {
+    static_assert(BITS == 4 || BITS == 8, "code width");
+    constexpr int LINES = BITS / 4;  // 128-byte lines of a row per run of 256 codes
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     constexpr int ROWS = RS * 16;   // weight rows per workgroup
     constexpr int TSTRIDE = ROWS;   // floats between tokens in the LDS partials
@@ -91,7 +98,7 @@ __global__ __launch_bounds__(NW* kWave) void qmv_tok16_kernel(const QmvArgs a) {
 #pragma unroll
         for (int ab = 0; ab < 2; ab++) {
             const int row = min(row0 + rs * 16 + (n & 7) + 8 * ab, N - 1);  // past N: a valid row, never stored
-            w_lane[rs][ab] = (uint32_t)row * (uint32_t)(K >> 1) + (uint32_t)(n >> 3) * 64u + (uint32_t)q * 16u;
+            w_lane[rs][ab] = (uint32_t)row * (uint32_t)(K * BITS / 8) + (uint32_t)(n >> 3) * 64u + (uint32_t)q * 16u;
         }
     // x: lane (i, q) of load `ab` of token set ts reads token 16 ts + (i % 8) + 8 ab, bytes 64 (i / 8) + 16 q of a
     // 128-byte step pair (TS sets of 16 tokens share every expanded weight)
@@ -100,8 +107,9 @@ __global__ __launch_bounds__(NW* kWave) void qmv_tok16_kernel(const QmvArgs a) {
     for (int ts = 0; ts < TS; ts++)
 #pragma unroll
         for (int ab = 0; ab < 2; ab++)
-            x_lane[ts][ab] = (uint32_t)min(16 * ts + (n & 7) + 8 * ab, M - 1) * (uint32_t)K * 2u + (uint32_t)(n >> 3) * 64u +
-                             (uint32_t)q * 16u;
+            x_lane[ts][ab] = (uint32_t)min(16 * ts + (n & 7) + 8 * ab, M - 1) * (uint32_t)K * 2u +
+                             (BITS == 4 ? (uint32_t)(n >> 3) * 64u + (uint32_t)q * 16u   // step pair: first 64 bytes | second
+                                        : (uint32_t)q * 32u + (uint32_t)(n >> 3) * 16u);  // group: first 16 of the lane's 32 | second
 
     const uint32_t mask = opaque_s(kNibbleMask);
     const uint32_t magic = opaque_v(kMagic128);
@@ -154,18 +162,20 @@ __global__ __launch_bounds__(NW* kWave) void qmv_tok16_kernel(const QmvArgs a) {
     // requests that are out at the same time come back in the order the memory likes, not in the order they are needed:
     // a set is therefore requested only RING sets ahead of its use, which keeps HBM busy during the arithmetic without
     // making the first set wait for the last.
-    uint4 ring[RING][QW][2];
+    uint4 ring[RING][QW][LINES][2];
     auto issue_set = [&](auto slot_tag, int rs_dyn, const int (&qds)[QW]) {
         constexpr int SL = decltype(slot_tag)::value;
 #pragma unroll
         for (int j = 0; j < QW; j++)
 #pragma unroll
-            for (int ab = 0; ab < 2; ab++) {
-                uint32_t base = 0;
+            for (int ln = 0; ln < LINES; ln++)
 #pragma unroll
-                for (int rs = 0; rs < RS; rs++) base = rs == rs_dyn ? w_lane[rs][ab] : base;
-                ring[SL][j][ab] = load_u128_at(wg, base + (uint32_t)qds[j] * 128u);
-            }
+                for (int ab = 0; ab < 2; ab++) {
+                    uint32_t base = 0;
+#pragma unroll
+                    for (int rs = 0; rs < RS; rs++) base = rs == rs_dyn ? w_lane[rs][ab] : base;
+                    ring[SL][j][ln][ab] = load_u128_at(wg, base + (uint32_t)qds[j] * (uint32_t)(128 * LINES) + (uint32_t)ln * 128u);
+                }
     };
     bool staged = false;
     for (int qbase = wave; qbase < quads; qbase += NW * QW) {
@@ -228,8 +238,12 @@ __global__ __launch_bounds__(NW* kWave) void qmv_tok16_kernel(const QmvArgs a) {
                     v.z = __builtin_amdgcn_update_dpp(vb.z, va.z, 0x108, 0xf, 0x3, false);
                     v.w = __builtin_amdgcn_update_dpp(vb.w, va.w, 0x108, 0xf, 0x3, false);
                 }
-                af[ts][j][st] = as_bf16x8(__builtin_amdgcn_perm(v.z, v.x, 0x05040100u), __builtin_amdgcn_perm(v.z, v.x, 0x07060302u),
-                                      __builtin_amdgcn_perm(v.w, v.y, 0x05040100u), __builtin_amdgcn_perm(v.w, v.y, 0x07060302u));
+                if constexpr (BITS == 4) {  // the order the expansion leaves the codes of a word in: 0 4 1 5 2 6 3 7
+                    af[ts][j][st] = as_bf16x8(__builtin_amdgcn_perm(v.z, v.x, 0x05040100u), __builtin_amdgcn_perm(v.z, v.x, 0x07060302u),
+                                              __builtin_amdgcn_perm(v.w, v.y, 0x05040100u), __builtin_amdgcn_perm(v.w, v.y, 0x07060302u));
+                } else {
+                    af[ts][j][st] = as_bf16x8(v.x, v.y, v.z, v.w);
+                }
                 float hs = (st & 1) ? ps[st >> 1] : 0.0f;
                 hs = dot2_bf16(v.x, ones, hs);
                 hs = dot2_bf16(v.y, ones, hs);
@@ -248,9 +262,11 @@ __global__ __launch_bounds__(NW* kWave) void qmv_tok16_kernel(const QmvArgs a) {
             const uint32_t u1 = __float_as_uint(r1) & 0xffff0000u;
             const float r2 = r1 - __uint_as_float(u1);
             const uint32_t u2 = __float_as_uint(r2) & 0xffff0000u;
-            const uint32_t m0 = __float_as_uint(-128.0f * __uint_as_float(u0));
-            const uint32_t m1 = __float_as_uint(-128.0f * __uint_as_float(u1));
-            const uint32_t m2 = __float_as_uint(-128.0f * __uint_as_float(u2));
+            // 4 bit: the expanded codes are 128 + code
+            const float off = BITS == 4 ? -128.0f : 0.0f;
+            const uint32_t m0 = __float_as_uint(off * __uint_as_float(u0));
+            const uint32_t m1 = __float_as_uint(off * __uint_as_float(u1));
+            const uint32_t m2 = __float_as_uint(off * __uint_as_float(u2));
             a2[ts][j] = as_bf16x8((u0 >> 16) | u1, (u2 >> 16) | m0, (m1 >> 16) | m2, 0u);
         }
 
@@ -261,18 +277,26 @@ __global__ __launch_bounds__(NW* kWave) void qmv_tok16_kernel(const QmvArgs a) {
             for (int j = 0; j < QW; j++) {
                 // first 64 bytes of all 16 rows (lanes i >= 8 from the second load's lanes i - 8), second 64 bytes (lanes
                 // i < 8 from the first load's lanes i + 8): as for x
-                const uint4 la = ring[SL][j][0], lb = ring[SL][j][1];
-                uint32_t f0 = __builtin_amdgcn_update_dpp(la.x, lb.x, 0x118, 0xf, 0xc, false);
-                uint32_t f1 = __builtin_amdgcn_update_dpp(la.y, lb.y, 0x118, 0xf, 0xc, false);
-                uint32_t f2 = __builtin_amdgcn_update_dpp(la.z, lb.z, 0x118, 0xf, 0xc, false);
-                uint32_t f3 = __builtin_amdgcn_update_dpp(la.w, lb.w, 0x118, 0xf, 0xc, false);
-                uint32_t g0 = __builtin_amdgcn_update_dpp(lb.x, la.x, 0x108, 0xf, 0x3, false);
-                uint32_t g1 = __builtin_amdgcn_update_dpp(lb.y, la.y, 0x108, 0xf, 0x3, false);
-                uint32_t g2 = __builtin_amdgcn_update_dpp(lb.z, la.z, 0x108, 0xf, 0x3, false);
-                uint32_t g3 = __builtin_amdgcn_update_dpp(lb.w, la.w, 0x108, 0xf, 0x3, false);
-                transpose(f0, f1, f2, f3);
-                transpose(g0, g1, g2, g3);
-                const uint32_t ww[8] = {f0, f1, f2, f3, g0, g1, g2, g3};
+                uint32_t ww[8 * LINES];  // 4 bit: the word of step st; 8 bit: the two words of step st at 2 st, 2 st + 1
+#pragma unroll
+                for (int ln = 0; ln < LINES; ln++) {
+                    const uint4 la = ring[SL][j][ln][0], lb = ring[SL][j][ln][1];
+                    uint32_t f0 = __builtin_amdgcn_update_dpp(la.x, lb.x, 0x118, 0xf, 0xc, false);
+                    uint32_t f1 = __builtin_amdgcn_update_dpp(la.y, lb.y, 0x118, 0xf, 0xc, false);
+                    uint32_t f2 = __builtin_amdgcn_update_dpp(la.z, lb.z, 0x118, 0xf, 0xc, false);
+                    uint32_t f3 = __builtin_amdgcn_update_dpp(la.w, lb.w, 0x118, 0xf, 0xc, false);
+                    uint32_t g0 = __builtin_amdgcn_update_dpp(lb.x, la.x, 0x108, 0xf, 0x3, false);
+                    uint32_t g1 = __builtin_amdgcn_update_dpp(lb.y, la.y, 0x108, 0xf, 0x3, false);
+                    uint32_t g2 = __builtin_amdgcn_update_dpp(lb.z, la.z, 0x108, 0xf, 0x3, false);
+                    uint32_t g3 = __builtin_amdgcn_update_dpp(lb.w, la.w, 0x108, 0xf, 0x3, false);
+                    if constexpr (BITS == 4) {
+                        transpose(f0, f1, f2, f3);
+                        transpose(g0, g1, g2, g3);
+                    }
+                    const uint32_t both[8] = {f0, f1, f2, f3, g0, g1, g2, g3};
+#pragma unroll
+                    for (int k = 0; k < 8; k++) ww[8 * ln + k] = both[k];
+                }
                 const uint4 sbv = sbq[(rs * 16 + n) * sb_pitch + qds[j]];
                 f32x4_t part[TS];
 #pragma unroll
@@ -285,7 +309,12 @@ __global__ __launch_bounds__(NW* kWave) void qmv_tok16_kernel(const QmvArgs a) {
 #pragma unroll
                     for (int half = 0; half < 2; half++) {
                         uint32_t e[4];
-                        unpack4_word(ww[2 * g + half], mask, magic, e);
+                        if constexpr (BITS == 4) {
+                            unpack4_word(ww[2 * g + half], mask, magic, e);
+                        } else {
+                            unpack8_word(ww[4 * g + 2 * half], e);
+                            unpack8_word(ww[4 * g + 2 * half + 1], e + 2);
+                        }
                         const bf16x8_t bop = as_bf16x8(e[0], e[1], e[2], e[3]);
 #pragma unroll
                         for (int ts = 0; ts < TS; ts++)
@@ -363,20 +392,22 @@ struct QmvTokEntry {
     int wg_rows;  // weight rows per workgroup
     int lds;      // bytes
 };
-#define AQ_QMVT16(NW, RS, QW, RING)                                                                       \
+#define AQ_QMVT16B(BITS, NW, RS, QW, RING)                                                                \
     {                                                                                                     \
-        {"qmvt_b4_m16_r" #RS "_w" #NW "_q" #QW "_d" #RING, 4, 16, RS, NW, RING, 0, QW, 6},                 \
-            qmv_tok16_kernel<NW, RS, QW, RING, 1>, 16 * RS, NW * 16 * (16 * RS) * 4                       \
+        {"qmvt_b" #BITS "_m16_r" #RS "_w" #NW "_q" #QW "_d" #RING, BITS, 16, RS, NW, RING, 0, QW, 6},      \
+            qmv_tok16_kernel<BITS, NW, RS, QW, RING, 1>, 16 * RS, NW * 16 * (16 * RS) * 4                 \
     }
+#define AQ_QMVT16(NW, RS, QW, RING) AQ_QMVT16B(4, NW, RS, QW, RING)
 // the same with two sets of 16 tokens per expanded weight: up to 32 rows of x
 #define AQ_QMVT16X2(NW, RS, QW, RING)                                                                     \
     {                                                                                                     \
         {"qmvt_b4_m32_s2_r" #RS "_w" #NW "_q" #QW "_d" #RING, 4, 32, RS, NW, RING, 0, QW, 6},              \
-            qmv_tok16_kernel<NW, RS, QW, RING, 2>, 16 * RS, NW * 32 * (16 * RS) * 4                       \
+            qmv_tok16_kernel<4, NW, RS, QW, RING, 2>, 16 * RS, NW * 32 * (16 * RS) * 4                    \
     }
 static const QmvTokEntry kQmvTokTable[] = {AQ_QMVT16(8, 4, 1, 2), AQ_QMVT16(8, 2, 1, 2), AQ_QMVT16(8, 1, 1, 1),
                                            AQ_QMVT16(16, 4, 1, 3), AQ_QMVT16(8, 4, 2, 2),
-                                           AQ_QMVT16X2(8, 4, 1, 2), AQ_QMVT16X2(8, 2, 1, 2), AQ_QMVT16X2(8, 1, 1, 1)};
+                                           AQ_QMVT16X2(8, 4, 1, 2), AQ_QMVT16X2(8, 2, 1, 2), AQ_QMVT16X2(8, 1, 1, 1),
+                                           AQ_QMVT16B(8, 8, 4, 1, 2), AQ_QMVT16B(8, 8, 2, 1, 2), AQ_QMVT16B(8, 8, 1, 1, 1)};
 
 int qmvt_variant_count() { return (int)(sizeof(kQmvTokTable) / sizeof(kQmvTokTable[0])); }
 const QmvVariant* qmvt_variant(int idx) {
@@ -386,13 +417,13 @@ const QmvVariant* qmvt_variant(int idx) {
 
 bool qmvt_fits(const QmvArgs& a, int bits, int group_size, int idx) {
     const QmvVariant* v = qmvt_variant(idx);
-    if (!v || bits != 4 || group_size != 64) return false;
+    if (!v || bits != v->bits || group_size != 64) return false;
     if (a.M < 1 || a.M > v->m || a.N < 1 || a.K < 256 || a.K % 256 != 0) return false;
     const uintptr_t al16 = reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.w);
     const uintptr_t al8 = reinterpret_cast<uintptr_t>(a.s) | reinterpret_cast<uintptr_t>(a.b);
     if ((al16 & 15) || (al8 & 7)) return false;
     // 32-bit byte offsets into the packed matrix and into x
-    if ((uint64_t)a.N * (uint64_t)(a.K / 2) >= (1ull << 32)) return false;
+    if ((uint64_t)a.N * (uint64_t)(a.K * bits / 8) >= (1ull << 32)) return false;
     // the 16-token form keeps its rows' scales and biases in LDS next to the partial sums
     if (((size_t)kQmvTokTable[idx].lds + (size_t)kQmvTokTable[idx].wg_rows * (a.K / 256 + 1) * 16 > 160 * 1024 ||
                        kQmvTokTable[idx].wg_rows * (a.K / 256) > tok16_stage_pieces(v->waves) * v->waves * kWave))
@@ -415,10 +446,9 @@ hipError_t qmvt_launch(int idx, const QmvArgs& a, hipStream_t stream) {
     return hipGetLastError();
 }
 
-// The variant for this shape, or -1: wavefronts so that each gets at least one run of four groups; two sets of rows per
-// wavefront while that still leaves a workgroup for most CUs.
-int qmvt_pick(int M, int K, int N, int cu_count) {
-    if (M < 1 || M > kTokMax || K < 256 || K % 256 != 0) return -1;
+// The variant for this shape, or -1.
+int qmvt_pick(int bits, int M, int K, int N, int cu_count) {
+    if (M < 1 || M > (bits == 4 ? kTokMax : 16) || K < 256 || K % 256 != 0) return -1;
     const int cus = cu_count > 0 ? cu_count : 256;
     if (K > 16384) return -1;
     // eight wavefronts, one run each per pass; one set of 16 tokens up to 16 rows of x, else two; as many sets of 16
@@ -427,7 +457,7 @@ int qmvt_pick(int M, int K, int N, int cu_count) {
     const int rs = (N + 63) / 64 >= (cus * 3) / 4 ? 4 : (N + 31) / 32 >= (cus * 3) / 4 ? 2 : 1;
     for (int i = 0; i < qmvt_variant_count(); i++) {
         const QmvVariant& v = kQmvTokTable[i].v;
-        if (v.m == most && v.waves == 8 && v.rows == rs && v.xmode == 1) return i;
+        if (v.bits == bits && v.m == most && v.waves == 8 && v.rows == rs && v.xmode == 1) return i;
     }
     return -1;
 }

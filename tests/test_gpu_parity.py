@@ -139,8 +139,6 @@ def _parse_variant(name):
         return "diag", parts["b"], parts["m"], parts["g"]
     if name.startswith("qmvt_"):
         return "tok", parts["b"], parts["m"], 0
-    if name.startswith("qmvd8_"):
-        return "d8", parts["b"], parts["m"], 0
     return "dot2", parts["b"], parts["m"], parts["g"]
 
 

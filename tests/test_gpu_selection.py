@@ -19,8 +19,8 @@ CASES = [
     (4, 64, 8, 4096 - 128, ("qmvd_",)),
     (4, 64, 16, 14336, ("qmvt_b4_m16_",)),           # token tile, 16-token form: 9..16 rows, K a multiple of 256
     (4, 32, 2, 1536, ("qmvd_",)),                    # groups of 32
-    (8, 64, 8, 4096, ("qmvd8_",)),                   # 8-bit MFMA: 5..16 rows
-    (8, 64, 16, 4096, ("qmvd8_",)),
+    (8, 64, 8, 4096, ("qmvt_b8_m16_",)),             # token tile, 8 bit: 5..16 rows
+    (8, 64, 16, 4096, ("qmvt_b8_m16_",)),
     (4, 64, 9, 4096, ("qmvt_b4_m16_",)),
     (4, 64, 17, 4096, ("qmvt_b4_m32_",)),            # token tile, 32-token form: 17..32 rows
     (4, 64, 32, 4096, ("qmvt_b4_m32_",)),

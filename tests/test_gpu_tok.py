@@ -23,29 +23,31 @@ def test_tok_every_variant(ctx, orc):
     import aq_mi355
     N = 150
     try:
-        for K in (256, 768, 2048, 2816, 4096, 14336):
-            words, s, b = F.synthetic_affine(N, K, 4, 64, seed=1500 + K // 256)
+        for K, bits in [(K, bits) for bits in (4, 8) for K in (256, 768, 2048, 2816, 4096, 14336)]:
+            words, s, b = F.synthetic_affine(N, K, bits, 64, seed=1500 + K // 256 + bits)
             x = F.synthetic_x(32, K, seed=1600 + K // 256)
-            ref = F.reference_f64(x, words, s, b, 4, 64, K)
+            ref = F.reference_f64(x, words, s, b, bits, 64, K)
             dw = DeviceAffine(ctx, words, s, b)
             for idx, name in _tok_variants():
+                if "_b%d_" % bits not in name:
+                    continue
                 ctx.force_variant(0, idx)
                 full = None
                 most = int(name.split("_m")[1].split("_")[0])  # rows of x the variant takes: 16, or 32 for the two-set forms
                 for rows in [r for r in (most, 1, 5, 9, 16, 17, 31) if r <= most]:
                     say("tok variant", name, "K", K, "rows", rows)
-                    acc = run_qmv(ctx, x[:rows], dw, rows, K, N, 64, 4, True)
+                    acc = run_qmv(ctx, x[:rows], dw, rows, K, N, 64, bits, True)
                     assert ctx.last_variant(0) == name
                     check_accumulators(acc, ref[:rows], "%s K=%d rows=%d" % (name, K, rows))
                     if full is None:
                         full = acc
                     assert np.array_equal(acc.view(np.uint32), full[:rows].view(np.uint32)), (name, K, rows)
                 some = min(17, most)
-                out = run_qmv(ctx, x[:some], dw, some, K, N, 64, 4, False)
+                out = run_qmv(ctx, x[:some], dw, some, K, N, 64, bits, False)
                 check_bf16_store(out, ref[:some], name)
                 assert np.array_equal(out, F.f32_to_bf16_bits(full[:some]).reshape(some, N))
             dw.free()
-        idx, name = [v for v in _tok_variants() if "_m32_" in v[1]][0]
+        idx, name = [v for v in _tok_variants() if "_b4_m32_" in v[1]][0]
         ctx.force_variant(0, idx)
         words, s, b = F.synthetic_affine(40, 16640, 4, 64, seed=1700)
         dw = DeviceAffine(ctx, words, s, b)
@@ -56,6 +58,32 @@ def test_tok_every_variant(ctx, orc):
         dw.free()
     finally:
         ctx.force_variant(0, -1)
+
+
+@pytest.mark.parametrize("M", [5, 8, 16])
+def test_tok_config2_full_shape_8bit(ctx, orc, M):
+    """cfg 2's 8-bit variant at its full shape (K = 4096, N = 14336): the default path; accumulators against the
+    float64 reference and, on sampled rows of x, the oracle's fp32-accumulated reference; bf16 store = RNE of the
+    accumulator; two runs give the same bytes."""
+    say("tok cfg2 8 bit", M)
+    K, N = 4096, 14336
+    words, s, b = F.synthetic_affine(N, K, 8, 64, seed=F.BASE_SEED + 2)
+    x = F.synthetic_x(M, K, seed=F.BASE_SEED + 3)
+    ref = F.reference_f64(x, words, s, b, 8, 64, K)
+    dw = DeviceAffine(ctx, words, s, b)
+    acc = run_qmv(ctx, x, dw, M, K, N, 64, 8, True)
+    assert ctx.last_variant(0).startswith("qmvt_b8_m16_"), ctx.last_variant(0)
+    check_accumulators(acc, ref, "tok cfg2 8 bit M=%d" % M)
+    rows = sorted({0, M - 1})
+    xf = F.bf16_bits_to_f32(x).reshape(M, K)
+    o32 = orc.hip_reference_projection_batch(xf[rows].reshape(-1), len(rows), words, s, b, N, K, 64, 8)
+    check_accumulators(acc[rows], o32, "tok cfg2 8 bit vs oracle M=%d" % M)
+    out = run_qmv(ctx, x, dw, M, K, N, 64, 8, False)
+    check_bf16_store(out, ref, "tok cfg2 8 bit bf16")
+    assert np.array_equal(out, F.f32_to_bf16_bits(acc).reshape(M, N))
+    again = run_qmv(ctx, x, dw, M, K, N, 64, 8, True)
+    assert np.array_equal(again.view(np.uint32), acc.view(np.uint32))
+    dw.free()
 
 
 @pytest.mark.parametrize("M", [9, 16, 17, 32])
