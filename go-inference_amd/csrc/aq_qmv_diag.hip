@@ -219,7 +219,18 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     const gptr_t wg = uniform_ptr(reinterpret_cast<const char*>(other ? a.w2 : a.w) + srow * (K >> 1));
     const gptr_t sg = uniform_ptr(reinterpret_cast<const char*>(other ? a.s2 : a.s) + srow * groups * 2);
     const gptr_t bg = uniform_ptr(reinterpret_cast<const char*>(other ? a.b2 : a.b) + srow * groups * 2);
-    const uint32_t w_lane = (uint32_t)row * (uint32_t)(K >> 1) + (uint32_t)j * 16;  // bytes
+    // Weights are requested as whole 128-byte lines of 8 rows per instruction (half as many requests at the L1 as 64
+    // bytes of each of 16 rows): lane (i = lane % 16, j) of load `ab` reads row 8 ab + i % 8 of the set, bytes
+    // 64 (i / 8) + 16 j of a chunk; two DPP moves per register pair then leave "lane (n, j): bytes 16 j .. 16 j + 15 of
+    // the first (second) 64 bytes of row n", the shape the B operands have.
+    uint32_t w_lane[2];
+#pragma unroll
+    for (int ab = 0; ab < 2; ab++) {
+        int r8 = row0 + (n & 7) + 8 * ab;
+        if (r8 >= N) r8 = N - 1;
+        w_lane[ab] = (uint32_t)r8 * (uint32_t)(K >> 1) + (uint32_t)j * 16;  // bytes
+    }
+    const uint32_t w_half = (uint32_t)(n >> 3) * 64;  // which 64 bytes of the chunk this lane requests
     // scales and biases: lane group j holds the four groups of chunk j of the step
     const uint32_t sb_lane = (uint32_t)row * (uint32_t)groups * 2 + (uint32_t)j * SBB;  // bytes
 
@@ -257,13 +268,16 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
         int sp = wave + u * NW;
         if (sp >= supers) sp = supers - 1;  // past the end: a valid address, the result is not used
         const int valid = min(CPS, chunks - CPS * sp);  // chunks of this step; the others re-read chunk 0 and are not used
-        const uint32_t wo = w_lane + (uint32_t)sp * (CPS * 128);
+        const uint32_t wo = (uint32_t)sp * (CPS * 128);
 #pragma unroll
         for (int cc = 0; cc < CPS; cc++) {
             const uint32_t co = cc < valid ? cc * 128 : 0;
-            wq[u][cc][0] = load_u128_at(wg, wo + co);
             // (the second half of a last chunk that is a single half: re-reads the first, not used)
-            wq[u][cc][1] = load_u128_at(wg, wo + co + (cc < valid && 2 * (CPS * sp + cc) + 1 < halves ? 64 : 0));
+            const uint32_t ho = cc < valid && 2 * (CPS * sp + cc) + 1 < halves ? w_half : 0;
+            const uint4 la = load_u128_at(wg, w_lane[0] + wo + co + ho);
+            const uint4 lb = load_u128_at(wg, w_lane[1] + wo + co + ho);
+            wq[u][cc][0] = la;
+            wq[u][cc][1] = lb;
         }
         // A last chunk of one half has two groups: its 8 bytes are read 4 bytes early (inside the row) and the
         // upper word, which holds the two groups, moves down.
@@ -371,7 +385,21 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
 #pragma unroll
                 for (int L = 0; L < 2; L++) {
                     if (L == 1 && 2 * (CPS * sp + cc) + 1 >= halves) break;  // a last chunk of one half
-                    const uint32_t ww[4] = {wq[u][cc][L].x, wq[u][cc][L].y, wq[u][cc][L].z, wq[u][cc][L].w};
+                    // first 64 bytes: lanes i >= 8 take rows 8..15 from the second load's lanes i - 8; second 64 bytes:
+                    // lanes i < 8 take rows 0..7 from the first load's lanes i + 8
+                    const uint4 la = wq[u][cc][0], lb = wq[u][cc][1];
+                    uint32_t ww[4];
+                    if (L == 0) {
+                        ww[0] = __builtin_amdgcn_update_dpp(la.x, lb.x, 0x118, 0xf, 0xc, false);
+                        ww[1] = __builtin_amdgcn_update_dpp(la.y, lb.y, 0x118, 0xf, 0xc, false);
+                        ww[2] = __builtin_amdgcn_update_dpp(la.z, lb.z, 0x118, 0xf, 0xc, false);
+                        ww[3] = __builtin_amdgcn_update_dpp(la.w, lb.w, 0x118, 0xf, 0xc, false);
+                    } else {
+                        ww[0] = __builtin_amdgcn_update_dpp(lb.x, la.x, 0x108, 0xf, 0x3, false);
+                        ww[1] = __builtin_amdgcn_update_dpp(lb.y, la.y, 0x108, 0xf, 0x3, false);
+                        ww[2] = __builtin_amdgcn_update_dpp(lb.z, la.z, 0x108, 0xf, 0x3, false);
+                        ww[3] = __builtin_amdgcn_update_dpp(lb.w, la.w, 0x108, 0xf, 0x3, false);
+                    }
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
                         uint32_t p[4];
