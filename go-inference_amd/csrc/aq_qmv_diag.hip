@@ -96,7 +96,8 @@ __host__ __device__ inline size_t qmvd_lds_bytes_for(int M, int K, int nw, int m
 // meet at the end.  Scales and biases are 16 bytes per chunk and lane.  K is then a multiple of 256.
 // HEAD (lm_head, one activation row): 4 stores every row's packed (score, row) instead of the score, 3 keeps the
 // best packed value of the 16 rows in a.partial[set] for fold_best_kernel (aq_qmv_head.hip).
-template <int NW, int SUP, int NR, bool PAIR, int MT = 1, bool GATHER = false, int CPS = 4, bool G32 = false, int HEAD = 0>
+template <int NW, int SUP, int NR, bool PAIR, int MT = 1, bool GATHER = false, int CPS = 4, bool G32 = false, int HEAD = 0,
+          bool LINES = true>
 __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block) {
     static_assert(HEAD == 0 || (!PAIR && !GATHER && MT == 1), "the head epilogues take one plain activation row");
     static_assert(!G32 || MT == 1, "group 32: one set of two activation rows");
@@ -219,18 +220,21 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     const gptr_t wg = uniform_ptr(reinterpret_cast<const char*>(other ? a.w2 : a.w) + srow * (K >> 1));
     const gptr_t sg = uniform_ptr(reinterpret_cast<const char*>(other ? a.s2 : a.s) + srow * groups * 2);
     const gptr_t bg = uniform_ptr(reinterpret_cast<const char*>(other ? a.b2 : a.b) + srow * groups * 2);
-    // Weights are requested as whole 128-byte lines of 8 rows per instruction (half as many requests at the L1 as 64
-    // bytes of each of 16 rows): lane (i = lane % 16, j) of load `ab` reads row 8 ab + i % 8 of the set, bytes
+    // LINES: weights are requested as whole 128-byte lines of 8 rows per instruction (half as many requests at the L1 as
+    // 64 bytes of each of 16 rows): lane (i = lane % 16, j) of load `ab` reads row 8 ab + i % 8 of the set, bytes
     // 64 (i / 8) + 16 j of a chunk; two DPP moves per register pair then leave "lane (n, j): bytes 16 j .. 16 j + 15 of
-    // the first (second) 64 bytes of row n", the shape the B operands have.
+    // the first (second) 64 bytes of row n", the shape the B operands have.  Otherwise load L of a chunk is that shape
+    // as it comes.  (Measured on one box, old shape -> lines: the four-launch layer 33.0 -> 32.3 us, 14336 -> 4096
+    // 9.0 -> 8.8 us, the MoE block 84.2 -> 82.4 us, but 4096 -> 14336 as a launch of its own 8.5 -> 8.6 us: the plain
+    // kernel of up to four wavefronts keeps the old shape.)
     uint32_t w_lane[2];
 #pragma unroll
     for (int ab = 0; ab < 2; ab++) {
-        int r8 = row0 + (n & 7) + 8 * ab;
+        int r8 = LINES ? row0 + (n & 7) + 8 * ab : row0 + n;
         if (r8 >= N) r8 = N - 1;
         w_lane[ab] = (uint32_t)r8 * (uint32_t)(K >> 1) + (uint32_t)j * 16;  // bytes
     }
-    const uint32_t w_half = (uint32_t)(n >> 3) * 64;  // which 64 bytes of the chunk this lane requests
+    const uint32_t w_half = LINES ? (uint32_t)(n >> 3) * 64 : 0;  // which 64 bytes of the chunk this lane requests
     // scales and biases: lane group j holds the four groups of chunk j of the step
     const uint32_t sb_lane = (uint32_t)row * (uint32_t)groups * 2 + (uint32_t)j * SBB;  // bytes
 
@@ -274,10 +278,9 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
             const uint32_t co = cc < valid ? cc * 128 : 0;
             // (the second half of a last chunk that is a single half: re-reads the first, not used)
             const uint32_t ho = cc < valid && 2 * (CPS * sp + cc) + 1 < halves ? w_half : 0;
-            const uint4 la = load_u128_at(wg, w_lane[0] + wo + co + ho);
-            const uint4 lb = load_u128_at(wg, w_lane[1] + wo + co + ho);
-            wq[u][cc][0] = la;
-            wq[u][cc][1] = lb;
+            const bool whole = cc < valid && 2 * (CPS * sp + cc) + 1 < halves;
+            wq[u][cc][0] = load_u128_at(wg, w_lane[0] + wo + co + ho);
+            wq[u][cc][1] = load_u128_at(wg, w_lane[1] + wo + co + (LINES ? ho : whole ? 64u : 0u));
         }
         // A last chunk of one half has two groups: its 8 bytes are read 4 bytes early (inside the row) and the
         // upper word, which holds the two groups, moves down.
@@ -389,7 +392,13 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
                     // lanes i < 8 take rows 0..7 from the first load's lanes i + 8
                     const uint4 la = wq[u][cc][0], lb = wq[u][cc][1];
                     uint32_t ww[4];
-                    if (L == 0) {
+                    if constexpr (!LINES) {
+                        const uint4 lv = L == 0 ? la : lb;
+                        ww[0] = lv.x;
+                        ww[1] = lv.y;
+                        ww[2] = lv.z;
+                        ww[3] = lv.w;
+                    } else if (L == 0) {
                         ww[0] = __builtin_amdgcn_update_dpp(la.x, lb.x, 0x118, 0xf, 0xc, false);
                         ww[1] = __builtin_amdgcn_update_dpp(la.y, lb.y, 0x118, 0xf, 0xc, false);
                         ww[2] = __builtin_amdgcn_update_dpp(la.z, lb.z, 0x118, 0xf, 0xc, false);
@@ -483,7 +492,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
 
 template <int NW, int SUP, int NR, int MT, int CPS>
 __global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_kernel(const QmvArgs a) {
-    qmv_diag_body<NW, SUP, NR, false, MT, false, CPS>(a, (int)blockIdx.x);
+    qmv_diag_body<NW, SUP, NR, false, MT, false, CPS, false, 0, (NW > 4)>(a, (int)blockIdx.x);
 }
 
 template <int NW, int SUP, int CPS>
