@@ -22,9 +22,9 @@
 
 namespace aq {
 
-template <int BITS, int M, int R, int NW, int DEPTH, bool GATHER, int XMODE>
+template <int BITS, int M, int R, int NW, int DEPTH, bool GATHER>
 __global__ __launch_bounds__(NW* kWave) void qmv_dot2_kernel(const QmvArgs a) {
-    qmv_dot2_body<BITS, M, R, NW, DEPTH, GATHER, XMODE>(a, blockIdx.x);
+    qmv_dot2_body<BITS, M, R, NW, DEPTH, GATHER>(a, blockIdx.x);
 }
 
 // Several weight matrices against the same activations in one launch (q|k|v, gate|up): the
@@ -41,7 +41,7 @@ __global__ __launch_bounds__(NW* kWave) void qmv_dot2_multi_kernel(const QmvMult
     a.b = ma.b[set];
     a.y = ma.y[set];
     a.N = ma.N[set];
-    qmv_dot2_body<BITS, M, R, NW, DEPTH, false, 0>(a, (int)blockIdx.x - (set ? ma.block_end[set - 1] : 0));
+    qmv_dot2_body<BITS, M, R, NW, DEPTH, false>(a, (int)blockIdx.x - (set ? ma.block_end[set - 1] : 0));
 }
 
 // ---- variant table --------------------------------------------------------
@@ -53,32 +53,19 @@ struct QmvEntry {
     QmvKernel fn;
 };
 
-#define AQ_QMV_X(BITS, M, R, NW, DEPTH, G, X)                                                           \
+// (names keep the "_x0" of the staging mode they have always had: x through LDS)
+#define AQ_QMV(BITS, M, R, NW, DEPTH, G)                                                                \
     {                                                                                                   \
-        {"qmv_b" #BITS "_m" #M "_r" #R "_w" #NW "_d" #DEPTH "_g" #G "_x" #X, BITS, M, R, NW, DEPTH, G, X}, \
-            qmv_dot2_kernel<BITS, M, R, NW, DEPTH, (G != 0), X>                                         \
+        {"qmv_b" #BITS "_m" #M "_r" #R "_w" #NW "_d" #DEPTH "_g" #G "_x0", BITS, M, R, NW, DEPTH, G, 0}, \
+            qmv_dot2_kernel<BITS, M, R, NW, DEPTH, (G != 0)>                                            \
     }
-#define AQ_QMV(BITS, M, R, NW, DEPTH, G) AQ_QMV_X(BITS, M, R, NW, DEPTH, G, 0)
-
-#define AQ_QMV_M1_SET(BITS, G)                                                                     \
-    AQ_QMV(BITS, 1, 1, 4, 2, G), AQ_QMV(BITS, 1, 1, 4, 4, G), AQ_QMV(BITS, 1, 1, 8, 2, G),         \
-        AQ_QMV(BITS, 1, 2, 2, 2, G), AQ_QMV(BITS, 1, 2, 4, 2, G), AQ_QMV(BITS, 1, 2, 4, 4, G),     \
-        AQ_QMV(BITS, 1, 2, 8, 2, G), AQ_QMV(BITS, 1, 4, 2, 2, G), AQ_QMV(BITS, 1, 4, 4, 2, G),     \
-        AQ_QMV(BITS, 1, 4, 4, 4, G), AQ_QMV(BITS, 1, 4, 8, 2, G), AQ_QMV(BITS, 1, 8, 2, 2, G),     \
-        AQ_QMV(BITS, 1, 8, 4, 2, G), AQ_QMV(BITS, 1, 7, 4, 2, G), AQ_QMV(BITS, 1, 7, 8, 2, G),       \
-        AQ_QMV_X(BITS, 1, 1, 4, 2, G, 1), AQ_QMV_X(BITS, 1, 2, 4, 2, G, 1), AQ_QMV_X(BITS, 1, 4, 4, 2, G, 1), \
-        AQ_QMV_X(BITS, 1, 2, 8, 2, G, 1), AQ_QMV_X(BITS, 1, 4, 8, 2, G, 1), AQ_QMV_X(BITS, 1, 4, 2, 2, G, 1), \
-        AQ_QMV_X(BITS, 1, 2, 4, 4, G, 1), AQ_QMV_X(BITS, 1, 8, 4, 2, G, 1), AQ_QMV_X(BITS, 1, 4, 1, 2, G, 1), \
-        AQ_QMV_X(BITS, 1, 2, 1, 2, G, 1), AQ_QMV_X(BITS, 1, 8, 1, 2, G, 1), AQ_QMV_X(BITS, 1, 4, 4, 1, G, 1)
-
-#define AQ_QMV_MN_SET(BITS, M)                                                                     \
-    AQ_QMV(BITS, M, 1, 4, 2, 0), AQ_QMV(BITS, M, 2, 4, 2, 0), AQ_QMV(BITS, M, 4, 4, 2, 0),         \
-        AQ_QMV(BITS, M, 2, 8, 2, 0), AQ_QMV(BITS, M, 4, 8, 2, 0)
+// four wavefronts a workgroup, two slices of K in flight, 1 / 2 / 4 rows per wavefront: what the selection picks from
+#define AQ_QMV_SET(BITS, M, G) AQ_QMV(BITS, M, 1, 4, 2, G), AQ_QMV(BITS, M, 2, 4, 2, G), AQ_QMV(BITS, M, 4, 4, 2, G)
 
 static const QmvEntry kQmvTable[] = {
-    AQ_QMV_M1_SET(4, 0), AQ_QMV_M1_SET(8, 0), AQ_QMV_M1_SET(4, 1), AQ_QMV_M1_SET(8, 1),
-    AQ_QMV_MN_SET(4, 2), AQ_QMV_MN_SET(4, 3), AQ_QMV_MN_SET(4, 4),
-    AQ_QMV_MN_SET(8, 2), AQ_QMV_MN_SET(8, 3), AQ_QMV_MN_SET(8, 4),
+    AQ_QMV_SET(4, 1, 0), AQ_QMV_SET(8, 1, 0), AQ_QMV_SET(4, 1, 1), AQ_QMV_SET(8, 1, 1),
+    AQ_QMV_SET(4, 2, 0), AQ_QMV_SET(4, 3, 0), AQ_QMV_SET(4, 4, 0),
+    AQ_QMV_SET(8, 2, 0), AQ_QMV_SET(8, 3, 0), AQ_QMV_SET(8, 4, 0),
 };
 
 int qmv_variant_count() { return (int)(sizeof(kQmvTable) / sizeof(kQmvTable[0])); }
@@ -90,7 +77,7 @@ const QmvVariant* qmv_variant(int idx) {
 
 size_t qmv_lds_bytes(int idx, const QmvArgs& a) {
     const QmvVariant* v = qmv_variant(idx);
-    if (!v || v->xmode == 1) return 0;
+    if (!v) return 0;
     return (size_t)v->m * (size_t)a.K * 2;
 }
 

@@ -19,7 +19,7 @@ namespace aq {
 
 template <int BITS, int R, bool GATHER, int FUSE>
 __global__ __launch_bounds__(4 * kWave) void qmv_act_kernel(const QmvArgs a) {
-    qmv_dot2_body<BITS, 1, R, 4, 2, GATHER, 0, FUSE>(a, blockIdx.x);
+    qmv_dot2_body<BITS, 1, R, 4, 2, GATHER, FUSE>(a, blockIdx.x);
 }
 
 typedef void (*QmvActKernel)(const QmvArgs);

@@ -397,14 +397,12 @@ struct BlkEntry {
             qmv_blk_kernel<BITS, MCAP, KI, D, (G != 0)>                                             \
     }
 // v.depth = K pieces per wavefront, v.waves = ring depth (row groups in flight per wavefront)
-#define AQ_BLK_M(BITS, MCAP, G)                                                                     \
-    AQ_BLK(BITS, MCAP, 1, 2, G), AQ_BLK(BITS, MCAP, 1, 4, G), AQ_BLK(BITS, MCAP, 2, 2, G),          \
-        AQ_BLK(BITS, MCAP, 4, 1, G), AQ_BLK(BITS, MCAP, 4, 2, G)
+// the ring depths the plan asks for: two row groups in flight with one or two K pieces per wavefront, one with four
+#define AQ_BLK_M(BITS, MCAP, G) AQ_BLK(BITS, MCAP, 1, 2, G), AQ_BLK(BITS, MCAP, 2, 2, G), AQ_BLK(BITS, MCAP, 4, 1, G)
 #define AQ_BLK_SET(BITS)                                                                            \
-    AQ_BLK_M(BITS, 1, 0), AQ_BLK(BITS, 1, 1, 8, 0), AQ_BLK(BITS, 1, 1, 3, 0), AQ_BLK(BITS, 1, 2, 1, 0), \
-        AQ_BLK(BITS, 1, 2, 4, 0), AQ_BLK_M(BITS, 2, 0), AQ_BLK_M(BITS, 3, 0), AQ_BLK_M(BITS, 4, 0), \
-        AQ_BLK(BITS, 8, 1, 2, 0), AQ_BLK(BITS, 8, 1, 4, 0), AQ_BLK(BITS, 8, 2, 2, 0),               \
-        AQ_BLK(BITS, 12, 1, 2, 0), AQ_BLK(BITS, 16, 1, 2, 0), AQ_BLK_M(BITS, 1, 1)
+    AQ_BLK_M(BITS, 1, 0), AQ_BLK_M(BITS, 2, 0), AQ_BLK_M(BITS, 3, 0), AQ_BLK_M(BITS, 4, 0),         \
+        AQ_BLK(BITS, 8, 1, 2, 0), AQ_BLK(BITS, 8, 2, 2, 0), AQ_BLK(BITS, 12, 1, 2, 0),              \
+        AQ_BLK(BITS, 16, 1, 2, 0), AQ_BLK_M(BITS, 1, 1)
 
 static const BlkEntry kBlkTable[] = {AQ_BLK_SET(4), AQ_BLK_SET(8)};
 

@@ -22,17 +22,15 @@ struct Codec<8> {
 };
 
 // One slice of R rows held in registers (plus, in direct-x mode, the lane's x chunk).
-template <int R, int XREGS>
+template <int R>
 struct Slice {
     uint4 w[R];
     uint16_t s[R];
     uint16_t b[R];
-    uint4 x[XREGS > 0 ? XREGS : 1];
 };
 
-// XMODE 0: x staged once per workgroup into LDS (x loads are issued before any weight load so the
-//          barrier never waits for HBM); XMODE 1 (M == 1 only): every lane pulls its own 64-byte
-//          x chunk straight from global/L2 with the slice, no LDS and no barrier.
+// x is staged once per workgroup into LDS (its loads are issued before any weight load so the barrier never waits
+// for HBM).
 // bx: this workgroup's position among those of one weight matrix (blockIdx.x for a plain launch).
 // FUSE 0: y = W x.
 // FUSE 1: a wavefront owns R rows of the `gate` matrix (w, s, b) and the same R rows of the `up` matrix
@@ -44,16 +42,13 @@ struct Slice {
 //         rocm_mlx_q4_projection_greedy accumulates with atomicMax
 //         (kernels/quant/affine_projection_fused.hipinc:190-248).
 // FUSE 4: every row's packed (score, row) is stored, as rocm_mlx_q4_projection_scores does (:411-446).
-template <int BITS, int M, int R, int NW, int DEPTH, bool GATHER, int XMODE, int FUSE = 0>
+template <int BITS, int M, int R, int NW, int DEPTH, bool GATHER, int FUSE = 0>
 __device__ __forceinline__ void qmv_dot2_body(const QmvArgs& a, const int bx) {
     using C = Codec<BITS>;
     constexpr int CPC = C::kCodesPerChunk;
     constexpr int PAIRS = C::kPairs;
-    constexpr int XREGS = XMODE == 1 ? PAIRS / 4 : 0;
-    static_assert(XMODE == 0 || M == 1, "direct x mode is single-row only");
-    static_assert(FUSE == 0 || XMODE == 0, "the fused kernels stage x through LDS");
     constexpr int RS = FUSE == 1 ? 2 * R : R;  // row slots a wavefront streams
-    extern __shared__ uint32_t xs[];  // [M][K/2] bf16 pairs, unpack order (XMODE 0)
+    extern __shared__ uint32_t xs[];  // [M][K/2] bf16 pairs, unpack order
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -110,12 +105,12 @@ __device__ __forceinline__ void qmv_dot2_body(const QmvArgs& a, const int bx) {
 #pragma unroll
     for (int r = 0; r < R; r++) rel[r] = (uint32_t)min(r, N - 1 - row_base_clamped);
 
-    // Stage x (XMODE 0): global loads first, so that nothing below queues ahead of them.
+    // Stage x: global loads first, so that nothing below queues ahead of them.
     constexpr int XPT = 4;  // 16-byte x pieces held per thread between load and LDS write
     uint4 xstage[XPT];
     uint4 xstage2[FUSE == 2 ? XPT : 1];
     const int pieces = M * (K / 8);
-    if constexpr (XMODE == 0) {
+    {
         const uint4* src = reinterpret_cast<const uint4*>(xrow);
 #pragma unroll
         for (int q = 0; q < XPT; q++) {
@@ -132,15 +127,10 @@ __device__ __forceinline__ void qmv_dot2_body(const QmvArgs& a, const int bx) {
         }
     }
 
-    auto load_slice = [&](Slice<RS, XREGS>& t, int sl) {
+    auto load_slice = [&](Slice<RS>& t, int sl) {
         const int c = sl * kWave + lane;
         if (sl < nslices && c < chunks_per_row) {
             const uint32_t g2 = (uint32_t)((c * CPC) >> a.gs_shift) * 2u;
-            if constexpr (XMODE == 1) {
-                const uint4* xp = reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(xrow) + (uint32_t)c * (PAIRS * 4u));
-#pragma unroll
-                for (int q = 0; q < XREGS; q++) t.x[q] = xp[q];
-            }
 #pragma unroll
             for (int r = 0; r < RS; r++) {
                 const bool up = FUSE == 1 && r >= R;
@@ -157,11 +147,11 @@ __device__ __forceinline__ void qmv_dot2_body(const QmvArgs& a, const int bx) {
         }
     };
 
-    Slice<RS, XREGS> ring[DEPTH];
+    Slice<RS> ring[DEPTH];
 #pragma unroll
     for (int d = 0; d < DEPTH; d++) load_slice(ring[d], d);
 
-    if constexpr (XMODE == 0) {
+    {
         auto permute = [](uint4 v) {
             if constexpr (BITS == 4) {
                 // (x0,x1)(x2,x3)(x4,x5)(x6,x7) -> (x0,x4)(x1,x5)(x2,x6)(x3,x7)
@@ -206,30 +196,14 @@ __device__ __forceinline__ void qmv_dot2_body(const QmvArgs& a, const int bx) {
     const uint32_t mask_s = opaque_s(kNibbleMask);   // both stay in registers so that
     const uint32_t magic_v = opaque_v(kMagic128);  // (w & mask) | magic is a single v_and_or_b32
 
-    auto compute_slice = [&](const Slice<RS, XREGS>& t, int sl) {
+    auto compute_slice = [&](const Slice<RS>& t, int sl) {
         const int c = sl * kWave + lane;
         if (sl < nslices && c < chunks_per_row) {
             uint32_t xq[M][PAIRS];
             float xsum[M];
 #pragma unroll
             for (int m = 0; m < M; m++) {
-                if constexpr (XMODE == 1) {
-#pragma unroll
-                    for (int q = 0; q < PAIRS / 4; q++) {
-                        const uint4 v = t.x[q];
-                        if constexpr (BITS == 4) {
-                            xq[m][4 * q + 0] = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);
-                            xq[m][4 * q + 1] = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);
-                            xq[m][4 * q + 2] = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);
-                            xq[m][4 * q + 3] = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
-                        } else {
-                            xq[m][4 * q + 0] = v.x;
-                            xq[m][4 * q + 1] = v.y;
-                            xq[m][4 * q + 2] = v.z;
-                            xq[m][4 * q + 3] = v.w;
-                        }
-                    }
-                } else {
+                {
                     const uint4* xp = reinterpret_cast<const uint4*>(xs + (size_t)m * (K / 2) + (size_t)c * PAIRS);
 #pragma unroll
                     for (int q = 0; q < PAIRS / 4; q++) {

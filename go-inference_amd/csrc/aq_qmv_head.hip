@@ -17,7 +17,7 @@ namespace aq {
 
 template <int BITS, int R, int FUSE>
 __global__ __launch_bounds__(4 * kWave) void qmv_head_kernel(const QmvArgs a) {
-    qmv_dot2_body<BITS, 1, R, 4, 2, false, 0, FUSE>(a, blockIdx.x);
+    qmv_dot2_body<BITS, 1, R, 4, 2, false, FUSE>(a, blockIdx.x);
 }
 
 typedef void (*QmvHeadKernel)(const QmvArgs);

@@ -405,7 +405,6 @@ struct QmvTokEntry {
             qmv_tok16_kernel<4, NW, RS, QW, RING, 2>, 16 * RS, NW * 32 * (16 * RS) * 4                    \
     }
 static const QmvTokEntry kQmvTokTable[] = {AQ_QMVT16(8, 4, 1, 2), AQ_QMVT16(8, 2, 1, 2), AQ_QMVT16(8, 1, 1, 1),
-                                           AQ_QMVT16(16, 4, 1, 3), AQ_QMVT16(8, 4, 2, 2),
                                            AQ_QMVT16X2(8, 4, 1, 2), AQ_QMVT16X2(8, 2, 1, 2), AQ_QMVT16X2(8, 1, 1, 1),
                                            AQ_QMVT16B(8, 8, 4, 1, 2), AQ_QMVT16B(8, 8, 2, 1, 2), AQ_QMVT16B(8, 8, 1, 1, 1)};
 
