@@ -81,7 +81,7 @@ struct QmvVariant {
     int waves;   // wavefronts per workgroup
     int depth;   // K slices in flight per wavefront
     int gather;  // 1: reads rhs/lhs on device, grid.y = routes
-    int xmode;   // 0: x staged through LDS, 1: every lane reads its x chunk from global
+    int xmode;   // family-specific (dot2: 0; diagonal: chunks per step when not 4; token tile: runs held per pass)
     int kind;    // 0: VALU dot2 kernel (aq_qmv.hip),
                  // 2: block-MFMA kernel (aq_qmv_blk.hip; m = most rows, depth = K pieces per wavefront),
                  // 4: diagonal-MFMA kernel (aq_qmv_diag.hip; m = most rows, rows = sets of 16 rows per workgroup,
