@@ -589,14 +589,28 @@ def main():
         h_logits, h_best, h_scores, h_top = ctx.alloc(HN * 2), ctx.alloc(8), ctx.alloc(HN * 8), ctx.alloc(40 * 8)
         head_bytes = HN * HK * BITS // 8 + 2 * HN * (HK // HG) * 2 + HK * 2
 
-        def head_time(fn, n=40):
+        def head_time(fn, n=40, graph=False):
+            # graph=True: a graph of n calls, replayed, so that the launches of a call of several kernels
+            # cost no host time; calls of one kernel are timed as plain launches on the stream
             for i in range(4):
                 fn(pool[i % 2])
             ctx.sync()
-            ctx.timer_start()
+            if not graph:
+                ctx.timer_start()
+                for i in range(n):
+                    fn(pool[i % 2])
+                return ctx.timer_stop() * 1e3 / n
+            ctx.capture_begin()
             for i in range(n):
                 fn(pool[i % 2])
-            return ctx.timer_stop() * 1e3 / n
+            g = ctx.capture_end()
+            ts = []
+            for _ in range(5):
+                ctx.timer_start()
+                ctx.graph_launch(g)
+                ts.append(ctx.timer_stop() * 1e3 / n)
+            ctx.graph_destroy(g)
+            return float(np.median(ts))
 
         us_logits = head_time(lambda t: ctx.qmv(hx, t[0], t[1], t[2], h_logits, 1, HK, HN, HG, BITS))
         k_logits = ctx.last_variant(0)
@@ -606,13 +620,13 @@ def main():
             ctx.qmv_scores(hx, t[0], t[1], t[2], h_scores, 1, HK, HN, HG, BITS)
             ctx.packed_topk(h_scores, HN, 40, h_top)
 
-        us_topk = head_time(topk40)
+        us_topk = head_time(topk40, graph=True)
 
         def sample40(t):
             topk40(t)
             ctx.packed_topk_sample(h_top, 40, 0.8, 0.95, 30.0, 0.37, h_best)
 
-        us_sample = head_time(sample40)
+        us_sample = head_time(sample40, graph=True)
         # the sampler kernel on its own list of 40 (the list the last call left)
         us_sampler = head_time(lambda t: ctx.packed_topk_sample(h_top, 40, 0.8, 0.95, 30.0, 0.37, h_best), n=200)
         head = {"N": HN, "K": HK, "group": HG, "bits": BITS, "weight_bytes": head_bytes,
@@ -622,7 +636,7 @@ def main():
                 "scores_then_top40": {"us": round(us_topk, 2), "GBps": round((head_bytes + HN * 8) / us_topk / 1e3, 1)},
                 "scores_top40_sample": {"us": round(us_sample, 2), "sampler_alone_us": round(us_sampler, 2)},
                 "note": "lm_head 262144 x 1536, 4-bit group 32 (251 MB), two copies alternated; greedy_fused = aq_qmv_greedy "
-                        "(8 bytes out); scores_then_top40 = aq_qmv_scores + aq_packed_topk"}
+                        "(8 bytes out); scores_then_top40 = aq_qmv_scores + aq_packed_topk (both top40 legs: a graph of 40 calls, replayed)"}
         for t in pool[0] + pool[1] + (hx, h_logits, h_best, h_scores, h_top):
             t.free()
 

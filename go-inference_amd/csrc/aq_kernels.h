@@ -178,6 +178,8 @@ hipError_t pack_scores_launch(const float* scores, int M, int N, const int32_t* 
 constexpr int kTopKMax = 64;
 constexpr int kTopKPerLane = 16;                    // values a lane sorts in registers
 constexpr int kTopKSegment = 64 * kTopKPerLane;     // values one wavefront reduces to top_k
+constexpr int kTopKCandidates = 1024;               // entries the threshold path orders in one workgroup
+constexpr int kTopKThresholdSegments = 1024;        // most segments whose maxima a wavefront holds in registers
 size_t packed_topk_scratch_entries(int64_t count, int top_k);
 hipError_t packed_topk_launch(const unsigned long long* in, int64_t count, int top_k, unsigned long long* out,
                               unsigned long long* scratch, hipStream_t stream);

@@ -178,11 +178,9 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
 // sorts its kTopKPerLane values in registers; then, top_k times, the wavefront takes the largest of the 64
 // list heads (high words first, then the low words of the lanes that hold that high word) and the winning
 // lane drops its head.  Entries past `count` read as 0, which is also the "no candidate" value.
-__global__ __launch_bounds__(256) void packed_topk_kernel(const unsigned long long* __restrict__ in, int64_t count, int top_k,
-                                                          unsigned long long* __restrict__ out) {
+__device__ __forceinline__ void topk_reduce_segment(const unsigned long long* __restrict__ in, int64_t count, int top_k,
+                                                    unsigned long long* __restrict__ out, int64_t segment, int lane) {
     constexpr int V = kTopKPerLane;
-    const int lane = threadIdx.x & (kWave - 1);
-    const int64_t segment = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     const int64_t begin = segment * kTopKSegment;
     if (begin >= count) return;  // whole wavefronts
     unsigned long long v[V];
@@ -227,28 +225,216 @@ __global__ __launch_bounds__(256) void packed_topk_kernel(const unsigned long lo
     if (lane < top_k) out[segment * top_k + lane] = mine;
 }
 
+// A round of the segment-by-segment reduction.  With `gate` set the round only runs when the candidate list of
+// the threshold path below has overflowed (*gate > kTopKCandidates); otherwise it leaves at once.
+__global__ __launch_bounds__(256) void packed_topk_kernel(const unsigned long long* __restrict__ in, int64_t count, int top_k,
+                                                          unsigned long long* __restrict__ out, const uint32_t* gate) {
+    if (gate && *gate <= (uint32_t)kTopKCandidates) return;
+    topk_reduce_segment(in, count, top_k, out, (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6), threadIdx.x & (kWave - 1));
+}
+
+// Threshold path, for inputs of many segments.  The top_k-th largest of the segment maxima is a value T that
+// at least top_k entries reach (the maxima themselves), so the top_k largest entries all lie among the entries
+// >= T; for scores that are not arranged by rank that set is a little over top_k entries, and one workgroup
+// orders it by counting.  Three launches: maxima, filter, finish.  When more than kTopKCandidates entries
+// reach T (long runs of equal scores, an input sorted by score) the finish launch runs the first round of the
+// segment-by-segment reduction instead and the gated rounds after it complete the answer.
+// A wavefront of these two kernels takes a piece of 64 * V entries: V is the largest of 16, 4, 1 that leaves at
+// least top_k pieces.
+template <int V>
+__global__ __launch_bounds__(256) void topk_segment_max_kernel(const unsigned long long* __restrict__ in, int64_t count,
+                                                               unsigned long long* __restrict__ segmax, uint32_t* counter) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t segment = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t begin = segment * (kWave * V);
+    if (blockIdx.x == 0 && threadIdx.x == 0) *counter = 0;
+    if (begin >= count) return;
+    unsigned long long m = 0;
+#pragma unroll
+    for (int j = 0; j < V; j++) {
+        const int64_t i = begin + j * kWave + lane;
+        const unsigned long long v = i < count ? in[i] : 0ull;
+        m = v > m ? v : m;
+    }
+    const uint32_t hi = (uint32_t)(m >> 32), lo = (uint32_t)m;
+    const uint32_t best_hi = wave_max_u32(hi);
+    const uint32_t best_lo = wave_max_u32(hi == best_hi ? lo : 0u);
+    if (lane == 0) segmax[segment] = ((unsigned long long)best_hi << 32) | best_lo;
+}
+
+// The largest t, a multiple of 2^kTopKThresholdShift, that at least top_k of the high words `key` (SV a lane, zero
+// where there is none) reach: built bit by bit from the top, every count one ballot.
+constexpr int kTopKThresholdShift = 8;
+
+template <int SV>
+__device__ __forceinline__ uint32_t topk_threshold_key(const uint32_t (&key)[SV], int top_k) {
+    uint32_t t = 0;
+    for (int bit = 31; bit >= kTopKThresholdShift; bit--) {
+        const uint32_t trial = t | (1u << bit);
+        int reach = 0;
+#pragma unroll
+        for (int j = 0; j < SV; j++) reach += __popcll(__ballot(key[j] >= trial));
+        if (reach >= top_k) t = trial;
+    }
+    return t;
+}
+
+template <int SV>
+__device__ __forceinline__ uint32_t topk_threshold(const unsigned long long* __restrict__ segmax, int segments, int top_k,
+                                                   int lane) {
+    uint32_t key[SV];
+#pragma unroll
+    for (int j = 0; j < SV; j++) key[j] = j * kWave + lane < segments ? (uint32_t)(segmax[j * kWave + lane] >> 32) : 0u;
+    return topk_threshold_key<SV>(key, top_k);
+}
+
+template <int V>
+__global__ __launch_bounds__(256) void topk_filter_kernel(const unsigned long long* __restrict__ in, int64_t count, int top_k,
+                                                          const unsigned long long* __restrict__ segmax, int segments,
+                                                          uint32_t* counter, unsigned long long* __restrict__ cand) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t segment = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t begin = segment * (kWave * V);
+    if (begin >= count) return;
+    unsigned long long v[V];
+#pragma unroll
+    for (int j = 0; j < V; j++) {
+        const int64_t i = begin + j * kWave + lane;
+        v[j] = i < count ? in[i] : 0ull;
+    }
+    // T: at least top_k segment maxima have a high word (the score) >= T's, so at least top_k entries reach T
+    // and the top_k largest are among them; every wavefront works T out for itself from the same list
+    const uint32_t t_key = segments <= 4 * kWave ? topk_threshold<4>(segmax, segments, top_k, lane)
+                                                 : topk_threshold<kTopKThresholdSegments / kWave>(segmax, segments, top_k, lane);
+    const unsigned long long t = (unsigned long long)t_key << 32;
+    unsigned long long mask[V];
+    int total = 0;
+#pragma unroll
+    for (int j = 0; j < V; j++) {
+        mask[j] = __ballot(v[j] >= t && v[j] != 0);
+        total += __popcll(mask[j]);
+    }
+    if (total == 0) return;  // uniform over the wavefront
+    uint32_t base = 0;
+    if (lane == 0) base = atomicAdd(counter, (uint32_t)total);
+    base = (uint32_t)__builtin_amdgcn_readfirstlane((int)base);
+    const unsigned long long below = (1ull << lane) - 1;
+#pragma unroll
+    for (int j = 0; j < V; j++) {
+        const uint32_t pos = base + (uint32_t)__popcll(mask[j] & below);
+        if (((mask[j] >> lane) & 1) && pos < (uint32_t)kTopKCandidates) cand[pos] = v[j];
+        base += (uint32_t)__popcll(mask[j]);
+    }
+}
+
+// The candidates are distinct unless the input repeats a value, so an entry's place in the output is the number
+// of candidates above it (equal values take consecutive places in list order).
+__global__ __launch_bounds__(256) void topk_finish_kernel(const unsigned long long* __restrict__ in, int64_t count, int top_k,
+                                                          const uint32_t* counter, const unsigned long long* __restrict__ cand,
+                                                          unsigned long long* __restrict__ out,
+                                                          unsigned long long* __restrict__ round_out) {
+    const uint32_t n = *counter;
+    if (n > (uint32_t)kTopKCandidates) {
+        topk_reduce_segment(in, count, top_k, round_out, (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6),
+                            threadIdx.x & (kWave - 1));
+        return;
+    }
+    if (blockIdx.x != 0) return;
+    constexpr int PER = kTopKCandidates / 256;
+    __shared__ unsigned long long c[kTopKCandidates];
+    unsigned long long mine[PER];
+    int rank[PER];
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+        const uint32_t idx = threadIdx.x + 256u * i;
+        mine[i] = idx < n ? cand[idx] : 0ull;
+        c[idx] = mine[i];
+        rank[i] = 0;
+    }
+    __syncthreads();
+    for (uint32_t o = 0; o < n; o++) {
+        const unsigned long long other = c[o];
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            const uint32_t idx = threadIdx.x + 256u * i;
+            rank[i] += (other > mine[i] || (other == mine[i] && o < idx)) ? 1 : 0;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+        const uint32_t idx = threadIdx.x + 256u * i;
+        if (idx < n && rank[i] < top_k) out[rank[i]] = mine[i];
+    }
+    if (threadIdx.x >= n && threadIdx.x < (uint32_t)top_k) out[threadIdx.x] = 0ull;  // fewer candidates than top_k
+}
+
 static int64_t topk_segments(int64_t count) { return (count + kTopKSegment - 1) / kTopKSegment; }
+
+// Entries a lane takes on the threshold path, 0 when the input goes segment by segment: the path needs at least
+// top_k maxima and a wavefront keeps the whole list of maxima in registers.
+static int topk_threshold_per_lane(int64_t count, int top_k) {
+    if (count <= kTopKSegment) return 0;
+    for (int v : {16, 4, 1}) {
+        const int64_t pieces = (count + kWave * v - 1) / (kWave * v);
+        if (pieces >= top_k && pieces <= kTopKThresholdSegments) return v;
+    }
+    return 0;
+}
+
+constexpr int kTopKHeader = 2;  // scratch[0]: candidate counter (its low word)
 
 size_t packed_topk_scratch_entries(int64_t count, int top_k) {
     if (count <= kTopKSegment) return 0;
     // first round's output, then the second round's beside it (every later round is smaller)
     const int64_t c1 = topk_segments(count) * top_k;
     const int64_t c2 = c1 > kTopKSegment ? topk_segments(c1) * top_k : 0;
-    return (size_t)(c1 + c2);
+    int64_t total = c1 + c2;
+    if (topk_threshold_per_lane(count, top_k)) total += kTopKHeader + kTopKThresholdSegments + kTopKCandidates;
+    return (size_t)total;
+}
+
+template <int V>
+static void topk_threshold_launch(const unsigned long long* in, int64_t count, int top_k, unsigned long long* segmax,
+                                  uint32_t* counter, unsigned long long* cand, hipStream_t stream) {
+    const int64_t pieces = (count + kWave * V - 1) / (kWave * V);
+    const dim3 grid((unsigned)((pieces + 3) / 4));
+    hipLaunchKernelGGL(topk_segment_max_kernel<V>, grid, dim3(256), 0, stream, in, count, segmax, counter);
+    hipLaunchKernelGGL(topk_filter_kernel<V>, grid, dim3(256), 0, stream, in, count, top_k, segmax, (int)pieces, counter, cand);
 }
 
 hipError_t packed_topk_launch(const unsigned long long* in, int64_t count, int top_k, unsigned long long* out,
                               unsigned long long* scratch, hipStream_t stream) {
     if (top_k <= 0 || top_k > kTopKMax || count <= 0) return hipErrorInvalidValue;
-    const int64_t c1 = topk_segments(count) * top_k;
+    const int64_t first = topk_segments(count);
+    const int64_t c1 = first * top_k;
     unsigned long long* bufs[2] = {scratch, scratch + c1};
+    const uint32_t* gate = nullptr;
     int which = 0;
     const unsigned long long* src = in;
     int64_t n = count;
+    if (const int per_lane = topk_threshold_per_lane(count, top_k)) {
+        const int64_t c2 = c1 > kTopKSegment ? topk_segments(c1) * top_k : 0;
+        unsigned long long* extra = scratch + c1 + c2;
+        uint32_t* counter = reinterpret_cast<uint32_t*>(extra);
+        unsigned long long* segmax = extra + kTopKHeader;
+        unsigned long long* cand = segmax + kTopKThresholdSegments;
+        if (per_lane == 16) topk_threshold_launch<16>(in, count, top_k, segmax, counter, cand, stream);
+        else if (per_lane == 4) topk_threshold_launch<4>(in, count, top_k, segmax, counter, cand, stream);
+        else topk_threshold_launch<1>(in, count, top_k, segmax, counter, cand, stream);
+        hipLaunchKernelGGL(topk_finish_kernel, dim3((unsigned)((first + 3) / 4)), dim3(256), 0, stream, in, count, top_k, counter,
+                           cand, out, bufs[0]);
+        hipError_t rc = hipGetLastError();
+        if (rc != hipSuccess) return rc;
+        gate = counter;
+        src = bufs[0];
+        n = c1;
+        which = 1;
+    }
     while (true) {
         const int64_t segments = topk_segments(n);
         unsigned long long* dst = segments == 1 ? out : bufs[which];
-        hipLaunchKernelGGL(packed_topk_kernel, dim3((unsigned)((segments + 3) / 4)), dim3(256), 0, stream, src, n, top_k, dst);
+        hipLaunchKernelGGL(packed_topk_kernel, dim3((unsigned)((segments + 3) / 4)), dim3(256), 0, stream, src, n, top_k, dst,
+                           gate);
         hipError_t rc = hipGetLastError();
         if (rc != hipSuccess || segments == 1) return rc;
         src = dst;

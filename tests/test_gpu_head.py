@@ -132,7 +132,8 @@ def test_greedy_ties_and_nonfinite_rows(ctx, orc):
     dw.free()
 
 
-@pytest.mark.parametrize("count,top_k", [(1, 1), (100, 8), (2048, 64), (2049, 5), (262144, 40), (70000, 64), (5, 8)])
+@pytest.mark.parametrize("count,top_k", [(1, 1), (100, 8), (2048, 64), (2049, 5), (262144, 40), (70000, 64), (5, 8), (32000, 40), (4097, 64),
+                                         (151936, 40), (1100000, 16)])
 def test_packed_topk_sorted_descending(ctx, count, top_k):
     import aq_mi355
     say("packed topk", count, top_k)
@@ -147,6 +148,40 @@ def test_packed_topk_sorted_descending(ctx, count, top_k):
     got = _u64(dout, top_k)
     want = np.sort(packed)[::-1][:top_k]
     want = np.concatenate([want, np.zeros(top_k - want.size, np.uint64)])
+    assert np.array_equal(got, want)
+    din.free()
+    dout.free()
+
+
+@pytest.mark.parametrize("shape", ["by_rank", "by_rank_reversed", "nearly_empty", "empty", "one_score", "repeats"])
+@pytest.mark.parametrize("count,top_k", [(262144, 40), (65536, 64), (9000, 8), (1048576, 3), (40000, 64), (5000, 50)])
+def test_packed_topk_arranged_inputs(ctx, shape, count, top_k):
+    """Inputs that defeat a threshold taken from per-segment maxima (scores arranged by rank, one score
+    everywhere) or leave fewer candidates than top_k still give the sorted top_k, zero-padded."""
+    say("packed topk arranged", shape, count, top_k)
+    rng = np.random.default_rng(count * 7 + top_k)
+    idx = np.arange(count, dtype=np.uint64)
+    low = np.uint64(0xFFFFFFFF) - idx
+    if shape == "by_rank":
+        packed = ((np.uint64(0x90000000) - idx) << np.uint64(32)) | low
+    elif shape == "by_rank_reversed":
+        packed = ((np.uint64(0x80000000) + idx) << np.uint64(32)) | low
+    elif shape == "nearly_empty":
+        packed = np.zeros(count, np.uint64)
+        where = rng.choice(count, top_k - 1, replace=False)
+        packed[where] = (np.uint64(0xC0000000) << np.uint64(32)) | low[where]
+    elif shape == "empty":
+        packed = np.zeros(count, np.uint64)
+    elif shape == "one_score":
+        packed = (np.uint64(0xC1234567) << np.uint64(32)) | low
+    else:
+        packed = rng.integers(1, 50, count).astype(np.uint64) << np.uint64(40)   # the same value many times over
+    din, dout = ctx.to_device(packed), ctx.to_device(np.full(top_k, 0xDEADBEEF, np.uint64))
+    for _ in range(2):                                                           # the workspace is reused
+        ctx.packed_topk(din, count, top_k, dout)
+    ctx.sync()
+    got = _u64(dout, top_k)
+    want = np.sort(packed)[::-1][:top_k]
     assert np.array_equal(got, want)
     din.free()
     dout.free()
