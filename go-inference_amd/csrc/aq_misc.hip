@@ -173,80 +173,120 @@ __global__ __launch_bounds__(256) void qmv_generic_kernel(const QmvArgs a, int b
     }
 }
 
-// Six-bit codes in groups of 16 or 32 (the layouts GGUF Q6_K and Q5_K tensors repack to): one wavefront per row as
-// above, but a lane takes 16 codes = three whole words at a time (a wavefront reads 768 contiguous bytes of codes per
-// step), decodes them with shifts of one 64-bit and one 32-bit piece, and uses the group form of the sum,
-// scale * sum(code * x) + bias * sum(x), with one scale and bias per lane and step (16 codes never straddle a group).
-template <int GS>
-__global__ __launch_bounds__(256) void qmv_six_kernel(const QmvArgs a, int gather) {
+// Six-bit codes in groups of 16, 32, 64 or 128 (16 / 32: the layouts GGUF Q6_K and Q5_K tensors repack to; 64: MLX's
+// own six-bit form).  A lane takes 16 codes = three whole words at a time (a wavefront reads 768 contiguous bytes
+// of codes per step), turns each pair of codes into a pair of bf16 128 + code (0x4300 | code, exact) and feeds
+// v_dot2_f32_bf16 with the matching pair of x; the group form of the sum, scale * sum((128 + code) * x) +
+// (bias - 128 * scale) * sum(x), has one scale and bias per lane and step (16 codes never straddle a group).
+// A wavefront carries R rows through the same slice of x, so x and its sum are fetched and formed once per R rows,
+// and up to MR rows of x share each decoded row.  14336 x 4096, groups of 64: 15.8 us for one row of x (the
+// float form one row at a time took 16.7, the any-width kernel 117); a form that kept x in LDS and the loads a
+// ring of four steps ahead over persistent wavefronts measured slower (16.3-17.0 us) and is not kept.
+__device__ __forceinline__ void six_pairs(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t (&p)[8]) {
+    const uint32_t f[8] = {w0,       w0 >> 12, __builtin_amdgcn_alignbit(w1, w0, 24), w1 >> 4,
+                           w1 >> 16, __builtin_amdgcn_alignbit(w2, w1, 28), w2 >> 8,  w2 >> 20};
+#pragma unroll
+    for (int i = 0; i < 8; i++) p[i] = (f[i] & 63u) | ((f[i] << 10) & 0x003F0000u) | 0x43004300u;
+}
+
+template <int GS, int MR, int R>
+__global__ __launch_bounds__(256) void qmv_six_kernel(const QmvArgs a, int gather, int m0) {
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
-    const int row = blockIdx.x * 4 + wave;
+    const int row0 = (blockIdx.x * 4 + wave) * R;
     const int K = a.K, N = a.N;
-    if (row >= N) return;
+    if (row0 >= N) return;
     const int64_t words = (int64_t)K * 6 / 32;
     const int gpr = K / GS;
     const uint32_t* wbase = a.w;
     const uint16_t* sbase = a.s;
     const uint16_t* bbase = a.b;
-    const uint16_t* xbase = a.x;
-    int64_t yoff = 0;
-    int m_count = a.M;
+    const uint16_t* xbase = a.x + (int64_t)m0 * K;
+    int64_t yoff = (int64_t)m0 * N;
+    int m_count = a.M - m0 < MR ? a.M - m0 : MR;
     bool ok = true;
     if (gather) {
         const int z = blockIdx.y;
         const int e = a.rhs[z];
         int xr = a.lhs ? a.lhs[z] : 0;
         ok = (unsigned)e < (unsigned)a.num_experts && (unsigned)xr < (unsigned)a.x_rows;
-        const int64_t row0 = ok ? ((int64_t)e * a.expert_rows + a.row_base) : 0;
+        const int64_t slab0 = ok ? ((int64_t)e * a.expert_rows + a.row_base) : 0;
         if (!ok) xr = 0;
-        wbase += row0 * words;
-        sbase += row0 * gpr;
-        bbase += row0 * gpr;
-        xbase += (int64_t)xr * K;
+        wbase += slab0 * words;
+        sbase += slab0 * gpr;
+        bbase += slab0 * gpr;
+        xbase = a.x + (int64_t)xr * K;
         yoff = (int64_t)z * N;
         m_count = 1;
     }
-    const uint32_t* wr = wbase + (int64_t)row * words;
-    const uint16_t* sr = sbase + (int64_t)row * gpr;
-    const uint16_t* br = bbase + (int64_t)row * gpr;
-    for (int m0 = 0; m0 < m_count; m0 += 4) {
-        float acc[4] = {0.f, 0.f, 0.f, 0.f};
-        for (int k0 = lane * 16; k0 < K; k0 += kWave * 16) {
-            const uint32_t* wp = wr + (k0 >> 4) * 3;
-            const uint32_t w0 = wp[0], w1 = wp[1], w2 = wp[2];
-            const float scale = bf16_bits_to_f32(sr[k0 / GS]), bias = bf16_bits_to_f32(br[k0 / GS]);
-            const uint64_t lo = (uint64_t)w0 | (uint64_t)w1 << 32;
-            float c[16];
+    const uint32_t* wr[R];
+    const uint16_t* sr[R];
+    const uint16_t* br[R];
 #pragma unroll
-            for (int i = 0; i < 10; i++) c[i] = (float)(uint32_t)((lo >> (6 * i)) & 63u);
-            c[10] = (float)((uint32_t)(lo >> 60) | ((w2 & 3u) << 4));
+    for (int r = 0; r < R; r++) {
+        const int row = row0 + r < N ? row0 + r : N - 1;  // a ragged last set repeats its last row
+        wr[r] = wbase + (int64_t)row * words;
+        sr[r] = sbase + (int64_t)row * gpr;
+        br[r] = bbase + (int64_t)row * gpr;
+    }
+    float acc[R][MR];
 #pragma unroll
-            for (int i = 0; i < 5; i++) c[11 + i] = (float)((w2 >> (2 + 6 * i)) & 63u);
+    for (int r = 0; r < R; r++)
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                if (m0 + j < m_count) {
-                    const uint4* xp = reinterpret_cast<const uint4*>(xbase + (int64_t)(m0 + j) * K + k0);
-                    const uint4 x0 = xp[0], x1 = xp[1];
-                    const uint32_t xw[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
-                    float dot = 0.f, xs = 0.f;
+        for (int m = 0; m < MR; m++) acc[r][m] = 0.f;
+#pragma unroll 2
+    for (int k0 = lane * 16; k0 < K; k0 += kWave * 16) {
+        uint32_t w[R][3];
+        uint32_t sb[R][2];
 #pragma unroll
-                    for (int i = 0; i < 8; i++) {
-                        const float xa = __uint_as_float(xw[i] << 16), xb = __uint_as_float(xw[i] & 0xffff0000u);
-                        dot = __fmaf_rn(c[2 * i], xa, dot);
-                        dot = __fmaf_rn(c[2 * i + 1], xb, dot);
-                        xs += xa + xb;
-                    }
-                    acc[j] += scale * dot + bias * xs;
-                }
-            }
+        for (int r = 0; r < R; r++) {
+            const uint32_t* wp = wr[r] + (k0 >> 4) * 3;
+            w[r][0] = wp[0];
+            w[r][1] = wp[1];
+            w[r][2] = wp[2];
+            sb[r][0] = sr[r][k0 / GS];
+            sb[r][1] = br[r][k0 / GS];
+        }
+        uint32_t xw[MR][8];
+        float xs[MR];
+#pragma unroll
+        for (int m = 0; m < MR; m++) {
+            const int mm = m < m_count ? m : 0;
+            const uint4* xp = reinterpret_cast<const uint4*>(xbase + (int64_t)mm * K + k0);
+            const uint4 x0 = xp[0], x1 = xp[1];
+            xw[m][0] = x0.x, xw[m][1] = x0.y, xw[m][2] = x0.z, xw[m][3] = x0.w;
+            xw[m][4] = x1.x, xw[m][5] = x1.y, xw[m][6] = x1.z, xw[m][7] = x1.w;
         }
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            float tot = wave_sum(acc[j]);
+        for (int m = 0; m < MR; m++) {
+            float t = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) t = dot2_bf16(xw[m][i], 0x3F803F80u, t);
+            xs[m] = t;
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            uint32_t p[8];
+            six_pairs(w[r][0], w[r][1], w[r][2], p);
+            const float scale = bf16_bits_to_f32(sb[r][0]), bias = bf16_bits_to_f32(sb[r][1]);
+            const float shift = __fmaf_rn(-128.f, scale, bias);
+#pragma unroll
+            for (int m = 0; m < MR; m++) {
+                float d = 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; i++) d = dot2_bf16(p[i], xw[m][i], d);
+                acc[r][m] += __fmaf_rn(scale, d, shift * xs[m]);
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+#pragma unroll
+        for (int m = 0; m < MR; m++) {
+            float tot = wave_sum(acc[r][m]);
             if (!ok) tot = 0.0f;
-            if (lane == 0 && m0 + j < m_count) {
-                const int64_t o = yoff + (int64_t)(m0 + j) * N + row;
+            if (lane == 0 && m < m_count && row0 + r < N) {
+                const int64_t o = yoff + (int64_t)m * N + row0 + r;
                 if (a.out_f32) {
                     reinterpret_cast<float*>(a.y)[o] = tot;
                 } else {
@@ -257,8 +297,25 @@ __global__ __launch_bounds__(256) void qmv_six_kernel(const QmvArgs a, int gathe
     }
 }
 
+template <int GS>
+static hipError_t qmv_six_launch(const QmvArgs& a, bool gather, hipStream_t stream) {
+    constexpr int R = 4;
+    const dim3 grid((unsigned)((a.N + 4 * R - 1) / (4 * R)), gather ? (unsigned)a.routes : 1u, 1u);
+    const int rows = gather ? 1 : a.M;
+    for (int m0 = 0; m0 < rows; m0 += 4) {
+        const int left = rows - m0;
+        if (left == 1)
+            hipLaunchKernelGGL((qmv_six_kernel<GS, 1, R>), grid, dim3(256), 0, stream, a, gather ? 1 : 0, m0);
+        else if (left == 2)
+            hipLaunchKernelGGL((qmv_six_kernel<GS, 2, R>), grid, dim3(256), 0, stream, a, gather ? 1 : 0, m0);
+        else
+            hipLaunchKernelGGL((qmv_six_kernel<GS, 4, R>), grid, dim3(256), 0, stream, a, gather ? 1 : 0, m0);
+    }
+    return hipGetLastError();
+}
+
 bool qmv_six_eligible(const QmvArgs& a, int bits, int group_size) {
-    return bits == 6 && (group_size == 16 || group_size == 32) && a.K % 16 == 0 &&
+    return bits == 6 && (group_size == 16 || group_size == 32 || group_size == 64 || group_size == 128) && a.K % 16 == 0 &&
            (reinterpret_cast<uintptr_t>(a.x) & 15) == 0 && (reinterpret_cast<uintptr_t>(a.w) & 3) == 0 &&
            (reinterpret_cast<uintptr_t>(a.s) & 1) == 0 && (reinterpret_cast<uintptr_t>(a.b) & 1) == 0;
 }
@@ -266,11 +323,9 @@ bool qmv_six_eligible(const QmvArgs& a, int bits, int group_size) {
 hipError_t qmv_generic_launch(const QmvArgs& a, int bits, int group_size, bool gather, hipStream_t stream) {
     dim3 grid((unsigned)((a.N + 3) / 4), gather ? (unsigned)a.routes : 1u, 1u);
     if (qmv_six_eligible(a, bits, group_size)) {
-        if (group_size == 16)
-            hipLaunchKernelGGL(qmv_six_kernel<16>, grid, dim3(256), 0, stream, a, gather ? 1 : 0);
-        else
-            hipLaunchKernelGGL(qmv_six_kernel<32>, grid, dim3(256), 0, stream, a, gather ? 1 : 0);
-        return hipGetLastError();
+        return group_size == 16 ? qmv_six_launch<16>(a, gather, stream)
+             : group_size == 32 ? qmv_six_launch<32>(a, gather, stream)
+             : group_size == 64 ? qmv_six_launch<64>(a, gather, stream) : qmv_six_launch<128>(a, gather, stream);
     }
     hipLaunchKernelGGL(qmv_generic_kernel, grid, dim3(256), 0, stream, a, bits, group_size, gather ? 1 : 0);
     return hipGetLastError();

@@ -108,7 +108,7 @@ int qmm_dispatch(hipStream_t stream, Workspace* ws, int cu_count, int forced, co
         q.M = M;
         q.out_f32 = out_f32 ? 1 : 0;
         q.routes = 1;
-        *last_variant = "qmv_generic";
+        *last_variant = qmv_six_eligible(q, bits, group_size) ? "qmv_six" : "qmv_generic";
         hipError_t rc = qmv_generic_launch(q, bits, group_size, false, stream);
         if (rc != hipSuccess) return fail((int)rc, "rocm.hip.hipLaunchKernel: HIP returned %d", (int)rc);
         return AQ_OK;

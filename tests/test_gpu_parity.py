@@ -110,7 +110,8 @@ def test_qmv_ragged_and_thin_shapes(ctx, orc, bits, gs, K, N, M):
 
 @pytest.mark.parametrize("bits,gs,K,N,M", [(2, 64, 640, 9, 1), (3, 64, 256, 9, 1), (5, 64, 256, 9, 2), (6, 32, 192, 11, 1),
                                            (6, 16, 64, 5, 3), (4, 16, 64, 5, 1), (2, 128, 256, 24, 5),
-                                           (6, 16, 1040, 33, 6), (6, 32, 4096, 70, 2), (6, 32, 1056, 7, 5), (6, 16, 16, 3, 1)])
+                                           (6, 16, 1040, 33, 6), (6, 32, 4096, 70, 2), (6, 32, 1056, 7, 5), (6, 16, 16, 3, 1),
+                                           (6, 64, 4096, 70, 1), (6, 64, 2112, 19, 3), (6, 128, 1280, 18, 4), (6, 64, 1088, 37, 7)])
 def test_qmv_other_widths_generic_kernel(ctx, orc, bits, gs, K, N, M):
     say("qmv generic", bits, gs, K, N, M)
     rng = np.random.default_rng(bits * 100 + K)
@@ -122,8 +123,8 @@ def test_qmv_other_widths_generic_kernel(ctx, orc, bits, gs, K, N, M):
     dw = DeviceAffine(ctx, words, s, b)
     acc = run_qmv(ctx, x, dw, M, K, N, gs, bits, True)
     check_accumulators(acc, ref, "generic")
-    # six-bit codes in groups of 16 / 32 (what GGUF Q6_K / Q5_K repack to) have a kernel of their own
-    if bits == 6 and gs in (16, 32) and K % 16 == 0 and M <= 4:
+    # six-bit codes in groups of 16 / 32 (what GGUF Q6_K / Q5_K repack to) and 64 / 128 have a kernel of their own
+    if bits == 6 and gs in (16, 32, 64, 128) and K % 16 == 0 and M <= 4:
         assert ctx.last_variant(0) == "qmv_six"
     else:                                # more than four rows go through the row-block loop, which reports its own name
         assert ctx.last_variant(0) in ("qmv_generic", "qmv_six")

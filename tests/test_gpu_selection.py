@@ -33,6 +33,8 @@ CASES = [
     (4, 64, 3, 2880, ("qmvb_", "qmv_b4_")),
     (3, 64, 2, 512, ("qmv_generic",)),               # any width
     (6, 32, 1, 512, ("qmv_six",)),
+    (6, 64, 1, 512, ("qmv_six",)),
+    (6, 64, 4, 4096, ("qmv_six",)),
     (4, 64, 48, 4096, ("qmmf_",)),                   # 33..64 rows, K a multiple of 256: K shared out over workgroups
     (8, 64, 24, 4096, ("qmmf_",)),                   # 8 bit beyond 16 rows
     (4, 64, 20, 320, ("qmmt_b4_mb1_nb2_wm1_wn4",)),  # fewer than 64 rows, K no multiple of 256: 32 x 256 tiles
