@@ -70,6 +70,7 @@ struct aq_ctx {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     std::mutex mu;
     int forced[2] = {-1, -1};
+    unsigned families_off = 0;  // bit per kernel family that AQ_MI355_DISABLE names: the selection skips them
     const char* last_variant[2] = {"", ""};
     int cu_count = 0;
     aq::Workspace ws;       // scratch of the matmul path and of the unfused fallbacks (aq_qmm.h)
@@ -143,6 +144,28 @@ enum { kFamDot2, kFamBlk, kFamDiag, kFamTok, kFamCount };
 // and the kernel that takes any geometry.
 enum { kFamTiles = kFamCount, kFamTilesLarge, kFamGeneric };
 
+// Route switches, the counterpart of the reference's GO_ROCM_DISABLE_* variables (hip_projection_launch.go:95-137):
+// AQ_MI355_DISABLE=name[,name...] over dot2, blk, diag, tok, tiles, read when a context is created, takes those
+// families out of the selection of every entry point, which then falls through to the next family that takes the
+// shape (the any-width kernel cannot be switched off).  There is no code-object override like
+// GO_ROCM_KERNEL_HSACO (hip_kernel_module.go:14-35): the kernels are linked into this library.
+unsigned families_off_from_env(const char* value) {
+    static const struct { const char* name; unsigned bits; } kNames[] = {
+        {"dot2", 1u << kFamDot2}, {"blk", 1u << kFamBlk}, {"diag", 1u << kFamDiag}, {"tok", 1u << kFamTok},
+        {"tiles", (1u << kFamTiles) | (1u << kFamTilesLarge)}};
+    unsigned off = 0;
+    if (!value) return off;
+    const char* p = value;
+    while (*p) {
+        const char* e = p;
+        while (*e && *e != ',') e++;
+        for (const auto& n : kNames)
+            if (strlen(n.name) == (size_t)(e - p) && strncmp(n.name, p, (size_t)(e - p)) == 0) off |= n.bits;
+        p = *e ? e + 1 : e;
+    }
+    return off;
+}
+
 struct QmvFamily {
     int (*count)();
     const aq::QmvVariant* (*variant)(int);
@@ -208,7 +231,7 @@ const QmvRule kQmvRules[] = {
     {8, 0, 0, 1, 1, kFamBlk},               // (a single row of 4-bit codes is faster on the dot2 kernels)
     {0, 0, 0, 5, INT32_MAX, kFamTiles},     // K shared out over workgroups for few rows; any geometry
     {0, 0, 0, 1, 4, kFamDot2},
-    {0, 0, 0, 1, 4, kFamGeneric},
+    {0, 0, 0, 1, INT32_MAX, kFamGeneric},   // beyond four rows only when the tile kernels are switched off
 };
 
 constexpr int kPass = INT32_MIN;  // a family's answer when the shape is not its to run
@@ -306,7 +329,7 @@ int launch_qmv_rows(aq_ctx* ctx, aq::QmvArgs a, int group_size, int bits, bool g
     }
     for (const QmvRule& r : kQmvRules) {
         if ((r.bits && r.bits != bits) || (r.group_size && r.group_size != group_size) || (r.gather != 0) != gather ||
-            a.M < r.m_lo || a.M > r.m_hi)
+            a.M < r.m_lo || a.M > r.m_hi || (ctx->families_off >> r.family & 1))
             continue;
         const int rc = run_family(r.family, ctx, a, group_size, bits, gather, -1);
         if (rc != kPass) return rc;
@@ -349,6 +372,7 @@ int aq_create(int device, aq_ctx** out) {
     if (!ctx) return fail(AQ_ERR_NOMEM, "aq_create: out of host memory");
     ctx->device = device;
     ctx->cu_count = prop.multiProcessorCount;
+    ctx->families_off = families_off_from_env(getenv("AQ_MI355_DISABLE"));
     snprintf(ctx->name, sizeof ctx->name, "%s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
     rc = hipStreamCreateWithFlags(&ctx->own_stream, hipStreamNonBlocking);
     if (rc == hipSuccess) rc = hipEventCreate(&ctx->ev0);
@@ -608,7 +632,7 @@ int aq_qmv_multi(aq_ctx* ctx, const void* x, int count, const void* const* packe
             std::lock_guard<std::mutex> lk(ctx->mu);
             // the kernels aq_qmv would pick for each member, in one grid
             // (every variant with the same split of K computes the same bytes, whatever the rows per workgroup)
-            const int di = aq::qmvd_pick(M, K, (int)total);
+            const int di = (ctx->families_off >> kFamDiag & 1) ? -1 : aq::qmvd_pick(M, K, (int)total);
             if (di >= 0 && aq::qmvd_multi_supported(di)) {
                 bool fits = true;
                 aq::QmvMultiArgs ma{};
@@ -808,7 +832,8 @@ int aq_qmv_gate_up(aq_ctx* ctx, const void* x, const void* gate_packed, const vo
     const bool out_f32 = (flags & AQ_OUT_F32) != 0;
     if (M <= 4 && ctx->forced[0] < 0) {
         // the diagonal-MFMA kernels with one set of wavefronts per matrix
-        const int di = aq::qmvd_pick(1, K, 1 << 20);  // the split of K that a single row gets; any row count shares its bytes
+        // the split of K that a single row gets; any row count shares its bytes
+        const int di = (ctx->families_off >> kFamDiag & 1) ? -1 : aq::qmvd_pick(1, K, 1 << 20);
         aq::QmvArgs a{};
         a.x = static_cast<const uint16_t*>(x);
         a.w = static_cast<const uint32_t*>(gate_packed);
@@ -905,7 +930,7 @@ int aq_gather_qmv_gate_up(aq_ctx* ctx, const void* x, const void* packed, const 
     const bool out_f32 = (flags & AQ_OUT_F32) != 0;
     if (ctx->forced[0] < 0) {
         // the gathered diagonal-MFMA pair kernel: one set of wavefronts on the gate rows, one on the up rows
-        const int di = aq::qmvd_pick_gather(K);
+        const int di = (ctx->families_off >> kFamDiag & 1) ? -1 : aq::qmvd_pick_gather(K);
         aq::QmvArgs a{};
         a.x = static_cast<const uint16_t*>(x);
         a.w = a.w2 = static_cast<const uint32_t*>(packed);
@@ -1193,7 +1218,8 @@ int head_call(aq_ctx* ctx, const char* op, int fuse, const void* x, const void* 
         std::lock_guard<std::mutex> lk(ctx->mu);
         {
             // the diagonal-MFMA kernel aq_qmv would pick for this projection, with the head epilogue
-            const int di = bits != 4 ? -1 : group_size == 32 ? aq::qmvd_pick_g32(1, K, N) : group_size == 64 ? aq::qmvd_pick(1, K, N) : -1;
+            const int di = bits != 4 || (ctx->families_off >> kFamDiag & 1) ? -1
+                           : group_size == 32 ? aq::qmvd_pick_g32(1, K, N) : group_size == 64 ? aq::qmvd_pick(1, K, N) : -1;
             aq::QmvArgs a{};
             a.x = static_cast<const uint16_t*>(x);
             a.w = static_cast<const uint32_t*>(packed);

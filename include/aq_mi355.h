@@ -378,7 +378,12 @@ int aq_proj_quant_matmul_host(aq_ctx *ctx, float *out, const float *x, size_t x_
 /* Kernel-variant introspection and override, for tuning sweeps and profiles.
  * op: 0 = qmv/gather (matvec kernel families), 1 = qmm (matmul kernel families).  variant -1 restores automatic
  * selection (the counterpart of the reference's shape->kernel selector tables,
- * go/engine/hip/hip_projection_launch.go:4925-5064 and its GO_ROCM_* route switches :107-137). */
+ * go/engine/hip/hip_projection_launch.go:4925-5064).
+ * Route switches (the reference's GO_ROCM_DISABLE_* variables, hip_projection_launch.go:95-137): the environment
+ * variable AQ_MI355_DISABLE=name[,name...] over dot2, blk, diag, tok, tiles is read by aq_create and takes those
+ * kernel families out of that context's selection; a call then runs on the next family that takes its shape (the
+ * any-width kernel at the end cannot be switched off).  aq_qmm with five rows and more is not affected.  There is
+ * no code-object override (GO_ROCM_KERNEL_HSACO, hip_kernel_module.go:14-35): the kernels are part of the library. */
 int aq_variant_count(int op);
 const char *aq_variant_name(int op, int variant);
 int aq_force_variant(aq_ctx *ctx, int op, int variant);

@@ -71,3 +71,32 @@ def test_matmul_of_few_rows_runs_as_matvec(ctx, M):
     assert ctx.last_variant(1) == name and name.startswith("qmvd_")
     assert np.array_equal(via_qmv.view(np.uint32), via_qmm.view(np.uint32))
     dw.free()
+
+
+@pytest.mark.parametrize("off,bits,M,K,prefixes", [
+    ("diag", 4, 1, 4096, ("qmv_b4_",)),                 # one row falls through to the dot2 kernels
+    ("diag,dot2", 4, 1, 4096, ("qmv_generic",)),        # ... and past them to the any-width kernel
+    ("tok", 4, 16, 4096, ("qmmf_", "qmvb_")),           # 16 rows without the token-tile kernels
+    ("tok,tiles,blk", 4, 16, 4096, ("qmv_generic",)),
+    ("blk", 8, 1, 4096, ("qmv_b8_",)),
+    ("nothing-by-that-name", 4, 1, 4096, ("qmvd_",)),   # unknown names switch nothing off
+])
+def test_route_switches_from_the_environment(monkeypatch, off, bits, M, K, prefixes):
+    """AQ_MI355_DISABLE, read when a context is created, takes kernel families out of the selection; the call then
+    runs on the next family that takes the shape, with a result inside the same tolerance."""
+    import aq_mi355
+    say("route switches", off, bits, M, K)
+    monkeypatch.setenv("AQ_MI355_DISABLE", off)
+    c = aq_mi355.Context(0)
+    try:
+        words, s, b = F.synthetic_affine(N, K, bits, 64, seed=1200 + bits + M)
+        x = F.synthetic_x(M, K, seed=1250 + M)
+        ref = F.reference_f64(x, words, s, b, bits, 64, K)
+        dw = DeviceAffine(c, words, s, b)
+        acc = run_qmv(c, x, dw, M, K, N, 64, bits, True)
+        name = c.last_variant(0)
+        assert name.startswith(prefixes), (name, prefixes)
+        check_accumulators(acc, ref, name)
+        dw.free()
+    finally:
+        c.close()
