@@ -220,7 +220,7 @@ const QmvRule kQmvRules[] = {
     {4, 64, 0, 1, 8, kFamDiag},             // one row up to 16 steps of 1024 codes, up to 8 rows at 2..4 steps: every row
                                             // of such a call has the bytes of a call with that row alone
     {4, 32, 0, 1, 2, kFamDiag},             // groups of 32: two tokens x eight groups as MFMA rows
-    {8, 64, 0, 5, 16, kFamTok},             // K a multiple of 256 up to 16384: one launch, weights streamed once, no scratch
+    {8, 64, 0, 5, 32, kFamTok},             // K a multiple of 256 up to 16384: one launch, weights streamed once, no scratch
                                             // (up to 4 rows the block-MFMA kernels stay: 14.2 / 15.9 against 14.9 / 14.8 us for
                                             // 1 / 4 rows of 4096 x 14336, and their rows have the bytes of single-row calls)
     {4, 64, 0, 5, 32, kFamTok},             // the same for 4-bit codes, up to 32 rows

@@ -399,14 +399,16 @@ struct QmvTokEntry {
     }
 #define AQ_QMVT16(NW, RS, QW, RING) AQ_QMVT16B(4, NW, RS, QW, RING)
 // the same with two sets of 16 tokens per expanded weight: up to 32 rows of x
-#define AQ_QMVT16X2(NW, RS, QW, RING)                                                                     \
+#define AQ_QMVT16X2B(BITS, NW, RS, QW, RING)                                                              \
     {                                                                                                     \
-        {"qmvt_b4_m32_s2_r" #RS "_w" #NW "_q" #QW "_d" #RING, 4, 32, RS, NW, RING, 0, QW, 6},              \
-            qmv_tok16_kernel<4, NW, RS, QW, RING, 2>, 16 * RS, NW * 32 * (16 * RS) * 4                    \
+        {"qmvt_b" #BITS "_m32_s2_r" #RS "_w" #NW "_q" #QW "_d" #RING, BITS, 32, RS, NW, RING, 0, QW, 6},   \
+            qmv_tok16_kernel<BITS, NW, RS, QW, RING, 2>, 16 * RS, NW * 32 * (16 * RS) * 4                 \
     }
+#define AQ_QMVT16X2(NW, RS, QW, RING) AQ_QMVT16X2B(4, NW, RS, QW, RING)
 static const QmvTokEntry kQmvTokTable[] = {AQ_QMVT16(8, 4, 1, 2), AQ_QMVT16(8, 2, 1, 2), AQ_QMVT16(8, 1, 1, 1),
                                            AQ_QMVT16X2(8, 4, 1, 2), AQ_QMVT16X2(8, 2, 1, 2), AQ_QMVT16X2(8, 1, 1, 1),
-                                           AQ_QMVT16B(8, 8, 4, 1, 2), AQ_QMVT16B(8, 8, 2, 1, 2), AQ_QMVT16B(8, 8, 1, 1, 1)};
+                                           AQ_QMVT16B(8, 8, 4, 1, 2), AQ_QMVT16B(8, 8, 2, 1, 2), AQ_QMVT16B(8, 8, 1, 1, 1),
+                                           AQ_QMVT16X2B(8, 8, 4, 1, 2), AQ_QMVT16X2B(8, 8, 2, 1, 2), AQ_QMVT16X2B(8, 8, 1, 1, 1)};
 
 int qmvt_variant_count() { return (int)(sizeof(kQmvTokTable) / sizeof(kQmvTokTable[0])); }
 const QmvVariant* qmvt_variant(int idx) {
@@ -447,7 +449,7 @@ hipError_t qmvt_launch(int idx, const QmvArgs& a, hipStream_t stream) {
 
 // The variant for this shape, or -1.
 int qmvt_pick(int bits, int M, int K, int N, int cu_count) {
-    if (M < 1 || M > (bits == 4 ? kTokMax : 16) || K < 256 || K % 256 != 0) return -1;
+    if (M < 1 || M > kTokMax || K < 256 || K % 256 != 0) return -1;
     const int cus = cu_count > 0 ? cu_count : 256;
     if (K > 16384) return -1;
     // eight wavefronts, one run each per pass; one set of 16 tokens up to 16 rows of x, else two; as many sets of 16

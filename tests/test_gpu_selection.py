@@ -36,7 +36,8 @@ CASES = [
     (6, 64, 1, 512, ("qmv_six",)),
     (6, 64, 4, 4096, ("qmv_six",)),
     (4, 64, 48, 4096, ("qmmf_",)),                   # 33..64 rows, K a multiple of 256: K shared out over workgroups
-    (8, 64, 24, 4096, ("qmmf_",)),                   # 8 bit beyond 16 rows
+    (8, 64, 24, 4096, ("qmvt_b8_m32_",)),            # token tile, 8 bit, 32-token form
+    (8, 64, 40, 4096, ("qmmf_",)),                   # 8 bit beyond 32 rows
     (4, 64, 20, 320, ("qmmt_b4_mb1_nb2_wm1_wn4",)),  # fewer than 64 rows, K no multiple of 256: 32 x 256 tiles
     (4, 64, 40, 320, ("qmmt_b4_mb2_nb2_wm1_wn4",)),  # ... 64 x 256 tiles
     (8, 64, 70, 320, ("qmmt_b8_mb2_nb2_wm2_wn2",)),  # 64 rows and more: 128 x 128 tiles
