@@ -134,18 +134,22 @@ int qmm_dispatch(hipStream_t stream, Workspace* ws, int cu_count, int forced, co
         // prefill sizes: the LDS-staged 128 x 128 tiles (four 64 x 64 wavefront tiles, two workgroups a CU);
         // the 128 x 64 wavefront tiles need more registers than two wavefronts a SIMD leave and measure slower
         tile_idx = find_qmmt(bits, 2, 2, 2, 2);
-        // 4 bit, enough 256 x 128 tiles to fill the chip twice over: the kernels whose MFMA operand carries
-        // scale * (code - 8) as fp16 (half the vector instructions per MFMA, no fp32 work on the accumulators;
-        // measured 10 % faster at 2048 x 14336)
-        if (bits == 4 && (int64_t)((M + 255) / 256) * ((N + 127) / 128) >= 2 * (cu_count > 0 ? cu_count : 256)) {
-            int half = find_qmmt_named("qmmh_b4_mb4_nb2_wm2_wn2_s2c");
-            // at least one 256 x 256 tile per CU: eight wavefronts on a tile that feeds twice the MFMAs per byte of x
-            // copied into LDS, three stages (the copies of x were at two thirds of what a CU takes in; measured
-            // 0.305 -> 0.277 ms at 2048 x 14336 x 4096)
-            if ((int64_t)((M + 255) / 256) * ((N + 255) / 256) >= (cu_count > 0 ? cu_count : 256)) {
-                const int wide = find_qmmt_named("qmmh_b4_mb4_nb2_wm2_wn4");
-                if (wide >= 0) half = wide;
-            }
+        // 4 bit: the kernels whose MFMA operand carries scale * (code - 8) as fp16 (half the vector instructions per
+        // MFMA, no fp32 work on the accumulators) once their tiles cover enough of the chip.  A round of 256 x 256
+        // tiles (eight wavefronts, twice the MFMAs per byte of x copied into LDS) takes 0.121 ms at K = 4096 however
+        // few tiles it holds, a round of 256 x 128 tiles 0.094-0.107 ms, a round of up to 512 of the 128 x 128 tiles
+        // 0.07-0.115 ms; measured on one box, 256 x 256 / 256 x 128 / 128 x 128 (ms): 2048 x 14336 0.277 / 0.305 / 0.32,
+        // 1024 x 14336 0.139 / 0.150 / 0.196, 768 x 14336 0.125 / 0.135 / 0.158, 768 x 12288 0.122 / 0.129 / 0.148,
+        // 768 x 10240 0.122 / 0.103 / 0.110, 2048 x 4096 0.126 / 0.107 / 0.117, 1536 x 4096 0.121 / 0.098 / 0.103,
+        // 512 x 10240 0.121 / 0.094 / 0.094, 512 x 8192 0.121 / 0.095 / 0.071, 256 x 14336 0.120 / 0.094 / 0.067.
+        // Hence: 256 x 256 from 9/16 of a tile per CU, else 256 x 128 above 5/8 of a tile per CU.
+        const int cus = cu_count > 0 ? cu_count : 256;
+        const int64_t mb = (M + 255) / 256;
+        if (bits == 4 && mb * ((N + 255) / 256) * 16 >= (int64_t)cus * 9) {
+            const int wide = find_qmmt_named("qmmh_b4_mb4_nb2_wm2_wn4");
+            if (wide >= 0) tile_idx = wide;
+        } else if (bits == 4 && mb * ((N + 127) / 128) * 8 > (int64_t)cus * 5) {
+            const int half = find_qmmt_named("qmmh_b4_mb4_nb2_wm2_wn2_s2c");
             if (half >= 0) tile_idx = half;
         }
     }
@@ -168,6 +172,14 @@ int qmm_dispatch(hipStream_t stream, Workspace* ws, int cu_count, int forced, co
             tile_idx = want;
             ksplit = ks;
         }
+    }
+    if (idx < 0 && M > 64 && tile_idx >= 0 && tile_idx == find_qmmt(bits, 2, 2, 2, 2) && (K / 64) % 4 == 0) {
+        // 128 x 128 tiles that leave CUs idle and a long K: K shared out over up to eight workgroups per tile, two
+        // workgroups a CU at most, 1024 codes of K each at least
+        const int cus = cu_count > 0 ? cu_count : 256;
+        const int64_t tiles = (int64_t)((M + 127) / 128) * ((N + 127) / 128);
+        for (int k = 2; k <= 8; k++)
+            if ((K / 64) % (4 * k) == 0 && tiles * k <= 2 * cus && (K / 64) / k >= 16) ksplit = k;
     }
     if (tile_idx < 0) {
         // fewer than 64 rows and a K that is no multiple of 256: 32 x 256 or 64 x 256 workgroup tiles

@@ -701,7 +701,9 @@ def test_gather_errors(ctx):
 
 @pytest.mark.parametrize("M,K,N,bits,gs", [(3, 512, 64, 4, 64), (5, 256, 40, 4, 64), (2, 128, 8, 8, 64), (33, 1024, 130, 4, 64),
                                            (64, 512, 256, 8, 64), (100, 2816, 96, 4, 64), (17, 704, 17, 4, 64), (40, 1408, 70, 4, 128),
-                                           (130, 384, 33, 8, 128), (256, 1024, 512, 4, 64)])
+                                           (130, 384, 33, 8, 128), (256, 1024, 512, 4, 64),
+                                           # more than 64 rows, few 128 x 128 tiles, long K: K shared out over workgroups
+                                           (130, 2048, 200, 4, 64), (100, 4096, 520, 8, 64), (200, 6144, 130, 4, 128)])
 def test_qmm_small_cases(ctx, orc, M, K, N, bits, gs):
     say("qmm", M, K, N, bits, gs)
     _qmv_case(ctx, orc, M, K, N, bits, gs, 900 + M + N, fn="qmm")

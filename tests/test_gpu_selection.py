@@ -101,3 +101,22 @@ def test_route_switches_from_the_environment(monkeypatch, off, bits, M, K, prefi
         dw.free()
     finally:
         c.close()
+
+
+@pytest.mark.parametrize("M,K,Nq,prefix", [
+    (1024, 2048, 14336, "qmmh_b4_mb4_nb2_wm2_wn4"),        # 224 tiles of 256 x 256: 7/8 of a tile per CU
+    (768, 2048, 10240, "qmmh_b4_mb4_nb2_wm2_wn2_s2c"),     # 120 such tiles, 240 of 256 x 128
+    (256, 2048, 14336, "qmmt_b4_mb2_nb2_wm2_wn2"),         # 112 tiles of 256 x 128: the 128 x 128 tiles
+])
+def test_selected_prefill_tiles(ctx, M, K, Nq, prefix):
+    """aq_qmm picks its tile kernel by how much of the chip the tiles cover; sampled output columns against float64."""
+    say("prefill selection", M, K, Nq)
+    words, s, b = F.synthetic_affine(Nq, K, 4, 64, seed=1300 + M)
+    x = F.synthetic_x(M, K, seed=1350 + M)
+    dw = DeviceAffine(ctx, words, s, b)
+    acc = run_qmv(ctx, x, dw, M, K, Nq, 64, 4, True, fn="qmm")
+    assert ctx.last_variant(1) == prefix, ctx.last_variant(1)
+    cols = np.random.default_rng(5).choice(Nq, 96, replace=False)
+    ref = F.reference_f64(x, words[cols], s[cols], b[cols], 4, 64, K)
+    check_accumulators(acc[:, cols], ref, prefix)
+    dw.free()
