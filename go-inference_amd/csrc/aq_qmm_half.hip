@@ -605,6 +605,8 @@ struct QmmHalfEntry {
 static const QmmHalfEntry kQmmHalfTable[] = {
     AQ_QMMH(4, 2, 2, 2, 2, 2, true, "_s2c"),  // 256 x 128, four wavefronts, two stages (every LDS address a constant)
     AQ_QMMH(4, 2, 2, 4, 3, 2, false, ""),     // 256 x 256, eight wavefronts, three stages (120 KiB): an A tile feeds twice the MFMAs
+    AQ_QMMH(3, 2, 2, 4, 3, 2, false, ""),     // 192 x 256: a round of these takes 0.82 of a round of those; for row counts
+                                              // that fill their rounds better (1536 rows: 8 bands instead of 6 of 256)
 };
 
 int qmmh_variant_count() { return (int)(sizeof(kQmmHalfTable) / sizeof(kQmmHalfTable[0])); }

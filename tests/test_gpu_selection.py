@@ -105,6 +105,7 @@ def test_route_switches_from_the_environment(monkeypatch, off, bits, M, K, prefi
 
 @pytest.mark.parametrize("M,K,Nq,prefix", [
     (1024, 2048, 14336, "qmmh_b4_mb4_nb2_wm2_wn4"),        # 224 tiles of 256 x 256: 7/8 of a tile per CU
+    (768, 2048, 14336, "qmmh_b4_mb3_nb2_wm2_wn4"),         # 168 such tiles or 224 of 192 x 256: one round either way
     (768, 2048, 10240, "qmmh_b4_mb4_nb2_wm2_wn2_s2c"),     # 120 such tiles, 240 of 256 x 128
     (256, 2048, 14336, "qmmt_b4_mb2_nb2_wm2_wn2"),         # 112 tiles of 256 x 128: the 128 x 128 tiles
 ])
