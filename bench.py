@@ -465,6 +465,30 @@ def main():
         for t in pools[8] + dom_extra:
             for d in t:
                 d.free()
+        # six-bit codes, groups of 64 (MLX 6 bit), one row of x: the same projection, 12 copies in turn
+        rng6 = np.random.Generator(np.random.PCG64(F.BASE_SEED + 31))
+        w6 = rng6.integers(0, 1 << 32, size=(N, K * 6 // 32), dtype=np.uint64).astype(np.uint32)
+        first6 = (ctx.to_device(w6), ctx.to_device(s8), ctx.to_device(b8))
+        pool6 = [first6]
+        for c in range(1, 12):
+            dst = tuple(ctx.alloc(t.nbytes) for t in first6)
+            for d, t in zip(dst, first6):
+                ctx._check(ctx.lib.aq_d2d(ctx.handle, d.ptr, t.ptr, t.nbytes))
+            pool6.append(dst)
+        xm = ctx.to_device(F.synthetic_x(1, K, seed=F.BASE_SEED + 1101))
+        ym = ctx.alloc(N * 2)
+        for i in range(6):
+            ctx.qmv(xm, *pool6[i % 12], ym, 1, K, N, GROUP, 6)
+        ctx.sync()
+        us = replay_ms(lambda i: ctx.qmv(xm, *pool6[i % 12], ym, 1, K, N, GROUP, 6), 120) * 1e3
+        by = qmv_bytes(K, N, 1, 6)
+        small_m["b6_m1"] = {"us": round(us, 3), "GBps": round(by / us / 1e3, 1),
+                            "pct_of_hbm_peak": round(by / us / 1e3 / HBM_PEAK_GBPS * 100, 2), "kernel": ctx.last_variant(0)}
+        xm.free()
+        ym.free()
+        for t in pool6:
+            for d in t:
+                d.free()
 
         # ---- extra: MoE gather_qmv decode (cfg 4): 128 experts, 8 tokens x top-8, ids read on device --
         E, TOK, TOPK, DM, DFF = 128, 8, 8, 2816, 1408
