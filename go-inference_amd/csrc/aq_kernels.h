@@ -28,6 +28,7 @@ struct QmvArgs {
     int row_base;     // gather only: first row of the slab used
     int x_rows;       // gather only: rows in x (bounds for lhs)
     int routes;       // gather only
+    int stream_w;     // diagonal-MFMA kernels: load the weights with the non-temporal hint (set by the launch functions)
     // activation-fused kernels only (aq_qmv_act.hip)
     const uint16_t* x2;  // x-load fusion: the `up` activations, same shape and row indexing as x (the `gate` ones)
     const uint32_t* w2;  // pair fusion: the `up` matrix (w, s, b are the `gate` one)

@@ -54,6 +54,12 @@ __device__ __forceinline__ uint4 load_u128_at(gptr_t base, uint32_t off) {
     const u32x4_t v = *reinterpret_cast<const __attribute__((address_space(1))) u32x4_t*>(base + off);
     return make_uint4(v[0], v[1], v[2], v[3]);
 }
+// The same with the non-temporal hint: the line leaves the L1 once it has been read.  Only for loads that take whole
+// 128-byte lines per instruction (a line requested in two halves would be fetched twice).
+__device__ __forceinline__ uint4 load_u128_stream_at(gptr_t base, uint32_t off) {
+    const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const __attribute__((address_space(1))) u32x4_t*>(base + off));
+    return make_uint4(v[0], v[1], v[2], v[3]);
+}
 __device__ __forceinline__ uint2 load_u64_at(gptr_t base, uint32_t off) {
     const u32x2_t v = *reinterpret_cast<const __attribute__((address_space(1))) u32x2_t*>(base + off);
     return make_uint2(v[0], v[1]);
@@ -97,8 +103,9 @@ __host__ __device__ inline size_t qmvd_lds_bytes_for(int M, int K, int nw, int m
 // HEAD (lm_head, one activation row): 4 stores every row's packed (score, row) instead of the score, 3 keeps the
 // best packed value of the 16 rows in a.partial[set] for fold_best_kernel (aq_qmv_head.hip).
 template <int NW, int SUP, int NR, bool PAIR, int MT = 1, bool GATHER = false, int CPS = 4, bool G32 = false, int HEAD = 0,
-          bool LINES = true>
+          bool LINES = true, bool STREAM = false>
 __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block) {
+    static_assert(!STREAM || LINES, "streaming loads take whole lines");
     static_assert(HEAD == 0 || (!PAIR && !GATHER && MT == 1), "the head epilogues take one plain activation row");
     static_assert(!G32 || MT == 1, "group 32: one set of two activation rows");
     constexpr int TPS = G32 ? 2 : 4;      // activation rows per set
@@ -279,8 +286,13 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
             // (the second half of a last chunk that is a single half: re-reads the first, not used)
             const uint32_t ho = cc < valid && 2 * (CPS * sp + cc) + 1 < halves ? w_half : 0;
             const bool whole = cc < valid && 2 * (CPS * sp + cc) + 1 < halves;
-            wq[u][cc][0] = load_u128_at(wg, w_lane[0] + wo + co + ho);
-            wq[u][cc][1] = load_u128_at(wg, w_lane[1] + wo + co + (LINES ? ho : whole ? 64u : 0u));
+            if constexpr (STREAM) {
+                wq[u][cc][0] = load_u128_stream_at(wg, w_lane[0] + wo + co + ho);
+                wq[u][cc][1] = load_u128_stream_at(wg, w_lane[1] + wo + co + ho);
+            } else {
+                wq[u][cc][0] = load_u128_at(wg, w_lane[0] + wo + co + ho);
+                wq[u][cc][1] = load_u128_at(wg, w_lane[1] + wo + co + (LINES ? ho : whole ? 64u : 0u));
+            }
         }
         // A last chunk of one half has two groups: its 8 bytes are read 4 bytes early (inside the row) and the
         // upper word, which holds the two groups, moves down.
@@ -492,12 +504,22 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
 
 template <int NW, int SUP, int NR, int MT, int CPS>
 __global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_kernel(const QmvArgs a) {
-    qmv_diag_body<NW, SUP, NR, false, MT, false, CPS, false, 0, (NW > 4)>(a, (int)blockIdx.x);
+    // a.stream_w (large matrices): whole lines with the non-temporal hint (same box: 4096 x 14336 8.70 -> 8.31 us, the
+    // four-launch layer 32.3 -> 30.9 us; 4096 x 4096 4.05 -> 4.17 us, which is why it is a choice per launch; a read of
+    // the same bytes with no arithmetic: 6.73 -> 6.17 us in contiguous pieces, but 7.47 -> 8.35 us in 64-byte pieces
+    // of rows, whose lines are then fetched twice); the arithmetic and its bytes are the same
+    if (a.stream_w)
+        qmv_diag_body<NW, SUP, NR, false, MT, false, CPS, false, 0, true, true>(a, (int)blockIdx.x);
+    else
+        qmv_diag_body<NW, SUP, NR, false, MT, false, CPS, false, 0, (NW > 4)>(a, (int)blockIdx.x);
 }
 
 template <int NW, int SUP, int CPS>
 __global__ __launch_bounds__(2 * NW* kWave) void qmv_diag_pair_kernel(const QmvArgs a) {
-    qmv_diag_body<NW, SUP, 2, true, 1, false, CPS>(a, (int)blockIdx.x);
+    if (a.stream_w)
+        qmv_diag_body<NW, SUP, 2, true, 1, false, CPS, false, 0, true, true>(a, (int)blockIdx.x);
+    else
+        qmv_diag_body<NW, SUP, 2, true, 1, false, CPS>(a, (int)blockIdx.x);
 }
 
 // Quantisation groups of 32 codes, up to two activation rows.
@@ -536,10 +558,17 @@ __global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_multi_kernel(const Qmv
     a.b = ma.b[set];
     a.y = ma.y[set];
     a.N = ma.N[set];
-    qmv_diag_body<NW, SUP, NR, false, 1, false, CPS>(a, (int)blockIdx.x - (set ? ma.block_end[set - 1] : 0));
+    if (a.stream_w)
+        qmv_diag_body<NW, SUP, NR, false, 1, false, CPS, false, 0, true, true>(a, (int)blockIdx.x - (set ? ma.block_end[set - 1] : 0));
+    else
+        qmv_diag_body<NW, SUP, NR, false, 1, false, CPS>(a, (int)blockIdx.x - (set ? ma.block_end[set - 1] : 0));
 }
 
 // ---- variant table --------------------------------------------------------
+
+// Packed bytes of a dense launch (all its matrices) from which the weights are loaded with the non-temporal hint; the
+// gathered kernels keep plain loads (the MoE block measured 80.7 against 83.1 us with the hint: routes share experts).
+constexpr int64_t kDiagStreamBytes = (int64_t)16 << 20;
 
 typedef void (*QmvDiagKernel)(const QmvArgs);
 struct QmvDiagEntry {
@@ -637,7 +666,9 @@ hipError_t qmvd_launch(int idx, const QmvArgs& a, hipStream_t stream) {
     }
     const int wg_rows = kDiagRows * e.v.rows;
     dim3 grid((unsigned)((a.N + wg_rows - 1) / wg_rows), e.v.gather ? (unsigned)a.routes : 1u, 1u);
-    hipLaunchKernelGGL(e.fn, grid, dim3((unsigned)(e.v.rows * e.v.waves * kWave)), lds, stream, a);
+    QmvArgs b = a;
+    b.stream_w = !e.v.gather && (int64_t)a.N * (a.K / 2) >= kDiagStreamBytes ? 1 : 0;
+    hipLaunchKernelGGL(e.fn, grid, dim3((unsigned)(e.v.rows * e.v.waves * kWave)), lds, stream, b);
     return hipGetLastError();
 }
 
@@ -721,7 +752,9 @@ hipError_t qmvd_pair_launch(int idx, const QmvArgs& a, bool gather, hipStream_t 
         if (rc != hipSuccess) return rc;
     }
     dim3 grid((unsigned)((a.N + kDiagRows - 1) / kDiagRows), gather ? (unsigned)a.routes : 1u, 1u);
-    hipLaunchKernelGGL(fn, grid, dim3((unsigned)(2 * e->nw * kWave)), lds, stream, a);
+    QmvArgs b = a;
+    b.stream_w = !gather && (int64_t)2 * a.N * (a.K / 2) >= kDiagStreamBytes ? 1 : 0;
+    hipLaunchKernelGGL(fn, grid, dim3((unsigned)(2 * e->nw * kWave)), lds, stream, b);
     return hipGetLastError();
 }
 
@@ -824,6 +857,9 @@ hipError_t qmvd_multi_launch(int idx, QmvMultiArgs ma, hipStream_t stream) {
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (rc != hipSuccess) return rc;
     }
+    int64_t bytes = 0;
+    for (int i = 0; i < ma.count; i++) bytes += (int64_t)ma.N[i] * (ma.common.K / 2);
+    ma.common.stream_w = bytes >= kDiagStreamBytes ? 1 : 0;
     hipLaunchKernelGGL(e->fn, dim3((unsigned)blocks), dim3((unsigned)(e->nw * e->nr * kWave)), lds, stream, ma);
     return hipGetLastError();
 }
