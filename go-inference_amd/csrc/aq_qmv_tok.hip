@@ -27,6 +27,12 @@ __device__ __forceinline__ uint4 load_u128_at(gptr_t base, uint32_t off) {
     const u32x4_t v = *reinterpret_cast<const __attribute__((address_space(1))) u32x4_t*>(base + off);
     return make_uint4(v[0], v[1], v[2], v[3]);
 }
+// The same with the non-temporal hint, for the weights: they are read once, in whole 128-byte lines per instruction, and
+// leave the L1 to x, scales and biases (4096 x 14336, 16 / 32 rows of x: 12.65 -> 12.28 / 17.14 -> 16.8 us).
+__device__ __forceinline__ uint4 load_u128_stream_at(gptr_t base, uint32_t off) {
+    const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const __attribute__((address_space(1))) u32x4_t*>(base + off));
+    return make_uint4(v[0], v[1], v[2], v[3]);
+}
 __device__ __forceinline__ uint2 load_u64_at(gptr_t base, uint32_t off) {
     const u32x2_t v = *reinterpret_cast<const __attribute__((address_space(1))) u32x2_t*>(base + off);
     return make_uint2(v[0], v[1]);
@@ -174,7 +180,7 @@ __global__ __launch_bounds__(NW* kWave) void qmv_tok16_kernel(const QmvArgs a) {
                     uint32_t base = 0;
 #pragma unroll
                     for (int rs = 0; rs < RS; rs++) base = rs == rs_dyn ? w_lane[rs][ab] : base;
-                    ring[SL][j][ln][ab] = load_u128_at(wg, base + (uint32_t)qds[j] * (uint32_t)(128 * LINES) + (uint32_t)ln * 128u);
+                    ring[SL][j][ln][ab] = load_u128_stream_at(wg, base + (uint32_t)qds[j] * (uint32_t)(128 * LINES) + (uint32_t)ln * 128u);
                 }
     };
     bool staged = false;
