@@ -179,7 +179,8 @@ __global__ __launch_bounds__(256) void qmv_generic_kernel(const QmvArgs a, int b
 // v_dot2_f32_bf16 with the matching pair of x; the group form of the sum, scale * sum((128 + code) * x) +
 // (bias - 128 * scale) * sum(x), has one scale and bias per lane and step (16 codes never straddle a group).
 // A wavefront carries R rows through the same slice of x, so x and its sum are fetched and formed once per R rows,
-// and up to MR rows of x share each decoded row.  14336 x 4096, groups of 64: 15.8 us for one row of x (the
+// and up to MR rows of x share each decoded row; the codes are loaded with the non-temporal hint (read once, whole
+// lines per wavefront and row: 15.5 -> 14.8 us).  14336 x 4096, groups of 64: 14.8 us for one row of x (the
 // float form one row at a time took 16.7, the any-width kernel 117); a form that kept x in LDS and the loads a
 // ring of four steps ahead over persistent wavefronts measured slower (16.3-17.0 us) and is not kept.
 __device__ __forceinline__ void six_pairs(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t (&p)[8]) {
@@ -241,9 +242,9 @@ __global__ __launch_bounds__(256) void qmv_six_kernel(const QmvArgs a, int gathe
 #pragma unroll
         for (int r = 0; r < R; r++) {
             const uint32_t* wp = wr[r] + (k0 >> 4) * 3;
-            w[r][0] = wp[0];
-            w[r][1] = wp[1];
-            w[r][2] = wp[2];
+            w[r][0] = __builtin_nontemporal_load(wp);
+            w[r][1] = __builtin_nontemporal_load(wp + 1);
+            w[r][2] = __builtin_nontemporal_load(wp + 2);
             sb[r][0] = sr[r][k0 / GS];
             sb[r][1] = br[r][k0 / GS];
         }
