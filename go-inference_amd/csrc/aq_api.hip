@@ -220,9 +220,12 @@ const QmvRule kQmvRules[] = {
     {4, 64, 0, 1, 8, kFamDiag},             // one row up to 16 steps of 1024 codes, up to 8 rows at 2..4 steps: every row
                                             // of such a call has the bytes of a call with that row alone
     {4, 32, 0, 1, 2, kFamDiag},             // groups of 32: two tokens x eight groups as MFMA rows
-    {8, 64, 0, 5, 32, kFamTok},             // K a multiple of 256 up to 16384: one launch, weights streamed once, no scratch
-                                            // (up to 4 rows the block-MFMA kernels stay: 14.2 / 15.9 against 14.9 / 14.8 us for
-                                            // 1 / 4 rows of 4096 x 14336, and their rows have the bytes of single-row calls)
+    {8, 0, 0, 1, 1, kFamDot2},              // one row of 8-bit codes: the dot2 kernel with its non-temporal loads, 12.4 us for
+                                            // 4096 x 14336 (63 % of the HBM peak) against 14.2 us on the block-MFMA kernel
+    {8, 64, 0, 2, 32, kFamTok},             // K a multiple of 256 up to 16384: one launch, weights streamed once, no scratch
+                                            // (4 rows of 4096 x 14336: 14.3 us against 15.0 on the block-MFMA kernels, 21.5 on
+                                            // the dot2 kernels; the reference states its rows-equal-single-rows contract for
+                                            // 4-bit codes only, qmv_rows_test.go:36-41)
     {4, 64, 0, 5, 32, kFamTok},             // the same for 4-bit codes, up to 32 rows
                                             // (5..8 rows: only where the diagonal kernels passed; they measure 11.2 us
                                             // against 14.4 us at 8 rows of 4096 x 14336, but not row by row the same bytes)

@@ -141,8 +141,15 @@ __device__ __forceinline__ void qmv_dot2_body(const QmvArgs& a, const int bx) {
 #pragma unroll
             for (int r = 0; r < RS; r++) {
                 const bool up = FUSE == 1 && r >= R;
-                t.w[r] = *reinterpret_cast<const uint4*>((up ? wbase2 : wbase) +
-                                                         (rel[up ? r - R : r] * row_bytes + (uint32_t)c * 16u));
+                const char* wp = (up ? wbase2 : wbase) + (rel[up ? r - R : r] * row_bytes + (uint32_t)c * 16u);
+                if constexpr (GATHER) {
+                    t.w[r] = *reinterpret_cast<const uint4*>(wp);
+                } else {
+                    // dense: read once, 1 KiB of a row per instruction: the non-temporal hint lets the L1 give the line up
+                    typedef uint32_t u32x4_nt __attribute__((ext_vector_type(4)));
+                    const u32x4_nt v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_nt*>(wp));
+                    t.w[r] = make_uint4(v[0], v[1], v[2], v[3]);
+                }
             }
         }
     };

@@ -24,8 +24,10 @@ CASES = [
     (4, 64, 9, 4096, ("qmvt_b4_m16_",)),
     (4, 64, 17, 4096, ("qmvt_b4_m32_",)),            # token tile, 32-token form: 17..32 rows
     (4, 64, 32, 4096, ("qmvt_b4_m32_",)),
-    (8, 64, 1, 4096, ("qmvb_",)),                    # block MFMA: one row of 8-bit codes
-    (8, 64, 4, 4096, ("qmvb_",)),                    # ... and 2..4 rows
+    (8, 64, 1, 4096, ("qmv_b8_",)),                  # dot2: one row of 8-bit codes
+    (8, 128, 1, 4096, ("qmv_b8_",)),
+    (8, 64, 4, 4096, ("qmvt_b8_m16_",)),             # token tile, 8 bit: 2..16 rows, K a multiple of 256
+    (8, 64, 4, 4096 + 64, ("qmvb_", "qmv_b8_")),     # ... block MFMA or dot2 for other K
     (4, 64, 8, 14336, ("qmvt_b4_m16_",)),            # 5..8 rows at a K the diagonal kernels take for one row only
     (4, 64, 8, 14336 + 128, ("qmvb_", "qmmf_", "qmmt_")),
     (4, 128, 1, 4096, ("qmv_b4_",)),                 # dot2: groups of 128

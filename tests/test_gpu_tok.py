@@ -60,7 +60,7 @@ def test_tok_every_variant(ctx, orc):
         ctx.force_variant(0, -1)
 
 
-@pytest.mark.parametrize("M", [5, 8, 16, 17, 32])
+@pytest.mark.parametrize("M", [2, 4, 5, 8, 16, 17, 32])
 def test_tok_config2_full_shape_8bit(ctx, orc, M):
     """cfg 2's 8-bit variant at its full shape (K = 4096, N = 14336): the default path; accumulators against the
     float64 reference and, on sampled rows of x, the oracle's fp32-accumulated reference; bf16 store = RNE of the
