@@ -156,7 +156,9 @@ def test_cfg4_at_128_experts(ctx, orc):
     ddn.free()
 
 
-@pytest.mark.parametrize("name,Ns", [("q|k|v", (4096, 1024, 1024)), ("gate|up", (14336, 14336))])
+# the third form crosses the size from which a launch loads its weights with the non-temporal hint (16 MB of codes):
+# the launch of both matrices is above it, the single calls it is compared with are below
+@pytest.mark.parametrize("name,Ns", [("q|k|v", (4096, 1024, 1024)), ("gate|up", (14336, 14336)), ("q|o", (4096, 4200))])
 def test_cfg1_multi_launch_forms(ctx, orc, name, Ns):
     """The launches the cfg 1 bench times: aq_qmv_multi over q|k|v and over gate|up = 2 x 14336 rows at K = 4096.
     Byte-identical to one aq_qmv per matrix (ConcatQuantRows' contract, go/model/quant_weight.go:32-44), and every
