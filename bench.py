@@ -179,8 +179,8 @@ def main():
 
     ctx = aq_mi355.Context(0)
     dev_name = ctx.device_name()
-    if dev_name.startswith(" ("):  # the driver reports no marketing name on some boxes
-        dev_name = "AMD Instinct MI355X" + dev_name
+    if dev_name.startswith("AMD Instinct MI350 series ("):  # the driver reports no marketing name on some boxes; 256 CUs: MI355X
+        dev_name = dev_name.replace("MI350 series", "MI355X", 1)
 
     # ---- synthetic layer, resident in HBM; copies made device-to-device -------------------------
     layer_bytes = sum(qmv_bytes(K, N) for _, K, N in LAYER)

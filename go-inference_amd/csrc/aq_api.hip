@@ -376,7 +376,9 @@ int aq_create(int device, aq_ctx** out) {
     ctx->device = device;
     ctx->cu_count = prop.multiProcessorCount;
     ctx->families_off = families_off_from_env(getenv("AQ_MI355_DISABLE"));
-    snprintf(ctx->name, sizeof ctx->name, "%s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
+    // (some hosts report no marketing name)
+    snprintf(ctx->name, sizeof ctx->name, "%s (%s, %d CUs)", prop.name[0] ? prop.name : "AMD Instinct MI350 series", prop.gcnArchName,
+             prop.multiProcessorCount);
     rc = hipStreamCreateWithFlags(&ctx->own_stream, hipStreamNonBlocking);
     if (rc == hipSuccess) rc = hipEventCreate(&ctx->ev0);
     if (rc == hipSuccess) rc = hipEventCreate(&ctx->ev1);
