@@ -163,9 +163,10 @@ int qmm_dispatch(hipStream_t stream, Workspace* ws, int cu_count, int forced, co
     // K is shared out as well and a small kernel adds the partial tiles.
     int ksplit = 1;
     if (idx < 0 && M > 4 && M <= 64 && (K / 64) % 4 == 0) {
-        // the kernels whose LDS stages hold four blocks of K: 32 or 64 rows by 256 (8 bit: 128) columns per workgroup
+        // the kernels whose LDS stages hold four blocks of K: 32 or 64 rows by 256 (8 bit: 128) columns per workgroup, eight
+        // (8 bit: four) wavefronts side by side
         const int bm = M <= 32 ? 32 : 64, bn = bits == 4 ? 256 : 128;
-        const int want = find_qmmt_named(bits == 4 ? (M <= 32 ? "qmmf_b4_mb1_nb2_wm1_wn4" : "qmmf_b4_mb2_nb2_wm1_wn4")
+        const int want = find_qmmt_named(bits == 4 ? (M <= 32 ? "qmmf_b4_mb1_nb1_wm1_wn8" : "qmmf_b4_mb2_nb1_wm1_wn8")
                                                    : (M <= 32 ? "qmmf_b8_mb1_nb1_wm1_wn4" : "qmmf_b8_mb2_nb1_wm1_wn4"));
         if (want >= 0) {
             const int tiles = ((M + bm - 1) / bm) * ((N + bn - 1) / bn);

@@ -12,7 +12,7 @@
 // next quad's scales, biases and block sums fetched with ordinary loads at the same point - by the end-of-quad
 // wait everything outstanding has landed, so the compiler's own wait at the first use of those registers finds
 // nothing to drain.  One workgroup per CU (two stages are 96 to 128 KiB of LDS); workgroup tiles are 32 or 64
-// rows by 256 columns (4 bit) or 128 columns (8 bit), four wavefronts side by side.
+// rows by 256 columns (4 bit, eight wavefronts side by side) or 128 columns (8 bit, four).
 #include "aq_device.h"
 #include "aq_kernels.h"
 #include "aq_lds_copy.h"
@@ -48,17 +48,19 @@ __device__ __forceinline__ uint32_t dup16(uint32_t h) { return (h & 0xffffu) | (
 
 // Operands: QmmTileArgs as the tile kernels take them (x rewritten by their pass over x; ksplit workgroups per
 // tile, each over gsplit blocks of K, a multiple of 4; partial tiles [ksplit][M][N] when ksplit > 1).
-template <int BITS, int MB>
-__global__ __launch_bounds__(4 * kWave, 1) void qmm_few_kernel(const QmmTileArgs a) {
-    constexpr int NB = BITS == 4 ? 2 : 1;
-    constexpr int WN = 4;
+// WN wavefronts side by side: four with two column blocks each (4 bit) or eight with one, which puts two
+// wavefronts on a SIMD (one's code expansion and scaling under the other's MFMAs) and halves both per wavefront.
+template <int BITS, int MB, int WN>
+__global__ __launch_bounds__(WN* kWave, 1) void qmm_few_kernel(const QmmTileArgs a) {
+    constexpr int NB = BITS == 4 ? 8 / WN : 1;
+    static_assert(WN == 4 || (WN == 8 && BITS == 4), "four wavefronts, or eight for 4-bit codes");
     constexpr int BM = MB * 32;
     constexpr int BN = WN * NB * 32;
     constexpr int WPB = BITS == 4 ? 8 : 16;       // packed words per row and 64-code block
     constexpr int A_BLK = MB * 4096;              // fragments of one block
     constexpr int B_BLK = BN * WPB * 4;           // packed codes of one block: 8 KiB either way
     constexpr int A_QUAD = 4 * A_BLK, B_QUAD = 4 * B_BLK;
-    constexpr int NA = MB * 4;                    // 1 KiB copies of A per wavefront and quad (MB * 16 fragments over 4)
+    constexpr int NA = MB * 16 / WN;              // 1 KiB copies of A per wavefront and quad (MB * 16 fragments)
     constexpr int NBC = B_QUAD / 1024 / WN;       // 1 KiB copies of codes per wavefront and quad
     constexpr float OFFSET = BITS == 4 ? 16.0f : 0.0f;
     static_assert(B_BLK == 8192, "a block of codes is 8 KiB for both widths");
@@ -373,12 +375,13 @@ struct QmmFewEntry {
     void (*fn)(const QmmTileArgs);
     int lds_bytes;
 };
-#define AQ_QMMF(BITS, MB, NB)                                                                               \
-    {                                                                                                       \
-        {"qmmf_b" #BITS "_mb" #MB "_nb" #NB "_wm1_wn4", BITS, MB, NB, 1, 4}, qmm_few_kernel<BITS, MB>,      \
-            2 * (4 * MB * 4096 + 4 * 8192)                                                                  \
+#define AQ_QMMF(BITS, MB, NB, WN)                                                                                  \
+    {                                                                                                              \
+        {"qmmf_b" #BITS "_mb" #MB "_nb" #NB "_wm1_wn" #WN, BITS, MB, NB, 1, WN}, qmm_few_kernel<BITS, MB, WN>,     \
+            2 * (4 * MB * 4096 + 4 * 8192)                                                                         \
     }
-static const QmmFewEntry kQmmFewTable[] = {AQ_QMMF(4, 1, 2), AQ_QMMF(4, 2, 2), AQ_QMMF(8, 1, 1), AQ_QMMF(8, 2, 1)};
+// 4 bit: eight wavefronts (64 x 14336 x 4096: 31.2 us against 34.1 us with four; 32 rows: 23.4 against 25.6 us)
+static const QmmFewEntry kQmmFewTable[] = {AQ_QMMF(4, 1, 1, 8), AQ_QMMF(4, 2, 1, 8), AQ_QMMF(8, 1, 1, 4), AQ_QMMF(8, 2, 1, 4)};
 
 int qmmf_variant_count() { return (int)(sizeof(kQmmFewTable) / sizeof(kQmmFewTable[0])); }
 const QmmVariant* qmmf_variant(int idx) {
@@ -396,7 +399,7 @@ hipError_t qmmf_launch_kernel(int idx, const QmmTileArgs& a, hipStream_t stream)
     hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e.fn), hipFuncAttributeMaxDynamicSharedMemorySize,
                                         e.lds_bytes);
     if (rc != hipSuccess) return rc;
-    hipLaunchKernelGGL(e.fn, dim3(grid), dim3(4 * kWave), (size_t)e.lds_bytes, stream, a);
+    hipLaunchKernelGGL(e.fn, dim3(grid), dim3((unsigned)(e.v.wn * kWave)), (size_t)e.lds_bytes, stream, a);
     return hipGetLastError();
 }
 
