@@ -916,3 +916,25 @@ def test_qmm_errors(ctx):
             ctx.qmm(buf, buf, buf, buf, buf, *args)
         assert e.value.code == aq_mi355.AQ_ERR_SHAPE
     buf.free()
+
+
+def test_rows_through_the_gather_have_single_row_bytes(ctx, orc):
+    """More than eight rows with the bytes of single-row calls: the reference's multi-row route rides its gather kernel
+    with one expert and lhs = the identity (go/engine/metal/qmv_rows.go:14-24, up to 24 rows); the same call here."""
+    say("rows through gather")
+    import aq_mi355
+    K, N, M = 4096, 528, 24
+    words, s, b = F.synthetic_affine(N, K, 4, 64, seed=1401)
+    x = F.synthetic_x(M, K, seed=1402)
+    dw = DeviceAffine(ctx, words, s, b)
+    dx, dl = ctx.to_device(x), ctx.to_device(np.arange(M, dtype=np.int32))
+    dr, dy = ctx.to_device(np.zeros(M, dtype=np.int32)), ctx.alloc(M * N * 2)
+    ctx.gather_qmv(dx, dw.w, dw.s, dw.b, dl, dr, dy, M, M, K, N, 1, N, 0, 64, 4, 0)
+    ctx.sync()
+    got = dy.download(np.uint16, M * N).reshape(M, N)
+    for m in range(M):
+        one = run_qmv(ctx, x[m:m + 1], dw, 1, K, N, 64, 4, False)
+        assert np.array_equal(got[m], one[0]), m
+    for t in (dx, dl, dr, dy):
+        t.free()
+    dw.free()
