@@ -105,6 +105,34 @@ def run_probe(which, variant=None):
         for i in range(60 * ncopy):
             ww, ss, bb = pool[i % ncopy]
             ctx.qmv(x, ww, ss, bb, y, M, K, N, GROUP, BITS)
+    elif which == "b8":
+        # cfg 2's 8-bit variant, one row of x: 14336 x 4096 (62.4 MB), 8 copies in turn
+        w8, s8, b8 = F.synthetic_affine(N, K, 8, GROUP, seed=F.BASE_SEED + 30)
+        first8 = (ctx.to_device(w8), ctx.to_device(s8), ctx.to_device(b8))
+        pool8 = [first8]
+        for _ in range(1, 8):
+            dst = tuple(ctx.alloc(t.nbytes) for t in first8)
+            for d, t in zip(dst, first8):
+                ctx._check(ctx.lib.aq_d2d(ctx.handle, d.ptr, t.ptr, t.nbytes))
+            pool8.append(dst)
+        x = ctx.to_device(F.synthetic_x(1, K, seed=F.BASE_SEED + 1000))
+        y = ctx.alloc(N * 2)
+        for i in range(1600):
+            ww, ss, bb = pool8[i % 8]
+            ctx.qmv(x, ww, ss, bb, y, 1, K, N, GROUP, 8)
+    elif which == "head":
+        # lm_head 262144 x 1536, 4 bit group 32 (251.7 MB): logits, two copies in turn
+        HN, HK, HG = 262144, 1536, 32
+        hw, hs, hb = F.synthetic_affine(HN, HK, BITS, HG, seed=F.BASE_SEED + 90)
+        firsth = (ctx.to_device(hw), ctx.to_device(hs), ctx.to_device(hb))
+        second = tuple(ctx.alloc(t.nbytes) for t in firsth)
+        for d, t in zip(second, firsth):
+            ctx._check(ctx.lib.aq_d2d(ctx.handle, d.ptr, t.ptr, t.nbytes))
+        x = ctx.to_device(F.synthetic_x(1, HK, seed=F.BASE_SEED + 1000))
+        y = ctx.alloc(HN * 2)
+        for i in range(600):
+            ww, ss, bb = (firsth, second)[i % 2]
+            ctx.qmv(x, ww, ss, bb, y, 1, HK, HN, HG, BITS)
     elif which == "read_floor":
         for i in range(200 * ncopy):
             ww, ss, bb = pool[i % ncopy]
@@ -154,7 +182,7 @@ def main():
                          "does not survive stream capture; its per-dispatch durations are what such a run is for)")
     ap.add_argument("--no-qmm", action="store_true", help="skip the prefill qmm extra")
     ap.add_argument("--no-extras", action="store_true", help="skip the small-M and MoE gather extras")
-    ap.add_argument("--probe", choices=["dominant", "qmm", "rows16", "rows32", "read_floor", "gather"], help="run only the named kernel a few times, preceded by two "
+    ap.add_argument("--probe", choices=["dominant", "qmm", "rows16", "rows32", "read_floor", "gather", "b8", "head"], help="run only the named kernel a few times, preceded by two "
                     "kernels of known traffic (a 256 MiB zero fill, a dequantisation of the gate tensor): the workload "
                     "of the rocprofv3 --pmc passes behind roofline.traffic")
     ap.add_argument("--variant", help="with --probe qmm: force this kernel variant (a name aq_variant_name lists)")
