@@ -25,6 +25,7 @@ AQ_OUT_F32 = 0x1
 AQ_IN_F32 = 2
 AQ_LOGITS_BF16 = 4
 AQ_BF16_STEPS = 8
+AQ_W_TILED = 0x10
 AQ_ACT_GELU_TANH = 1
 AQ_ACT_SILU = 2
 OP_QMV = 0
@@ -112,6 +113,9 @@ PROTOTYPES = {
     "aq_upload_fused_gate_up": (_i, [_vp, _c.POINTER(HostLinear), _c.POINTER(HostLinear), _c.POINTER(DeviceLinear)]),
     "aq_free_device_linear": (_i, [_vp, _c.POINTER(DeviceLinear)]),
     "aq_dequant_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _c.c_int64, _i, _i, _i]),
+    "aq_tiled_bytes": (_c.c_int64, [_c.c_int64, _i, _i, _i]),
+    "aq_tile_weights": (_i, [_vp, _vp, _vp, _vp, _c.c_int64, _i, _i, _i, _vp]),
+    "aq_untile_weights": (_i, [_vp, _vp, _c.c_int64, _i, _i, _i, _vp, _vp, _vp]),
     "aq_packed_topk_sample": (_i, [_vp, _vp, _i, _c.c_float, _c.c_float, _c.c_float, _c.c_double, _vp]),
     "aq_gguf_affine_layout_of": (_i, [_i, _c.c_int64, _c.c_int64, _c.POINTER(GgufAffineLayout)]),
     "aq_gguf_to_affine": (_i, [_vp, _i, _vp, _c.c_uint64, _c.c_int64, _c.c_int64, _vp, _vp, _vp]),
@@ -140,6 +144,10 @@ PROTOTYPES = {
     "aqh_repack_b1_to_b2": (_i, [_vp, _sz, _sz, _sz, _i, _i, _i, _vp, _sz]),
     "aqh_affine_geometry": (None, [_i, _i, _i, _c.POINTER(_i), _c.POINTER(_i)]),
 }
+
+
+def tiled_bytes(N, K, group_size=64, bits=4):
+    return load().aq_tiled_bytes(N, K, group_size, bits)
 
 
 class AqError(RuntimeError):
@@ -303,6 +311,18 @@ class Context:
         fn, check, h = self.lib.aq_qmv_multi, self._check, self.handle
         args = (_ptr(x), n, arr(ws), arr(ss), arr(bs), arr(ys), (_c.c_int * n)(*Ns), M, K, group_size, bits, flags)
         return lambda: check(fn(h, *args))
+
+    def tile_weights(self, w, s, b, N, K, group_size=64, bits=4):
+        """The tile-major tensor (a new device buffer) of the MLX arrays w, s, b."""
+        n = tiled_bytes(N, K, group_size, bits)
+        if n < 0:
+            raise AqError(AQ_ERR_UNSUPPORTED, "no tile-major layout for this geometry")
+        out = self.alloc(n)
+        self._check(self.lib.aq_tile_weights(self.handle, _ptr(w), _ptr(s), _ptr(b), N, K, group_size, bits, out.ptr))
+        return out
+
+    def untile_weights(self, tiled, N, K, w, s, b, group_size=64, bits=4):
+        self._check(self.lib.aq_untile_weights(self.handle, _ptr(tiled), N, K, group_size, bits, _ptr(w), _ptr(s), _ptr(b)))
 
     def reserve_workspace(self, M, K):
         self._check(self.lib.aq_reserve_workspace(self.handle, M, K))

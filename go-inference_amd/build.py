@@ -14,7 +14,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libaq_mi355.so")
 
-HIP_SOURCES = ["aq_qmv.hip", "aq_qmv_blk.hip", "aq_qmv_diag.hip", "aq_qmv_tok.hip", "aq_qmv_act.hip", "aq_moe.hip", "aq_qmv_head.hip", "aq_qmm.hip", "aq_qmm_tile.hip", "aq_qmm_half.hip", "aq_qmm_few.hip", "aq_misc.hip", "aq_gguf.hip", "aq_api.hip"]
+HIP_SOURCES = ["aq_qmv.hip", "aq_qmv_blk.hip", "aq_qmv_diag.hip", "aq_qmv_tok.hip", "aq_qmv_act.hip", "aq_moe.hip", "aq_qmv_head.hip", "aq_qmm.hip", "aq_qmm_tile.hip", "aq_qmm_half.hip", "aq_qmm_few.hip", "aq_misc.hip", "aq_tile.hip", "aq_gguf.hip", "aq_api.hip"]
 CXX_SOURCES = [os.path.join("host", f) for f in ("quant_registry.cc", "quant_weight.cc", "rocm_affine.cc", "safetensors.cc", "host_capi.cc")]
 
 COMMON = ["-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function"]

@@ -18,6 +18,7 @@
 
 #include "aq_kernels.h"
 #include "aq_qmm.h"
+#include "aq_tile.h"
 
 namespace {
 
@@ -340,6 +341,46 @@ int launch_qmv_rows(aq_ctx* ctx, aq::QmvArgs a, int group_size, int bits, bool g
     return fail(AQ_ERR_UNSUPPORTED, "aq_qmv: no kernel for bits=%d group=%d rows=%d K=%d N=%d", bits, group_size, a.M, a.K, a.N);
 }
 
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+// The MLX arrays of a tile-major tensor, written into the context's workspace at byte offset `base` (which the
+// caller has reserved up to base + untiled_bytes(N, K)): the route of calls that no tile-major kernel takes.
+size_t untiled_bytes(int64_t N, int K) { return align256((size_t)N * (K / 2)) + 2 * align256((size_t)N * (K / 64) * 2); }
+int untile_into_ws(aq_ctx* ctx, size_t base, const void* tiled, int64_t N, int K, const uint32_t** w, const uint16_t** s,
+                   const uint16_t** b) {
+    char* p = static_cast<char*>(ctx->ws.ptr) + base;
+    char* ps = p + align256((size_t)N * (K / 2));
+    char* pb = ps + align256((size_t)N * (K / 64) * 2);
+    AQ_HIP(aq::tile_unpack_launch(tiled, p, ps, pb, N, K, ctx->stream), "hipLaunchKernel");
+    *w = reinterpret_cast<const uint32_t*>(p);
+    *s = reinterpret_cast<const uint16_t*>(ps);
+    *b = reinterpret_cast<const uint16_t*>(pb);
+    return AQ_OK;
+}
+
+// A dense matvec call whose weights are in the tile-major layout (a.w; a.s and a.b unset): the diagonal-MFMA
+// kernels read it as it lies; any other kernel gets the MLX arrays rebuilt in the workspace first.
+int launch_qmv_tiled(aq_ctx* ctx, aq::QmvArgs a, int group_size, int bits) {
+    a.gs_shift = ilog2(group_size);
+    a.tiled = 1;
+    int family = -1, local = -1;
+    const int forced = ctx->forced[0];
+    if (forced >= 0 && !qmv_locate(forced, &family, &local)) return fail(AQ_ERR_ARG, "aq_qmv: forced variant %d does not exist", forced);
+    if (forced >= 0 ? family == kFamDiag : !(ctx->families_off >> kFamDiag & 1)) {
+        const int rc = run_diag(ctx, a, group_size, bits, false, forced >= 0 ? local : -1);
+        if (rc != kPass) return rc;
+        if (forced >= 0)
+            return fail(AQ_ERR_ARG, "aq_qmv: forced variant %d does not fit tile-major weights with rows=%d K=%d N=%d", forced, a.M,
+                        a.K, a.N);
+    }
+    const size_t region = aq::qmm_scratch_bytes(a.M, a.K, a.N);
+    AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    if (int rc = aq::workspace_reserve(ctx->stream, &ctx->ws, region + untiled_bytes(a.N, a.K), fail)) return rc;
+    if (int rc = untile_into_ws(ctx, region, a.w, a.N, a.K, &a.w, &a.s, &a.b)) return rc;
+    a.tiled = 0;
+    return launch_qmv_rows(ctx, a, group_size, bits, false);
+}
+
 }  // namespace
 
 namespace {
@@ -590,7 +631,14 @@ int aq_qmv(aq_ctx* ctx, const void* x, const void* packed, const void* scales, c
     if (M < 0 || K < 0 || N < 0) return fail(AQ_ERR_SHAPE, "aq_qmv: M, K, N must be non-negative");
     if (M == 0 || N == 0 || K == 0) return AQ_OK;
     if (int rc = check_geometry("aq_qmv", K, group_size, bits)) return rc;
-    if (!x || !packed || !scales || !biases || !y) return fail(AQ_ERR_ARG, "aq_qmv: null operand");
+    const bool tiled = (flags & AQ_W_TILED) != 0;
+    if (tiled) {
+        if (aq::tile_total_bytes(N, K, group_size, bits) < 0)
+            return fail(AQ_ERR_UNSUPPORTED, "aq_qmv: no tile-major layout for bits=%d group=%d K=%d", bits, group_size, K);
+        if (!aligned(packed, 16)) return fail(AQ_ERR_ARG, "aq_qmv: a tile-major tensor is 16-byte aligned");
+        scales = biases = nullptr;
+    }
+    if (!x || !packed || (!tiled && (!scales || !biases)) || !y) return fail(AQ_ERR_ARG, "aq_qmv: null operand");
     if (!aligned(x, 2) || !aligned(packed, 4) || !aligned(scales, 2) || !aligned(biases, 2) || !aligned(y, 2))
         return fail(AQ_ERR_ARG, "aq_qmv: operand pointer is not element-aligned");
     std::lock_guard<std::mutex> lk(ctx->mu);
@@ -605,6 +653,7 @@ int aq_qmv(aq_ctx* ctx, const void* x, const void* packed, const void* scales, c
     a.M = M;
     a.out_f32 = (flags & AQ_OUT_F32) ? 1 : 0;
     a.routes = 1;
+    if (tiled) return launch_qmv_tiled(ctx, a, group_size, bits);
     return launch_qmv_rows(ctx, a, group_size, bits, false);
 }
 
@@ -614,14 +663,20 @@ int aq_qmv_multi(aq_ctx* ctx, const void* x, int count, const void* const* packe
     if (!ctx) return fail(AQ_ERR_ARG, "aq_qmv_multi: ctx is null");
     if (count < 0 || count > aq::kQmvMultiMax) return fail(AQ_ERR_ARG, "aq_qmv_multi: count must be 0..%d", aq::kQmvMultiMax);
     if (count == 0) return AQ_OK;
-    if (!packed || !scales || !biases || !y || !N) return fail(AQ_ERR_ARG, "aq_qmv_multi: null array");
+    if (!packed || !y || !N) return fail(AQ_ERR_ARG, "aq_qmv_multi: null array");
     if (M < 0 || K < 0) return fail(AQ_ERR_SHAPE, "aq_qmv_multi: M, K must be non-negative");
     bool fused = M >= 1 && M <= 4 && K > 0 && bits == 4 && ctx->forced[0] < 0;
+    const bool tiled = (flags & AQ_W_TILED) != 0;  // every member is a tile-major tensor; scales and biases are not read
+    if (!tiled && (!scales || !biases)) return fail(AQ_ERR_ARG, "aq_qmv_multi: null array");
+    const void* const kNoArrays[aq::kQmvMultiMax] = {nullptr, nullptr, nullptr, nullptr};
+    if (tiled) scales = biases = kNoArrays;
     for (int i = 0; i < count; i++) {
         if (N[i] < 0) return fail(AQ_ERR_SHAPE, "aq_qmv_multi: N[%d] must be non-negative", i);
         if (N[i] == 0) fused = false;  // an empty member: leave the bookkeeping to aq_qmv
-        if (N[i] > 0 && K > 0 && M > 0 && (!packed[i] || !scales[i] || !biases[i] || !y[i]))
+        if (N[i] > 0 && K > 0 && M > 0 && (!packed[i] || (!tiled && (!scales[i] || !biases[i])) || !y[i]))
             return fail(AQ_ERR_ARG, "aq_qmv_multi: null operand in member %d", i);
+        if (tiled && N[i] > 0 && K > 0 && M > 0 && (aq::tile_total_bytes(N[i], K, group_size, bits) < 0 || !aligned(packed[i], 16)))
+            fused = false;  // aq_qmv names the problem
     }
     if (fused) {
         if (int rc = check_geometry("aq_qmv_multi", K, group_size, bits)) return rc;
@@ -647,6 +702,7 @@ int aq_qmv_multi(aq_ctx* ctx, const void* x, int count, const void* const* packe
                 ma.common.gs_shift = ilog2(group_size);
                 ma.common.out_f32 = (flags & AQ_OUT_F32) ? 1 : 0;
                 ma.common.routes = 1;
+                ma.common.tiled = tiled ? 1 : 0;
                 ma.count = count;
                 for (int i = 0; i < count; i++) {
                     ma.w[i] = static_cast<const uint32_t*>(packed[i]);
@@ -668,7 +724,7 @@ int aq_qmv_multi(aq_ctx* ctx, const void* x, int count, const void* const* packe
                     return AQ_OK;
                 }
             }
-            const int idx = M == 1 ? pick_qmv_variant(ctx, bits, 1, false, (int)total, K, 1) : -1;
+            const int idx = M == 1 && !tiled ? pick_qmv_variant(ctx, bits, 1, false, (int)total, K, 1) : -1;
             const int rows = idx >= 0 ? aq::qmv_variant(idx)->rows : 0;
             if (rows > 0 && aq::qmv_multi_supported(bits, 1, rows)) {
                 aq::QmvMultiArgs ma{};
@@ -829,7 +885,15 @@ int aq_qmv_gate_up(aq_ctx* ctx, const void* x, const void* gate_packed, const vo
     if (M == 0 || N == 0) return AQ_OK;
     if (K == 0) return fail(AQ_ERR_SHAPE, "aq_qmv_gate_up: K must be positive when there is output to write");
     if (int rc = check_geometry("aq_qmv_gate_up", K, group_size, bits)) return rc;
-    if (!x || !gate_packed || !gate_scales || !gate_biases || !up_packed || !up_scales || !up_biases || !y)
+    const bool tiled = (flags & AQ_W_TILED) != 0;  // gate_packed and up_packed are tile-major tensors
+    if (tiled) {
+        if (aq::tile_total_bytes(N, K, group_size, bits) < 0)
+            return fail(AQ_ERR_UNSUPPORTED, "aq_qmv_gate_up: no tile-major layout for bits=%d group=%d K=%d", bits, group_size, K);
+        if (!aligned(gate_packed, 16) || !aligned(up_packed, 16))
+            return fail(AQ_ERR_ARG, "aq_qmv_gate_up: a tile-major tensor is 16-byte aligned");
+        gate_scales = gate_biases = up_scales = up_biases = nullptr;
+    }
+    if (!x || !gate_packed || !up_packed || !y || (!tiled && (!gate_scales || !gate_biases || !up_scales || !up_biases)))
         return fail(AQ_ERR_ARG, "aq_qmv_gate_up: null operand");
     if (!aligned(x, 2) || !aligned(gate_packed, 4) || !aligned(up_packed, 4) || !aligned(gate_scales, 2) ||
         !aligned(gate_biases, 2) || !aligned(up_scales, 2) || !aligned(up_biases, 2) || !aligned(y, 2))
@@ -855,6 +919,7 @@ int aq_qmv_gate_up(aq_ctx* ctx, const void* x, const void* gate_packed, const vo
         a.out_f32 = out_f32 ? 1 : 0;
         a.routes = 1;
         a.act = act;
+        a.tiled = tiled ? 1 : 0;
         aq::QmvArgs up = a;
         up.w = a.w2;
         up.s = a.s2;
@@ -867,6 +932,20 @@ int aq_qmv_gate_up(aq_ctx* ctx, const void* x, const void* gate_packed, const vo
             AQ_HIP(aq::qmvd_pair_launch(di, a, false, ctx->stream), "hipLaunchKernel");
             return AQ_OK;
         }
+    }
+    if (tiled) {
+        // no fused tile-major kernel for this call: the MLX arrays of both matrices are rebuilt behind the scratch
+        // of the unfused route, which then runs as for any other call
+        const size_t region = qmm_region(M, K, N) + 2 * align256((size_t)M * N * 4);
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+        if (int rc = aq::workspace_reserve(ctx->stream, &ctx->ws, region + 2 * untiled_bytes(N, K), fail)) return rc;
+        const uint32_t* w[2];
+        const uint16_t *sc[2], *bi[2];
+        if (int rc = untile_into_ws(ctx, region, gate_packed, N, K, &w[0], &sc[0], &bi[0])) return rc;
+        if (int rc = untile_into_ws(ctx, region + untiled_bytes(N, K), up_packed, N, K, &w[1], &sc[1], &bi[1])) return rc;
+        gate_packed = w[0], gate_scales = sc[0], gate_biases = bi[0];
+        up_packed = w[1], up_scales = sc[1], up_biases = bi[1];
     }
     if (M == 1 && ctx->forced[0] < 0 && dot2_eligible(K, group_size, bits, x, gate_packed, (size_t)K * 2) &&
         aligned(up_packed, 16)) {
@@ -1490,6 +1569,39 @@ int aq_free_device_linear(aq_ctx* ctx, aq_device_linear* lin) {
     for (void* p : {lin->weight, lin->scales, lin->biases})
         if (p) AQ_HIP(hipFree(p), "hipFree");
     memset(lin, 0, sizeof *lin);
+    return AQ_OK;
+}
+
+int64_t aq_tiled_bytes(int64_t N, int K, int group_size, int bits) { return aq::tile_total_bytes(N, K, group_size, bits); }
+
+int aq_tile_weights(aq_ctx* ctx, const void* packed, const void* scales, const void* biases, int64_t N, int K, int group_size,
+                    int bits, void* tiled) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_tile_weights: ctx is null");
+    if (N <= 0 || K <= 0) return fail(AQ_ERR_SHAPE, "aq_tile_weights: N and K must be positive");
+    if (int rc = check_geometry("aq_tile_weights", K, group_size, bits)) return rc;
+    if (aq::tile_total_bytes(N, K, group_size, bits) < 0)
+        return fail(AQ_ERR_UNSUPPORTED, "aq_tile_weights: no tile-major layout for bits=%d group=%d K=%d (4-bit codes in groups of 64, K a multiple of 128)",
+                    bits, group_size, K);
+    if (!packed || !scales || !biases || !tiled) return fail(AQ_ERR_ARG, "aq_tile_weights: null operand");
+    if (!aligned(packed, 16) || !aligned(tiled, 16) || !aligned(scales, 2) || !aligned(biases, 2))
+        return fail(AQ_ERR_ARG, "aq_tile_weights: packed and tiled must be 16-byte aligned, scales and biases 2-byte aligned");
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    AQ_HIP(aq::tile_repack_launch(packed, scales, biases, tiled, N, K, ctx->stream), "hipLaunchKernel");
+    return AQ_OK;
+}
+
+int aq_untile_weights(aq_ctx* ctx, const void* tiled, int64_t N, int K, int group_size, int bits, void* packed, void* scales,
+                      void* biases) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_untile_weights: ctx is null");
+    if (N <= 0 || K <= 0) return fail(AQ_ERR_SHAPE, "aq_untile_weights: N and K must be positive");
+    if (int rc = check_geometry("aq_untile_weights", K, group_size, bits)) return rc;
+    if (aq::tile_total_bytes(N, K, group_size, bits) < 0)
+        return fail(AQ_ERR_UNSUPPORTED, "aq_untile_weights: no tile-major layout for bits=%d group=%d K=%d", bits, group_size, K);
+    if (!packed || !scales || !biases || !tiled) return fail(AQ_ERR_ARG, "aq_untile_weights: null operand");
+    if (!aligned(packed, 16) || !aligned(tiled, 16) || !aligned(scales, 2) || !aligned(biases, 2))
+        return fail(AQ_ERR_ARG, "aq_untile_weights: packed and tiled must be 16-byte aligned, scales and biases 2-byte aligned");
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    AQ_HIP(aq::tile_unpack_launch(tiled, packed, scales, biases, N, K, ctx->stream), "hipLaunchKernel");
     return AQ_OK;
 }
 

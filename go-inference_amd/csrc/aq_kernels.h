@@ -29,6 +29,8 @@ struct QmvArgs {
     int x_rows;       // gather only: rows in x (bounds for lhs)
     int routes;       // gather only
     int stream_w;     // diagonal-MFMA kernels: load the weights with the non-temporal hint (set by the launch functions)
+    int early_wgs;    // diagonal-MFMA kernels: workgroups (by index) that request their weights before they stage x
+    int tiled;        // diagonal-MFMA kernels, dense: w (and w2) hold the tile-major layout of aq_tile.h; s, b are not read
     // activation-fused kernels only (aq_qmv_act.hip)
     const uint16_t* x2;  // x-load fusion: the `up` activations, same shape and row indexing as x (the `gate` ones)
     const uint32_t* w2;  // pair fusion: the `up` matrix (w, s, b are the `gate` one)
@@ -217,6 +219,10 @@ bool qmv_six_eligible(const QmvArgs& a, int bits, int group_size);
 // in the access shape of the diagonal-MFMA matvec (mode 0) or as contiguous 1 KiB pieces (mode 1).
 hipError_t read_probe_launch(const void* w, const void* s, const void* b, int64_t rows, int row_bytes, int sb_bytes, int mode,
                              uint32_t* out, hipStream_t stream);
+
+// MLX layout <-> tile-major layout of a 4-bit group-64 tensor (aq_tile.hip, layout in aq_tile.h).  w 16-byte aligned.
+hipError_t tile_repack_launch(const void* w, const void* s, const void* b, void* tiled, int64_t N, int K, hipStream_t stream);
+hipError_t tile_unpack_launch(const void* tiled, void* w, void* s, void* b, int64_t N, int K, hipStream_t stream);
 
 // fp32 dequantisation of a whole tensor, bits in {1,2,4,8} (word-clean widths)
 // or {3,5,6} through the straddling path.

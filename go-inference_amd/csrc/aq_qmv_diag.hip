@@ -36,6 +36,10 @@
 // whatever the number of activation rows, and so does the multi-matrix launch.
 #include "aq_device.h"
 #include "aq_kernels.h"
+#include "aq_tile.h"
+
+#include <cstdlib>
+#include <type_traits>
 
 namespace aq {
 
@@ -77,6 +81,9 @@ constexpr int kDiagChunk = 256;    // codes of a row per MFMA chain (four groups
 // A wavefront step is CPS chunks (a template parameter: 4, or 3 where that shares K out more evenly, e.g. the 11
 // chunks of K = 2816 as 3 + 3 + 3 + 2 over four wavefronts instead of 4 + 4 + 3 + none).
 constexpr int kDiagZeroBytes = 128;
+#ifndef AQ_DIAG_AHEAD
+#define AQ_DIAG_AHEAD 2  // chunks of a step requested before its arithmetic starts; chunk c + 2 when chunk c is about to be multiplied
+#endif
 #ifndef AQ_DIAG_WROWS
 #define AQ_DIAG_WROWS 1  // most activation rows a wavefront stages for itself (4 measured slower for every row count)
 #endif
@@ -103,9 +110,10 @@ __host__ __device__ inline size_t qmvd_lds_bytes_for(int M, int K, int nw, int m
 // HEAD (lm_head, one activation row): 4 stores every row's packed (score, row) instead of the score, 3 keeps the
 // best packed value of the 16 rows in a.partial[set] for fold_best_kernel (aq_qmv_head.hip).
 template <int NW, int SUP, int NR, bool PAIR, int MT = 1, bool GATHER = false, int CPS = 4, bool G32 = false, int HEAD = 0,
-          bool LINES = true, bool STREAM = false>
+          bool LINES = true, bool STREAM = false, bool TILED = false>
 __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block) {
-    static_assert(!STREAM || LINES, "streaming loads take whole lines");
+    static_assert(!STREAM || LINES || TILED, "streaming loads take whole lines");
+    static_assert(!TILED || (!G32 && !GATHER && HEAD == 0), "the tile-major layout: dense group-64 projections");
     static_assert(HEAD == 0 || (!PAIR && !GATHER && MT == 1), "the head epilogues take one plain activation row");
     static_assert(!G32 || MT == 1, "group 32: one set of two activation rows");
     constexpr int TPS = G32 ? 2 : 4;      // activation rows per set
@@ -149,7 +157,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     const gptr_t xg = uniform_ptr(reinterpret_cast<const char*>(a.x) + x_row * K * 2);
     const int ppt = K >> 3;        // 16-byte pieces of a token (K % 128 == 0: whole groups of eight)
     const int pieces = M * ppt;
-    auto stage = [&](int p, const uint4 v) {
+    auto stage = [&](int p, uint32_t t, const uint4 v) {  // piece p of x, which belongs to activation row t
         uint4 o;
         o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);  // (x0, x4)
         o.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);  // (x1, x5)
@@ -177,7 +185,6 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
             const uint32_t n1 = __float_as_uint(-128.0f * __uint_as_float(u1));
             const uint32_t n2 = __float_as_uint(-128.0f * __uint_as_float(u2));
             // group g of token t: 12 bytes at [t][chunk g / 4][g % 4]
-            const uint32_t t = (uint32_t)p / (uint32_t)ppt;
             const uint32_t g = ((uint32_t)p - t * (uint32_t)ppt) >> (G32 ? 2 : 3);
             uint32_t* e = G32 ? reinterpret_cast<uint32_t*>(lds_raw + a2_off + (t * chunks + (g >> 3)) * 96 + (g & 7) * 12)
                               : reinterpret_cast<uint32_t*>(lds_raw + a2_off + (t * chunks + (g >> 2)) * 48 + (g & 3) * 12);
@@ -242,9 +249,115 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
         w_lane[ab] = (uint32_t)r8 * (uint32_t)(K >> 1) + (uint32_t)j * 16;  // bytes
     }
     const uint32_t w_half = LINES ? (uint32_t)(n >> 3) * 64 : 0;  // which 64 bytes of the chunk this lane requests
+    // TILED (aq_tile.h): a step of a set of 16 rows is one contiguous tile, 1 KiB of scales and biases and then 1 KiB
+    // per 128-code half, each KiB in lane order, so every load instruction of a wavefront takes 1 KiB of consecutive
+    // bytes and the registers arrive in operand order
+    // (a workgroup of several sets may reach past the last set of the tensor: it reads the last one again and stores nothing)
+    const uint32_t t_lane = TILED ? (uint32_t)min(row0 / kDiagRows, (N + kDiagRows - 1) / kDiagRows - 1) * tile_set_bytes(K, CPS) + (uint32_t)lane * 16 : 0;
     // scales and biases: lane group j holds the four groups of chunk j of the step
     const uint32_t sb_lane = (uint32_t)row * (uint32_t)groups * 2 + (uint32_t)j * SBB;  // bytes
 
+    // the lane that holds the scales of chunk 0 of the step for this lane's row (ds_bpermute byte address)
+    const int sc_addr = n * 4;
+
+    const uint32_t mask = opaque_s(kNibbleMask);
+    const uint32_t magic = opaque_v(kMagic128);
+
+    uint4 wq[SUP][CPS][2];
+    uint4 sq[SUP], bq[SUP];  // (group 64: x and y only)
+    // Scales and biases are requested before the codes: loads come back in the order they went out, and every chunk's
+    // arithmetic needs them, so the first chunk can be worked on while the later ones are still on the way.
+    auto step_of = [&](int u) {
+        const int sp = wave + u * NW;
+        return sp >= supers ? supers - 1 : sp;  // past the end: a valid address, the result is not used
+    };
+    auto issue_scales = [&](int u) {
+        const int sp = step_of(u);
+        const int valid = min(CPS, chunks - CPS * sp);  // chunks of this step
+        if constexpr (TILED) {
+            const uint32_t to = t_lane + (uint32_t)sp * tile_step_bytes(CPS);
+            const uint4 sb = STREAM ? load_u128_stream_at(wg, to) : load_u128_at(wg, to);
+            sq[u] = make_uint4(sb.x, sb.y, 0, 0);
+            bq[u] = make_uint4(sb.z, sb.w, 0, 0);
+        } else {
+            // A last chunk of one half has two groups: its 8 bytes are read 4 bytes early (inside the row) and the
+            // upper word, which holds the two groups, moves down.
+            const bool halfl = (halves & 1) && j < CPS && CPS * sp + j == chunks - 1;
+            const uint32_t so = sb_lane + (uint32_t)sp * (CPS * SBB) - (j < valid ? 0u : (uint32_t)j * SBB) - (halfl ? 4u : 0u);
+            if constexpr (G32) {
+                sq[u] = load_u128_at(sg, so);
+                bq[u] = load_u128_at(bg, so);
+            } else {
+                const uint2 s2 = load_u64_at(sg, so), b2 = load_u64_at(bg, so);
+                sq[u] = make_uint4(s2.x, s2.y, 0, 0);
+                bq[u] = make_uint4(b2.x, b2.y, 0, 0);
+            }
+            if (!G32 && (halves & 1)) {
+                sq[u].x = halfl ? sq[u].y : sq[u].x;
+                bq[u].x = halfl ? bq[u].y : bq[u].x;
+            }
+        }
+    };
+    auto issue_chunk = [&](int u, int cc) {
+        const int sp = step_of(u);
+        const int valid = min(CPS, chunks - CPS * sp);  // chunks of this step; the others re-read chunk 0 and are not used
+        if constexpr (TILED) {
+            const uint32_t to = t_lane + (uint32_t)sp * tile_step_bytes(CPS);
+#pragma unroll
+            for (int L = 0; L < 2; L++) {
+                // (a half past the end of the row: re-reads the tile's first, not used)
+                const uint32_t ho = cc < valid && 2 * (CPS * sp + cc) + L < halves ? (uint32_t)(2 * cc + L) * 1024 : 0;
+                wq[u][cc][L] = STREAM ? load_u128_stream_at(wg, to + 1024 + ho) : load_u128_at(wg, to + 1024 + ho);
+            }
+        } else {
+            const uint32_t wo = (uint32_t)sp * (CPS * 128);
+            const uint32_t co = cc < valid ? cc * 128 : 0;
+            // (the second half of a last chunk that is a single half: re-reads the first, not used)
+            const uint32_t ho = cc < valid && 2 * (CPS * sp + cc) + 1 < halves ? w_half : 0;
+            const bool whole = cc < valid && 2 * (CPS * sp + cc) + 1 < halves;
+            if constexpr (STREAM) {
+                wq[u][cc][0] = load_u128_stream_at(wg, w_lane[0] + wo + co + ho);
+                wq[u][cc][1] = load_u128_stream_at(wg, w_lane[1] + wo + co + ho);
+            } else {
+                wq[u][cc][0] = load_u128_at(wg, w_lane[0] + wo + co + ho);
+                wq[u][cc][1] = load_u128_at(wg, w_lane[1] + wo + co + (LINES ? ho : whole ? 64u : 0u));
+            }
+        }
+    };
+    auto stage_x = [&]() {
+#pragma unroll
+        for (int q = 0; q < PRE; q++)
+            if (pre_p[q] < pieces) stage(pre_p[q], wstage ? (uint32_t)(q >> 1) : (uint32_t)pre_p[q] / (uint32_t)ppt, pre[q]);
+        if (wstage) {
+            // LDS operations of one wavefront complete in order: what its lanes wrote is there for its later reads
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        } else {
+            for (int p = tid + 2 * NR * NW * kWave; p < pieces; p += NR * NW * kWave)
+                stage(p, (uint32_t)p / (uint32_t)ppt, load_u128_at(xg, (uint32_t)p * 16));
+            __syncthreads();  // x, sums and zeros are in LDS
+        }
+    };
+    // A CU takes the loads of its workgroups roughly in the order the workgroups arrived: the first workgroup of a CU
+    // gets its requests out at once, the later ones wait for up to microseconds before theirs are accepted.  Those
+    // stage x BEFORE they request their weights (they would wait anyway), so that nothing but the arithmetic on the
+    // weights is left to do once their loads, the last of the launch, have come back; the first a.early_wgs
+    // workgroups request first and stage while the memory system is starting up.
+    // (Several activation rows are staged by the workgroup together, behind a barrier: always first; measured at eight
+    // rows of 4096 x 14336: 13.4 -> 11.1 us.)
+    const bool late = !wstage || (int)(blockIdx.x + blockIdx.y * gridDim.x) >= a.early_wgs;
+    if (late) stage_x();
+    // AHEAD chunks are requested before the arithmetic starts; chunk cc + AHEAD when chunk cc is about to be worked on
+    constexpr int AHEAD = SUP == 1 && AQ_DIAG_AHEAD < CPS ? AQ_DIAG_AHEAD : CPS;
+#pragma unroll
+    for (int u = 0; u < SUP; u++) {
+        issue_scales(u);
+#pragma unroll
+        for (int cc = 0; cc < AHEAD; cc++) issue_chunk(u, cc);
+    }
+    // (nothing below is needed to request the weights: it must not delay the requests of the workgroups that start first)
+    __builtin_amdgcn_sched_barrier(0);
     // A fragments: load L (0, 1) of a chunk holds groups 2L and 2L + 1; lane group j holds codes of group
     // 2L + (j >> 1).  The lane's A row (at, ag) is non-zero in load L iff ag == 2L + (j >> 1).
     // affine-term A: rows (t, 0) carry the split sums of the four groups of chunk j of the step, 48 bytes
@@ -266,64 +379,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
         a2_base[tg] = d2 ? a2_off + ((uint32_t)token * chunks + j) * A2B : zero_off;
         a2_mul[tg] = d2 ? CPS * A2B : 0;
     }
-    // the lane that holds the scales of chunk 0 of the step for this lane's row (ds_bpermute byte address)
-    const int sc_addr = n * 4;
-
-    const uint32_t mask = opaque_s(kNibbleMask);
-    const uint32_t magic = opaque_v(kMagic128);
-
-    uint4 wq[SUP][CPS][2];
-    uint4 sq[SUP], bq[SUP];  // (group 64: x and y only)
-#pragma unroll
-    for (int u = 0; u < SUP; u++) {
-        int sp = wave + u * NW;
-        if (sp >= supers) sp = supers - 1;  // past the end: a valid address, the result is not used
-        const int valid = min(CPS, chunks - CPS * sp);  // chunks of this step; the others re-read chunk 0 and are not used
-        const uint32_t wo = (uint32_t)sp * (CPS * 128);
-#pragma unroll
-        for (int cc = 0; cc < CPS; cc++) {
-            const uint32_t co = cc < valid ? cc * 128 : 0;
-            // (the second half of a last chunk that is a single half: re-reads the first, not used)
-            const uint32_t ho = cc < valid && 2 * (CPS * sp + cc) + 1 < halves ? w_half : 0;
-            const bool whole = cc < valid && 2 * (CPS * sp + cc) + 1 < halves;
-            if constexpr (STREAM) {
-                wq[u][cc][0] = load_u128_stream_at(wg, w_lane[0] + wo + co + ho);
-                wq[u][cc][1] = load_u128_stream_at(wg, w_lane[1] + wo + co + ho);
-            } else {
-                wq[u][cc][0] = load_u128_at(wg, w_lane[0] + wo + co + ho);
-                wq[u][cc][1] = load_u128_at(wg, w_lane[1] + wo + co + (LINES ? ho : whole ? 64u : 0u));
-            }
-        }
-        // A last chunk of one half has two groups: its 8 bytes are read 4 bytes early (inside the row) and the
-        // upper word, which holds the two groups, moves down.
-        const bool halfl = (halves & 1) && j < CPS && CPS * sp + j == chunks - 1;
-        const uint32_t so = sb_lane + (uint32_t)sp * (CPS * SBB) - (j < valid ? 0u : (uint32_t)j * SBB) - (halfl ? 4u : 0u);
-        if constexpr (G32) {
-            sq[u] = load_u128_at(sg, so);
-            bq[u] = load_u128_at(bg, so);
-        } else {
-            const uint2 s2 = load_u64_at(sg, so), b2 = load_u64_at(bg, so);
-            sq[u] = make_uint4(s2.x, s2.y, 0, 0);
-            bq[u] = make_uint4(b2.x, b2.y, 0, 0);
-        }
-        if (!G32 && (halves & 1)) {
-            sq[u].x = halfl ? sq[u].y : sq[u].x;
-            bq[u].x = halfl ? bq[u].y : bq[u].x;
-        }
-    }
-
-#pragma unroll
-    for (int q = 0; q < PRE; q++)
-        if (pre_p[q] < pieces) stage(pre_p[q], pre[q]);
-    if (wstage) {
-        // LDS operations of one wavefront complete in order: what its lanes wrote is there for its later reads
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    } else {
-        for (int p = tid + 2 * NR * NW * kWave; p < pieces; p += NR * NW * kWave) stage(p, load_u128_at(xg, (uint32_t)p * 16));
-        __syncthreads();  // x, sums and zeros are in LDS
-    }
+    if (!late) stage_x();
 
     float acc[MT];
     f32x4_t dsum[MT];  // affine term, register 0 is the one that is used
@@ -372,18 +428,30 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
                 a_addr0[tg] = a_base0[tg] + (uint32_t)sp * a_mul0[tg];
                 a_addr1[tg] = a_base1[tg] + (uint32_t)sp * a_mul1[tg];
             }
+            // The A fragments of chunk cc + 1 are read from LDS while chunk cc is multiplied: every register of `af` is
+            // loaded again as soon as the MFMA that read it has been issued, so the wavefront never waits for LDS.
+            bf16x8_t af[MT][2][4];
+            auto read_af = [&](int tg, int L, int i, int cc) {
+                af[tg][L][i] = *reinterpret_cast<const bf16x8_t*>(lds_raw + (L == 0 ? a_addr0[tg] + cc * a_chunk0[tg] : a_addr1[tg] + cc * a_chunk1[tg]) + i * 16);
+            };
+            // (Two sets of activation rows: the registers do not allow it; a chunk's fragments are read when it starts.)
+            constexpr bool PF = MT == 1 && SUP == 1;
+            auto read_chunk_af = [&](int cc) {
 #pragma unroll
-            for (int cc = 0; cc < CPS; cc++) {
-                if (cc >= valid) break;
-                bf16x8_t af[MT][2][4];
-#pragma unroll
-                for (int tg = 0; tg < MT; tg++) {
+                for (int tg = 0; tg < MT; tg++)
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
-                        af[tg][0][i] = *reinterpret_cast<const bf16x8_t*>(lds_raw + a_addr0[tg] + cc * a_chunk0[tg] + i * 16);
-                        af[tg][1][i] = *reinterpret_cast<const bf16x8_t*>(lds_raw + a_addr1[tg] + cc * a_chunk1[tg] + i * 16);
+                        read_af(tg, 0, i, cc);
+                        read_af(tg, 1, i, cc);
                     }
-                }
+            };
+            if constexpr (PF) read_chunk_af(0);
+#pragma unroll
+            for (int cc = 0; cc < CPS; cc++) {
+                if (cc + AHEAD < CPS) issue_chunk(u, cc + AHEAD);
+                if (cc >= valid) break;
+                if constexpr (!PF) read_chunk_af(cc);
+                const int cnext = min(cc + 1, valid - 1);  // (the last chunk reads its own fragments again: not used)
                 // the four scales of chunk cc of this lane's row sit in lane group cc
                 uint32_t sx = (uint32_t)__builtin_amdgcn_ds_bpermute(sc_addr + cc * 64, (int)sv.x);
                 uint32_t sy = (uint32_t)__builtin_amdgcn_ds_bpermute(sc_addr + cc * 64, (int)sv.y);
@@ -394,51 +462,58 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
                     sx = (j & 1) ? sz : sx;
                     sy = (j & 1) ? sw2 : sy;
                 }
-                f32x4_t dq[MT];
+                // Two chains of MFMAs, one per 128-code half, that take turns: the rows of A that are not zero in
+                // half L are those of groups 2 L and 2 L + 1 (group 32: 4 L .. 4 L + 3), so chain L is the whole of
+                // those groups' sums and adds exact zeros to the others; the sums are the bits one chain over both
+                // halves would give, at half the dependent length.
+                f32x4_t dq[MT][2];
 #pragma unroll
-                for (int tg = 0; tg < MT; tg++) dq[tg] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-                for (int L = 0; L < 2; L++) {
-                    if (L == 1 && 2 * (CPS * sp + cc) + 1 >= halves) break;  // a last chunk of one half
-                    // first 64 bytes: lanes i >= 8 take rows 8..15 from the second load's lanes i - 8; second 64 bytes:
-                    // lanes i < 8 take rows 0..7 from the first load's lanes i + 8
-                    const uint4 la = wq[u][cc][0], lb = wq[u][cc][1];
-                    uint32_t ww[4];
-                    if constexpr (!LINES) {
-                        const uint4 lv = L == 0 ? la : lb;
-                        ww[0] = lv.x;
-                        ww[1] = lv.y;
-                        ww[2] = lv.z;
-                        ww[3] = lv.w;
-                    } else if (L == 0) {
-                        ww[0] = __builtin_amdgcn_update_dpp(la.x, lb.x, 0x118, 0xf, 0xc, false);
-                        ww[1] = __builtin_amdgcn_update_dpp(la.y, lb.y, 0x118, 0xf, 0xc, false);
-                        ww[2] = __builtin_amdgcn_update_dpp(la.z, lb.z, 0x118, 0xf, 0xc, false);
-                        ww[3] = __builtin_amdgcn_update_dpp(la.w, lb.w, 0x118, 0xf, 0xc, false);
-                    } else {
-                        ww[0] = __builtin_amdgcn_update_dpp(lb.x, la.x, 0x108, 0xf, 0x3, false);
-                        ww[1] = __builtin_amdgcn_update_dpp(lb.y, la.y, 0x108, 0xf, 0x3, false);
-                        ww[2] = __builtin_amdgcn_update_dpp(lb.z, la.z, 0x108, 0xf, 0x3, false);
-                        ww[3] = __builtin_amdgcn_update_dpp(lb.w, la.w, 0x108, 0xf, 0x3, false);
-                    }
+                for (int tg = 0; tg < MT; tg++) dq[tg][0] = dq[tg][1] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+                const uint4 la = wq[u][cc][0], lb = wq[u][cc][1];
+                auto multiply = [&](auto both_halves) {  // straight-line code in either case
+                    constexpr int NL = decltype(both_halves)::value ? 2 : 1;
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
-                        uint32_t p[4];
-                        unpack4_word(ww[i], mask, magic, p);
-                        const bf16x8_t bfrag = as_bf16x8(p[0], p[1], p[2], p[3]);
 #pragma unroll
-                        for (int tg = 0; tg < MT; tg++)
-                            dq[tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[tg][L][i], bfrag, dq[tg], 0, 0, 0);
+                        for (int L = 0; L < NL; L++) {
+                            // LINES, first 64 bytes: lanes i >= 8 take rows 8..15 from the second load's lanes i - 8;
+                            // second 64 bytes: lanes i < 8 take rows 0..7 from the first load's lanes i + 8
+                            const uint32_t wa = i == 0 ? la.x : i == 1 ? la.y : i == 2 ? la.z : la.w;
+                            const uint32_t wb = i == 0 ? lb.x : i == 1 ? lb.y : i == 2 ? lb.z : lb.w;
+                            uint32_t ww;
+                            if constexpr (!LINES || TILED)
+                                ww = L == 0 ? wa : wb;
+                            else if (L == 0)
+                                ww = __builtin_amdgcn_update_dpp(wa, wb, 0x118, 0xf, 0xc, false);
+                            else
+                                ww = __builtin_amdgcn_update_dpp(wb, wa, 0x108, 0xf, 0x3, false);
+                            uint32_t p[4];
+                            unpack4_word(ww, mask, magic, p);
+                            const bf16x8_t bfrag = as_bf16x8(p[0], p[1], p[2], p[3]);
+#pragma unroll
+                            for (int tg = 0; tg < MT; tg++) {
+                                dq[tg][L] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[tg][L][i], bfrag, dq[tg][L], 0, 0, 0);
+                                if (PF && cc + 1 < CPS) read_af(tg, L, i, cnext);
+                            }
+                        }
                     }
-                }
+                };
+                if (2 * (CPS * sp + cc) + 1 < halves)  // (a last chunk may be a single half)
+                    multiply(std::true_type{});
+                else
+                    multiply(std::false_type{});
                 const float s0 = bf16_bits_to_f32(sx & 0xffffu), s1 = __uint_as_float(sx & 0xffff0000u);
                 const float s2 = bf16_bits_to_f32(sy & 0xffffu), s3 = __uint_as_float(sy & 0xffff0000u);
 #pragma unroll
                 for (int tg = 0; tg < MT; tg++) {
-                    acc[tg] = __builtin_fmaf(s0, dq[tg][0], acc[tg]);
-                    acc[tg] = __builtin_fmaf(s1, dq[tg][1], acc[tg]);
-                    acc[tg] = __builtin_fmaf(s2, dq[tg][2], acc[tg]);
-                    acc[tg] = __builtin_fmaf(s3, dq[tg][3], acc[tg]);
+                    // group 64: registers 0, 1 come from the first half, 2, 3 from the second; group 32: all four from
+                    // the half of this lane's token slot
+                    const f32x4_t d0 = dq[tg][0], d1 = dq[tg][1];
+                    const bool odd = G32 && (j & 1);
+                    acc[tg] = __builtin_fmaf(s0, odd ? d1[0] : d0[0], acc[tg]);
+                    acc[tg] = __builtin_fmaf(s1, odd ? d1[1] : d0[1], acc[tg]);
+                    acc[tg] = __builtin_fmaf(s2, (G32 && !odd) ? d0[2] : d1[2], acc[tg]);
+                    acc[tg] = __builtin_fmaf(s3, (G32 && !odd) ? d0[3] : d1[3], acc[tg]);
                 }
             }
         }
@@ -503,20 +578,29 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
 }
 
 template <int NW, int SUP, int NR, int MT, int CPS>
-__global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_kernel(const QmvArgs a) {
+__global__ __launch_bounds__(NR* NW* kWave, 4) void qmv_diag_kernel(const QmvArgs a) {
     // a.stream_w (large matrices): whole lines with the non-temporal hint (same box: 4096 x 14336 8.70 -> 8.31 us, the
     // four-launch layer 32.3 -> 30.9 us; 4096 x 4096 4.05 -> 4.17 us, which is why it is a choice per launch; a read of
     // the same bytes with no arithmetic: 6.73 -> 6.17 us in contiguous pieces, but 7.47 -> 8.35 us in 64-byte pieces
     // of rows, whose lines are then fetched twice); the arithmetic and its bytes are the same
-    if (a.stream_w)
+    // a.tiled: a.w is the tensor in the tile-major layout of aq_tile.h (a.s and a.b are not read)
+    if (a.tiled && a.stream_w)
+        qmv_diag_body<NW, SUP, NR, false, MT, false, CPS, false, 0, false, true, true>(a, (int)blockIdx.x);
+    else if (a.tiled)
+        qmv_diag_body<NW, SUP, NR, false, MT, false, CPS, false, 0, false, false, true>(a, (int)blockIdx.x);
+    else if (a.stream_w)
         qmv_diag_body<NW, SUP, NR, false, MT, false, CPS, false, 0, true, true>(a, (int)blockIdx.x);
     else
         qmv_diag_body<NW, SUP, NR, false, MT, false, CPS, false, 0, (NW > 4)>(a, (int)blockIdx.x);
 }
 
 template <int NW, int SUP, int CPS>
-__global__ __launch_bounds__(2 * NW* kWave) void qmv_diag_pair_kernel(const QmvArgs a) {
-    if (a.stream_w)
+__global__ __launch_bounds__(2 * NW* kWave, 4) void qmv_diag_pair_kernel(const QmvArgs a) {
+    if (a.tiled && a.stream_w)
+        qmv_diag_body<NW, SUP, 2, true, 1, false, CPS, false, 0, false, true, true>(a, (int)blockIdx.x);
+    else if (a.tiled)
+        qmv_diag_body<NW, SUP, 2, true, 1, false, CPS, false, 0, false, false, true>(a, (int)blockIdx.x);
+    else if (a.stream_w)
         qmv_diag_body<NW, SUP, 2, true, 1, false, CPS, false, 0, true, true>(a, (int)blockIdx.x);
     else
         qmv_diag_body<NW, SUP, 2, true, 1, false, CPS>(a, (int)blockIdx.x);
@@ -524,7 +608,7 @@ __global__ __launch_bounds__(2 * NW* kWave) void qmv_diag_pair_kernel(const QmvA
 
 // Quantisation groups of 32 codes, up to two activation rows.
 template <int NW, int SUP, int NR, int CPS>
-__global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_g32_kernel(const QmvArgs a) {
+__global__ __launch_bounds__(NR* NW* kWave, 4) void qmv_diag_g32_kernel(const QmvArgs a) {
     if (a.stream_w)
         qmv_diag_body<NW, SUP, NR, false, 1, false, CPS, true, 0, true, true>(a, (int)blockIdx.x);
     else
@@ -533,25 +617,25 @@ __global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_g32_kernel(const QmvAr
 
 // lm_head forms (one activation row): packed scores (4) or the best packed value per 16 rows (3).
 template <int NW, int SUP, int NR, int CPS, bool G32, int HEAD>
-__global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_head_kernel(const QmvArgs a) {
+__global__ __launch_bounds__(NR* NW* kWave, 4) void qmv_diag_head_kernel(const QmvArgs a) {
     // always with the non-temporal hint: an lm_head is hundreds of megabytes (262144 x 1536, group 32: 42.0 -> 37.4-38.6 us)
     qmv_diag_body<NW, SUP, NR, false, 1, false, CPS, G32, HEAD, true, true>(a, (int)blockIdx.x);
 }
 
 // Gathered forms: grid.y = routes.
 template <int NW, int SUP, int NR, int CPS>
-__global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_gather_kernel(const QmvArgs a) {
+__global__ __launch_bounds__(NR* NW* kWave, 4) void qmv_diag_gather_kernel(const QmvArgs a) {
     qmv_diag_body<NW, SUP, NR, false, 1, true, CPS>(a, (int)blockIdx.x);
 }
 template <int NW, int SUP, int CPS>
-__global__ __launch_bounds__(2 * NW* kWave) void qmv_diag_gather_pair_kernel(const QmvArgs a) {
+__global__ __launch_bounds__(2 * NW* kWave, 4) void qmv_diag_gather_pair_kernel(const QmvArgs a) {
     qmv_diag_body<NW, SUP, 2, true, 1, true, CPS>(a, (int)blockIdx.x);
 }
 
 // Several weight matrices against the same activations in one launch (q|k|v, gate|up): the workgroups of all
 // matrices form one grid, and each looks up which matrix it belongs to.
 template <int NW, int SUP, int NR, int CPS>
-__global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_multi_kernel(const QmvMultiArgs ma) {
+__global__ __launch_bounds__(NR* NW* kWave, 4) void qmv_diag_multi_kernel(const QmvMultiArgs ma) {
     int set = 0;
 #pragma unroll
     for (int i = 1; i < kQmvMultiMax; i++)
@@ -562,10 +646,15 @@ __global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_multi_kernel(const Qmv
     a.b = ma.b[set];
     a.y = ma.y[set];
     a.N = ma.N[set];
-    if (a.stream_w)
-        qmv_diag_body<NW, SUP, NR, false, 1, false, CPS, false, 0, true, true>(a, (int)blockIdx.x - (set ? ma.block_end[set - 1] : 0));
+    const int block = (int)blockIdx.x - (set ? ma.block_end[set - 1] : 0);
+    if (a.tiled && a.stream_w)
+        qmv_diag_body<NW, SUP, NR, false, 1, false, CPS, false, 0, false, true, true>(a, block);
+    else if (a.tiled)
+        qmv_diag_body<NW, SUP, NR, false, 1, false, CPS, false, 0, false, false, true>(a, block);
+    else if (a.stream_w)
+        qmv_diag_body<NW, SUP, NR, false, 1, false, CPS, false, 0, true, true>(a, block);
     else
-        qmv_diag_body<NW, SUP, NR, false, 1, false, CPS>(a, (int)blockIdx.x - (set ? ma.block_end[set - 1] : 0));
+        qmv_diag_body<NW, SUP, NR, false, 1, false, CPS>(a, block);
 }
 
 // ---- variant table --------------------------------------------------------
@@ -573,6 +662,23 @@ __global__ __launch_bounds__(NR* NW* kWave) void qmv_diag_multi_kernel(const Qmv
 // Packed bytes of a dense launch (all its matrices) from which the weights are loaded with the non-temporal hint; the
 // gathered kernels keep plain loads (the MoE block measured 80.7 against 83.1 us with the hint: routes share experts).
 constexpr int64_t kDiagStreamBytes = (int64_t)16 << 20;
+
+// Workgroups that request their weights before staging x: as many as the device has CUs (the first workgroup each CU
+// receives; later ones find the CU's memory queue busy).
+static int diag_early_wgs() {
+    static int cached = -1;
+    if (cached < 0) {
+        const char* e = getenv("AQ_DIAG_EARLY");
+        int dev = 0, cus = 0;
+        if (e)
+            cached = atoi(e);
+        else if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0)
+            cached = cus;
+        else
+            cached = 256;
+    }
+    return cached;
+}
 
 typedef void (*QmvDiagKernel)(const QmvArgs);
 struct QmvDiagEntry {
@@ -628,14 +734,7 @@ static int cps_of(const QmvVariant& v) { return v.xmode ? v.xmode : 4; }
 static bool g32_of(const QmvVariant& v) { return v.kind == 5; }
 // Steps of cps chunks of 256 codes that cover K (its last chunk may be a single half of 128 codes).
 static int steps_for(int K, int cps) { return ((K + kDiagChunk - 1) / kDiagChunk + cps - 1) / cps; }
-// Chunks per step for this K: three where the even number of wavefronts that four would need holds them too (the
-// heaviest wavefront then has three chunks instead of four).  A function of K alone, so that every launch form
-// splits a row the same way and computes the same bytes.
-static int cps_for(int K) {
-    const int chunks = (K + kDiagChunk - 1) / kDiagChunk;
-    const int nw4 = ((chunks + 3) / 4 + 1) & ~1;
-    return (nw4 <= 4 && (chunks + 2) / 3 <= nw4) ? 3 : 4;
-}
+static int cps_for(int K) { return tile_cps_for(K); }
 
 int qmvd_variant_count() { return (int)(sizeof(kQmvDiagTable) / sizeof(kQmvDiagTable[0])); }
 const QmvVariant* qmvd_variant(int idx) {
@@ -656,6 +755,12 @@ bool qmvd_fits(const QmvArgs& a, int bits, int group_size, bool gather, int idx)
     if ((al16 & 15) || (al8 & 7)) return false;
     // 32-bit byte offsets into the packed matrix
     if ((uint64_t)a.N * (uint64_t)(a.K / 2) >= (1ull << 32)) return false;
+    if (a.tiled) {
+        // the layout is cut for one split of K; 32-bit byte offsets into it
+        if (gather || g32_of(*v) || cps_of(*v) != tile_cps_for(a.K)) return false;
+        const int64_t total = tile_total_bytes(a.N, a.K, group_size, bits);
+        if (total < 0 || total >= ((int64_t)1 << 32)) return false;
+    }
     return qmvd_lds_bytes_for(a.M, a.K, v->waves * v->rows, (v->m + 3) / 4, g32_of(*v)) <= 96 * 1024;
 }
 
@@ -672,6 +777,7 @@ hipError_t qmvd_launch(int idx, const QmvArgs& a, hipStream_t stream) {
     dim3 grid((unsigned)((a.N + wg_rows - 1) / wg_rows), e.v.gather ? (unsigned)a.routes : 1u, 1u);
     QmvArgs b = a;
     b.stream_w = !e.v.gather && (int64_t)a.N * (a.K / 2) >= kDiagStreamBytes ? 1 : 0;
+    b.early_wgs = diag_early_wgs();
     hipLaunchKernelGGL(e.fn, grid, dim3((unsigned)(e.v.rows * e.v.waves * kWave)), lds, stream, b);
     return hipGetLastError();
 }
@@ -758,6 +864,7 @@ hipError_t qmvd_pair_launch(int idx, const QmvArgs& a, bool gather, hipStream_t 
     dim3 grid((unsigned)((a.N + kDiagRows - 1) / kDiagRows), gather ? (unsigned)a.routes : 1u, 1u);
     QmvArgs b = a;
     b.stream_w = !gather && (int64_t)2 * a.N * (a.K / 2) >= kDiagStreamBytes ? 1 : 0;
+    b.early_wgs = diag_early_wgs();
     hipLaunchKernelGGL(fn, grid, dim3((unsigned)(2 * e->nw * kWave)), lds, stream, b);
     return hipGetLastError();
 }
@@ -814,8 +921,10 @@ hipError_t qmvd_head_launch(int idx, int fuse, const QmvArgs& a, hipStream_t str
         if (rc != hipSuccess) return rc;
     }
     const int wg_rows = kDiagRows * e->nr;
+    QmvArgs b = a;
+    b.early_wgs = diag_early_wgs();
     hipLaunchKernelGGL(e->fn, dim3((unsigned)((a.N + wg_rows - 1) / wg_rows)), dim3((unsigned)(e->nw * e->nr * kWave)), lds,
-                       stream, a);
+                       stream, b);
     return hipGetLastError();
 }
 
@@ -864,6 +973,7 @@ hipError_t qmvd_multi_launch(int idx, QmvMultiArgs ma, hipStream_t stream) {
     int64_t bytes = 0;
     for (int i = 0; i < ma.count; i++) bytes += (int64_t)ma.N[i] * (ma.common.K / 2);
     ma.common.stream_w = bytes >= kDiagStreamBytes ? 1 : 0;
+    ma.common.early_wgs = diag_early_wgs();
     hipLaunchKernelGGL(e->fn, dim3((unsigned)blocks), dim3((unsigned)(e->nw * e->nr * kWave)), lds, stream, ma);
     return hipGetLastError();
 }

@@ -47,6 +47,9 @@ extern "C" {
 #define AQ_IN_F32 0x2u      /* aq_moe_combine: the route rows are float32 instead of bf16           */
 #define AQ_LOGITS_BF16 0x4u /* aq_moe_route: the router scores are bf16 instead of float32          */
 #define AQ_BF16_STEPS 0x8u  /* aq_moe_combine: round every product and partial sum to bf16          */
+#define AQ_W_TILED 0x10u    /* aq_qmv, aq_qmv_multi, aq_qmv_gate_up: the packed pointers are tile-major tensors
+                               made by aq_tile_weights; they hold scales and biases too, so the scale and bias
+                               arguments are not read (NULL will do)                                          */
 
 typedef struct aq_ctx aq_ctx;
 
@@ -352,6 +355,24 @@ typedef struct aq_gguf_affine_layout {
 int aq_gguf_affine_layout_of(int gguf_type, int64_t rows, int64_t cols, aq_gguf_affine_layout *out);
 int aq_gguf_to_affine(aq_ctx *ctx, int gguf_type, const void *src, uint64_t src_bytes, int64_t rows, int64_t cols,
                       void *packed, void *scales, void *biases);
+
+/* A device layout made once at load time, as the reference synthesises the device layouts of GGUF tensors at load
+ * (go/engine/hip/hip_gguf_affine_adapter.go:199-218).  The tile-major form of a 4-bit group-64 tensor (K a multiple
+ * of 128) stores, for every set of 16 rows and every step of K that one wavefront of the matvec kernels works on, the
+ * codes AND that step's scales and biases as one contiguous tile whose every KiB is in lane order, so a load
+ * instruction of a wavefront takes 1 KiB of consecutive bytes instead of 64 bytes of each of 16 rows (the MLX
+ * row-major arrays cost the single-row projection 4096 -> 14336 about 1.5 us of 8).  aq_tiled_bytes gives the
+ * size of the tile-major tensor (as many bytes as the three MLX arrays when N is a multiple of 16; -1 when the
+ * geometry has no such form); aq_tile_weights writes it from the MLX arrays (device to device, stream-ordered, may
+ * be captured); aq_untile_weights is its exact inverse.  Calls that take AQ_W_TILED compute the same bytes as the
+ * same call on the MLX arrays (same kernels, same order of additions); shapes no tile-major kernel takes (more
+ * than eight rows of x, K beyond 16384, forced variants of other families) rebuild the MLX arrays in the context's
+ * workspace first (one extra pass over the tensor; the workspace grows on demand, not during capture). */
+int64_t aq_tiled_bytes(int64_t N, int K, int group_size, int bits);
+int aq_tile_weights(aq_ctx *ctx, const void *packed, const void *scales, const void *biases, int64_t N, int K,
+                    int group_size, int bits, void *tiled);
+int aq_untile_weights(aq_ctx *ctx, const void *tiled, int64_t N, int K, int group_size, int bits, void *packed,
+                      void *scales, void *biases);
 
 /* mlxaffine.DequantizeTensor on device (go/model/quant/mlxaffine/mlxaffine.go:178-208):
  * out_f32[N,K] = scale*code + bias, bit-exact with the CPU path. */

@@ -229,3 +229,46 @@ def reference_f64(x_bits, words, s_bits, b_bits, bits, group_size, K):
     w = numpy_dequant(words, s_bits, b_bits, bits, group_size, K).astype(np.float64)
     x = bf16_bits_to_f32(x_bits).astype(np.float64).reshape(-1, K)
     return x @ w.T
+
+
+# ---- tile-major device layout (4-bit, group 64), written independently of the library's kernels --------------------
+
+def tile_cps(k):
+    """Chunks of 256 codes per wavefront step for this K (3 where that shares K out evenly over 2 or 4 wavefronts)."""
+    chunks = (k + 255) // 256
+    nw4 = ((chunks + 3) // 4 + 1) & ~1
+    return 3 if (nw4 <= 4 and (chunks + 2) // 3 <= nw4) else 4
+
+
+def tile_major(words, s_bits, b_bits, n, k):
+    """MLX arrays of a 4-bit group-64 tensor -> the tile-major byte string aq_tile_weights must produce.
+
+    Sets of 16 rows (zero-padded); per set, steps of `cps` chunks of 256 codes; per step 1 KiB of scales and biases
+    (lane l = (row l % 16, chunk l // 16 of the step): four scales then four biases, zeros where there is no group),
+    then 1 KiB per 128-code half (lane l: bytes [16 (l // 16), +16) of that half of row l % 16)."""
+    assert k % 128 == 0
+    cps = tile_cps(k)
+    halves, groups = k // 128, k // 64
+    chunks = (halves + 1) // 2
+    steps = (chunks + cps - 1) // cps
+    sets = (n + 15) // 16
+    wb = np.zeros((sets * 16, k // 2), dtype=np.uint8)
+    wb[:n] = np.ascontiguousarray(words, dtype=np.uint32).reshape(n, k // 8).view(np.uint8)
+    sp = np.zeros((sets * 16, steps * cps * 4), dtype=np.uint16)
+    bp = np.zeros_like(sp)
+    sp[:n, :groups] = np.asarray(s_bits, dtype=np.uint16).reshape(n, groups)
+    bp[:n, :groups] = np.asarray(b_bits, dtype=np.uint16).reshape(n, groups)
+    out = []
+    for st in range(sets):
+        rows = slice(16 * st, 16 * st + 16)
+        for step in range(steps):
+            sb = np.zeros((4, 16, 8), dtype=np.uint16)  # [lane group j][row n][4 scales | 4 biases]
+            for j in range(cps):
+                g0 = 4 * (step * cps + j)
+                sb[j, :, :4] = sp[rows, g0:g0 + 4]
+                sb[j, :, 4:] = bp[rows, g0:g0 + 4]
+            out.append(sb.tobytes())
+            for h in range(2 * step * cps, min(2 * (step + 1) * cps, halves)):
+                piece = wb[rows, 64 * h:64 * h + 64].reshape(16, 4, 16)  # [row][j][16 bytes]
+                out.append(np.ascontiguousarray(piece.transpose(1, 0, 2)).tobytes())
+    return np.frombuffer(b"".join(out), dtype=np.uint8)

@@ -103,3 +103,18 @@ def test_pack_and_unpack_best_match_the_oracle(aqlib, orc):
         with pytest.raises(aq_mi355.AqError) as e:
             aq_mi355.unpack_best(*args)
         assert e.value.code == code
+
+
+def test_tiled_bytes_needs_no_device(aqlib):
+    """aq_tiled_bytes is pure arithmetic: it agrees with the numpy statement of the tile-major layout."""
+    import aq_mi355
+    for n, k in ((14336, 4096), (17, 4096), (33, 2816), (64, 3200), (5, 128), (100, 16384)):
+        w, s, b = F.synthetic_affine(min(n, 40), k, 4, 64, seed=n + k)
+        sets_ref = (min(n, 40) + 15) // 16
+        per_set = F.tile_major(w, s, b, min(n, 40), k).size // sets_ref
+        assert aq_mi355.tiled_bytes(n, k) == (n + 15) // 16 * per_set
+    assert aq_mi355.tiled_bytes(14336, 4096) == 14336 * 4096 // 2 + 2 * 14336 * 64 * 2
+    for n, k, gs, bits in ((16, 4096, 64, 8), (16, 4096, 32, 4), (16, 4096, 128, 4), (16, 192, 64, 4), (0, 4096, 64, 4)):
+        assert aq_mi355.tiled_bytes(n, k, gs, bits) == -1
+    assert aqlib.aq_tile_weights(None, None, None, None, 16, 4096, 64, 4, None) == aq_mi355.AQ_ERR_ARG
+    assert aqlib.aq_untile_weights(None, None, 16, 4096, 64, 4, None, None, None) == aq_mi355.AQ_ERR_ARG
