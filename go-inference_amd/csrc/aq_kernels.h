@@ -215,6 +215,10 @@ hipError_t qmv_generic_launch(const QmvArgs& a, int bits, int group_size, bool g
 // Six-bit codes in groups of 16 or 32 with K a multiple of 16 take a kernel of their own inside that launch.
 bool qmv_six_eligible(const QmvArgs& a, int bits, int group_size);
 
+// Allows `lds` bytes of dynamic LDS for kernel function fn when that is beyond the 48 KiB every kernel may use: one
+// hipFuncSetAttribute per device and function (for the largest size asked so far) instead of one per launch.
+hipError_t ensure_dynamic_lds(const void* fn, size_t lds);
+
 // Measurement aid (aq_misc.hip): reads the codes, scales and biases of a 4-bit group-64 tensor once with no arithmetic,
 // in the access shape of the diagonal-MFMA matvec (mode 0) or as contiguous 1 KiB pieces (mode 1).
 hipError_t read_probe_launch(const void* w, const void* s, const void* b, int64_t rows, int row_bytes, int sb_bytes, int mode,

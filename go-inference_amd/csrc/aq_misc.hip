@@ -12,10 +12,31 @@
 // (go/engine/hip/hip_projection_reference.go:92-116, unpack :200-222) for
 // widths the tuned kernels do not cover (2,3,5,6 bit; groups other than
 // 32/64/128), one wavefront per output row.
+#include <map>
+#include <mutex>
+#include <utility>
 #include "aq_device.h"
 #include "aq_kernels.h"
 
 namespace aq {
+
+// Dynamic LDS beyond 48 KiB has to be allowed per kernel function: done once per device and function (for the
+// largest size asked so far), not per launch.
+hipError_t ensure_dynamic_lds(const void* fn, size_t lds) {
+    if (lds <= 48 * 1024) return hipSuccess;
+    static std::mutex mu;
+    static std::map<std::pair<int, const void*>, size_t> allowed;
+    int dev = 0;
+    hipError_t rc = hipGetDevice(&dev);
+    if (rc != hipSuccess) return rc;
+    std::lock_guard<std::mutex> lk(mu);
+    size_t& have = allowed[{dev, fn}];
+    if (have >= lds) return hipSuccess;
+    rc = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (rc == hipSuccess) have = lds;
+    return rc;
+}
+
 
 __device__ __forceinline__ float affine_weight(float scale, float code, float bias) {
 #pragma clang fp contract(off)

@@ -396,9 +396,7 @@ hipError_t qmmf_launch_kernel(int idx, const QmmTileArgs& a, hipStream_t stream)
     if (a.ksplit < 1 || a.gsplit % 4 != 0) return hipErrorInvalidValue;
     const int T = a.tiles_m * a.tiles_n * a.ksplit;
     const unsigned grid = (unsigned)(((T + 7) / 8) * 8);
-    hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e.fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                        e.lds_bytes);
-    if (rc != hipSuccess) return rc;
+    if (hipError_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(e.fn), (size_t)e.lds_bytes)) return rc;
     hipLaunchKernelGGL(e.fn, dim3(grid), dim3((unsigned)(e.v.wn * kWave)), (size_t)e.lds_bytes, stream, a);
     return hipGetLastError();
 }

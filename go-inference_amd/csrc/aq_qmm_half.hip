@@ -650,11 +650,8 @@ hipError_t qmmh_launch(int idx, const QmmArgs& q, void* workspace, hipStream_t s
     a.partial = nullptr;
     const int T = a.tiles_m * a.tiles_n;
     const unsigned grid = (unsigned)(((T + 7) / 8) * 8);
-    if (e.lds_bytes > 48 * 1024) {
-        rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e.fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                 e.lds_bytes);
-        if (rc != hipSuccess) return rc;
-    }
+    rc = ensure_dynamic_lds(reinterpret_cast<const void*>(e.fn), (size_t)e.lds_bytes);
+    if (rc != hipSuccess) return rc;
     hipLaunchKernelGGL(e.fn, dim3(grid), dim3((unsigned)(e.v.wm * e.v.wn * kWave)), (size_t)e.lds_bytes, stream, a);
     return hipGetLastError();
 }

@@ -578,11 +578,8 @@ hipError_t qmmt_launch_splitk(int idx, const QmmArgs& q, void* workspace, int ks
     if (few >= 0) {
         rc = qmmf_launch_kernel(few, a, stream);
     } else {
-        if (e.lds_bytes > 48 * 1024) {
-            rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e.fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     e.lds_bytes);
-            if (rc != hipSuccess) return rc;
-        }
+        rc = ensure_dynamic_lds(reinterpret_cast<const void*>(e.fn), (size_t)e.lds_bytes);
+        if (rc != hipSuccess) return rc;
         hipLaunchKernelGGL(e.fn, dim3(grid), dim3((unsigned)(e.v.wm * e.v.wn * kWave)), (size_t)e.lds_bytes, stream, a);
         rc = hipGetLastError();
     }

@@ -88,11 +88,7 @@ hipError_t qmv_launch(int idx, const QmvArgs& a, hipStream_t stream) {
     dim3 grid((unsigned)((a.N + rows_per_wg - 1) / rows_per_wg), e.v.gather ? (unsigned)a.routes : 1u, 1u);
     dim3 block((unsigned)(e.v.waves * kWave), 1u, 1u);
     const size_t lds = qmv_lds_bytes(idx, a);
-    if (lds > 48 * 1024) {
-        hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e.fn),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (rc != hipSuccess) return rc;
-    }
+    if (hipError_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(e.fn), (size_t)lds)) return rc;
     hipLaunchKernelGGL(e.fn, grid, block, lds, stream, a);
     return hipGetLastError();
 }
@@ -127,11 +123,7 @@ hipError_t qmv_multi_launch(int bits, int m, int rows, QmvMultiArgs ma, hipStrea
         ma.block_end[i] = blocks;
     }
     const size_t lds = (size_t)m * (size_t)ma.common.K * 2;
-    if (lds > 48 * 1024) {
-        hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e->fn),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (rc != hipSuccess) return rc;
-    }
+    if (hipError_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(e->fn), (size_t)lds)) return rc;
     hipLaunchKernelGGL(e->fn, dim3((unsigned)blocks), dim3(4 * kWave), lds, stream, ma);
     return hipGetLastError();
 }

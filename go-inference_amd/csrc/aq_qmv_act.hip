@@ -47,11 +47,7 @@ hipError_t qmv_act_launch(int bits, int fuse, int rows, bool gather, const QmvAr
     const int rows_per_wg = rows * 4;
     dim3 grid((unsigned)((a.N + rows_per_wg - 1) / rows_per_wg), gather ? (unsigned)a.routes : 1u, 1u);
     const size_t lds = (size_t)a.K * 2;
-    if (lds > 48 * 1024) {
-        hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e->fn),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (rc != hipSuccess) return rc;
-    }
+    if (hipError_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(e->fn), (size_t)lds)) return rc;
     hipLaunchKernelGGL(e->fn, grid, dim3(4 * kWave), lds, stream, a);
     return hipGetLastError();
 }

@@ -507,11 +507,7 @@ hipError_t qmvb_launch(const BlkPlan& p, const QmvArgs& a, hipStream_t stream) {
     const BlkEntry& e = kBlkTable[p.idx];
     dim3 grid((unsigned)p.nwg, e.v.gather ? (unsigned)a.routes : 1u, 1u);
     dim3 block((unsigned)(p.nw * kWave), 1u, 1u);
-    if (p.lds > 48 * 1024) {
-        hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e.fn),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)p.lds);
-        if (rc != hipSuccess) return rc;
-    }
+    if (hipError_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(e.fn), (size_t)p.lds)) return rc;
     hipLaunchKernelGGL(e.fn, grid, block, p.lds, stream, a, p.geom);
     return hipGetLastError();
 }

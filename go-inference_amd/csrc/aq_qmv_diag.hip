@@ -107,10 +107,12 @@ __host__ __device__ inline size_t qmvd_lds_bytes_for(int M, int K, int nw, int m
 // (token, group slot) for TWO tokens and the eight groups of a chunk, row (t, g) is non-zero in load L for lane
 // group j iff g == 4 L + j, D lands as lane (2 t + g / 4, n), register g % 4, and the two halves of a token's sum
 // meet at the end.  Scales and biases are 16 bytes per chunk and lane.  K is then a multiple of 256.
+// EVEN: K is a whole number of steps of CPS chunks (the caller has checked): no step is short and no chunk a single half,
+// and what deals with those is not compiled in.
 // HEAD (lm_head, one activation row): 4 stores every row's packed (score, row) instead of the score, 3 keeps the
 // best packed value of the 16 rows in a.partial[set] for fold_best_kernel (aq_qmv_head.hip).
 template <int NW, int SUP, int NR, bool PAIR, int MT = 1, bool GATHER = false, int CPS = 4, bool G32 = false, int HEAD = 0,
-          bool LINES = true, bool STREAM = false, bool TILED = false>
+          bool LINES = true, bool STREAM = false, bool TILED = false, bool EVEN = false>
 __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block) {
     static_assert(!STREAM || LINES || TILED, "streaming loads take whole lines");
     static_assert(!TILED || (!G32 && !GATHER && HEAD == 0), "the tile-major layout: dense group-64 projections");
@@ -191,7 +193,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
             e[0] = (u0 >> 16) | u1;  // (X0, X1)
             e[1] = (u2 >> 16) | n0;  // (X2, -128 X0)
             e[2] = (n1 >> 16) | n2;  // (-128 X1, -128 X2)
-            if (!G32 && (halves & 1) && (int)g == groups - 1) {
+            if (!EVEN && !G32 && (halves & 1) && (int)g == groups - 1) {
                 // a last chunk of one half: its two missing groups must add nothing to the affine term
 #pragma unroll
                 for (int q = 3; q < 9; q++) e[q] = 0;
@@ -273,7 +275,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     };
     auto issue_scales = [&](int u) {
         const int sp = step_of(u);
-        const int valid = min(CPS, chunks - CPS * sp);  // chunks of this step
+        const int valid = EVEN ? CPS : min(CPS, chunks - CPS * sp);  // chunks of this step
         if constexpr (TILED) {
             const uint32_t to = t_lane + (uint32_t)sp * tile_step_bytes(CPS);
             const uint4 sb = STREAM ? load_u128_stream_at(wg, to) : load_u128_at(wg, to);
@@ -282,7 +284,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
         } else {
             // A last chunk of one half has two groups: its 8 bytes are read 4 bytes early (inside the row) and the
             // upper word, which holds the two groups, moves down.
-            const bool halfl = (halves & 1) && j < CPS && CPS * sp + j == chunks - 1;
+            const bool halfl = !EVEN && (halves & 1) && j < CPS && CPS * sp + j == chunks - 1;
             const uint32_t so = sb_lane + (uint32_t)sp * (CPS * SBB) - (j < valid ? 0u : (uint32_t)j * SBB) - (halfl ? 4u : 0u);
             if constexpr (G32) {
                 sq[u] = load_u128_at(sg, so);
@@ -292,7 +294,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
                 sq[u] = make_uint4(s2.x, s2.y, 0, 0);
                 bq[u] = make_uint4(b2.x, b2.y, 0, 0);
             }
-            if (!G32 && (halves & 1)) {
+            if (!EVEN && !G32 && (halves & 1)) {
                 sq[u].x = halfl ? sq[u].y : sq[u].x;
                 bq[u].x = halfl ? bq[u].y : bq[u].x;
             }
@@ -300,21 +302,21 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     };
     auto issue_chunk = [&](int u, int cc) {
         const int sp = step_of(u);
-        const int valid = min(CPS, chunks - CPS * sp);  // chunks of this step; the others re-read chunk 0 and are not used
+        const int valid = EVEN ? CPS : min(CPS, chunks - CPS * sp);  // chunks of this step; the others re-read chunk 0 and are not used
         if constexpr (TILED) {
             const uint32_t to = t_lane + (uint32_t)sp * tile_step_bytes(CPS);
 #pragma unroll
             for (int L = 0; L < 2; L++) {
                 // (a half past the end of the row: re-reads the tile's first, not used)
-                const uint32_t ho = cc < valid && 2 * (CPS * sp + cc) + L < halves ? (uint32_t)(2 * cc + L) * 1024 : 0;
+                const uint32_t ho = EVEN || (cc < valid && 2 * (CPS * sp + cc) + L < halves) ? (uint32_t)(2 * cc + L) * 1024 : 0;
                 wq[u][cc][L] = STREAM ? load_u128_stream_at(wg, to + 1024 + ho) : load_u128_at(wg, to + 1024 + ho);
             }
         } else {
             const uint32_t wo = (uint32_t)sp * (CPS * 128);
             const uint32_t co = cc < valid ? cc * 128 : 0;
             // (the second half of a last chunk that is a single half: re-reads the first, not used)
-            const uint32_t ho = cc < valid && 2 * (CPS * sp + cc) + 1 < halves ? w_half : 0;
-            const bool whole = cc < valid && 2 * (CPS * sp + cc) + 1 < halves;
+            const uint32_t ho = EVEN || (cc < valid && 2 * (CPS * sp + cc) + 1 < halves) ? w_half : 0;
+            const bool whole = EVEN || (cc < valid && 2 * (CPS * sp + cc) + 1 < halves);
             if constexpr (STREAM) {
                 wq[u][cc][0] = load_u128_stream_at(wg, w_lane[0] + wo + co + ho);
                 wq[u][cc][1] = load_u128_stream_at(wg, w_lane[1] + wo + co + ho);
@@ -392,7 +394,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     for (int u = 0; u < SUP; u++) {
         const int sp = wave + u * NW;
         if (sp < supers) {
-            const int valid = min(CPS, chunks - CPS * sp);
+            const int valid = EVEN ? CPS : min(CPS, chunks - CPS * sp);
             const uint4 sv = sq[u], bv = bq[u];
             // affine term of the groups of the step: six k-slots per group (b b b s s s), 24 (group 32: 48) per lane
             {
@@ -448,7 +450,10 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
             if constexpr (PF) read_chunk_af(0);
 #pragma unroll
             for (int cc = 0; cc < CPS; cc++) {
-                if (cc + AHEAD < CPS) issue_chunk(u, cc + AHEAD);
+                if (cc + AHEAD < CPS) {
+                    issue_chunk(u, cc + AHEAD);
+                    __builtin_amdgcn_sched_barrier(0);  // (the request goes out before chunk cc is waited for, not behind its arithmetic)
+                }
                 if (cc >= valid) break;
                 if constexpr (!PF) read_chunk_af(cc);
                 const int cnext = min(cc + 1, valid - 1);  // (the last chunk reads its own fragments again: not used)
@@ -498,7 +503,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
                         }
                     }
                 };
-                if (2 * (CPS * sp + cc) + 1 < halves)  // (a last chunk may be a single half)
+                if (EVEN || 2 * (CPS * sp + cc) + 1 < halves)  // (a last chunk may be a single half)
                     multiply(std::true_type{});
                 else
                     multiply(std::false_type{});
@@ -577,42 +582,38 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     }
 }
 
-template <int NW, int SUP, int NR, int MT, int CPS>
-__global__ __launch_bounds__(NR* NW* kWave, 4) void qmv_diag_kernel(const QmvArgs a) {
-    // a.stream_w (large matrices): whole lines with the non-temporal hint (same box: 4096 x 14336 8.70 -> 8.31 us, the
-    // four-launch layer 32.3 -> 30.9 us; 4096 x 4096 4.05 -> 4.17 us, which is why it is a choice per launch; a read of
-    // the same bytes with no arithmetic: 6.73 -> 6.17 us in contiguous pieces, but 7.47 -> 8.35 us in 64-byte pieces
-    // of rows, whose lines are then fetched twice); the arithmetic and its bytes are the same
-    // a.tiled: a.w is the tensor in the tile-major layout of aq_tile.h (a.s and a.b are not read)
-    if (a.tiled && a.stream_w)
-        qmv_diag_body<NW, SUP, NR, false, MT, false, CPS, false, 0, false, true, true>(a, (int)blockIdx.x);
-    else if (a.tiled)
-        qmv_diag_body<NW, SUP, NR, false, MT, false, CPS, false, 0, false, false, true>(a, (int)blockIdx.x);
-    else if (a.stream_w)
-        qmv_diag_body<NW, SUP, NR, false, MT, false, CPS, false, 0, true, true>(a, (int)blockIdx.x);
-    else
-        qmv_diag_body<NW, SUP, NR, false, MT, false, CPS, false, 0, (NW > 4)>(a, (int)blockIdx.x);
+// MODE of the dense kernels, chosen per launch on the host (one kernel per mode, so that a launch carries only the code
+// it runs): bit 0 = the weights are loaded with the non-temporal hint, as whole lines (large matrices; same box:
+// 4096 x 14336 8.70 -> 8.31 us, the four-launch layer 32.3 -> 30.9 us, but 4096 x 4096 4.05 -> 4.17 us; a read of the
+// same bytes with no arithmetic: 6.73 -> 6.17 us in contiguous pieces, but 7.47 -> 8.35 us in 64-byte pieces of rows,
+// whose lines are then fetched twice); bit 1 = a.w (and a.w2) hold the tile-major layout of aq_tile.h and a.s, a.b
+// are not read; bit 2 = K is a whole number of steps (no code for short steps and half chunks).  The arithmetic and
+// its bytes are the same in every mode.
+template <int NW, int SUP, int NR, bool PAIR, int MT, int CPS, bool G32, int MODE>
+__device__ __forceinline__ void qmv_diag_dense(const QmvArgs& a, const int block) {
+    constexpr bool STREAM = (MODE & 1) != 0, TILED = (MODE & 2) != 0, EVEN = (MODE & 4) != 0;
+    constexpr bool LINES = !TILED;
+    qmv_diag_body<NW, SUP, NR, PAIR, MT, false, CPS, G32, 0, LINES, STREAM, TILED, EVEN>(a, block);
 }
 
-template <int NW, int SUP, int CPS>
-__global__ __launch_bounds__(2 * NW* kWave, 4) void qmv_diag_pair_kernel(const QmvArgs a) {
-    if (a.tiled && a.stream_w)
-        qmv_diag_body<NW, SUP, 2, true, 1, false, CPS, false, 0, false, true, true>(a, (int)blockIdx.x);
-    else if (a.tiled)
-        qmv_diag_body<NW, SUP, 2, true, 1, false, CPS, false, 0, false, false, true>(a, (int)blockIdx.x);
-    else if (a.stream_w)
-        qmv_diag_body<NW, SUP, 2, true, 1, false, CPS, false, 0, true, true>(a, (int)blockIdx.x);
+template <int NW, int SUP, int NR, int MT, int CPS, int MODE>
+__global__ __launch_bounds__(NR* NW* kWave, 4) void qmv_diag_kernel(const QmvArgs a) {
+    if constexpr ((MODE & 3) == 0)  // (the plain kernel of up to four wavefronts keeps 64-byte pieces of 16 rows, see the body)
+        qmv_diag_body<NW, SUP, NR, false, MT, false, CPS, false, 0, (NW > 4), false, false, (MODE & 4) != 0>(a, (int)blockIdx.x);
     else
-        qmv_diag_body<NW, SUP, 2, true, 1, false, CPS>(a, (int)blockIdx.x);
+        qmv_diag_dense<NW, SUP, NR, false, MT, CPS, false, MODE>(a, (int)blockIdx.x);
+}
+
+template <int NW, int SUP, int CPS, int MODE>
+__global__ __launch_bounds__(2 * NW* kWave, 4) void qmv_diag_pair_kernel(const QmvArgs a) {
+    qmv_diag_dense<NW, SUP, 2, true, 1, CPS, false, MODE>(a, (int)blockIdx.x);
 }
 
 // Quantisation groups of 32 codes, up to two activation rows.
-template <int NW, int SUP, int NR, int CPS>
+template <int NW, int SUP, int NR, int CPS, int MODE>
 __global__ __launch_bounds__(NR* NW* kWave, 4) void qmv_diag_g32_kernel(const QmvArgs a) {
-    if (a.stream_w)
-        qmv_diag_body<NW, SUP, NR, false, 1, false, CPS, true, 0, true, true>(a, (int)blockIdx.x);
-    else
-        qmv_diag_body<NW, SUP, NR, false, 1, false, CPS, true>(a, (int)blockIdx.x);
+    static_assert((MODE & 2) == 0, "groups of 32 have no tile-major form");
+    qmv_diag_dense<NW, SUP, NR, false, 1, CPS, true, MODE>(a, (int)blockIdx.x);
 }
 
 // lm_head forms (one activation row): packed scores (4) or the best packed value per 16 rows (3).
@@ -634,7 +635,7 @@ __global__ __launch_bounds__(2 * NW* kWave, 4) void qmv_diag_gather_pair_kernel(
 
 // Several weight matrices against the same activations in one launch (q|k|v, gate|up): the workgroups of all
 // matrices form one grid, and each looks up which matrix it belongs to.
-template <int NW, int SUP, int NR, int CPS>
+template <int NW, int SUP, int NR, int CPS, int MODE>
 __global__ __launch_bounds__(NR* NW* kWave, 4) void qmv_diag_multi_kernel(const QmvMultiArgs ma) {
     int set = 0;
 #pragma unroll
@@ -647,14 +648,7 @@ __global__ __launch_bounds__(NR* NW* kWave, 4) void qmv_diag_multi_kernel(const 
     a.y = ma.y[set];
     a.N = ma.N[set];
     const int block = (int)blockIdx.x - (set ? ma.block_end[set - 1] : 0);
-    if (a.tiled && a.stream_w)
-        qmv_diag_body<NW, SUP, NR, false, 1, false, CPS, false, 0, false, true, true>(a, block);
-    else if (a.tiled)
-        qmv_diag_body<NW, SUP, NR, false, 1, false, CPS, false, 0, false, false, true>(a, block);
-    else if (a.stream_w)
-        qmv_diag_body<NW, SUP, NR, false, 1, false, CPS, false, 0, true, true>(a, block);
-    else
-        qmv_diag_body<NW, SUP, NR, false, 1, false, CPS>(a, block);
+    qmv_diag_dense<NW, SUP, NR, false, 1, CPS, false, MODE>(a, block);
 }
 
 // ---- variant table --------------------------------------------------------
@@ -681,44 +675,49 @@ static int diag_early_wgs() {
 }
 
 typedef void (*QmvDiagKernel)(const QmvArgs);
+// Index into a variant's kernels for this launch.
+static int diag_mode(int K, int cps, bool tiled, bool stream) {
+    return (K % (cps * kDiagChunk) == 0 ? 4 : 0) + (tiled ? 2 : 0) + (stream ? 1 : 0);
+}
 struct QmvDiagEntry {
     QmvVariant v;
-    QmvDiagKernel fn;
+    QmvDiagKernel fn[8];  // by mode (bit 0: non-temporal weight loads, bit 1: tile-major weights, bit 2: whole steps); gathered: [0] only
 };
+#define AQ_DIAG_MODES(K, ...) {K<__VA_ARGS__, 0>, K<__VA_ARGS__, 1>, K<__VA_ARGS__, 2>, K<__VA_ARGS__, 3>, K<__VA_ARGS__, 4>, K<__VA_ARGS__, 5>, K<__VA_ARGS__, 6>, K<__VA_ARGS__, 7>}
 // name, bits, m (most rows), sets of 16 rows per workgroup, wavefronts per set, steps per wavefront, gather,
 // xmode = chunks per step when not 4, kind.  waves x depth steps cover K.
 #define AQ_QMVD(NW, SUP, NR)                                                                                    \
     {                                                                                                           \
-        {"qmvd_b4_m4_r" #NR "_w" #NW "_d" #SUP "_g0", 4, 4, NR, NW, SUP, 0, 0, 4}, qmv_diag_kernel<NW, SUP, NR, 1, 4> \
+        {"qmvd_b4_m4_r" #NR "_w" #NW "_d" #SUP "_g0", 4, 4, NR, NW, SUP, 0, 0, 4}, AQ_DIAG_MODES(qmv_diag_kernel, NW, SUP, NR, 1, 4) \
     }
 #define AQ_QMVD3(NW, SUP, NR)                                                                                      \
     {                                                                                                              \
-        {"qmvd_b4_m4_r" #NR "_w" #NW "_d" #SUP "_g0_c3", 4, 4, NR, NW, SUP, 0, 3, 4}, qmv_diag_kernel<NW, SUP, NR, 1, 3> \
+        {"qmvd_b4_m4_r" #NR "_w" #NW "_d" #SUP "_g0_c3", 4, 4, NR, NW, SUP, 0, 3, 4}, AQ_DIAG_MODES(qmv_diag_kernel, NW, SUP, NR, 1, 3) \
     }
 #define AQ_QMVDG(NW, SUP, NR)                                                                                          \
     {                                                                                                                  \
-        {"qmvd_b4_m1_r" #NR "_w" #NW "_d" #SUP "_g1", 4, 1, NR, NW, SUP, 1, 0, 4}, qmv_diag_gather_kernel<NW, SUP, NR, 4> \
+        {"qmvd_b4_m1_r" #NR "_w" #NW "_d" #SUP "_g1", 4, 1, NR, NW, SUP, 1, 0, 4}, {qmv_diag_gather_kernel<NW, SUP, NR, 4>, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr} \
     }
 #define AQ_QMVDG3(NW, SUP, NR)                                                                                            \
     {                                                                                                                     \
-        {"qmvd_b4_m1_r" #NR "_w" #NW "_d" #SUP "_g1_c3", 4, 1, NR, NW, SUP, 1, 3, 4}, qmv_diag_gather_kernel<NW, SUP, NR, 3> \
+        {"qmvd_b4_m1_r" #NR "_w" #NW "_d" #SUP "_g1_c3", 4, 1, NR, NW, SUP, 1, 3, 4}, {qmv_diag_gather_kernel<NW, SUP, NR, 3>, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr} \
     }
 #define AQ_QMVD8(NW, SUP, NR)                                                                                   \
     {                                                                                                           \
-        {"qmvd_b4_m8_r" #NR "_w" #NW "_d" #SUP "_g0", 4, 8, NR, NW, SUP, 0, 0, 4}, qmv_diag_kernel<NW, SUP, NR, 2, 4> \
+        {"qmvd_b4_m8_r" #NR "_w" #NW "_d" #SUP "_g0", 4, 8, NR, NW, SUP, 0, 0, 4}, AQ_DIAG_MODES(qmv_diag_kernel, NW, SUP, NR, 2, 4) \
     }
 #define AQ_QMVD83(NW, SUP, NR)                                                                                     \
     {                                                                                                              \
-        {"qmvd_b4_m8_r" #NR "_w" #NW "_d" #SUP "_g0_c3", 4, 8, NR, NW, SUP, 0, 3, 4}, qmv_diag_kernel<NW, SUP, NR, 2, 3> \
+        {"qmvd_b4_m8_r" #NR "_w" #NW "_d" #SUP "_g0_c3", 4, 8, NR, NW, SUP, 0, 3, 4}, AQ_DIAG_MODES(qmv_diag_kernel, NW, SUP, NR, 2, 3) \
     }
 // kind 5: quantisation groups of 32 codes
 #define AQ_QMVDS(NW, SUP, NR)                                                                                          \
     {                                                                                                                  \
-        {"qmvd_b4_m2_r" #NR "_w" #NW "_d" #SUP "_g0_s32", 4, 2, NR, NW, SUP, 0, 0, 5}, qmv_diag_g32_kernel<NW, SUP, NR, 4> \
+        {"qmvd_b4_m2_r" #NR "_w" #NW "_d" #SUP "_g0_s32", 4, 2, NR, NW, SUP, 0, 0, 5}, {qmv_diag_g32_kernel<NW, SUP, NR, 4, 0>, qmv_diag_g32_kernel<NW, SUP, NR, 4, 1>, nullptr, nullptr, qmv_diag_g32_kernel<NW, SUP, NR, 4, 4>, qmv_diag_g32_kernel<NW, SUP, NR, 4, 5>, nullptr, nullptr} \
     }
 #define AQ_QMVDS3(NW, SUP, NR)                                                                                            \
     {                                                                                                                     \
-        {"qmvd_b4_m2_r" #NR "_w" #NW "_d" #SUP "_g0_s32_c3", 4, 2, NR, NW, SUP, 0, 3, 5}, qmv_diag_g32_kernel<NW, SUP, NR, 3> \
+        {"qmvd_b4_m2_r" #NR "_w" #NW "_d" #SUP "_g0_s32_c3", 4, 2, NR, NW, SUP, 0, 3, 5}, {qmv_diag_g32_kernel<NW, SUP, NR, 3, 0>, qmv_diag_g32_kernel<NW, SUP, NR, 3, 1>, nullptr, nullptr, qmv_diag_g32_kernel<NW, SUP, NR, 3, 4>, qmv_diag_g32_kernel<NW, SUP, NR, 3, 5>, nullptr, nullptr} \
     }
 static const QmvDiagEntry kQmvDiagTable[] = {
     AQ_QMVD(4, 1, 1), AQ_QMVD(4, 1, 2), AQ_QMVD(4, 1, 4), AQ_QMVD(2, 2, 2), AQ_QMVD(2, 1, 2), AQ_QMVD(8, 1, 1),
@@ -768,17 +767,16 @@ hipError_t qmvd_launch(int idx, const QmvArgs& a, hipStream_t stream) {
     if (idx < 0 || idx >= qmvd_variant_count()) return hipErrorInvalidValue;
     const QmvDiagEntry& e = kQmvDiagTable[idx];
     const size_t lds = qmvd_lds_bytes_for(a.M, a.K, e.v.waves * e.v.rows, (e.v.m + 3) / 4, g32_of(e.v));
-    if (lds > 48 * 1024) {
-        hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e.fn),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (rc != hipSuccess) return rc;
-    }
+    const int stream_w = !e.v.gather && (int64_t)a.N * (a.K / 2) >= kDiagStreamBytes ? 1 : 0;
+    const QmvDiagKernel fn = e.fn[e.v.gather ? 0 : diag_mode(a.K, cps_of(e.v), a.tiled != 0, stream_w != 0)];
+    if (!fn) return hipErrorInvalidValue;
+    if (hipError_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(fn), lds)) return rc;
     const int wg_rows = kDiagRows * e.v.rows;
     dim3 grid((unsigned)((a.N + wg_rows - 1) / wg_rows), e.v.gather ? (unsigned)a.routes : 1u, 1u);
     QmvArgs b = a;
-    b.stream_w = !e.v.gather && (int64_t)a.N * (a.K / 2) >= kDiagStreamBytes ? 1 : 0;
+    b.stream_w = stream_w;
     b.early_wgs = diag_early_wgs();
-    hipLaunchKernelGGL(e.fn, grid, dim3((unsigned)(e.v.rows * e.v.waves * kWave)), lds, stream, b);
+    hipLaunchKernelGGL(fn, grid, dim3((unsigned)(e.v.rows * e.v.waves * kWave)), lds, stream, b);
     return hipGetLastError();
 }
 
@@ -835,9 +833,9 @@ int qmvd_pick_g32(int M, int K, int N) {
 // act(gate . x) * (up . x) with the variant's (wavefronts, steps) split of K; a.w2 / a.s2 / a.b2 are the `up` matrix.
 struct QmvDiagPairEntry {
     int nw, sup, cps;
-    QmvDiagKernel fn, gather_fn;
+    QmvDiagKernel fn[8], gather_fn;
 };
-#define AQ_QMVD_PAIR(NW, SUP, CPS) {NW, SUP, CPS, qmv_diag_pair_kernel<NW, SUP, CPS>, qmv_diag_gather_pair_kernel<NW, SUP, CPS>}
+#define AQ_QMVD_PAIR(NW, SUP, CPS) {NW, SUP, CPS, AQ_DIAG_MODES(qmv_diag_pair_kernel, NW, SUP, CPS), qmv_diag_gather_pair_kernel<NW, SUP, CPS>}
 static const QmvDiagPairEntry kQmvDiagPairTable[] = {
     AQ_QMVD_PAIR(2, 1, 4), AQ_QMVD_PAIR(4, 1, 4), AQ_QMVD_PAIR(6, 1, 4), AQ_QMVD_PAIR(8, 1, 4),
     AQ_QMVD_PAIR(2, 1, 3), AQ_QMVD_PAIR(4, 1, 3),
@@ -854,16 +852,13 @@ bool qmvd_pair_supported(int idx) { return find_pair(idx) != nullptr; }
 hipError_t qmvd_pair_launch(int idx, const QmvArgs& a, bool gather, hipStream_t stream) {
     const QmvDiagPairEntry* e = find_pair(idx);
     if (!e) return hipErrorInvalidValue;
-    const QmvDiagKernel fn = gather ? e->gather_fn : e->fn;
+    const int stream_w = !gather && (int64_t)2 * a.N * (a.K / 2) >= kDiagStreamBytes ? 1 : 0;
+    const QmvDiagKernel fn = gather ? e->gather_fn : e->fn[diag_mode(a.K, e->cps, a.tiled != 0, stream_w != 0)];
     const size_t lds = qmvd_lds_bytes_for(gather ? 1 : a.M, a.K, 2 * e->nw);
-    if (lds > 48 * 1024) {
-        hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                            (int)lds);
-        if (rc != hipSuccess) return rc;
-    }
+    if (hipError_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(fn), lds)) return rc;
     dim3 grid((unsigned)((a.N + kDiagRows - 1) / kDiagRows), gather ? (unsigned)a.routes : 1u, 1u);
     QmvArgs b = a;
-    b.stream_w = !gather && (int64_t)2 * a.N * (a.K / 2) >= kDiagStreamBytes ? 1 : 0;
+    b.stream_w = stream_w;
     b.early_wgs = diag_early_wgs();
     hipLaunchKernelGGL(fn, grid, dim3((unsigned)(2 * e->nw * kWave)), lds, stream, b);
     return hipGetLastError();
@@ -915,11 +910,7 @@ hipError_t qmvd_head_launch(int idx, int fuse, const QmvArgs& a, hipStream_t str
     const QmvDiagHeadEntry* e = find_head(idx, fuse);
     if (!e || a.M != 1 || (fuse == 3 && !a.partial)) return hipErrorInvalidValue;
     const size_t lds = qmvd_lds_bytes_for(1, a.K, e->nw * e->nr, 1, e->g32 != 0);
-    if (lds > 48 * 1024) {
-        hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e->fn),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (rc != hipSuccess) return rc;
-    }
+    if (hipError_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(e->fn), lds)) return rc;
     const int wg_rows = kDiagRows * e->nr;
     QmvArgs b = a;
     b.early_wgs = diag_early_wgs();
@@ -931,10 +922,10 @@ hipError_t qmvd_head_launch(int idx, int fuse, const QmvArgs& a, hipStream_t str
 typedef void (*QmvDiagMultiKernel)(const QmvMultiArgs);
 struct QmvDiagMultiEntry {
     int nw, sup, nr, cps;
-    QmvDiagMultiKernel fn;
+    QmvDiagMultiKernel fn[8];
 };
-#define AQ_QMVD_MULTI(NW, SUP, NR) {NW, SUP, NR, 4, qmv_diag_multi_kernel<NW, SUP, NR, 4>}
-#define AQ_QMVD_MULTI3(NW, SUP, NR) {NW, SUP, NR, 3, qmv_diag_multi_kernel<NW, SUP, NR, 3>}
+#define AQ_QMVD_MULTI(NW, SUP, NR) {NW, SUP, NR, 4, AQ_DIAG_MODES(qmv_diag_multi_kernel, NW, SUP, NR, 4)}
+#define AQ_QMVD_MULTI3(NW, SUP, NR) {NW, SUP, NR, 3, AQ_DIAG_MODES(qmv_diag_multi_kernel, NW, SUP, NR, 3)}
 static const QmvDiagMultiEntry kQmvDiagMultiTable[] = {
     AQ_QMVD_MULTI(4, 1, 1), AQ_QMVD_MULTI(4, 1, 2), AQ_QMVD_MULTI(4, 1, 4), AQ_QMVD_MULTI(2, 1, 2), AQ_QMVD_MULTI(2, 1, 4),
     AQ_QMVD_MULTI(6, 1, 1), AQ_QMVD_MULTI(8, 1, 1), AQ_QMVD_MULTI(10, 1, 1), AQ_QMVD_MULTI(12, 1, 1), AQ_QMVD_MULTI(14, 1, 1),
@@ -965,16 +956,13 @@ hipError_t qmvd_multi_launch(int idx, QmvMultiArgs ma, hipStream_t stream) {
         ma.block_end[i] = blocks;
     }
     const size_t lds = qmvd_lds_bytes_for(ma.common.M, ma.common.K, e->nw * e->nr);
-    if (lds > 48 * 1024) {
-        hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e->fn),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (rc != hipSuccess) return rc;
-    }
     int64_t bytes = 0;
     for (int i = 0; i < ma.count; i++) bytes += (int64_t)ma.N[i] * (ma.common.K / 2);
     ma.common.stream_w = bytes >= kDiagStreamBytes ? 1 : 0;
     ma.common.early_wgs = diag_early_wgs();
-    hipLaunchKernelGGL(e->fn, dim3((unsigned)blocks), dim3((unsigned)(e->nw * e->nr * kWave)), lds, stream, ma);
+    const QmvDiagMultiKernel fn = e->fn[diag_mode(ma.common.K, e->cps, ma.common.tiled != 0, ma.common.stream_w != 0)];
+    if (hipError_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(fn), lds)) return rc;
+    hipLaunchKernelGGL(fn, dim3((unsigned)blocks), dim3((unsigned)(e->nw * e->nr * kWave)), lds, stream, ma);
     return hipGetLastError();
 }
 

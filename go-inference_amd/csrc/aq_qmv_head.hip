@@ -101,11 +101,7 @@ hipError_t qmv_head_launch(int bits, int fuse, int rows, const QmvArgs& a, hipSt
     if (!e || a.M != 1) return hipErrorInvalidValue;
     const int rows_per_wg = rows * 4;
     const size_t lds = (size_t)a.K * 2;
-    if (lds > 48 * 1024) {
-        hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e->fn),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (rc != hipSuccess) return rc;
-    }
+    if (hipError_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(e->fn), (size_t)lds)) return rc;
     if (fuse == 3 && (!a.partial || !a.fold)) return hipErrorInvalidValue;
     hipLaunchKernelGGL(e->fn, dim3((unsigned)((a.N + rows_per_wg - 1) / rows_per_wg)), dim3(4 * kWave), lds, stream, a);
     hipError_t rc = hipGetLastError();

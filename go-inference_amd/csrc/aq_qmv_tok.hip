@@ -443,11 +443,7 @@ hipError_t qmvt_launch(int idx, const QmvArgs& a, hipStream_t stream) {
     const QmvTokEntry& e = kQmvTokTable[idx];
     // the 16-token form also stages 16 bytes of scales and biases per row and run of 256 codes (rows a run apart plus 16 bytes)
     const size_t lds = (size_t)e.lds + (size_t)e.wg_rows * (a.K / 256 + 1) * 16;
-    if (lds > 48 * 1024) {
-        hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(e.fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                            (int)lds);
-        if (rc != hipSuccess) return rc;
-    }
+    if (hipError_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(e.fn), (size_t)lds)) return rc;
     const int wg_rows = e.wg_rows;
     hipLaunchKernelGGL(e.fn, dim3((unsigned)((a.N + wg_rows - 1) / wg_rows)), dim3((unsigned)(e.v.waves * kWave)), lds, stream, a);
     return hipGetLastError();
