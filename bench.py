@@ -4,7 +4,9 @@
 A "step" is one pass of the decode hot path over one Gemma-style decoder layer: the seven 4-bit
 group-64 quantized GEMVs at batch 1 (q, k, v, o, gate, up, down).  Weights are synthetic (seeded),
 resident in HBM before the timed region, and the steps rotate over enough distinct layer copies that
-no launch finds its weights in the 256 MB Infinity Cache.  The printed JSON line carries the
+no launch finds its weights in the 256 MB Infinity Cache.  The weights are used in the device layout the library
+makes at load time (tile-major, aq_tile_weights: same bytes of storage, same results bit for bit; the same steps on
+the MLX arrays as uploaded are reported beside it).  The printed JSON line carries the
 whole-layer GB/s (`value`), the roofline of the dominant kernel (the 4096 -> 14336 qmv), and as extras
 the prefill qmm at M = 2048, the M = 1..32 sweep at 4 and 8 bit, the MoE gather block, and the
 reference CPU path timed on this box's host cores.
@@ -69,7 +71,7 @@ def traffic_from_profiles(name, kernel):
     return int(m.group(1)), "rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE on %s (profiles/%s)" % (kernel, name)
 
 
-def run_probe(which, variant=None):
+def run_probe(which, variant=None, layout="tiled"):
     import numpy as np
     import aq_mi355
     import fixtures as F
@@ -91,12 +93,17 @@ def run_probe(which, variant=None):
     deq = ctx.alloc(N * K * 4)
     ctx.dequant_f32(first[0], first[1], first[2], deq, N, K, GROUP, BITS)
     ctx.sync()
+    tiles = [ctx.tile_weights(*t, N, K, GROUP, BITS) for t in pool] if layout == "tiled" else None
+    ctx.sync()
     if which == "dominant":
         x = ctx.to_device(F.synthetic_x(1, K, seed=F.BASE_SEED + 1000))
         y = ctx.alloc(N * 2)
         for i in range(200 * ncopy):  # long enough for the clocks to settle: the first few hundred launches run slower
-            ww, ss, bb = pool[i % ncopy]
-            ctx.qmv(x, ww, ss, bb, y, 1, K, N, GROUP, BITS)
+            if tiles:
+                ctx.qmv(x, tiles[i % ncopy], None, None, y, 1, K, N, GROUP, BITS, aq_mi355.AQ_W_TILED)
+            else:
+                ww, ss, bb = pool[i % ncopy]
+                ctx.qmv(x, ww, ss, bb, y, 1, K, N, GROUP, BITS)
     elif which in ("rows16", "rows32"):
         # cfg 2: 16 / 32 rows of x against the same tensor
         M = int(which[4:])
@@ -135,8 +142,11 @@ def run_probe(which, variant=None):
             ctx.qmv(x, ww, ss, bb, y, 1, HK, HN, HG, BITS)
     elif which == "read_floor":
         for i in range(200 * ncopy):
-            ww, ss, bb = pool[i % ncopy]
-            ctx.probe_read(ww, ss, bb, K, N, 0)
+            if tiles:
+                ctx.probe_read(tiles[i % ncopy], None, None, K, N, 2)
+            else:
+                ww, ss, bb = pool[i % ncopy]
+                ctx.probe_read(ww, ss, bb, K, N, 1)
     elif which == "gather":
         # cfg 4: the fused gate|up gather and the down gather, 128 experts, 8 tokens x top-8
         E, TOK, TOPK, DM, DFF = 128, 8, 8, 2816, 1408
@@ -165,7 +175,7 @@ def run_probe(which, variant=None):
             ww, ss, bb = pool[i % ncopy]
             ctx.qmm(x, ww, ss, bb, y, M, K, N, GROUP, BITS)
     ctx.sync()
-    print(json.dumps({"probe": which, "fill_zero_bytes_written": 256 << 20,
+    print(json.dumps({"probe": which, "layout": layout, "fill_zero_bytes_written": 256 << 20,
                       "dequant_bytes_read": w.nbytes + s.nbytes + b.nbytes, "dequant_bytes_written": N * K * 4,
                       "kernel": ctx.last_variant(1 if which == "qmm" else 0)}))
     ctx.close()
@@ -186,6 +196,8 @@ def main():
                     "kernels of known traffic (a 256 MiB zero fill, a dequantisation of the gate tensor): the workload "
                     "of the rocprofv3 --pmc passes behind roofline.traffic")
     ap.add_argument("--variant", help="with --probe qmm: force this kernel variant (a name aq_variant_name lists)")
+    ap.add_argument("--layout", choices=["tiled", "mlx"], default="tiled", help="with --probe dominant / read_floor: the weights "
+                    "as the tile-major tensor made at load (default) or as the MLX arrays")
     ap.add_argument("--pmc-summary", metavar="DIR", help="print per-kernel averages of the counters a rocprofv3 --pmc "
                     "--output-format csv run left under DIR, and exit")
     args = ap.parse_args()
@@ -198,7 +210,7 @@ def main():
         sys.exit(2)
 
     if args.probe:
-        run_probe(args.probe, args.variant)
+        run_probe(args.probe, args.variant, args.layout)
         return
 
     import numpy as np
@@ -206,9 +218,7 @@ def main():
     import fixtures as F
 
     ctx = aq_mi355.Context(0)
-    dev_name = ctx.device_name()
-    if dev_name.startswith("AMD Instinct MI350 series ("):  # the driver reports no marketing name on some boxes; 256 CUs: MI355X
-        dev_name = dev_name.replace("MI350 series", "MI355X", 1)
+    dev_name = ctx.device_name()  # what the runtime reports (name, architecture, CUs, clock), unchanged
 
     # ---- synthetic layer, resident in HBM; copies made device-to-device -------------------------
     layer_bytes = sum(qmv_bytes(K, N) for _, K, N in LAYER)
@@ -231,6 +241,9 @@ def main():
                     ctx._check(ctx.lib.aq_d2d(ctx.handle, d.ptr, t.ptr, t.nbytes))
                 tensors[name] = dst
         layers.append(tensors)
+    # the device layout made at load: every tensor once more as a tile-major tensor (device to device)
+    T = aq_mi355.AQ_W_TILED
+    tiled = [{name: ctx.tile_weights(*t[name], dims_N, dims_K, GROUP, BITS) for name, dims_K, dims_N in LAYER} for t in layers]
     x4096 = ctx.to_device(F.synthetic_x(1, 4096, seed=F.BASE_SEED + 1000))
     x14336 = ctx.to_device(F.synthetic_x(1, 14336, seed=F.BASE_SEED + 1001))
     ys = {name: ctx.alloc(N * 2) for name, K, N in LAYER}
@@ -255,10 +268,22 @@ def main():
         return (pm(("q", "k", "v")), ctx.prepared_qmv(x4096, *t["o"], ys["o"], 1, 4096, 4096, GROUP, BITS),
                 pm(("gate", "up")), ctx.prepared_qmv(x14336, *t["down"], ys["down"], 1, 14336, 4096, GROUP, BITS))
 
-    calls = [prepare(t) for t in layers]
+    def prepare_tiled(t):
+        def pm(names):
+            return ctx.prepared_qmv_multi(x4096, [t[n] for n in names], [None] * len(names), [None] * len(names),
+                                          [ys[n] for n in names], [dims[n][1] for n in names], 1, 4096, GROUP, BITS, T)
+        return (pm(("q", "k", "v")), ctx.prepared_qmv(x4096, t["o"], None, None, ys["o"], 1, 4096, 4096, GROUP, BITS, T),
+                pm(("gate", "up")), ctx.prepared_qmv(x14336, t["down"], None, None, ys["down"], 1, 14336, 4096, GROUP, BITS, T))
+
+    calls_mlx = [prepare(t) for t in layers]
+    calls = [prepare_tiled(t) for t in tiled]
 
     def step(i):
         for call in calls[i % copies]:
+            call()
+
+    def step_mlx(i):
+        for call in calls_mlx[i % copies]:
             call()
 
     def replay_ms(launch, reps, replays=5):
@@ -302,15 +327,19 @@ def main():
     ms_stream = ctx.timer_stop() / args.steps
     ctx.sync()
     t_host = time.perf_counter() - t_host0
-    # the same layer as seven separate launches
+    # the same steps on the MLX arrays as they were uploaded (no load-time layout)
+    for i in range(args.warmup):
+        step_mlx(i)
+    ctx.sync()
+    ms_mlx = replay_ms(lambda i: step_mlx(args.warmup + i), args.steps)
+    # the same layer as seven separate launches (MLX arrays)
     for i in range(args.warmup):
         step_separate(i)
     ctx.sync()
     ms_separate = replay_ms(lambda i: step_separate(args.warmup + i), args.steps)
     variants = {}
     for name, K, N in LAYER:
-        w, s, b = layers[0][name]
-        ctx.qmv(x14336 if K == 14336 else x4096, w, s, b, ys[name], 1, K, N, GROUP, BITS)
+        ctx.qmv(x14336 if K == 14336 else x4096, tiled[0][name], None, None, ys[name], 1, K, N, GROUP, BITS, T)
         variants[name] = ctx.last_variant(0)
     ctx.sync()
 
@@ -330,54 +359,80 @@ def main():
     # ---- dominant kernel: qmv K=4096 -> N=14336, hipEvents on the launch stream ------------------
     dom = [layers[c][n] for c in range(copies) for n in ("gate", "up")]
     dom, dom_extra = widen_pool(dom)  # 640 MB of distinct tensors: every launch streams from HBM
+    dom_t = [tiled[c][n] for c in range(copies) for n in ("gate", "up")]
+    dom_t_extra = [ctx.tile_weights(*t, 14336, 4096, GROUP, BITS) for t in dom_extra]
+    dom_t = dom_t + dom_t_extra
     reps = 240
-    for i in range(24):
-        w, s, b = dom[i % len(dom)]
-        ctx.qmv(x4096, w, s, b, ys["gate"], 1, 4096, 14336, GROUP, BITS)
-    ctx.sync()
 
     def dom_launch(i):
+        ctx.qmv(x4096, dom_t[i % len(dom_t)], None, None, ys["gate"], 1, 4096, 14336, GROUP, BITS, T)
+
+    def dom_launch_mlx(i):
         w, s, b = dom[i % len(dom)]
         ctx.qmv(x4096, w, s, b, ys["gate"], 1, 4096, 14336, GROUP, BITS)
 
+    for i in range(24):
+        dom_launch(i)
+        dom_launch_mlx(i)
+    ctx.sync()
     dom_us = replay_ms(dom_launch, reps) * 1e3
+    dom_mlx_us = replay_ms(dom_launch_mlx, reps) * 1e3
     dom_bytes = qmv_bytes(4096, 14336)
     dom_gbps = dom_bytes / (dom_us * 1e-6) / 1e9
     # cached (same tensor every launch), reported separately
     dom_cached_us = replay_ms(lambda i: dom_launch(0), reps) * 1e3
-    # read floor: the same tensors, rotation and load instructions with the arithmetic, the activations and the store
-    # removed (mode 0: the matvec's own access shape; mode 1: contiguous 1 KiB per instruction)
+    # read floors: the same tensors in the same rotation and graph through the load instructions alone (no
+    # activations, no arithmetic, no store): mode 2 = the loads of the kernel timed above (tile-major tensor, 1 KiB of
+    # consecutive bytes per instruction, non-temporal), mode 1 = the loads of the matvec on the MLX arrays (whole lines
+    # of 8 rows per instruction, non-temporal), mode 3 = the MLX arrays as consecutive 1 KiB pieces, plain loads
     floor_us = {}
-    for mode in (0, 1):
+    for mode in (2, 1, 3):
         def floor_launch(i, mode=mode):
-            w, s, b = dom[i % len(dom)]
-            ctx.probe_read(w, s, b, 4096, 14336, mode)
+            if mode == 2:
+                ctx.probe_read(dom_t[i % len(dom_t)], None, None, 4096, 14336, 2)
+            else:
+                w, s, b = dom[i % len(dom)]
+                ctx.probe_read(w, s, b, 4096, 14336, mode)
         for i in range(24):
             floor_launch(i)
         ctx.sync()
         floor_us[mode] = replay_ms(floor_launch, reps) * 1e3
+    # an empty kernel in the same graph position: what a launch costs before it reads anything
+    empty = ctx.alloc(256)
+    for i in range(24):
+        ctx.fill_zero(empty, 16)
+    ctx.sync()
+    launch_us = replay_ms(lambda i: ctx.fill_zero(empty, 16), reps) * 1e3
+    empty.free()
 
     per_shape = {}
     for name, K, N in LAYER:
         pool, extra = widen_pool([layers[c][name] for c in range(copies)])
         xin = x14336 if K == 14336 else x4096
         n = max(240, len(pool))
+        pool_t = [tiled[c][name] for c in range(copies)] + [ctx.tile_weights(*t, N, K, GROUP, BITS) for t in extra]
+
+        def shape_launch(i, pool_t=pool_t, xin=xin, name=name, K=K, N=N):
+            ctx.qmv(xin, pool_t[i % len(pool_t)], None, None, ys[name], 1, K, N, GROUP, BITS, T)
+
+        def shape_launch_mlx(i, pool=pool, xin=xin, name=name, K=K, N=N):
+            w, s, b = pool[i % len(pool)]
+            ctx.qmv(xin, w, s, b, ys[name], 1, K, N, GROUP, BITS)
+
         for i in range(12):
-            w, s, b = pool[i % len(pool)]
-            ctx.qmv(xin, w, s, b, ys[name], 1, K, N, GROUP, BITS)
+            shape_launch(i)
+            shape_launch_mlx(i)
         ctx.sync()
-
-        def shape_launch(i, pool=pool, xin=xin, name=name, K=K, N=N):
-            w, s, b = pool[i % len(pool)]
-            ctx.qmv(xin, w, s, b, ys[name], 1, K, N, GROUP, BITS)
-
         us = replay_ms(shape_launch, n) * 1e3
+        us_mlx = replay_ms(shape_launch_mlx, n) * 1e3
         per_shape[name] = {"K": K, "N": N, "us": round(us, 3), "GBps": round(qmv_bytes(K, N) / us / 1e3, 1),
-                           "kernel": variants[name], "tensors_rotated": len(pool)}
+                           "us_mlx_layout": round(us_mlx, 3), "kernel": variants[name], "tensors_rotated": len(pool)}
         ctx.sync()
         for t in extra:
             for d in t:
                 d.free()
+        for d in pool_t[copies:]:
+            d.free()
 
     # ---- extra: prefill qmm at M = 2048 (cfg 3), bf16 MFMA roofline -------------------------------
     qmm = None
@@ -474,25 +529,41 @@ def main():
                 xm = ctx.to_device(F.synthetic_x(M, K, seed=F.BASE_SEED + 1100 + M))
                 ym = ctx.alloc(M * N * 2)
                 n = 120 if M <= 8 else 60
+                # up to eight rows of 4-bit codes run on the tile-major tensors (the kernels that read them take up to
+                # eight rows); everything else on the MLX arrays
+                use_tiles = bits == 4 and M <= 8
+
+                def m_launch(i, pool=pool, xm=xm, ym=ym, M=M, bits=bits, use_tiles=use_tiles):
+                    if use_tiles:
+                        ctx.qmv(xm, dom_t[i % len(dom_t)], None, None, ym, M, K, N, GROUP, bits, T)
+                    else:
+                        w, s, b = pool[i % len(pool)]
+                        ctx.qmv(xm, w, s, b, ym, M, K, N, GROUP, bits)
+
                 for i in range(6):
-                    w, s, b = pool[i % len(pool)]
-                    ctx.qmv(xm, w, s, b, ym, M, K, N, GROUP, bits)
+                    m_launch(i)
                 ctx.sync()
-
-                def m_launch(i, pool=pool, xm=xm, ym=ym, M=M, bits=bits):
-                    w, s, b = pool[i % len(pool)]
-                    ctx.qmv(xm, w, s, b, ym, M, K, N, GROUP, bits)
-
                 us = replay_ms(m_launch, n) * 1e3
                 by = qmv_bytes(K, N, M, bits)
                 small_m["b%d_m%d" % (bits, M)] = {"us": round(us, 3), "GBps": round(by / us / 1e3, 1),
                                                   "pct_of_hbm_peak": round(by / us / 1e3 / HBM_PEAK_GBPS * 100, 2),
-                                                  "kernel": ctx.last_variant(0) or ctx.last_variant(1)}
+                                                  "kernel": ctx.last_variant(0) or ctx.last_variant(1),
+                                                  "weights": "tile-major" if use_tiles else "MLX arrays"}
+                if use_tiles:
+                    def m_launch_mlx(i, pool=pool, xm=xm, ym=ym, M=M, bits=bits):
+                        w, s, b = pool[i % len(pool)]
+                        ctx.qmv(xm, w, s, b, ym, M, K, N, GROUP, bits)
+                    for i in range(6):
+                        m_launch_mlx(i)
+                    ctx.sync()
+                    small_m["b%d_m%d" % (bits, M)]["us_mlx_layout"] = round(replay_ms(m_launch_mlx, n) * 1e3, 3)
                 xm.free()
                 ym.free()
         for t in pools[8] + dom_extra:
             for d in t:
                 d.free()
+        for d in dom_t_extra:
+            d.free()
         # six-bit codes, groups of 64 (MLX 6 bit), one row of x: the same projection, 12 copies in turn
         rng6 = np.random.Generator(np.random.PCG64(F.BASE_SEED + 31))
         w6 = rng6.integers(0, 1 << 32, size=(N, K * 6 // 32), dtype=np.uint64).astype(np.uint32)
@@ -519,78 +590,112 @@ def main():
                 d.free()
 
         # ---- extra: MoE gather_qmv decode (cfg 4): 128 experts, 8 tokens x top-8, ids read on device --
+        # HBM-cold by construction: three copies of the expert slabs (2.6 GB) taken in turn and four seeded id sets
+        # (each 8 tokens x top-8 without replacement) taken in turn, so that between two uses of one slab copy about
+        # 700 MB of other expert rows have gone through the 256 MB Infinity Cache; every leg is a captured graph of 24
+        # blocks, replayed.
         E, TOK, TOPK, DM, DFF = 128, 8, 8, 2816, 1408
         routes = TOK * TOPK
+        NSLAB, NSETS, NBLOCKS = 3, 4, 24
         rng = np.random.Generator(np.random.PCG64(F.BASE_SEED + 77))
-        rhs = np.concatenate([rng.permutation(E)[:TOPK] for _ in range(TOK)]).astype(np.int32)
+        id_sets = [np.concatenate([rng.permutation(E)[:TOPK] for _ in range(TOK)]).astype(np.int32) for _ in range(NSETS)]
         lhs_tok = np.repeat(np.arange(TOK, dtype=np.int32), TOPK)
         lhs_route = np.arange(routes, dtype=np.int32)
         gu = F.synthetic_affine(E * 2 * DFF, DM, BITS, GROUP, seed=F.BASE_SEED + 40)  # [E, gate|up = 2*DFF, DM]
         down = F.synthetic_affine(E * DM, DFF, BITS, GROUP, seed=F.BASE_SEED + 41)    # [E, DM, DFF]: K = 1408 -> N = 2816
-        dgu = tuple(ctx.to_device(t) for t in gu)
-        dd = tuple(ctx.to_device(t) for t in down)
+        slabs = []
+        for c in range(NSLAB):
+            if c == 0:
+                slabs.append((tuple(ctx.to_device(t) for t in gu), tuple(ctx.to_device(t) for t in down)))
+            else:
+                pair = []
+                for src in slabs[0]:
+                    dst = tuple(ctx.alloc(t.nbytes) for t in src)
+                    for d, t in zip(dst, src):
+                        ctx._check(ctx.lib.aq_d2d(ctx.handle, d.ptr, t.ptr, t.nbytes))
+                    pair.append(dst)
+                slabs.append(tuple(pair))
         xt = ctx.to_device(F.synthetic_x(TOK, DM, seed=F.BASE_SEED + 1200))
-        d_rhs, d_tok, d_route = ctx.to_device(rhs), ctx.to_device(lhs_tok), ctx.to_device(lhs_route)
+        d_sets = [ctx.to_device(ids) for ids in id_sets]
+        d_tok, d_route = ctx.to_device(lhs_tok), ctx.to_device(lhs_route)
         yg, yu, yh = ctx.alloc(routes * DFF * 2), ctx.alloc(routes * DFF * 2), ctx.alloc(routes * DFF * 2)
         yd = ctx.alloc(routes * DM * 2)
 
-        def moe_unfused():
+        def moe_unfused(i):
+            dgu, dd = slabs[i % NSLAB]
+            d_rhs = d_sets[i % NSETS]
             ctx.gather_qmv(xt, dgu[0], dgu[1], dgu[2], d_tok, d_rhs, yg, routes, TOK, DM, DFF, E, 2 * DFF, 0, GROUP, BITS)
             ctx.gather_qmv(xt, dgu[0], dgu[1], dgu[2], d_tok, d_rhs, yu, routes, TOK, DM, DFF, E, 2 * DFF, DFF, GROUP, BITS)
             ctx.act_mul(yg, yu, yh, routes * DFF, aq_mi355.AQ_ACT_GELU_TANH)
             ctx.gather_qmv(yh, dd[0], dd[1], dd[2], d_route, d_rhs, yd, routes, routes, DFF, DM, E, DM, 0, GROUP, BITS)
 
-        def moe_fused():
+        def moe_fused(i):
+            dgu, dd = slabs[i % NSLAB]
+            d_rhs = d_sets[i % NSETS]
             ctx.gather_qmv_gate_up(xt, dgu[0], dgu[1], dgu[2], d_tok, d_rhs, yh, routes, TOK, DM, DFF, E, 2 * DFF, 0, DFF,
                                    GROUP, BITS, aq_mi355.AQ_ACT_GELU_TANH)
             ctx.gather_qmv(yh, dd[0], dd[1], dd[2], d_route, d_rhs, yd, routes, routes, DFF, DM, E, DM, 0, GROUP, BITS)
 
-        def time_us(fn, n=50):
-            for _ in range(5):
-                fn()
+        def moe_same(i):  # the same ids on the same slab copy every block: what the Infinity Cache makes of repeats
+            moe_fused(0)
+
+        def time_us(fn, n=NBLOCKS):
+            for i in range(6):
+                fn(i)
             ctx.sync()
-            ctx.timer_start()
-            for _ in range(n):
-                fn()
-            return ctx.timer_stop() * 1e3 / n
+            return replay_ms(fn, n) * 1e3
 
         us_unfused = time_us(moe_unfused)
         us = time_us(moe_fused)
         moe_kernel = ctx.last_variant(0)
+        us_same = time_us(moe_same)
 
         # the whole routed block on the device: scores -> router -> gathers -> combine, no host visit
+        # (four sets of router scores in turn, so the ids change from block to block here too)
         rng_l = np.random.Generator(np.random.PCG64(F.BASE_SEED + 78))
-        d_logits = ctx.to_device(rng_l.normal(0.0, 1.0, size=(TOK, E)).astype(np.float32))
+        d_logits = [ctx.to_device(rng_l.normal(0.0, 1.0, size=(TOK, E)).astype(np.float32)) for _ in range(NSETS)]
         d_ids, d_wts, d_tor = ctx.alloc(routes * 4), ctx.alloc(routes * 4), ctx.alloc(routes * 4)
         y_out = ctx.alloc(TOK * DM * 2)
 
-        def moe_block():
-            ctx.moe_route(d_logits, TOK, E, TOPK, d_ids, d_wts, d_tor)
+        def moe_block(i):
+            dgu, dd = slabs[i % NSLAB]
+            ctx.moe_route(d_logits[i % NSETS], TOK, E, TOPK, d_ids, d_wts, d_tor)
             ctx.gather_qmv_gate_up(xt, dgu[0], dgu[1], dgu[2], d_tor, d_ids, yh, routes, TOK, DM, DFF, E, 2 * DFF, 0, DFF,
                                    GROUP, BITS, aq_mi355.AQ_ACT_GELU_TANH)
             ctx.gather_qmv(yh, dd[0], dd[1], dd[2], d_route, d_ids, yd, routes, routes, DFF, DM, E, DM, 0, GROUP, BITS)
             ctx.moe_combine(yd, d_wts, y_out, TOK, TOPK, DM)
 
         us_block = time_us(moe_block)
-        for t in (d_logits, d_ids, d_wts, d_tor, y_out):
+        for t in d_logits + [d_ids, d_wts, d_tor, y_out]:
             t.free()
         per_route = 2 * qmv_bytes(DM, DFF) + qmv_bytes(DFF, DM)
-        distinct = len(set(rhs.tolist()))
+        distinct = [len(set(ids.tolist())) for ids in id_sets]
+        mean_distinct = sum(distinct) / len(distinct)
         # bytes of the distinct experts touched, each expert's three matrices counted once
         expert_bytes = 3 * (DFF * DM * BITS // 8 + 2 * DFF * (DM // GROUP) * 2)
-        gather = {"experts": E, "tokens": TOK, "top_k": TOPK, "routes": routes, "distinct_experts": distinct,
+        act_bytes = TOK * DM * 2 + 2 * routes * DFF * 2 + routes * DM * 2  # x, the gated rows written and read, y
+        distinct_bytes = mean_distinct * expert_bytes + act_bytes
+        gather = {"experts": E, "tokens": TOK, "top_k": TOPK, "routes": routes, "id_sets": NSETS, "slab_copies": NSLAB,
+                  "distinct_experts_per_set": distinct,
                   "us_per_moe_block": round(us, 3), "launches": 2,
+                  "GBps_distinct_expert_bytes": round(distinct_bytes / us / 1e3, 1),
+                  "pct_of_hbm_peak": round(distinct_bytes / us / 1e3 / HBM_PEAK_GBPS * 100, 2),
+                  "GBps_route_bytes": round(routes * per_route / us / 1e3, 1),
                   "us_per_moe_block_unfused": round(us_unfused, 3), "launches_unfused": 4,
                   "us_per_moe_block_with_router_and_combine": round(us_block, 3), "launches_with_router_and_combine": 4,
-                  "GBps_route_bytes": round(routes * per_route / us / 1e3, 1),
-                  "pct_of_hbm_peak": round(routes * per_route / us / 1e3 / HBM_PEAK_GBPS * 100, 2),
-                  "GBps_distinct_expert_bytes": round(distinct * expert_bytes / us / 1e3, 1),
+                  "us_per_moe_block_same_ids_same_slab": round(us_same, 3),
                   "note": "experts hold a fused gate|up slab [2*1408, 2816] and a down matrix [2816, 1408]; fused = "
                           "aq_gather_qmv_gate_up (GELU-tanh epilogue) + down gather; unfused = gate gather, up gather, "
-                          "aq_act_mul, down gather; route bytes = routes x one expert's codes+scales+biases+x+y; the "
-                          "same expert ids every step, so repeated experts may hit cache",
+                          "aq_act_mul, down gather.  HBM-cold: 3 slab copies (2.6 GB) and 4 seeded id sets in turn, a "
+                          "graph of 24 blocks replayed, so ~700 MB of other expert rows pass between two uses of a slab "
+                          "copy.  The headline figure counts every distinct expert of a block once (mean over the id "
+                          "sets) plus the activations; route bytes count an expert once per route that uses it; "
+                          "same_ids_same_slab repeats one block and shows what the cache makes of that",
                   "kernel": moe_kernel}
-        for t in dgu + dd + (xt, d_rhs, d_tok, d_route, yg, yu, yh, yd):
+        for pair in slabs:
+            for t in pair[0] + pair[1]:
+                t.free()
+        for t in d_sets + [xt, d_tok, d_route, yg, yu, yh, yd]:
             t.free()
 
         # ---- extra: the dense MLP of the layer with the activation fused (GELU-tanh) ----------------
@@ -598,13 +703,18 @@ def main():
         mlp_bytes = 2 * qmv_bytes(4096, 14336) + qmv_bytes(14336, 4096)
 
         def mlp_three(i):
-            L = layers[i % copies]
-            ctx.qmv_multi(x4096, [L["gate"][0], L["up"][0]], [L["gate"][1], L["up"][1]], [L["gate"][2], L["up"][2]],
-                          [hg, hu], [14336, 14336], 1, 4096, GROUP, BITS)
+            L = tiled[i % copies]
+            ctx.qmv_multi(x4096, [L["gate"], L["up"]], [None, None], [None, None], [hg, hu], [14336, 14336], 1, 4096, GROUP, BITS, T)
             ctx.act_mul(hg, hu, hh, 14336, aq_mi355.AQ_ACT_GELU_TANH)
-            ctx.qmv(hh, L["down"][0], L["down"][1], L["down"][2], ys["down"], 1, 14336, 4096, GROUP, BITS)
+            ctx.qmv(hh, L["down"], None, None, ys["down"], 1, 14336, 4096, GROUP, BITS, T)
 
         def mlp_pair(i):
+            L = tiled[i % copies]
+            ctx.qmv_gate_up(x4096, (L["gate"], None, None), (L["up"], None, None), hh, 1, 4096, 14336, GROUP, BITS,
+                            aq_mi355.AQ_ACT_GELU_TANH, T)
+            ctx.qmv(hh, L["down"], None, None, ys["down"], 1, 14336, 4096, GROUP, BITS, T)
+
+        def mlp_pair_mlx(i):
             L = layers[i % copies]
             ctx.qmv_gate_up(x4096, L["gate"], L["up"], hh, 1, 4096, 14336, GROUP, BITS, aq_mi355.AQ_ACT_GELU_TANH)
             ctx.qmv(hh, L["down"][0], L["down"][1], L["down"][2], ys["down"], 1, 14336, 4096, GROUP, BITS)
@@ -617,13 +727,14 @@ def main():
                         aq_mi355.AQ_ACT_GELU_TANH)
 
         mlp = {"bytes": mlp_bytes}
-        for key, fn, launches in (("three_launches", mlp_three, 3), ("gate_up_fused", mlp_pair, 2), ("x_load_fused", mlp_xload, 2)):
-            counter = iter(range(10 ** 9))
-            t_us = time_us(lambda: fn(next(counter)), n=120)
+        for key, fn, launches in (("three_launches", mlp_three, 3), ("gate_up_fused", mlp_pair, 2),
+                                  ("gate_up_fused_mlx_layout", mlp_pair_mlx, 2), ("x_load_fused_mlx_layout", mlp_xload, 2)):
+            t_us = time_us(fn, n=120)
             mlp[key] = {"us": round(t_us, 3), "launches": launches, "GBps": round(mlp_bytes / t_us / 1e3, 1),
                         "pct_of_hbm_peak": round(mlp_bytes / t_us / 1e3 / HBM_PEAK_GBPS * 100, 2)}
-        mlp["note"] = ("gate, up 4096->14336 and down 14336->4096 of the cfg1 layer with GELU-tanh: multi-matrix launch + "
-                       "aq_act_mul + down; aq_qmv_gate_up + down; multi-matrix launch + aq_qmv_act")
+        mlp["note"] = ("gate, up 4096->14336 and down 14336->4096 of the cfg1 layer with GELU-tanh, tile-major weights unless "
+                       "the key says otherwise: multi-matrix launch + aq_act_mul + down; aq_qmv_gate_up + down; the same on the "
+                       "MLX arrays; multi-matrix launch + aq_qmv_act (MLX arrays); graphs of 120 MLPs, replayed")
         for t in (hg, hu, hh):
             t.free()
 
@@ -802,12 +913,15 @@ def main():
         "vs_baseline": None,
         "dtype": "bf16 activations x 4-bit affine codes, fp32 accumulate",
         "data": "synthetic (seeded PCG64: uniform codes, scale=|N(0,0.02)|+1e-3, bias=-8*scale+N(0,1e-3), x~N(0,1)); "
-                "weights resident in HBM, %d layer copies rotated (%.0f MB)" % (copies, copies * weight_bytes / 1e6),
+                "weights resident in HBM in the tile-major layout made at load (aq_tile_weights), %d layer copies rotated "
+                "(%.0f MB)" % (copies, copies * weight_bytes / 1e6),
         "config": {"workload": "cfg1: Gemma-style decoder layer at batch 1, 4-bit group-64: q/o 4096x4096, k/v 4096->1024, "
                                "gate/up 4096->14336, down 14336->4096; %d algorithmic bytes per step" % layer_bytes,
                    "device": dev_name, "launches_per_step": 4,
                    "launches": "q|k|v fused, o, gate|up fused, down (aq_qmv_multi: one grid over projections that share x)"},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "mlx_layout": {"ms_per_step": round(ms_mlx, 5), "GBps": round(layer_bytes / (ms_mlx * 1e-3) / 1e9, 1),
+                       "note": "the same steps on the MLX arrays as uploaded (no load-time layout); same output bytes"},
         "ms_per_step_stream_launches": round(ms_stream, 5),
         "timing": "the K steps are captured into one HIP graph and replayed between two HIP events on the library's "
                   "stream (median of 5 replays); ms_per_step_stream_launches is the same K steps launched one by one "
@@ -820,11 +934,18 @@ def main():
                      "frac": round(dom_gbps / HBM_PEAK_GBPS, 4), "traffic": dom_traffic, "traffic_note": dom_traffic_note,
                      "bytes_per_launch": dom_bytes, "us_per_launch": round(dom_us, 3),
                      "us_per_launch_cached": round(dom_cached_us, 3),
-                     "read_floor": {"us_same_access_shape": round(floor_us[0], 3), "us_contiguous": round(floor_us[1], 3),
-                                    "frac_of_read_floor": round(floor_us[0] / dom_us, 4),
-                                    "note": "aq_probe_read over the same tensors in the same rotation and graph: the "
-                                            "matvec's load instructions (codes, scales, biases) with no activations, "
-                                            "arithmetic or store; frac_of_read_floor = that time / the matvec's"}},
+                     "weights": "tile-major (aq_tile_weights)", "us_per_launch_mlx_layout": round(dom_mlx_us, 3),
+                     "frac_mlx_layout": round(dom_bytes / (dom_mlx_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                     "read_floor": {"us_same_loads": round(floor_us[2], 3), "us_mlx_layout_loads": round(floor_us[1], 3),
+                                    "us_mlx_contiguous_plain": round(floor_us[3], 3), "us_empty_launch": round(launch_us, 3),
+                                    "frac_of_read_floor": round(floor_us[2] / dom_us, 4),
+                                    "note": "aq_probe_read over the same tensors in the same rotation and graph, loads only "
+                                            "(no activations, arithmetic or store): same_loads = the load instructions of "
+                                            "the kernel timed here (tile-major tensor, 1 KiB of consecutive bytes per "
+                                            "instruction, non-temporal); mlx_layout_loads = those of the matvec on the MLX "
+                                            "arrays (whole 128-byte lines of 8 rows, non-temporal); empty_launch = a "
+                                            "16-byte fill kernel in the same graph; frac_of_read_floor = same_loads / "
+                                            "the matvec's time"}},
         "cpu_baseline": cpu,
         "per_shape": per_shape,
         "qmm": qmm,

@@ -218,8 +218,12 @@ const QmvRule kQmvRules[] = {
     {4, 64, 1, 1, 1, kFamDiag},             // K a multiple of 128 in 2..8 steps of 1024 codes
     {0, 0, 1, 1, 1, kFamDot2},              // 4 / 8 bit, groups of 32 / 64 / 128, 16-byte chunks inside one group
     {0, 0, 1, 1, 1, kFamGeneric},
-    {4, 64, 0, 1, 8, kFamDiag},             // one row up to 16 steps of 1024 codes, up to 8 rows at 2..4 steps: every row
-                                            // of such a call has the bytes of a call with that row alone
+    {4, 64, 0, 1, 8, kFamDiag},             // K from 1152 to 16384: up to 8 rows in one launch at 2..4 steps of 1024 codes,
+                                            // up to 4 per launch at longer K; every row of such a call has the bytes of a
+                                            // call with that row alone
+    {4, 64, 0, 2, 8, kFamDot2},             // K the diagonal kernels do not take (up to 1024, no multiple of 128, beyond
+                                            // 16384): the kernel a single row of such a K runs on, four rows a launch, so
+                                            // that rows keep the bytes of single-row calls here too
     {4, 32, 0, 1, 2, kFamDiag},             // groups of 32: two tokens x eight groups as MFMA rows
     {8, 0, 0, 1, 1, kFamDot2},              // one row of 8-bit codes: the dot2 kernel with its non-temporal loads, 12.4 us for
                                             // 4096 x 14336 (63 % of the HBM peak) against 14.2 us on the block-MFMA kernel
@@ -228,8 +232,10 @@ const QmvRule kQmvRules[] = {
                                             // the dot2 kernels; the reference states its rows-equal-single-rows contract for
                                             // 4-bit codes only, qmv_rows_test.go:36-41)
     {4, 64, 0, 5, 32, kFamTok},             // the same for 4-bit codes, up to 32 rows
-                                            // (5..8 rows: only where the diagonal kernels passed; they measure 11.2 us
-                                            // against 14.4 us at 8 rows of 4096 x 14336, but not row by row the same bytes)
+                                            // (5..8 rows get here only when the two rules that keep the bytes of single-row
+                                            // calls have passed, e.g. on operands that are not 16-byte aligned, or with the
+                                            // diagonal and dot2 families switched off: this kernel is faster at long K,
+                                            // 15.6 against 2 x 9 us at 8 rows of 14336 x 4096, but not row by row the same bytes)
     {0, 0, 0, 9, 64, kFamTilesLarge},       // 16 Mi codes and more: the 16-row block-MFMA kernel is bound by its 4x4x4 MFMAs
     {0, 0, 0, 2, 16, kFamBlk},              // the whole call in one launch of up to 16 rows (4 where K is long)
     {8, 0, 0, 1, 1, kFamBlk},               // (a single row of 4-bit codes is faster on the dot2 kernels)
@@ -279,10 +285,32 @@ int run_diag(aq_ctx* ctx, const aq::QmvArgs& a, int group_size, int bits, bool g
                    : gather           ? aq::qmvd_pick_gather(a.K)
                    : group_size == 32 ? aq::qmvd_pick_g32(a.M, a.K, a.N)
                                       : aq::qmvd_pick(a.M, a.K, a.N);
-    if (di < 0 || !aq::qmvd_fits(a, bits, group_size, gather, di)) return kPass;
-    ctx->last_variant[0] = aq::qmvd_variant(di)->name;
-    AQ_HIP(aq::qmvd_launch(di, a, ctx->stream), "hipLaunchKernel");
-    return AQ_OK;
+    if (di >= 0 && aq::qmvd_fits(a, bits, group_size, gather, di)) {
+        ctx->last_variant[0] = aq::qmvd_variant(di)->name;
+        AQ_HIP(aq::qmvd_launch(di, a, ctx->stream), "hipLaunchKernel");
+        return AQ_OK;
+    }
+    // Five to eight rows of a K that one launch takes for up to four: two launches.  Every row of a call has the bytes
+    // of a call with that row alone (go/engine/metal/qmv_rows.go:14-24), which the other families do not give.
+    if (forced < 0 && !gather && group_size == 64 && a.M > 4 && a.M <= 8) {
+        const int d4 = aq::qmvd_pick(4, a.K, a.N);
+        aq::QmvArgs part = a;
+        part.M = 4;
+        if (d4 >= 0 && aq::qmvd_fits(part, bits, group_size, false, d4)) {
+            const size_t esize = a.out_f32 ? 4 : 2;
+            for (int m0 = 0; m0 < a.M; m0 += 4) {
+                part.M = a.M - m0 < 4 ? a.M - m0 : 4;
+                part.x = a.x + (size_t)m0 * a.K;
+                part.y = static_cast<char*>(a.y) + (size_t)m0 * a.N * esize;
+                const int dp = aq::qmvd_pick(part.M, a.K, a.N);
+                if (dp < 0 || !aq::qmvd_fits(part, bits, group_size, false, dp)) return kPass;
+                ctx->last_variant[0] = aq::qmvd_variant(dp)->name;
+                AQ_HIP(aq::qmvd_launch(dp, part, ctx->stream), "hipLaunchKernel");
+            }
+            return AQ_OK;
+        }
+    }
+    return kPass;
 }
 
 int run_tok(aq_ctx* ctx, const aq::QmvArgs& a, int group_size, int bits, bool gather, int forced) {
@@ -417,9 +445,11 @@ int aq_create(int device, aq_ctx** out) {
     ctx->device = device;
     ctx->cu_count = prop.multiProcessorCount;
     ctx->families_off = families_off_from_env(getenv("AQ_MI355_DISABLE"));
-    // (some hosts report no marketing name)
-    snprintf(ctx->name, sizeof ctx->name, "%s (%s, %d CUs)", prop.name[0] ? prop.name : "AMD Instinct MI350 series", prop.gcnArchName,
-             prop.multiProcessorCount);
+    // what the runtime reports, unchanged; a host that reports no marketing name shows the architecture instead
+    char arch_only[80];
+    snprintf(arch_only, sizeof arch_only, "%.60s device (no name reported)", prop.gcnArchName);
+    snprintf(ctx->name, sizeof ctx->name, "%s (%s, %d CUs, %d MHz)", prop.name[0] ? prop.name : arch_only, prop.gcnArchName,
+             prop.multiProcessorCount, prop.clockRate / 1000);
     rc = hipStreamCreateWithFlags(&ctx->own_stream, hipStreamNonBlocking);
     if (rc == hipSuccess) rc = hipEventCreate(&ctx->ev0);
     if (rc == hipSuccess) rc = hipEventCreate(&ctx->ev1);
@@ -616,8 +646,8 @@ void aq_graph_destroy(aq_graph* graph) {
 int aq_probe_read(aq_ctx* ctx, const void* packed, const void* scales, const void* biases, int K, int N, int mode) {
     if (!ctx) return fail(AQ_ERR_ARG, "aq_probe_read: ctx is null");
     if (K <= 0 || N <= 0 || K % 1024 != 0) return fail(AQ_ERR_SHAPE, "aq_probe_read: K must be a positive multiple of 1024, N positive");
-    if (mode != 0 && mode != 1) return fail(AQ_ERR_ARG, "aq_probe_read: mode is 0 or 1");
-    if (!packed || !scales || !biases) return fail(AQ_ERR_ARG, "aq_probe_read: null operand");
+    if (mode < 0 || mode > 3) return fail(AQ_ERR_ARG, "aq_probe_read: mode is 0..3");
+    if (!packed || (mode != 2 && (!scales || !biases))) return fail(AQ_ERR_ARG, "aq_probe_read: null operand");
     if (!aligned(packed, 16) || !aligned(scales, 8) || !aligned(biases, 8))
         return fail(AQ_ERR_ARG, "aq_probe_read: packed must be 16-byte, scales and biases 8-byte aligned");
     std::lock_guard<std::mutex> lk(ctx->mu);

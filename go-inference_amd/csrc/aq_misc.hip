@@ -353,31 +353,53 @@ hipError_t qmv_generic_launch(const QmvArgs& a, int bits, int group_size, bool g
     return hipGetLastError();
 }
 
-// ---- measurement aid: the bytes of an affine tensor read once, no arithmetic ----------------------------------
-// mode 0: the access shape of the diagonal-MFMA matvec (a wavefront reads 512 bytes of each of 16 rows as eight 16-byte
-// loads per lane, 64 contiguous bytes per row and instruction, plus 8 bytes of scales and of biases per lane);
-// mode 1: the same bytes as contiguous 1 KiB per instruction.  Nothing is written unless the data xor to a magic value.
+// Measurement aid: streams a 4-bit group-64 tensor once through the load instructions of the single-row matvec and does
+// nothing with the data (no activations, no arithmetic, no store): the time of a launch that only reads.
+//   mode 0: MLX arrays, 64 bytes of each of 16 rows per instruction, plain loads (the matvec of small matrices)
+//   mode 1: MLX arrays, whole 128-byte lines of 8 rows per instruction with the non-temporal hint (the matvec of
+//           matrices of 16 MB and more)
+//   mode 2: tile-major tensor (aq_tile.h), 1 KiB of consecutive bytes per instruction with the hint (the matvec on
+//           tile-major weights); w is that tensor, s and b are not read
+//   mode 3: MLX arrays as consecutive 1 KiB pieces, plain loads
+// Nothing is written unless the data xor to a magic value.
 typedef uint32_t probe_u32x4_t __attribute__((ext_vector_type(4)));
 template <int MODE>
 __global__ __launch_bounds__(256) void read_probe_kernel(const char* __restrict__ w, const char* __restrict__ s,
                                                           const char* __restrict__ b, int64_t rows, int row_bytes, int sb_bytes,
                                                           uint32_t* out) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int64_t unit = ((int64_t)blockIdx.x * 4 + wave);  // 8 KiB of codes each
+    const int64_t unit = ((int64_t)blockIdx.x * 4 + wave);  // 8 KiB of codes each: a step of 1024 codes of 16 rows
     probe_u32x4_t v[8];
-    uint2 sv, bv;
-    if (MODE == 0) {
+    uint2 sv = make_uint2(0, 0), bv = make_uint2(0, 0);
+    if (MODE == 0 || MODE == 1) {
         const int steps = row_bytes / 512;                  // wavefront steps per row
         const int64_t rset = unit / steps;
         const int step = (int)(unit - rset * steps);
         int64_t row = rset * 16 + (lane & 15);
         if (row >= rows) row = rows - 1;
-        const char* p = w + row * row_bytes + step * 512 + (lane >> 4) * 16;
+        if (MODE == 0) {
+            const char* p = w + row * row_bytes + step * 512 + (lane >> 4) * 16;
 #pragma unroll
-        for (int c = 0; c < 8; c++) v[c] = *reinterpret_cast<const probe_u32x4_t*>(p + c * 64);
+            for (int c = 0; c < 8; c++) v[c] = *reinterpret_cast<const probe_u32x4_t*>(p + c * 64);
+        } else {
+#pragma unroll
+            for (int c = 0; c < 8; c++) {
+                int64_t r8 = rset * 16 + (lane & 7) + 8 * (c & 1);
+                if (r8 >= rows) r8 = rows - 1;
+                const char* p = w + r8 * row_bytes + step * 512 + (c >> 1) * 128 + ((lane & 15) >> 3) * 64 + (lane >> 4) * 16;
+                v[c] = __builtin_nontemporal_load(reinterpret_cast<const probe_u32x4_t*>(p));
+            }
+        }
         const int64_t so = row * sb_bytes + step * 32 + (lane >> 4) * 8;
         sv = *reinterpret_cast<const uint2*>(s + so);
         bv = *reinterpret_cast<const uint2*>(b + so);
+    } else if (MODE == 2) {
+        const char* p = w + unit * 9216 + lane * 16;
+        const probe_u32x4_t sb = __builtin_nontemporal_load(reinterpret_cast<const probe_u32x4_t*>(p));
+        sv = make_uint2(sb[0], sb[1]);
+        bv = make_uint2(sb[2], sb[3]);
+#pragma unroll
+        for (int c = 0; c < 8; c++) v[c] = __builtin_nontemporal_load(reinterpret_cast<const probe_u32x4_t*>(p + 1024 + c * 1024));
     } else {
         const int64_t total = rows * row_bytes;
         int64_t base = unit * 8192 + lane * 16;
@@ -398,18 +420,22 @@ __global__ __launch_bounds__(256) void read_probe_kernel(const char* __restrict_
     if (acc == 0x9E3779B9u && out) out[threadIdx.x & 63] = acc;
 }
 
+// (mode 2 is only defined for K a multiple of 1024: every tile then has the full 9 KiB)
 hipError_t read_probe_launch(const void* w, const void* s, const void* b, int64_t rows, int row_bytes, int sb_bytes, int mode,
                              uint32_t* out, hipStream_t stream) {
     if (rows <= 0 || row_bytes < 512 || row_bytes % 512 != 0 || sb_bytes * 16 != row_bytes)  // (4-bit codes, groups of 64)
         return hipErrorInvalidValue;
     const int64_t units = ((rows + 15) / 16) * 16 * (int64_t)row_bytes / 8192;
-    const unsigned grid = (unsigned)((units + 3) / 4);
-    if (mode == 0)
-        hipLaunchKernelGGL(read_probe_kernel<0>, dim3(grid), dim3(256), 0, stream, static_cast<const char*>(w),
-                           static_cast<const char*>(s), static_cast<const char*>(b), rows, row_bytes, sb_bytes, out);
-    else
-        hipLaunchKernelGGL(read_probe_kernel<1>, dim3(grid), dim3(256), 0, stream, static_cast<const char*>(w),
-                           static_cast<const char*>(s), static_cast<const char*>(b), rows, row_bytes, sb_bytes, out);
+    if (units % 4 != 0) return hipErrorInvalidValue;  // whole workgroups of four wavefronts (K a multiple of 1024)
+    const unsigned grid = (unsigned)(units / 4);
+    const char *wc = static_cast<const char*>(w), *sc = static_cast<const char*>(s), *bc = static_cast<const char*>(b);
+    switch (mode) {
+        case 0: hipLaunchKernelGGL(read_probe_kernel<0>, dim3(grid), dim3(256), 0, stream, wc, sc, bc, rows, row_bytes, sb_bytes, out); break;
+        case 1: hipLaunchKernelGGL(read_probe_kernel<1>, dim3(grid), dim3(256), 0, stream, wc, sc, bc, rows, row_bytes, sb_bytes, out); break;
+        case 2: hipLaunchKernelGGL(read_probe_kernel<2>, dim3(grid), dim3(256), 0, stream, wc, sc, bc, rows, row_bytes, sb_bytes, out); break;
+        case 3: hipLaunchKernelGGL(read_probe_kernel<3>, dim3(grid), dim3(256), 0, stream, wc, sc, bc, rows, row_bytes, sb_bytes, out); break;
+        default: return hipErrorInvalidValue;
+    }
     return hipGetLastError();
 }
 

@@ -760,7 +760,9 @@ bool qmvd_fits(const QmvArgs& a, int bits, int group_size, bool gather, int idx)
         const int64_t total = tile_total_bytes(a.N, a.K, group_size, bits);
         if (total < 0 || total >= ((int64_t)1 << 32)) return false;
     }
-    return qmvd_lds_bytes_for(a.M, a.K, v->waves * v->rows, (v->m + 3) / 4, g32_of(*v)) <= 96 * 1024;
+    // (up to four steps: two workgroups per CU; longer K: whatever one workgroup may use)
+    return qmvd_lds_bytes_for(a.M, a.K, v->waves * v->rows, (v->m + 3) / 4, g32_of(*v)) <=
+           (size_t)(steps_for(a.K, cps_of(*v)) <= 4 ? 96 : 156) * 1024;
 }
 
 hipError_t qmvd_launch(int idx, const QmvArgs& a, hipStream_t stream) {
@@ -794,8 +796,9 @@ int qmvd_pick(int M, int K, int N) {
     } else if (steps == 3 || steps == 4) {
         nw = 4;
         nr = M == 1 ? 1 : M == 2 ? 2 : 4;
-    } else if (steps <= 16 && M == 1) {
-        // one step per wavefront (an idle one when the count is odd); more rows would stage too much x per workgroup
+    } else if (steps <= 16 && M <= 4) {
+        // one step per wavefront (an idle one when the count is odd) and one set of rows per workgroup: up to four
+        // activation rows of this length fit the LDS (more go in further launches, see run_diag)
         nw = (steps + 1) & ~1;
         nr = 1;
     } else {

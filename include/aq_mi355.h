@@ -103,10 +103,17 @@ int aq_capture_end(aq_ctx *ctx, aq_graph **out);
 int aq_graph_launch(aq_ctx *ctx, aq_graph *graph);
 void aq_graph_destroy(aq_graph *graph);
 
-/* Measurement aid with no counterpart in the reference: streams the packed codes, scales and biases of a 4-bit
- * group-64 tensor [N, K] through the same load instructions the single-row matvec issues (mode 0: 64 contiguous
- * bytes of each of 16 rows per instruction; mode 1: contiguous 1 KiB pieces) and does nothing with them.  Its time
- * is the floor any matvec over that tensor can reach on this device: the benchmark reports the matvec beside it.
+/* Measurement aid with no counterpart in the reference: streams the codes, scales and biases of a 4-bit group-64
+ * tensor [N, K] once through the load instructions of the single-row matvec and does nothing with them (no
+ * activations, no arithmetic, no store).  Its time is what a launch that only reads that tensor costs on this device;
+ * the benchmark reports the matvec beside the mode whose loads it issues.
+ *   mode 0: MLX arrays, 64 contiguous bytes of each of 16 rows per instruction, plain loads (the matvec's loads on
+ *           matrices under 16 MB)
+ *   mode 1: MLX arrays, whole 128-byte lines of 8 rows per instruction with the non-temporal hint (its loads on
+ *           larger matrices)
+ *   mode 2: `packed` is a tile-major tensor (aq_tile_weights), read as 1 KiB of consecutive bytes per instruction with
+ *           the hint (its loads on tile-major weights); scales and biases are not read and may be NULL
+ *   mode 3: MLX arrays as consecutive 1 KiB pieces, plain loads
  * K a multiple of 1024.  Stream-ordered; writes nothing. */
 int aq_probe_read(aq_ctx *ctx, const void *packed, const void *scales, const void *biases, int K, int N, int mode);
 

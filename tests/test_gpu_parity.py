@@ -262,11 +262,12 @@ def test_qmv_block_family_many_batches(ctx, orc):
     batch of staged scales holds (K = 512: one wavefront per workgroup, 4096 workgroups)."""
     M, K, N = 3, 512, 4 * 4096 * 19 + 8
     say("many batches", M, K, N)
-    words, s, b = F.synthetic_affine(N, K, 4, 64, seed=5)
+    # (groups of 128: few rows of group-64 codes go to the kernels whose rows carry the bytes of single-row calls)
+    words, s, b = F.synthetic_affine(N, K, 4, 128, seed=5)
     x = F.synthetic_x(M, K, seed=6)
-    ref = F.reference_f64(x, words, s, b, 4, 64, K)
+    ref = F.reference_f64(x, words, s, b, 4, 128, K)
     dw = DeviceAffine(ctx, words, s, b)
-    acc = run_qmv(ctx, x, dw, M, K, N, 64, 4, True)
+    acc = run_qmv(ctx, x, dw, M, K, N, 128, 4, True)
     assert ctx.last_variant(0).startswith("qmvb_"), ctx.last_variant(0)
     check_accumulators(acc, ref, "many batches")
     dw.free()
@@ -303,8 +304,11 @@ def test_qmvd_every_variant(ctx, orc):
                 dw, x, ref = data[(K, gs)]
                 ctx.force_variant(0, idx)
                 for rows in ((1, 2) if m == 2 else (1, 2, 3, 4) if m == 4 else (1, 4, 5, 7, 8)):
-                    if rows * K * 2 + rows * ((K + 255) // 256) * (96 if gs == 32 else 48) + 128 + wg_waves * max(1, m // 4) * 256 > 96 * 1024:
-                        # the activations of all rows and their group sums sit in LDS: beyond 96 KiB the variant refuses
+                    k_steps = -(-(-(-K // 256)) // (3 if name.endswith("_c3") else 4))
+                    lds_limit = (96 if k_steps <= 4 else 156) * 1024
+                    if rows * K * 2 + rows * ((K + 255) // 256) * (96 if gs == 32 else 48) + 128 + wg_waves * max(1, m // 4) * 256 > lds_limit:
+                        # the activations of all rows and their group sums sit in LDS: beyond 96 KiB (two workgroups a
+                        # CU; 156 KiB for K of more than four steps) the variant refuses
                         with pytest.raises(aq_mi355.AqError) as ei:
                             run_qmv(ctx, x[:rows], dw, rows, K, N, gs, bits, True)
                         assert ei.value.code == aq_mi355.AQ_ERR_ARG
@@ -369,9 +373,9 @@ def test_qmvd_gather_every_variant(ctx, orc):
 
 
 def test_qmvd_is_the_default_for_few_rows(ctx, orc):
-    """4-bit group-64 codes: 1..8 activation rows with K of 2, 3 or 4 steps of 1024 codes, and one row with up to 16
-    steps, land on the diagonal-MFMA kernels without forcing, rows beyond the last full 16 included; other K, more
-    rows at a long K, and 8 bit do not."""
+    """4-bit group-64 codes: 1..8 activation rows with K of 2..16 steps of 1024 codes land on the diagonal-MFMA kernels
+    without forcing (beyond four steps: up to four rows a launch), rows beyond the last full 16 included; other K and
+    8 bit do not."""
     for K, N in ((4096, 16 * 9 + 5), (3072, 64), (2048, 33)):
         words, s, b = F.synthetic_affine(N, K, 4, 64, seed=810 + K // 1024)
         x = F.synthetic_x(8, K, seed=820 + K // 1024)
@@ -405,7 +409,16 @@ def test_qmvd_is_the_default_for_few_rows(ctx, orc):
             assert ctx.last_variant(0).startswith("qmvd_") and "_s32" in ctx.last_variant(0), ctx.last_variant(0)
             check_accumulators(acc, ref[:rows], "diag g32 K=%d rows=%d" % (K, rows))
         dw.free()
-    for K, bits, rows in ((17408, 4, 1), (1024, 4, 1), (4096, 8, 1), (8192, 4, 2), (2880, 4, 1)):
+    for K, rows in ((8192, 2), (14336, 4), (14336, 7), (16384, 8), (11008, 3)):
+        words, s, b = F.synthetic_affine(40, K, 4, 64, seed=880 + K // 1024)
+        x = F.synthetic_x(rows, K, seed=881 + K // 1024)
+        dw = DeviceAffine(ctx, words, s, b)
+        say("default rows at a long K", K, rows)
+        acc = run_qmv(ctx, x, dw, rows, K, 40, 64, 4, True)
+        assert ctx.last_variant(0).startswith("qmvd_b4_m4_"), ctx.last_variant(0)
+        check_accumulators(acc, F.reference_f64(x, words, s, b, 4, 64, K), "diag default K=%d rows=%d" % (K, rows))
+        dw.free()
+    for K, bits, rows in ((17408, 4, 1), (1024, 4, 1), (4096, 8, 1), (17408, 4, 2), (2880, 4, 1)):
         words, s, b = F.synthetic_affine(32, K, bits, 64, seed=830)
         x = F.synthetic_x(rows, K, seed=831)
         dw = DeviceAffine(ctx, words, s, b)

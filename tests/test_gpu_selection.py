@@ -28,8 +28,10 @@ CASES = [
     (8, 128, 1, 4096, ("qmv_b8_",)),
     (8, 64, 4, 4096, ("qmvt_b8_m16_",)),             # token tile, 8 bit: 2..16 rows, K a multiple of 256
     (8, 64, 4, 4096 + 64, ("qmvb_", "qmv_b8_")),     # ... block MFMA or dot2 for other K
-    (4, 64, 8, 14336, ("qmvt_b4_m16_",)),            # 5..8 rows at a K the diagonal kernels take for one row only
-    (4, 64, 8, 14336 + 128, ("qmvb_", "qmmf_", "qmmt_")),
+    (4, 64, 8, 14336, ("qmvd_b4_m4_",)),             # 5..8 rows at a K of more than four steps: two launches of four rows
+    (4, 64, 3, 14336 + 128, ("qmvd_b4_m4_",)),       # ... up to four rows in one (15 steps, the last one short)
+    (4, 64, 8, 16384 + 128, ("qmv_b4_",)),           # K beyond the diagonal kernels: the dot2 kernels, four rows a launch
+    (4, 64, 12, 16384 + 128, ("qmvb_", "qmmf_", "qmmt_")),
     (4, 128, 1, 4096, ("qmv_b4_",)),                 # dot2: groups of 128
     (4, 64, 1, 2880, ("qmv_b4_",)),                  # dot2: K = 45 groups
     (4, 64, 3, 2880, ("qmvb_", "qmv_b4_")),
