@@ -104,6 +104,7 @@ PROTOTYPES = {
     "aq_moe_combine": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _u]),
     "aq_qmv_greedy": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i]),
     "aq_probe_read": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i]),
+    "aq_qmv_greedy_selected": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i]),
     "aq_qmv_greedy_static": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i]),
     "aq_qmv_scores": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i]),
     "aq_packed_topk": (_i, [_vp, _vp, _c.c_int64, _i, _vp]),
@@ -376,6 +377,10 @@ class Context:
 
     def probe_read(self, w, s, b, K, N, mode=0):
         self._check(self.lib.aq_probe_read(self.handle, _ptr(w), _ptr(s), _ptr(b), K, N, mode))
+
+    def qmv_greedy_selected(self, x, w, s, b, rows, count, best, K, N, group_size=64, bits=4):
+        self._check(self.lib.aq_qmv_greedy_selected(self.handle, _ptr(x), _ptr(w), _ptr(s), _ptr(b), _ptr(rows), count,
+                                                    _ptr(best), K, N, group_size, bits))
 
     def qmv_greedy_static(self, x, w, s, b, best, K, N, group_size=64, bits=4, suppress=None, suppress_count=0):
         self._check(self.lib.aq_qmv_greedy_static(self.handle, _ptr(x), _ptr(w), _ptr(s), _ptr(b), _ptr(suppress),

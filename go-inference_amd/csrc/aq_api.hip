@@ -1432,6 +1432,55 @@ int aq_qmv_greedy(aq_ctx* ctx, const void* x, const void* packed, const void* sc
                      group_size, bits);
 }
 
+int aq_qmv_greedy_selected(aq_ctx* ctx, const void* x, const void* packed, const void* scales, const void* biases,
+                           const int32_t* rows, int count, uint64_t* best, int K, int N, int group_size, int bits) {
+    const char* op = "aq_qmv_greedy_selected";
+    if (!ctx) return fail(AQ_ERR_ARG, "%s: ctx is null", op);
+    if (K < 0 || N < 0 || count < 0) return fail(AQ_ERR_SHAPE, "%s: K, N, count must be non-negative", op);
+    if (!best) return fail(AQ_ERR_ARG, "%s: null output", op);
+    if (!aligned(best, 8)) return fail(AQ_ERR_ARG, "%s: output pointer is not 8-byte aligned", op);
+    if (count > 0 && !rows) return fail(AQ_ERR_ARG, "%s: count without a list of rows", op);
+    if (rows && !aligned(rows, 4)) return fail(AQ_ERR_ARG, "%s: operand pointer is not element-aligned", op);
+    if (count == 0 || N == 0) {  // nothing to choose from: "no result"
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        AQ_HIP(aq::fill_zero_launch(best, 8, ctx->stream), "hipLaunchKernel");
+        return AQ_OK;
+    }
+    if (K == 0) return fail(AQ_ERR_SHAPE, "%s: K must be positive when there are rows to score", op);
+    if (int rc = check_geometry(op, K, group_size, bits)) return rc;
+    if (!x || !packed || !scales || !biases) return fail(AQ_ERR_ARG, "%s: null operand", op);
+    if (!aligned(x, 2) || !aligned(packed, 4) || !aligned(scales, 2) || !aligned(biases, 2))
+        return fail(AQ_ERR_ARG, "%s: operand pointer is not element-aligned", op);
+    if (count > 65535) return fail(AQ_ERR_UNSUPPORTED, "%s: at most 65535 candidates per call", op);
+    const int width = N < 16 ? N : 16;
+    const size_t start_bytes = align256((size_t)count * 4), need = start_bytes + (size_t)count * width * 4;
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    if (int rc = aq::workspace_reserve(ctx->stream, &ctx->ws, need, fail)) return rc;
+    int32_t* start = static_cast<int32_t*>(ctx->ws.ptr);
+    float* scores = reinterpret_cast<float*>(static_cast<char*>(ctx->ws.ptr) + start_bytes);
+    AQ_HIP(aq::selected_windows_launch(rows, count, N, width, start, ctx->stream), "hipLaunchKernel");
+    aq::QmvArgs a{};
+    a.x = static_cast<const uint16_t*>(x);
+    a.w = static_cast<const uint32_t*>(packed);
+    a.s = static_cast<const uint16_t*>(scales);
+    a.b = static_cast<const uint16_t*>(biases);
+    a.y = scores;
+    a.rhs = start;  // the "expert" of candidate z is the row its window starts at: a slab of experts one row apart
+    a.K = K;
+    a.N = width;
+    a.M = 1;
+    a.out_f32 = 1;
+    a.num_experts = N - width + 1;
+    a.expert_rows = 1;
+    a.x_rows = 1;
+    a.routes = count;
+    if (int rc = launch_qmv_rows(ctx, a, group_size, bits, true)) return rc;
+    AQ_HIP(aq::selected_pick_launch(scores, rows, start, count, width, reinterpret_cast<unsigned long long*>(best), ctx->stream),
+           "hipLaunchKernel");
+    return AQ_OK;
+}
+
 int aq_qmv_greedy_static(aq_ctx* ctx, const void* x, const void* packed, const void* scales, const void* biases,
                          const int32_t* suppress, int suppress_count, uint64_t* best, int K, int N, int group_size, int bits) {
     return head_call(ctx, "aq_qmv_greedy_static", 3, x, packed, scales, biases, suppress, suppress_count, best, 1, K, N,

@@ -173,6 +173,11 @@ bool qmv_head_supported(int bits, int fuse, int rows);
 // Slots a.partial must hold for the argmax of N rows at `rows` rows per wavefront.
 size_t qmv_head_partials(int N, int rows);
 hipError_t qmv_head_launch(int bits, int fuse, int rows, const QmvArgs& a, hipStream_t stream);
+// Greedy over a candidate list (aq_qmv_head.hip): the window of `width` rows each candidate is scored in (-1: id out of
+// range), and the maximum of pack(score, row) over the candidates' own rows of the gathered scores [count, width].
+hipError_t selected_windows_launch(const int32_t* rows, int count, int N, int width, int32_t* start, hipStream_t stream);
+hipError_t selected_pick_launch(const float* scores, const int32_t* rows, const int32_t* start, int count, int width,
+                                unsigned long long* best, hipStream_t stream);
 // The same two epilogues over fp32 scores that are already in memory: scores [M, N] -> best[M] / packed[M, N].
 hipError_t pack_scores_launch(const float* scores, int M, int N, const int32_t* suppress, int suppress_count,
                               unsigned long long* best_or_null, unsigned long long* packed_or_null, hipStream_t stream);

@@ -112,6 +112,57 @@ hipError_t qmv_head_launch(int bits, int fuse, int rows, const QmvArgs& a, hipSt
     return hipGetLastError();
 }
 
+// Greedy over a list of candidate rows (rocm_mlx_q4_projection_selected_greedy,
+// go/engine/hip/kernels/quant/affine_projection_fused.hipinc:485-546).  The scores come from the gathered matvec: every
+// candidate r is scored as one row of the window of `width` rows that starts at min(r, N - width) (an "expert" of a
+// slab whose experts are one row apart), so a candidate costs width rows of weights and no kernel of its own is needed.
+// windows: start[z] = first row of candidate z's window, -1 for an id outside [0, N).
+__global__ __launch_bounds__(256) void selected_windows_kernel(const int32_t* __restrict__ rows, int count, int N, int width,
+                                                               int32_t* __restrict__ start) {
+    const int z = blockIdx.x * 256 + threadIdx.x;
+    if (z >= count) return;
+    const int r = rows[z];
+    start[z] = (r >= 0 && r < N) ? min(r, N - width) : -1;
+}
+// pick: best[0] = max over the valid candidates with a finite score of pack(score, row); 0 when there is none.
+__global__ __launch_bounds__(256) void selected_pick_kernel(const float* __restrict__ scores, const int32_t* __restrict__ rows,
+                                                            const int32_t* __restrict__ start, int count, int width,
+                                                            unsigned long long* __restrict__ best) {
+    unsigned long long mine = 0;
+    for (int z = threadIdx.x; z < count; z += 256) {
+        const int e = start[z];
+        if (e < 0) continue;
+        const int r = rows[z];
+        const float v = scores[(int64_t)z * width + (r - e)];
+        if (isfinite(v)) {
+            const unsigned long long p = pack_score_index(v, (uint32_t)r);
+            mine = p > mine ? p : mine;
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const unsigned long long other = __shfl_xor(mine, o, kWave);
+        mine = other > mine ? other : mine;
+    }
+    __shared__ unsigned long long wave_best[4];
+    if ((threadIdx.x & (kWave - 1)) == 0) wave_best[threadIdx.x >> 6] = mine;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned long long b = wave_best[0];
+        for (int i = 1; i < 4; i++) b = wave_best[i] > b ? wave_best[i] : b;
+        best[0] = b;
+    }
+}
+hipError_t selected_windows_launch(const int32_t* rows, int count, int N, int width, int32_t* start, hipStream_t stream) {
+    hipLaunchKernelGGL(selected_windows_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, rows, count, N, width, start);
+    return hipGetLastError();
+}
+hipError_t selected_pick_launch(const float* scores, const int32_t* rows, const int32_t* start, int count, int width,
+                                unsigned long long* best, hipStream_t stream) {
+    hipLaunchKernelGGL(selected_pick_kernel, dim3(1), dim3(256), 0, stream, scores, rows, start, count, width, best);
+    return hipGetLastError();
+}
+
 hipError_t head_fold_launch(const unsigned long long* partial, int count, unsigned long long* fold, unsigned long long* best,
                             hipStream_t stream) {
     hipLaunchKernelGGL(fold_best_kernel, dim3(kHeadFoldGroups), dim3(256), 0, stream, partial, count, fold, best);

@@ -269,6 +269,17 @@ int aq_qmv_greedy(aq_ctx *ctx, const void *x, const void *packed, const void *sc
                   const int32_t *suppress, int suppress_count, uint64_t *best, int M, int K, int N, int group_size,
                   int bits);
 
+/* Greedy over a list of candidate rows (speculative or constrained decoding): best[0] = max over the candidates r of
+ * pack(x . dequant(w)[r,:], r), rows being a device int32[count] read on the device.  Ids outside [0, N) are skipped,
+ * duplicates are harmless, non-finite scores never win, best[0] == 0 means no candidate qualified; ties go to the lowest
+ * row id (the packing's order).  Replaces rocm_mlx_q4_projection_selected_greedy
+ * (go/engine/hip/kernels/quant/affine_projection_fused.hipinc:485-546; like it, this form has no suppress list: the
+ * list IS the selection).  One activation row.  A candidate is scored by the gathered matvec as one row of a window of
+ * 16 weight rows, so it costs 16 rows of weights; scratch comes from the context's workspace (count * 68 bytes; grows
+ * on demand, not during capture).  count <= 65535. */
+int aq_qmv_greedy_selected(aq_ctx *ctx, const void *x, const void *packed, const void *scales, const void *biases,
+                           const int32_t *rows, int count, uint64_t *best, int K, int N, int group_size, int bits);
+
 /* aq_qmv_greedy for one activation row with NO allocation of any kind (no hipMalloc / hipFree, no workspace
  * growth): it has no counterpart in the reference and exists for callers that cannot allocate - code under
  * HIP graph capture, tight serving loops, harnesses that forbid it.  The partial maxima and the fold tickets

@@ -374,3 +374,74 @@ def test_graph_is_refused_once_the_workspace_has_moved(orc):
         dw.free()
     finally:
         c.close()
+
+
+@pytest.mark.parametrize("bits,gs,K,N,exact", [(4, 64, 2048, 1000, True), (4, 64, 4096, 5000, True), (4, 64, 14336, 300, False),
+                                               (4, 32, 1536, 4099, False), (8, 64, 512, 50, False), (4, 64, 256, 10, False),
+                                               (6, 32, 192, 301, False)])
+def test_greedy_over_a_candidate_list(ctx, orc, bits, gs, K, N, exact):
+    """aq_qmv_greedy_selected (rocm_mlx_q4_projection_selected_greedy, affine_projection_fused.hipinc:485-546): the winner
+    is the oracle's greedy token over the logits with every row outside the list suppressed; ids out of range are
+    skipped, duplicates are harmless, equal scores go to the lowest id, an empty or all-invalid list gives 0.  exact:
+    shapes whose gathered and dense kernels compute the same bytes (the device's own logits decide); elsewhere the
+    float64 reference decides, within the matvec tolerance."""
+    say("selected greedy", bits, gs, K, N)
+    rng = np.random.default_rng(K + N)
+    if 32 % bits == 0:
+        words, s, b = F.synthetic_affine(N, K, bits, gs, seed=F.BASE_SEED + 140)
+    else:
+        words = F.pack_codes(rng.integers(0, 1 << bits, size=(N, K)), bits)
+        s = F.f32_to_bf16_bits((np.abs(rng.normal(0, 0.02, (N, K // gs))) + 1e-3).astype(np.float32))
+        b = F.f32_to_bf16_bits(rng.normal(0, 0.05, (N, K // gs)).astype(np.float32))
+    # rows 3 and 7 equal row 5: equal scores, the lowest id among the listed ones must win when they lead
+    for dup in (3, 7):
+        if N > 8:
+            words[dup], s[dup], b[dup] = words[5], s[5], b[5]
+    x = F.synthetic_x(1, K, seed=F.BASE_SEED + 141)
+    dw = DeviceAffine(ctx, words, s, b)
+    ref = F.reference_f64(x, words, s, b, bits, gs, K)[0]
+    logits = run_qmv(ctx, x, dw, 1, K, N, gs, bits, True)[0]
+    dx = ctx.to_device(np.ascontiguousarray(x, np.uint16))
+    best = ctx.to_device(np.full(1, 0xDEADBEEF, np.uint64))
+    top = int(np.argmax(ref))
+    lists = [rng.integers(0, N, size=n).tolist() for n in (1, 7, 40, min(N, 600))]
+    lists.append([top, -1, N, N + 5, top, 2 ** 31 - 1])               # ids out of range around the best row
+    if N > 8:
+        lists.append([7, 5, 3, 7])                                     # three equal rows: id 3 wins
+        lists.append(sorted(set(range(N)) - {top})[:2000])             # everything but the best row
+    lists.append([-5, N, N + 1])                                       # nothing valid
+    for cand in lists:
+        dc = ctx.to_device(np.asarray(cand, np.int32))
+        ctx.qmv_greedy_selected(dx, dw.w, dw.s, dw.b, dc, len(cand), best, K, N, gs, bits)
+        ctx.sync()
+        got = int(_u64(best, 1)[0])
+        valid = sorted({c for c in cand if 0 <= c < N})
+        if not valid:
+            assert got == 0
+            continue
+        tok, score = _unpack(got)
+        assert tok in valid
+        others = np.array(sorted(set(range(N)) - set(valid)), np.int32)
+        if exact:
+            want, want_score = orc.greedy_sample_suppress(logits, others)
+            assert (tok, score) == (want, want_score), (cand[:8], tok, want)
+        else:
+            assert abs(score - ref[tok]) <= MAX_ABS + 2e-3 * abs(ref[tok])
+            assert ref[tok] >= max(ref[v] for v in valid) - 2 * (MAX_ABS + 2e-3 * abs(ref[tok]))
+        if cand == [7, 5, 3, 7]:
+            assert tok == 3
+        dc.free()
+    # an empty list and an empty vocabulary: "no result"
+    ctx.qmv_greedy_selected(dx, dw.w, dw.s, dw.b, None, 0, best, K, N, gs, bits)
+    ctx.sync()
+    assert int(_u64(best, 1)[0]) == 0
+    import aq_mi355
+    with pytest.raises(aq_mi355.AqError) as e:
+        ctx.qmv_greedy_selected(dx, dw.w, dw.s, dw.b, None, 3, best, K, N, gs, bits)
+    assert e.value.code == aq_mi355.AQ_ERR_ARG
+    with pytest.raises(aq_mi355.AqError) as e:
+        ctx.qmv_greedy_selected(dx, dw.w, dw.s, dw.b, best, 70000, best, K, N, gs, bits)
+    assert e.value.code == aq_mi355.AQ_ERR_UNSUPPORTED
+    for t in (dx, best):
+        t.free()
+    dw.free()
