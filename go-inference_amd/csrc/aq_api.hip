@@ -1014,6 +1014,17 @@ int aq_qmv_gate_up(aq_ctx* ctx, const void* x, const void* gate_packed, const vo
     float* g = reinterpret_cast<float*>(static_cast<char*>(ctx->ws.ptr) + region);
     float* u = reinterpret_cast<float*>(static_cast<char*>(ctx->ws.ptr) + region + each);
     if (int rc = aq_qmv(ctx, x, gate_packed, gate_scales, gate_biases, g, M, K, N, group_size, bits, AQ_OUT_F32)) return rc;
+    if (M > 32 && ctx->forced[0] < 0 && !(ctx->families_off >> kFamTiles & 1) &&
+        aq::qmm_takes_gate(x, up_packed, K, group_size, bits)) {
+        // prefill sizes: the `up` projection runs on the matmul tiles anyway, and their stores apply act(gate) * up on
+        // the way out (rocm_mlx_q4_gelu_tanh_multiply_batch, go/engine/hip/kernels/quant/affine_gelu_tanh.hipinc:921-1109):
+        // one [M, N] fp32 matrix is written and read instead of two written and two read.  Same bytes as the route below.
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        const int rc = aq::qmm_dispatch(ctx->stream, &ctx->ws, ctx->cu_count, ctx->forced[1], &ctx->last_variant[1], x, up_packed,
+                                        up_scales, up_biases, y, M, K, N, group_size, bits, out_f32, fail, g, act);
+        if (rc == AQ_OK) ctx->last_variant[0] = "qmv_gate_up_tiles";
+        return rc;
+    }
     if (int rc = aq_qmv(ctx, x, up_packed, up_scales, up_biases, u, M, K, N, group_size, bits, AQ_OUT_F32)) return rc;
     std::lock_guard<std::mutex> lk(ctx->mu);
     AQ_HIP(aq::act_mul_f32_launch(g, u, y, (int64_t)M * N, act, out_f32 ? 1 : 0, ctx->stream), "hipLaunchKernel");

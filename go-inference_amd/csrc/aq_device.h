@@ -104,6 +104,29 @@ __device__ __forceinline__ float fmul_unfused(float a, float b) {
     return a * b;
 }
 
+// Eight consecutive outputs of the `up` projection (columns n .. n + 7 of a row of N, element offset o) times the
+// activation of the `gate` projection's fp32 sums at the same places: the element-wise step of a gated MLP as the
+// epilogue of the second projection.  The same two operations, in the same order, as the stand-alone kernel over two
+// fp32 matrices (act_mul_f32_launch), so the fused and the unfused route store the same bytes.
+__device__ __forceinline__ void gate_mul8(const float* gate, int act, int64_t o, int n, int N, float4& lo, float4& hi) {
+    float g[8];
+    if ((reinterpret_cast<uintptr_t>(gate) & 15) == 0 && (N & 3) == 0 && n + 8 <= N) {
+        const float4 a = *reinterpret_cast<const float4*>(gate + o), b = *reinterpret_cast<const float4*>(gate + o + 4);
+        g[0] = a.x, g[1] = a.y, g[2] = a.z, g[3] = a.w, g[4] = b.x, g[5] = b.y, g[6] = b.z, g[7] = b.w;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++) g[e] = n + e < N ? gate[o + e] : 0.0f;
+    }
+    lo.x = fmul_unfused(act_value(act, g[0]), lo.x);
+    lo.y = fmul_unfused(act_value(act, g[1]), lo.y);
+    lo.z = fmul_unfused(act_value(act, g[2]), lo.z);
+    lo.w = fmul_unfused(act_value(act, g[3]), lo.w);
+    hi.x = fmul_unfused(act_value(act, g[4]), hi.x);
+    hi.y = fmul_unfused(act_value(act, g[5]), hi.y);
+    hi.z = fmul_unfused(act_value(act, g[6]), hi.z);
+    hi.w = fmul_unfused(act_value(act, g[7]), hi.w);
+}
+
 // bf16(act(gate) * up): fp32 inside, one rounding at the end, as lthn_gelu_gate_mul_one
 // (go/engine/metal/kernels/moe/lthn_gelu_qmv_impl.h:24-33).
 __device__ __forceinline__ uint32_t act_mul_bf16x2(uint32_t g, uint32_t u, int act) {

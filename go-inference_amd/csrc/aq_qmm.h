@@ -17,6 +17,8 @@ struct QmmArgs {
     int M, K, N;
     int gs_blocks;  // 64-code blocks per quantisation group (1 for group 64, 2 for 128)
     int out_f32;
+    const float* gate;  // not null: y = act(gate[m, n]) * (x . w^T)[m, n], gate being fp32 [M, N] (a gated MLP's other projection)
+    int act;            // kActGeluTanh or kActSilu
 };
 
 struct QmmVariant {
@@ -43,6 +45,8 @@ struct QmmTileArgs {
     int ksplit;            // workgroups that share a tile along K (1: none)
     int gsplit;            // 64-code blocks of K per workgroup (a multiple of 4)
     float* partial;        // ksplit > 1: fp32 partial tiles [ksplit][M][N]
+    const float* gate;     // as in QmmArgs (applied where the final value is stored)
+    int act;
 };
 
 // (the variants of the fp16-operand kernels, aq_qmm_half.hip, are listed behind those of the tile kernels)
@@ -98,8 +102,11 @@ int qmm_reserve(hipStream_t stream, Workspace* ws, int M, int K, FailFn fail);
 // Validated-shape dispatch used by aq_qmm and by aq_qmv for calls the matvec families pass on.
 // Returns an AQ_* / hipError_t code through `fail`.
 // `forced` indexes the tile variants (qmmt_variant), or is negative.
+// gate (fp32 [M, N], or null) and act: the gated-MLP epilogue, see QmmArgs; only where qmm_takes_gate says so.
 int qmm_dispatch(hipStream_t stream, Workspace* ws, int cu_count, int forced, const char** last_variant, const void* x,
                  const void* packed, const void* scales, const void* biases, void* y, int M, int K, int N,
-                 int group_size, int bits, bool out_f32, FailFn fail);
+                 int group_size, int bits, bool out_f32, FailFn fail, const float* gate = nullptr, int act = 0);
+// Whether qmm_dispatch runs this call on the tile kernels, whose stores can carry the gated-MLP epilogue.
+bool qmm_takes_gate(const void* x, const void* packed, int K, int group_size, int bits);
 
 }  // namespace aq

@@ -68,7 +68,13 @@ int workspace_reserve(hipStream_t stream, Workspace* ws, size_t need, FailFn fai
 
 size_t qmm_scratch_bytes(int M, int K, int N) {
     const size_t xbytes = (qmmt_workspace_bytes(M, K) + 255) & ~(size_t)255;
-    const size_t partial = (M > 4 && M <= 64) ? qmmt_splitk_bytes(M, N, 16) : 0;
+    size_t partial = (M > 4 && M <= 64) ? qmmt_splitk_bytes(M, N, 16) : 0;
+    if (M > 64 && (K / 64) % 8 == 0 && K >= 2048) {
+        // 128 x 128 tiles that leave CUs idle share K out over up to 8 workgroups, at most two workgroups a CU in all
+        // (qmm_dispatch): k partial tiles of M x N with (M / 128) (N / 128) k <= 2 CUs, bounded here for up to 512 CUs
+        const size_t by_k = qmmt_splitk_bytes(M, N, 8), by_cus = (size_t)2 * 512 * 128 * 128 * 4 + ((size_t)M + N) * 128 * 8 * 4;
+        partial = by_k < by_cus ? by_k : by_cus;
+    }
     return xbytes + ((partial + 255) & ~(size_t)255);
 }
 
@@ -90,12 +96,17 @@ static int find_qmmt_named(const char* name) {
     return -1;
 }
 
+bool qmm_takes_gate(const void* x, const void* packed, int K, int group_size, int bits) {
+    return (bits == 4 || bits == 8) && (group_size == 64 || group_size == 128) && K % 64 == 0 &&
+           (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(packed) & 15) == 0;
+}
+
 int qmm_dispatch(hipStream_t stream, Workspace* ws, int cu_count, int forced, const char** last_variant, const void* x,
                  const void* packed, const void* scales, const void* biases, void* y, int M, int K, int N,
-                 int group_size, int bits, bool out_f32, FailFn fail) {
-    const bool mfma_ok = (bits == 4 || bits == 8) && (group_size == 64 || group_size == 128) && K % 64 == 0 &&
-                         (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(packed) & 15) == 0;
+                 int group_size, int bits, bool out_f32, FailFn fail, const float* gate, int act) {
+    const bool mfma_ok = qmm_takes_gate(x, packed, K, group_size, bits);
     if (!mfma_ok) {
+        if (gate) return fail(AQ_ERR_UNSUPPORTED, "aq_qmm: the gated epilogue needs the tile kernels (4 / 8 bit, groups of 64 / 128)");
         // any other geometry: the any-width matvec kernel walks the rows of x
         QmvArgs q{};
         q.x = static_cast<const uint16_t*>(x);
@@ -124,6 +135,8 @@ int qmm_dispatch(hipStream_t stream, Workspace* ws, int cu_count, int forced, co
     a.N = N;
     a.gs_blocks = group_size / 64;
     a.out_f32 = out_f32 ? 1 : 0;
+    a.gate = gate;
+    a.act = act;
     const int idx = forced;
     int tile_idx = -1;
     if (idx >= 0) {

@@ -334,10 +334,11 @@ __global__ __launch_bounds__(WN* kWave, 1) void qmm_few_kernel(const QmmTileArgs
         for (int p = 0; p < 32 / RPP; p++) {
             const int row = p * RPP + row_in;
             const int m = mtop + row;
-            const float4 lo = *reinterpret_cast<const float4*>(stage + row * CW + c8);
-            const float4 hi = *reinterpret_cast<const float4*>(stage + row * CW + c8 + 4);
+            float4 lo = *reinterpret_cast<const float4*>(stage + row * CW + c8);
+            float4 hi = *reinterpret_cast<const float4*>(stage + row * CW + c8 + 4);
             if (m >= M || n >= N) continue;
             const int64_t o = (int64_t)m * N + n;
+            if (a.gate && !a.partial) gate_mul8(a.gate, a.act, o, n, N, lo, hi);
             if (wide && n + 8 <= N) {
                 if (y_f32) {
                     float4* dst = reinterpret_cast<float4*>(reinterpret_cast<float*>(ybase) + o);

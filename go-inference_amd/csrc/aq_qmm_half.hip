@@ -553,10 +553,11 @@ __global__ __launch_bounds__(WM* WN* kWave, OCC) void qmmh_kernel(const QmmTileA
         for (int p = 0; p < 32 / RPP; p++) {
             const int row = p * RPP + row_in;
             const int m = mtop + row;
-            const float4 lo = *reinterpret_cast<const float4*>(stage + row * CW + c8);
-            const float4 hi = *reinterpret_cast<const float4*>(stage + row * CW + c8 + 4);
+            float4 lo = *reinterpret_cast<const float4*>(stage + row * CW + c8);
+            float4 hi = *reinterpret_cast<const float4*>(stage + row * CW + c8 + 4);
             if (m >= M || n >= N) continue;
             const int64_t o = (int64_t)m * N + n;
+            if (a.gate && !a.partial) gate_mul8(a.gate, a.act, o, n, N, lo, hi);
             if (wide && n + 8 <= N) {
                 if (a.out_f32) {
                     float4* dst = reinterpret_cast<float4*>(reinterpret_cast<float*>(a.y) + o);
@@ -641,6 +642,8 @@ hipError_t qmmh_launch(int idx, const QmmArgs& q, void* workspace, hipStream_t s
     a.N = q.N;
     a.gs_blocks = q.gs_blocks;
     a.out_f32 = q.out_f32;
+    a.gate = q.gate;
+    a.act = q.act;
     a.mblks = mblks;
     const int bm = e.v.wm * e.v.mb * 32, bn = e.v.wn * e.v.nb * 32;
     a.tiles_m = (q.M + bm - 1) / bm;

@@ -436,10 +436,11 @@ __global__ __launch_bounds__(WM* WN* kWave, 2) void qmm_tile_kernel(const QmmTil
         for (int p = 0; p < 32 / RPP; p++) {
             const int row = p * RPP + row_in;
             const int m = mtop + row;
-            const float4 lo = *reinterpret_cast<const float4*>(stage + row * CW + c8);
-            const float4 hi = *reinterpret_cast<const float4*>(stage + row * CW + c8 + 4);
+            float4 lo = *reinterpret_cast<const float4*>(stage + row * CW + c8);
+            float4 hi = *reinterpret_cast<const float4*>(stage + row * CW + c8 + 4);
             if (m >= M || n >= N) continue;
             const int64_t o = (int64_t)m * N + n;
+            if (a.gate && !a.partial) gate_mul8(a.gate, a.act, o, n, N, lo, hi);
             if (wide && n + 8 <= N) {
                 if (y_f32) {
                     float4* dst = reinterpret_cast<float4*>(reinterpret_cast<float*>(ybase) + o);
@@ -509,10 +510,12 @@ size_t qmmt_workspace_bytes(int M, int K) {
 
 // Adds the ksplit partial tiles [ksplit][M*N] in split order and stores bf16 or fp32.
 __global__ __launch_bounds__(256) void qmm_splitk_reduce_kernel(const float* __restrict__ partial, int ksplit, int64_t mn,
-                                                                 void* __restrict__ y, int out_f32) {
+                                                                 void* __restrict__ y, int out_f32, const float* __restrict__ gate,
+                                                                 int act) {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < mn; i += (int64_t)gridDim.x * 256) {
         float acc = partial[i];
         for (int s = 1; s < ksplit; s++) acc += partial[(int64_t)s * mn + i];
+        if (gate) acc = fmul_unfused(act_value(act, gate[i]), acc);  // the gated-MLP epilogue (QmmArgs::gate)
         if (out_f32) {
             static_cast<float*>(y)[i] = acc;
         } else {
@@ -562,6 +565,8 @@ hipError_t qmmt_launch_splitk(int idx, const QmmArgs& q, void* workspace, int ks
     a.N = q.N;
     a.gs_blocks = q.gs_blocks;
     a.out_f32 = q.out_f32;
+    a.gate = q.gate;
+    a.act = q.act;
     a.mblks = mblks;
     const int bm = v.wm * v.mb * 32, bn = v.wn * v.nb * 32;
     a.tiles_m = (q.M + bm - 1) / bm;
@@ -588,7 +593,7 @@ hipError_t qmmt_launch_splitk(int idx, const QmmArgs& q, void* workspace, int ks
     int64_t blocks = (mn + 255) / 256;
     if (blocks > 4096) blocks = 4096;
     hipLaunchKernelGGL(qmm_splitk_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, a.partial, ksplit, mn, q.y,
-                       q.out_f32);
+                       q.out_f32, q.gate, q.act);
     return hipGetLastError();
 }
 

@@ -169,6 +169,30 @@ def test_gate_up_unfused_shapes(ctx, orc, bits, gs, M, K, N):
     du.free()
 
 
+@pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("bits,gs,M,K,N", [(4, 64, 256, 4096, 520), (4, 64, 2048, 2048, 1024), (8, 64, 100, 1024, 203),
+                                           (4, 64, 40, 1024, 300), (4, 128, 64, 512, 96), (4, 64, 33, 320, 77)])
+def test_gate_up_prefill_rows(ctx, orc, act, bits, gs, M, K, N):
+    """More than 32 rows (rocm_mlx_q4_gelu_tanh_multiply_batch, affine_gelu_tanh.hipinc:921-1109): the `up` projection
+    runs on the matmul tiles and their stores apply act(gate) * up, over every tile family (fp16-operand tiles, bf16-code
+    tiles, few-rows kernels with their K-split sum) and ragged N.  Checked against the device's own two projections."""
+    say("gate_up prefill", act, bits, gs, M, K, N)
+    gw, gsb, gb = F.synthetic_affine(N, K, bits, gs, seed=F.BASE_SEED + 170)
+    uw, usb, ub = F.synthetic_affine(N, K, bits, gs, seed=F.BASE_SEED + 171)
+    x = F.synthetic_x(M, K, seed=F.BASE_SEED + 172)
+    dg, du = DeviceAffine(ctx, gw, gsb, gb), DeviceAffine(ctx, uw, usb, ub)
+    got = _run_gate_up(ctx, x, dg, du, M, K, N, gs, bits, act)
+    assert ctx.last_variant(0) == "qmv_gate_up_tiles"
+    g_gpu = run_qmv(ctx, x, dg, M, K, N, gs, bits, True)
+    u_gpu = run_qmv(ctx, x, du, M, K, N, gs, bits, True)
+    _check_fused(got, g_gpu, u_gpu, F.reference_f64(x, gw, gsb, gb, bits, gs, K), F.reference_f64(x, uw, usb, ub, bits, gs, K),
+                 act, orc, "gate_up prefill")
+    out = _run_gate_up(ctx, x, dg, du, M, K, N, gs, bits, act, f32=False)
+    assert np.array_equal(out, F.f32_to_bf16_bits(got).reshape(M, N))
+    dg.free()
+    du.free()
+
+
 def _gather_inputs(ctx, E, expert_rows, K, bits, gs, x_rows, lhs, rhs, seed):
     words, s, b = F.synthetic_affine(E * expert_rows, K, bits, gs, seed=seed)
     x = F.synthetic_x(x_rows, K, seed=seed + 1)
