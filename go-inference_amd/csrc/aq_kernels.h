@@ -11,25 +11,27 @@ namespace aq {
 // MLX group-affine format (go/model/quant/mlxaffine/mlxaffine.go:14-20):
 //   w [rows, K*bits/32] u32, s/b [rows, K/group] bf16, x [x_rows, K] bf16.
 struct QmvArgs {
+    // (What a kernel needs before it can request its weights sits in the first 64 bytes of the kernel arguments: one
+    // scalar load and one wait at the start of a wavefront instead of one per cache line.)
     const uint16_t* x;
     const uint32_t* w;
-    const uint16_t* s;
-    const uint16_t* b;
-    void* y;             // [M, N] (plain) or [routes, N] (gather); bf16 or f32
-    const int32_t* lhs;  // gather only: route -> x row, nullptr = row 0 for all
-    const int32_t* rhs;  // gather only: route -> expert id
+    void* y;          // [M, N] (plain) or [routes, N] (gather); bf16 or f32
     int K;
     int N;
     int M;            // activation rows (plain); 1 for gather
+    int early_wgs;    // diagonal-MFMA kernels: workgroups (by index) that request their weights before they stage x
+    const uint16_t* s;
+    const uint16_t* b;
     int gs_shift;     // log2(group size)
     int out_f32;      // 0: bf16 stores, 1: f32 stores
+    const int32_t* lhs;  // gather only: route -> x row, nullptr = row 0 for all
+    const int32_t* rhs;  // gather only: route -> expert id
     int num_experts;  // gather only
     int expert_rows;  // gather only: rows per expert in the slab
     int row_base;     // gather only: first row of the slab used
     int x_rows;       // gather only: rows in x (bounds for lhs)
     int routes;       // gather only
     int stream_w;     // diagonal-MFMA kernels: load the weights with the non-temporal hint (set by the launch functions)
-    int early_wgs;    // diagonal-MFMA kernels: workgroups (by index) that request their weights before they stage x
     int tiled;        // diagonal-MFMA kernels, dense: w (and w2) hold the tile-major layout of aq_tile.h; s, b are not read
     // activation-fused kernels only (aq_qmv_act.hip)
     const uint16_t* x2;  // x-load fusion: the `up` activations, same shape and row indexing as x (the `gate` ones)

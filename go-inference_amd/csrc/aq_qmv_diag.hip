@@ -348,7 +348,11 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     // workgroups request first and stage while the memory system is starting up.
     // (Several activation rows are staged by the workgroup together, behind a barrier: always first; measured at eight
     // rows of 4096 x 14336: 13.4 -> 11.1 us.)
-    const bool late = !wstage || (int)(blockIdx.x + blockIdx.y * gridDim.x) >= a.early_wgs;
+    // (a.early_wgs is read with the first kernel arguments, whether or not it is used: a scalar load behind a branch
+    // would be a second wait in front of the first request.  Only the gathered grids have a second dimension.)
+    const int early_wgs = a.early_wgs;
+    const int linear_block = GATHER ? (int)(blockIdx.x + blockIdx.y * gridDim.x) : (int)blockIdx.x;
+    const bool late = linear_block >= early_wgs || !wstage;
     if (late) stage_x();
     // AHEAD chunks are requested before the arithmetic starts; chunk cc + AHEAD when chunk cc is about to be worked on
     constexpr int AHEAD = SUP == 1 && AQ_DIAG_AHEAD < CPS ? AQ_DIAG_AHEAD : CPS;
