@@ -92,6 +92,7 @@ PROTOTYPES = {
     "aq_qmv_multi": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _u]),
     "aq_reserve_workspace": (_i, [_vp, _i, _i]),
     "aq_reserve_workspace_bytes": (_i, [_vp, _sz]),
+    "aq_workspace_bytes": (_sz, [_vp]),
     "aq_gather_qmv": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _u]),
     "aq_qmv_gate_up": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _u]),
     "aq_gather_qmv_gate_up": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i,
@@ -330,6 +331,9 @@ class Context:
 
     def reserve_workspace_bytes(self, nbytes):
         self._check(self.lib.aq_reserve_workspace_bytes(self.handle, nbytes))
+
+    def workspace_bytes(self):
+        return int(self.lib.aq_workspace_bytes(self.handle))
 
     def gather_qmv(self, x, w, s, b, lhs, rhs, y, routes, x_rows, K, N, num_experts, expert_rows, row_base=0,
                    group_size=64, bits=4, flags=0):

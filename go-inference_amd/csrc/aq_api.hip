@@ -147,8 +147,10 @@ enum { kFamTiles = kFamCount, kFamTilesLarge, kFamGeneric };
 
 // Route switches, the counterpart of the reference's GO_ROCM_DISABLE_* variables (hip_projection_launch.go:95-137):
 // AQ_MI355_DISABLE=name[,name...] over dot2, blk, diag, tok, tiles, read when a context is created, takes those
-// families out of the selection of every entry point, which then falls through to the next family that takes the
-// shape (the any-width kernel cannot be switched off).  There is no code-object override like
+// families out of the selection of aq_qmv, aq_gather_qmv and the calls built on them, which then fall through to the
+// next family that takes the shape (the any-width kernel cannot be switched off).  The fused head, gate|up and
+// multi-matrix calls honour `diag` only: with it off they run their dot2 kernels, which have no switch, because the
+// unfused route behind them is the selection above.  There is no code-object override like
 // GO_ROCM_KERNEL_HSACO (hip_kernel_module.go:14-35): the kernels are linked into this library.
 unsigned families_off_from_env(const char* value) {
     static const struct { const char* name; unsigned bits; } kNames[] = {
@@ -831,6 +833,12 @@ int aq_reserve_workspace_bytes(aq_ctx* ctx, size_t bytes) {
     return aq::workspace_reserve(ctx->stream, &ctx->ws, bytes, fail);
 }
 
+size_t aq_workspace_bytes(aq_ctx* ctx) {
+    if (!ctx) return 0;
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    return ctx->ws.bytes + ctx->head_ws.bytes;
+}
+
 int aq_gather_qmv(aq_ctx* ctx, const void* x, const void* packed, const void* scales, const void* biases,
                   const int32_t* lhs, const int32_t* rhs, void* y, int routes, int x_rows, int K, int N,
                   int num_experts, int expert_rows, int row_base, int group_size, int bits, unsigned flags) {
@@ -1322,7 +1330,9 @@ int head_call(aq_ctx* ctx, const char* op, int fuse, const void* x, const void* 
     if (!aligned(out, 8)) return fail(AQ_ERR_ARG, "%s: output pointer is not 8-byte aligned", op);
     if (suppress_count > 0 && !suppress) return fail(AQ_ERR_ARG, "%s: suppress_count without a suppress list", op);
     if (suppress && !aligned(suppress, 4)) return fail(AQ_ERR_ARG, "%s: operand pointer is not element-aligned", op);
-    const bool fused = M == 1 && N > 0 && K > 0 && ctx->forced[0] < 0 && (bits == 4 || bits == 8) && x && packed &&
+    // (a forced matvec variant sends the other head calls through aq_qmv and scratch memory; the entry point that
+    // allocates nothing has no such route and keeps to the fused kernels)
+    const bool fused = M == 1 && N > 0 && K > 0 && (ctx->forced[0] < 0 || no_alloc) && (bits == 4 || bits == 8) && x && packed &&
                        dot2_eligible(K, group_size, bits, x, packed, (size_t)K * 2);
     if (no_alloc && !fused && M > 0 && N > 0 && K > 0)
         return fail(AQ_ERR_UNSUPPORTED,

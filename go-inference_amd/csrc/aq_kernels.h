@@ -155,7 +155,7 @@ hipError_t head_fold_launch(const unsigned long long* partial, int count, unsign
 bool qmvd_multi_supported(int idx);
 hipError_t qmvd_multi_launch(int idx, QmvMultiArgs ma, hipStream_t stream);
 
-// Token-tile MFMA matvec kernels (aq_qmv_tok.hip; group-64 codes, 4 bit up to 32 and 8 bit up to 16 activation rows as
+// Token-tile MFMA matvec kernels (aq_qmv_tok.hip; group-64 codes of 4 or 8 bits, up to 32 activation rows as
 // the rows of 16x16x32 MFMAs, K a multiple of 256 up to 16384; one launch, no scratch memory).  kind 6 in QmvVariant.
 int qmvt_variant_count();
 const QmvVariant* qmvt_variant(int idx);

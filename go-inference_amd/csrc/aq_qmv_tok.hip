@@ -1,4 +1,4 @@
-// affine_qmv for 5..32 rows of x on gfx950 (batched / speculative-verify decode), 4-bit (8-bit: up to 16 rows) codes in
+// affine_qmv for 5..32 rows of x on gfx950 (batched / speculative-verify decode), 4- and 8-bit codes in
 // groups of 64: one launch, the weights streamed exactly once, no pass over x beforehand and no partial tiles in memory.
 //
 // Same contract as the other matvec kernels: replaces rocm_mlx_q4_projection_batch*
@@ -425,7 +425,8 @@ const QmvVariant* qmvt_variant(int idx) {
 bool qmvt_fits(const QmvArgs& a, int bits, int group_size, int idx) {
     const QmvVariant* v = qmvt_variant(idx);
     if (!v || bits != v->bits || group_size != 64) return false;
-    if (a.M < 1 || a.M > v->m || a.N < 1 || a.K < 256 || a.K % 256 != 0) return false;
+    // (K up to 16384, as qmvt_pick has it: what the tests cover; longer rows go to the kernels that split K)
+    if (a.M < 1 || a.M > v->m || a.N < 1 || a.K < 256 || a.K % 256 != 0 || a.K > 16384) return false;
     const uintptr_t al16 = reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.w);
     const uintptr_t al8 = reinterpret_cast<uintptr_t>(a.s) | reinterpret_cast<uintptr_t>(a.b);
     if ((al16 & 15) || (al8 & 7)) return false;

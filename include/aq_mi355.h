@@ -157,6 +157,9 @@ int aq_reserve_workspace(aq_ctx *ctx, int M, int K);
  * more than is there grows it (not possible while a capture is open): run such a call once before capturing,
  * or reserve its bytes here. */
 int aq_reserve_workspace_bytes(aq_ctx *ctx, size_t bytes);
+/* Device bytes the context holds as scratch right now (the workspace above plus the partial maxima of
+ * aq_qmv_greedy): lets a caller, or a test, see whether a call made either of them grow.  No reference counterpart. */
+size_t aq_workspace_bytes(aq_ctx *ctx);
 
 /* gather_qmv: for each route z, y[z,:N] = x[lhs[z] or 0, :K] . dequant(W_e)^T with
  * e = rhs[z] read ON DEVICE; W_e = rows [row_base, row_base+N) of expert e's slab.
@@ -287,7 +290,8 @@ int aq_qmv_greedy_selected(aq_ctx *ctx, const void *x, const void *packed, const
  * process ends.  Limits: M == 1; 4- or 8-bit codes whose rows are 16-byte aligned (the shapes the fused
  * kernels take, anything else returns AQ_ERR_UNSUPPORTED); at most 262144 partial maxima (one per 16 rows for
  * 4-bit group-32/64 codes with K > 1024, else one per 1..4 rows), i.e. vocabularies of up to 4 M rows on the
- * fast path and at least 262144 rows otherwise: beyond that AQ_ERR_SIZE.  best[0] is bit-identical to
+ * fast path and at least 262144 rows otherwise: beyond that AQ_ERR_SIZE.  A variant forced with aq_force_variant
+ * is not consulted (the fused kernels are the only route that needs no scratch).  best[0] is bit-identical to
  * aq_qmv_greedy's.  All calls on one GPU share that GPU's array (also across contexts): calls that overlap on
  * one GPU race; order them on one stream. */
 int aq_qmv_greedy_static(aq_ctx *ctx, const void *x, const void *packed, const void *scales, const void *biases,
@@ -421,7 +425,8 @@ int aq_proj_quant_matmul_host(aq_ctx *ctx, float *out, const float *x, size_t x_
  * Route switches (the reference's GO_ROCM_DISABLE_* variables, hip_projection_launch.go:95-137): the environment
  * variable AQ_MI355_DISABLE=name[,name...] over dot2, blk, diag, tok, tiles is read by aq_create and takes those
  * kernel families out of that context's selection; a call then runs on the next family that takes its shape (the
- * any-width kernel at the end cannot be switched off).  aq_qmm with five rows and more is not affected.  There is
+ * any-width kernel at the end cannot be switched off).  aq_qmm with five rows and more is not affected, and the
+ * fused head, gate|up and multi-matrix calls honour `diag` only (their dot2 kernels have no switch).  There is
  * no code-object override (GO_ROCM_KERNEL_HSACO, hip_kernel_module.go:14-35): the kernels are part of the library. */
 int aq_variant_count(int op);
 const char *aq_variant_name(int op, int variant);

@@ -39,6 +39,69 @@ def test_static_greedy_matches_greedy(ctx, orc, bits, gs, K, shapes):
         dw.free()
 
 
+def _free_device_bytes():
+    """hipMemGetInfo's free bytes, asked of the HIP runtime the library has loaded."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    free, total = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+    return free.value
+
+
+@pytest.mark.parametrize("bits,gs,K,N", [(4, 64, 2048, 9000), (8, 64, 1024, 3000), (4, 64, 512, 5000)])
+def test_static_greedy_allocates_nothing_and_replays_in_a_graph(ctx, bits, gs, K, N):
+    """On a context that has run nothing else: the call leaves the free device memory and the context's scratch sizes
+    as they were; captured into a graph it gives aq_qmv_greedy's packed best on every replay, also after the
+    activations have changed between replays."""
+    import aq_mi355
+    say("greedy static, fresh context", bits, gs, K, N)
+    fresh = aq_mi355.Context(0)
+    try:
+        words, s, b = F.synthetic_affine(N, K, bits, gs, seed=F.BASE_SEED + 140)
+        dw = DeviceAffine(fresh, words, s, b)
+        x0, x1 = F.synthetic_x(1, K, seed=F.BASE_SEED + 141), F.synthetic_x(1, K, seed=F.BASE_SEED + 142)
+        dx = fresh.to_device(x0)
+        dsup = fresh.to_device(np.array([2, N - 2], dtype=np.int32))
+        got = fresh.alloc(8)
+        fresh.fill_zero(got)
+        fresh.sync()
+        free0, scratch0 = _free_device_bytes(), fresh.workspace_bytes()
+        fresh.qmv_greedy_static(dx, dw.w, dw.s, dw.b, got, K, N, gs, bits, dsup, 2)
+        fresh.sync()
+        first = _best(got)
+        assert (_free_device_bytes(), fresh.workspace_bytes()) == (free0, scratch0)
+        fresh.force_variant(0, 0)                # a forced matvec variant is not consulted: same kernels, same answer
+        fresh.fill_zero(got)
+        fresh.qmv_greedy_static(dx, dw.w, dw.s, dw.b, got, K, N, gs, bits, dsup, 2)
+        fresh.force_variant(0, -1)
+        fresh.sync()
+        assert _best(got) == first
+        assert (_free_device_bytes(), fresh.workspace_bytes()) == (free0, scratch0)
+        # the same call under capture: nothing runs until the replays
+        fresh.fill_zero(got)
+        fresh.capture_begin()
+        fresh.qmv_greedy_static(dx, dw.w, dw.s, dw.b, got, K, N, gs, bits, dsup, 2)
+        graph = fresh.capture_end()
+        assert fresh.workspace_bytes() == scratch0
+        want = ctx.alloc(8)
+        for replay, xv in enumerate((x0, x1, x0)):
+            dx.upload(xv)
+            ctx.qmv_greedy(dx, dw.w, dw.s, dw.b, want, 1, K, N, gs, bits, dsup, 2)
+            ctx.sync()
+            fresh.fill_zero(got)
+            fresh.graph_launch(graph)
+            fresh.sync()
+            assert _best(got) == _best(want) != 0, replay
+            if replay == 0:
+                assert _best(got) == first
+        fresh.graph_destroy(graph)
+        for t in (dx, dsup, got, want):
+            t.free()
+        dw.free()
+    finally:
+        fresh.close()
+
+
 def test_static_greedy_limits(ctx):
     import aq_mi355
     buf = ctx.alloc(1 << 16)
