@@ -125,6 +125,13 @@ int pick_qmv_variant(const aq_ctx* ctx, int bits, int m, bool gather, int N, int
         }
     }
     if (m > 1 && want_rows > 4) want_rows = 4;
+    // one row of a large 8-bit matrix: one row per wavefront with four slices of it in flight (4096 x 14336: 12.1 us
+    // against 12.5 with two rows and two slices; the arithmetic of a row, and so its bytes, are the same)
+    if (bits == 8 && m == 1 && !gather && slices >= 4 && (int64_t)N * K >= ((int64_t)40 << 20))
+        for (int i = 0; i < aq::qmv_variant_count(); i++) {
+            const aq::QmvVariant* v = aq::qmv_variant(i);
+            if (v->bits == 8 && v->m == 1 && !v->gather && v->waves == 4 && v->depth == 4 && v->rows == 1 && v->xmode == 0) return i;
+        }
     int best = -1;
     for (int i = 0; i < aq::qmv_variant_count(); i++) {
         const aq::QmvVariant* v = aq::qmv_variant(i);
@@ -227,6 +234,9 @@ const QmvRule kQmvRules[] = {
                                             // 16384): the kernel a single row of such a K runs on, four rows a launch, so
                                             // that rows keep the bytes of single-row calls here too
     {4, 32, 0, 1, 2, kFamDiag},             // groups of 32: two tokens x eight groups as MFMA rows
+    {8, 64, 0, 1, 4, kFamDiag},             // up to four rows of 8-bit codes, K of 2048, 4096 or 8192, up to 40 Mi codes (where
+                                            // measured ahead of the next two rules, see qmvd_pick); a row of such a call
+                                            // has the bytes of a call with that row alone
     {8, 0, 0, 1, 1, kFamDot2},              // one row of 8-bit codes: the dot2 kernel with its non-temporal loads, 12.4 us for
                                             // 4096 x 14336 (63 % of the HBM peak) against 14.2 us on the block-MFMA kernel
     {8, 64, 0, 2, 32, kFamTok},             // K a multiple of 256 up to 16384: one launch, weights streamed once, no scratch
@@ -286,7 +296,7 @@ int run_diag(aq_ctx* ctx, const aq::QmvArgs& a, int group_size, int bits, bool g
     const int di = forced >= 0        ? forced
                    : gather           ? aq::qmvd_pick_gather(a.K)
                    : group_size == 32 ? aq::qmvd_pick_g32(a.M, a.K, a.N)
-                                      : aq::qmvd_pick(a.M, a.K, a.N);
+                                      : aq::qmvd_pick(a.M, a.K, a.N, bits);
     if (di >= 0 && aq::qmvd_fits(a, bits, group_size, gather, di)) {
         ctx->last_variant[0] = aq::qmvd_variant(di)->name;
         AQ_HIP(aq::qmvd_launch(di, a, ctx->stream), "hipLaunchKernel");
@@ -294,7 +304,7 @@ int run_diag(aq_ctx* ctx, const aq::QmvArgs& a, int group_size, int bits, bool g
     }
     // Five to eight rows of a K that one launch takes for up to four: two launches.  Every row of a call has the bytes
     // of a call with that row alone (go/engine/metal/qmv_rows.go:14-24), which the other families do not give.
-    if (forced < 0 && !gather && group_size == 64 && a.M > 4 && a.M <= 8) {
+    if (forced < 0 && !gather && group_size == 64 && bits == 4 && a.M > 4 && a.M <= 8) {
         const int d4 = aq::qmvd_pick(4, a.K, a.N);
         aq::QmvArgs part = a;
         part.M = 4;

@@ -129,13 +129,14 @@ const QmvVariant* qmvb_variant(int idx);
 bool qmvb_plan(const QmvArgs& a, int bits, int group_size, bool gather, int cu_count, int forced_idx, BlkPlan* out);
 hipError_t qmvb_launch(const BlkPlan& p, const QmvArgs& a, hipStream_t stream);
 
-// Diagonal-MFMA matvec kernels (aq_qmv_diag.hip; 4-bit group-64 codes, M <= 8, K a multiple of 256 in 2..16 steps of 1024).
+// Diagonal-MFMA matvec kernels (aq_qmv_diag.hip; 4-bit group-64 codes, M <= 8, K a multiple of 128 in 2..16 steps of 1024;
+// 8-bit group-64 codes, M <= 4, in steps of 512).
 int qmvd_variant_count();
 const QmvVariant* qmvd_variant(int idx);
 bool qmvd_fits(const QmvArgs& a, int bits, int group_size, bool gather, int idx);
 hipError_t qmvd_launch(int idx, const QmvArgs& a, hipStream_t stream);
 // The variant the library picks for M rows and this K, or -1 when another family takes the shape.
-int qmvd_pick(int M, int K, int N);
+int qmvd_pick(int M, int K, int N, int bits = 4);  // (8-bit codes: up to four rows)
 // The same for quantisation groups of 32 codes (up to two rows, K a multiple of 256).
 int qmvd_pick_g32(int M, int K, int N);
 // y = act(gate . x) * (up . x) with variant idx's split of K (a.w2, a.s2, a.b2: the `up` matrix; a.act); the two

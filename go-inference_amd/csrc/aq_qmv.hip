@@ -66,6 +66,7 @@ static const QmvEntry kQmvTable[] = {
     AQ_QMV_SET(4, 1, 0), AQ_QMV_SET(8, 1, 0), AQ_QMV_SET(4, 1, 1), AQ_QMV_SET(8, 1, 1),
     AQ_QMV_SET(4, 2, 0), AQ_QMV_SET(4, 3, 0), AQ_QMV_SET(4, 4, 0),
     AQ_QMV_SET(8, 2, 0), AQ_QMV_SET(8, 3, 0), AQ_QMV_SET(8, 4, 0),
+    AQ_QMV(8, 1, 1, 4, 4, 0),  // one row of a large 8-bit matrix: every slice of a 4096-code row in flight (4096 x 14336: 12.1 against 12.5 us)
 };
 
 int qmv_variant_count() { return (int)(sizeof(kQmvTable) / sizeof(kQmvTable[0])); }

@@ -1,5 +1,6 @@
 // affine_qmv / gather_qmv for gfx950, 4-bit codes in groups of 64 (1..8 activation rows) or 32 (1..2): the
-// diagonal-MFMA kernels, with their multi-matrix, gate|up pair, gathered and lm_head forms.
+// diagonal-MFMA kernels, with their multi-matrix, gate|up pair, gathered and lm_head forms; and a dense form for
+// 8-bit codes in groups of 64 (1..4 rows; the reference's q8 decode kernels, affine_projection.hipinc:105-149).
 //
 // Same contract as the dot2 kernel (aq_qmv.hip): replaces rocm_mlx_q4_projection*
 // (go/engine/hip/kernels/quant/affine_projection.hipinc:3-266), semantics of MLX affine_qmv
@@ -64,6 +65,9 @@ __device__ __forceinline__ uint4 load_u128_stream_at(gptr_t base, uint32_t off) 
     const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const __attribute__((address_space(1))) u32x4_t*>(base + off));
     return make_uint4(v[0], v[1], v[2], v[3]);
 }
+__device__ __forceinline__ uint32_t load_u32_at(gptr_t base, uint32_t off) {
+    return *reinterpret_cast<const __attribute__((address_space(1))) uint32_t*>(base + off);
+}
 __device__ __forceinline__ uint2 load_u64_at(gptr_t base, uint32_t off) {
     const u32x2_t v = *reinterpret_cast<const __attribute__((address_space(1))) u32x2_t*>(base + off);
     return make_uint2(v[0], v[1]);
@@ -90,8 +94,10 @@ constexpr int kDiagZeroBytes = 128;
 
 // LDS: activations in expansion order [M][K] bf16, the split group sums [M][chunks of 256 codes] x 48 B, 64 zero bytes,
 // the partial sums of the wavefronts [NW][sets of four activation rows][64] fp32.
-__host__ __device__ inline size_t qmvd_lds_bytes_for(int M, int K, int nw, int mt = 1, bool g32 = false) {
-    return (size_t)M * K * 2 + (size_t)M * ((K + kDiagChunk - 1) / kDiagChunk) * (g32 ? 96 : 48) + kDiagZeroBytes +
+// (8-bit codes: chunks of 128 codes and 32 bytes of sums each.)
+__host__ __device__ inline size_t qmvd_lds_bytes_for(int M, int K, int nw, int mt = 1, bool g32 = false, bool b8 = false) {
+    const int chunk = b8 ? kDiagChunk / 2 : kDiagChunk;
+    return (size_t)M * K * 2 + (size_t)M * ((K + chunk - 1) / chunk) * (g32 ? 96 : b8 ? 32 : 48) + kDiagZeroBytes +
            (size_t)nw * mt * 64 * 4;
 }
 
@@ -111,16 +117,27 @@ __host__ __device__ inline size_t qmvd_lds_bytes_for(int M, int K, int nw, int m
 // and what deals with those is not compiled in.
 // HEAD (lm_head, one activation row): 4 stores every row's packed (score, row) instead of the score, 3 keeps the
 // best packed value of the 16 rows in a.partial[set] for fold_best_kernel (aq_qmv_head.hip).
+// B8: 8-bit codes.  The bytes of a row keep the geometry of the 4-bit kernel (64-byte halves, 128-byte chunks, 16 bytes
+// per lane and half), so the loads are the same instructions; a half is then ONE group of 64 codes and a chunk two:
+// row (t, g) of A is non-zero in half L iff g == L, whatever the lane group, a lane's 16 codes of a half are two MFMAs
+// (cvt_f32_ubyte + v_perm give bf16 pairs in the order of the codes, every code 0..255 exact), D registers 0 and 1 of
+// the two halves are the two group sums, and the affine term is bias * X alone (the codes travel as themselves).
+// K is then a multiple of 128, so no chunk is a single half.
 template <int NW, int SUP, int NR, bool PAIR, int MT = 1, bool GATHER = false, int CPS = 4, bool G32 = false, int HEAD = 0,
-          bool LINES = true, bool STREAM = false, bool TILED = false, bool EVEN = false>
+          bool LINES = true, bool STREAM = false, bool TILED = false, bool EVEN = false, bool B8 = false>
 __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block) {
+    static_assert(!B8 || (!G32 && !TILED && !GATHER && !PAIR && HEAD == 0), "8-bit codes: dense group-64 projections");
     static_assert(!STREAM || LINES || TILED, "streaming loads take whole lines");
     static_assert(!TILED || (!G32 && !GATHER && HEAD == 0), "the tile-major layout: dense group-64 projections");
     static_assert(HEAD == 0 || (!PAIR && !GATHER && MT == 1), "the head epilogues take one plain activation row");
     static_assert(!G32 || MT == 1, "group 32: one set of two activation rows");
     constexpr int TPS = G32 ? 2 : 4;      // activation rows per set
-    constexpr int A2B = G32 ? 96 : 48;    // bytes of split group sums per chunk and activation row
-    constexpr int SBB = G32 ? 16 : 8;     // bytes of scales (or biases) per chunk and weight row
+    constexpr int A2B = G32 ? 96 : B8 ? 32 : 48;  // bytes of split group sums per chunk and activation row (8 bit: 24 + 8 of zeros)
+    constexpr int SBB = G32 ? 16 : B8 ? 4 : 8;    // bytes of scales (or biases) per chunk and weight row
+    constexpr int HSH = B8 ? 6 : 7;               // log2 of the codes in a 64-byte half of a row
+    constexpr int XH = B8 ? 128 : 256;            // bytes of activations per half
+    constexpr int PPC = B8 ? 16 : 32;             // 16-byte pieces of activations per chunk
+    constexpr int NI = B8 ? 2 : 4;                // MFMAs per half
     static_assert(!PAIR || NR == 2, "the pair kernel runs one set per matrix");
     static_assert(!GATHER || MT == 1, "a route has one activation row");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
@@ -131,7 +148,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     const int rg = wave_wg / NW;    // which 16 rows of the workgroup's NR x 16
     const int K = a.K, N = a.N, M = GATHER ? 1 : a.M;
     const int groups = K >> (G32 ? 5 : 6);
-    const int halves = K >> 7;             // 128-code halves of a row (K % 128 == 0)
+    const int halves = K >> HSH;           // 64-byte halves of a row (K % 128 == 0)
     const int chunks = (halves + 1) >> 1;  // the last chunk may be a single half
     static_assert(CPS >= 2 && CPS <= 4, "a step holds 2..4 chunks (one lane group per chunk for the scales)");
     const int supers = (chunks + CPS - 1) / CPS;  // the last step may hold fewer chunks
@@ -160,11 +177,13 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     const int ppt = K >> 3;        // 16-byte pieces of a token (K % 128 == 0: whole groups of eight)
     const int pieces = M * ppt;
     auto stage = [&](int p, uint32_t t, const uint4 v) {  // piece p of x, which belongs to activation row t
-        uint4 o;
-        o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);  // (x0, x4)
-        o.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);  // (x1, x5)
-        o.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);  // (x2, x6)
-        o.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);  // (x3, x7)
+        uint4 o = v;  // (8-bit codes expand in their own order)
+        if constexpr (!B8) {
+            o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);  // (x0, x4)
+            o.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);  // (x1, x5)
+            o.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);  // (x2, x6)
+            o.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);  // (x3, x7)
+        }
         *reinterpret_cast<uint4*>(lds_raw + xs_off + (uint32_t)p * 16) = o;
         const uint32_t ones = 0x3f803f80u;
         float sum = dot2_bf16(v.x, ones, 0.0f);
@@ -183,17 +202,20 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
             const uint32_t u1 = __float_as_uint(r1) & 0xffff0000u;
             const float r2 = r1 - __uint_as_float(u1);
             const uint32_t u2 = __float_as_uint(r2) & 0xffff0000u;
-            const uint32_t n0 = __float_as_uint(-128.0f * __uint_as_float(u0));
-            const uint32_t n1 = __float_as_uint(-128.0f * __uint_as_float(u1));
-            const uint32_t n2 = __float_as_uint(-128.0f * __uint_as_float(u2));
+            // (8-bit codes carry no offset: the scale slots of the affine term multiply zeros)
+            const uint32_t n0 = B8 ? 0u : __float_as_uint(-128.0f * __uint_as_float(u0));
+            const uint32_t n1 = B8 ? 0u : __float_as_uint(-128.0f * __uint_as_float(u1));
+            const uint32_t n2 = B8 ? 0u : __float_as_uint(-128.0f * __uint_as_float(u2));
             // group g of token t: 12 bytes at [t][chunk g / 4][g % 4]
             const uint32_t g = ((uint32_t)p - t * (uint32_t)ppt) >> (G32 ? 2 : 3);
-            uint32_t* e = G32 ? reinterpret_cast<uint32_t*>(lds_raw + a2_off + (t * chunks + (g >> 3)) * 96 + (g & 7) * 12)
-                              : reinterpret_cast<uint32_t*>(lds_raw + a2_off + (t * chunks + (g >> 2)) * 48 + (g & 3) * 12);
+            uint32_t* e = G32  ? reinterpret_cast<uint32_t*>(lds_raw + a2_off + (t * chunks + (g >> 3)) * 96 + (g & 7) * 12)
+                          : B8 ? reinterpret_cast<uint32_t*>(lds_raw + a2_off + (t * chunks + (g >> 1)) * 32 + (g & 1) * 12)
+                               : reinterpret_cast<uint32_t*>(lds_raw + a2_off + (t * chunks + (g >> 2)) * 48 + (g & 3) * 12);
             e[0] = (u0 >> 16) | u1;  // (X0, X1)
             e[1] = (u2 >> 16) | n0;  // (X2, -128 X0)
             e[2] = (n1 >> 16) | n2;  // (-128 X1, -128 X2)
-            if (!EVEN && !G32 && (halves & 1) && (int)g == groups - 1) {
+            if (B8 && (g & 1)) e[3] = e[4] = 0;  // the last 8 of a chunk's 32 bytes
+            if (!EVEN && !G32 && !B8 && (halves & 1) && (int)g == groups - 1) {
                 // a last chunk of one half: its two missing groups must add nothing to the affine term
 #pragma unroll
                 for (int q = 3; q < 9; q++) e[q] = 0;
@@ -212,8 +234,8 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
 #pragma unroll
     for (int q = 0; q < PRE; q++) {
         if (wstage) {
-            const int pl = wave * (CPS * 32) + (q & 1) * 64 + lane;  // piece of row q / 2
-            pre_p[q] = (q >> 1) < M && pl < ppt && (q & 1) * 64 + lane < CPS * 32 ? (q >> 1) * ppt + pl : pieces;
+            const int pl = wave * (CPS * PPC) + (q & 1) * 64 + lane;  // piece of row q / 2
+            pre_p[q] = (q >> 1) < M && pl < ppt && (q & 1) * 64 + lane < CPS * PPC ? (q >> 1) * ppt + pl : pieces;
         } else {
             pre_p[q] = q < 2 ? tid + q * NR * NW * kWave : pieces;
         }
@@ -248,7 +270,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     for (int ab = 0; ab < 2; ab++) {
         int r8 = LINES ? row0 + (n & 7) + 8 * ab : row0 + n;
         if (r8 >= N) r8 = N - 1;
-        w_lane[ab] = (uint32_t)r8 * (uint32_t)(K >> 1) + (uint32_t)j * 16;  // bytes
+        w_lane[ab] = (uint32_t)r8 * (uint32_t)(B8 ? K : K >> 1) + (uint32_t)j * 16;  // bytes
     }
     const uint32_t w_half = LINES ? (uint32_t)(n >> 3) * 64 : 0;  // which 64 bytes of the chunk this lane requests
     // TILED (aq_tile.h): a step of a set of 16 rows is one contiguous tile, 1 KiB of scales and biases and then 1 KiB
@@ -284,17 +306,20 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
         } else {
             // A last chunk of one half has two groups: its 8 bytes are read 4 bytes early (inside the row) and the
             // upper word, which holds the two groups, moves down.
-            const bool halfl = !EVEN && (halves & 1) && j < CPS && CPS * sp + j == chunks - 1;
+            const bool halfl = !EVEN && !B8 && (halves & 1) && j < CPS && CPS * sp + j == chunks - 1;
             const uint32_t so = sb_lane + (uint32_t)sp * (CPS * SBB) - (j < valid ? 0u : (uint32_t)j * SBB) - (halfl ? 4u : 0u);
             if constexpr (G32) {
                 sq[u] = load_u128_at(sg, so);
                 bq[u] = load_u128_at(bg, so);
+            } else if constexpr (B8) {
+                sq[u] = make_uint4(load_u32_at(sg, so), 0, 0, 0);
+                bq[u] = make_uint4(load_u32_at(bg, so), 0, 0, 0);
             } else {
                 const uint2 s2 = load_u64_at(sg, so), b2 = load_u64_at(bg, so);
                 sq[u] = make_uint4(s2.x, s2.y, 0, 0);
                 bq[u] = make_uint4(b2.x, b2.y, 0, 0);
             }
-            if (!EVEN && !G32 && (halves & 1)) {
+            if (!EVEN && !G32 && !B8 && (halves & 1)) {
                 sq[u].x = halfl ? sq[u].y : sq[u].x;
                 bq[u].x = halfl ? bq[u].y : bq[u].x;
             }
@@ -372,15 +397,15 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     for (int tg = 0; tg < MT; tg++) {
         const int token = tg * TPS + at;
         const bool tok = token < M;
-        const bool d0 = tok && ag == (G32 ? j : j >> 1);
-        const bool d1 = tok && ag == (G32 ? 4 + j : 2 + (j >> 1));
-        const uint32_t x_lane = xs_off + (uint32_t)token * K * 2 + (uint32_t)j * 64;  // codes j*32.. of a 128-code load
+        const bool d0 = tok && ag == (G32 ? j : B8 ? 0 : j >> 1);
+        const bool d1 = tok && ag == (G32 ? 4 + j : B8 ? 1 : 2 + (j >> 1));
+        const uint32_t x_lane = xs_off + (uint32_t)token * K * 2 + (uint32_t)j * (XH / 4);  // the lane group's quarter of a half
         a_base0[tg] = d0 ? x_lane : zero_off;
-        a_base1[tg] = d1 ? x_lane + 256 : zero_off;
-        a_mul0[tg] = d0 ? CPS * 512 : 0;
-        a_mul1[tg] = d1 ? CPS * 512 : 0;
-        a_chunk0[tg] = d0 ? 512 : 0;
-        a_chunk1[tg] = d1 ? 512 : 0;
+        a_base1[tg] = d1 ? x_lane + XH : zero_off;
+        a_mul0[tg] = d0 ? CPS * 2 * XH : 0;
+        a_mul1[tg] = d1 ? CPS * 2 * XH : 0;
+        a_chunk0[tg] = d0 ? 2 * XH : 0;
+        a_chunk1[tg] = d1 ? 2 * XH : 0;
         const bool d2 = tok && ag == 0;
         a2_base[tg] = d2 ? a2_off + ((uint32_t)token * chunks + j) * A2B : zero_off;
         a2_mul[tg] = d2 ? CPS * A2B : 0;
@@ -403,9 +428,10 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
             // affine term of the groups of the step: six k-slots per group (b b b s s s), 24 (group 32: 48) per lane
             {
                 const uint32_t lo2 = 0x01000100u, hi2 = 0x03020302u, lolo = 0x05040100u, hihi = 0x07060302u;
-                constexpr int NWORD = G32 ? 4 : 2;  // words of two groups each
+                constexpr int NWORD = G32 ? 4 : B8 ? 1 : 2;  // words of two groups each
                 const uint32_t sw[4] = {sv.x, sv.y, sv.z, sv.w}, bw[4] = {bv.x, bv.y, bv.z, bv.w};
-                uint32_t e[6 * NWORD];
+                uint32_t e[B8 ? 8 : 6 * NWORD];
+                if constexpr (B8) e[6] = e[7] = 0;
 #pragma unroll
                 for (int w = 0; w < NWORD; w++) {
                     // (b0 b0 | b0 s0 | s0 s0 | b1 b1 | b1 s1 | s1 s1) of the word's two groups
@@ -421,7 +447,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
                     // (lane groups past the last chunk of the row contribute zeros)
                     const uint32_t a2_addr = j < valid ? a2_base[tg] + (uint32_t)sp * a2_mul[tg] : zero_off;
 #pragma unroll
-                    for (int q = 0; q < 6 * NWORD / 4; q++) {
+                    for (int q = 0; q < (B8 ? 2 : 6 * NWORD / 4); q++) {
                         const bf16x8_t a2 = *reinterpret_cast<const bf16x8_t*>(lds_raw + a2_addr + q * 16);
                         dsum[tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
                             a2, as_bf16x8(e[4 * q], e[4 * q + 1], e[4 * q + 2], e[4 * q + 3]), dsum[tg], 0, 0, 0);
@@ -436,7 +462,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
             }
             // The A fragments of chunk cc + 1 are read from LDS while chunk cc is multiplied: every register of `af` is
             // loaded again as soon as the MFMA that read it has been issued, so the wavefront never waits for LDS.
-            bf16x8_t af[MT][2][4];
+            bf16x8_t af[MT][2][NI];
             auto read_af = [&](int tg, int L, int i, int cc) {
                 af[tg][L][i] = *reinterpret_cast<const bf16x8_t*>(lds_raw + (L == 0 ? a_addr0[tg] + cc * a_chunk0[tg] : a_addr1[tg] + cc * a_chunk1[tg]) + i * 16);
             };
@@ -446,7 +472,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
 #pragma unroll
                 for (int tg = 0; tg < MT; tg++)
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
+                    for (int i = 0; i < NI; i++) {
                         read_af(tg, 0, i, cc);
                         read_af(tg, 1, i, cc);
                     }
@@ -482,22 +508,28 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
                 auto multiply = [&](auto both_halves) {  // straight-line code in either case
                     constexpr int NL = decltype(both_halves)::value ? 2 : 1;
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
+                    for (int i = 0; i < NI; i++) {
 #pragma unroll
                         for (int L = 0; L < NL; L++) {
                             // LINES, first 64 bytes: lanes i >= 8 take rows 8..15 from the second load's lanes i - 8;
                             // second 64 bytes: lanes i < 8 take rows 0..7 from the first load's lanes i + 8
-                            const uint32_t wa = i == 0 ? la.x : i == 1 ? la.y : i == 2 ? la.z : la.w;
-                            const uint32_t wb = i == 0 ? lb.x : i == 1 ? lb.y : i == 2 ? lb.z : lb.w;
-                            uint32_t ww;
-                            if constexpr (!LINES || TILED)
-                                ww = L == 0 ? wa : wb;
-                            else if (L == 0)
-                                ww = __builtin_amdgcn_update_dpp(wa, wb, 0x118, 0xf, 0xc, false);
-                            else
-                                ww = __builtin_amdgcn_update_dpp(wb, wa, 0x108, 0xf, 0x3, false);
+                            auto word = [&](int q) {
+                                const uint32_t wa = q == 0 ? la.x : q == 1 ? la.y : q == 2 ? la.z : la.w;
+                                const uint32_t wb = q == 0 ? lb.x : q == 1 ? lb.y : q == 2 ? lb.z : lb.w;
+                                if constexpr (!LINES || TILED)
+                                    return L == 0 ? wa : wb;
+                                else if (L == 0)
+                                    return (uint32_t)__builtin_amdgcn_update_dpp(wa, wb, 0x118, 0xf, 0xc, false);
+                                else
+                                    return (uint32_t)__builtin_amdgcn_update_dpp(wb, wa, 0x108, 0xf, 0x3, false);
+                            };
                             uint32_t p[4];
-                            unpack4_word(ww, mask, magic, p);
+                            if constexpr (B8) {
+                                unpack8_word(word(2 * i), p);
+                                unpack8_word(word(2 * i + 1), p + 2);
+                            } else {
+                                unpack4_word(word(i), mask, magic, p);
+                            }
                             const bf16x8_t bfrag = as_bf16x8(p[0], p[1], p[2], p[3]);
 #pragma unroll
                             for (int tg = 0; tg < MT; tg++) {
@@ -519,10 +551,16 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
                     // the half of this lane's token slot
                     const f32x4_t d0 = dq[tg][0], d1 = dq[tg][1];
                     const bool odd = G32 && (j & 1);
-                    acc[tg] = __builtin_fmaf(s0, odd ? d1[0] : d0[0], acc[tg]);
-                    acc[tg] = __builtin_fmaf(s1, odd ? d1[1] : d0[1], acc[tg]);
-                    acc[tg] = __builtin_fmaf(s2, (G32 && !odd) ? d0[2] : d1[2], acc[tg]);
-                    acc[tg] = __builtin_fmaf(s3, (G32 && !odd) ? d0[3] : d1[3], acc[tg]);
+                    if constexpr (B8) {
+                        // two groups a chunk: register 0 of the first half's sums, register 1 of the second's
+                        acc[tg] = __builtin_fmaf(s0, d0[0], acc[tg]);
+                        acc[tg] = __builtin_fmaf(s1, d1[1], acc[tg]);
+                    } else {
+                        acc[tg] = __builtin_fmaf(s0, odd ? d1[0] : d0[0], acc[tg]);
+                        acc[tg] = __builtin_fmaf(s1, odd ? d1[1] : d0[1], acc[tg]);
+                        acc[tg] = __builtin_fmaf(s2, (G32 && !odd) ? d0[2] : d1[2], acc[tg]);
+                        acc[tg] = __builtin_fmaf(s3, (G32 && !odd) ? d0[3] : d1[3], acc[tg]);
+                    }
                 }
             }
         }
@@ -620,6 +658,14 @@ __global__ __launch_bounds__(NR* NW* kWave, 4) void qmv_diag_g32_kernel(const Qm
     qmv_diag_dense<NW, SUP, NR, false, 1, CPS, true, MODE>(a, (int)blockIdx.x);
 }
 
+// 8-bit codes in groups of 64, up to four activation rows (whole lines of 8 rows per load instruction, as the 4-bit
+// kernels of more than four wavefronts have them).
+template <int NW, int SUP, int NR, int CPS, int MODE>
+__global__ __launch_bounds__(NR* NW* kWave, 4) void qmv_diag_b8_kernel(const QmvArgs a) {
+    static_assert((MODE & 2) == 0, "8-bit codes have no tile-major form");
+    qmv_diag_body<NW, SUP, NR, false, 1, false, CPS, false, 0, true, (MODE & 1) != 0, false, (MODE & 4) != 0, true>(a, (int)blockIdx.x);
+}
+
 // lm_head forms (one activation row): packed scores (4) or the best packed value per 16 rows (3).
 template <int NW, int SUP, int NR, int CPS, bool G32, int HEAD>
 __global__ __launch_bounds__(NR* NW* kWave, 4) void qmv_diag_head_kernel(const QmvArgs a) {
@@ -680,6 +726,7 @@ static int diag_early_wgs() {
 
 typedef void (*QmvDiagKernel)(const QmvArgs);
 // Index into a variant's kernels for this launch.
+// (K: in codes of 4 bits; a row of 8-bit codes counts as one of twice the length, which has the same bytes)
 static int diag_mode(int K, int cps, bool tiled, bool stream) {
     return (K % (cps * kDiagChunk) == 0 ? 4 : 0) + (tiled ? 2 : 0) + (stream ? 1 : 0);
 }
@@ -723,6 +770,15 @@ struct QmvDiagEntry {
     {                                                                                                                     \
         {"qmvd_b4_m2_r" #NR "_w" #NW "_d" #SUP "_g0_s32_c3", 4, 2, NR, NW, SUP, 0, 3, 5}, {qmv_diag_g32_kernel<NW, SUP, NR, 3, 0>, qmv_diag_g32_kernel<NW, SUP, NR, 3, 1>, nullptr, nullptr, qmv_diag_g32_kernel<NW, SUP, NR, 3, 4>, qmv_diag_g32_kernel<NW, SUP, NR, 3, 5>, nullptr, nullptr} \
     }
+// 8-bit codes (bits = 8; the split of K is that of a 4-bit row of the same bytes)
+#define AQ_QMVDB(NW, SUP, NR)                                                                                          \
+    {                                                                                                                  \
+        {"qmvd_b8_m4_r" #NR "_w" #NW "_d" #SUP "_g0", 8, 4, NR, NW, SUP, 0, 0, 4}, {qmv_diag_b8_kernel<NW, SUP, NR, 4, 0>, qmv_diag_b8_kernel<NW, SUP, NR, 4, 1>, nullptr, nullptr, qmv_diag_b8_kernel<NW, SUP, NR, 4, 4>, qmv_diag_b8_kernel<NW, SUP, NR, 4, 5>, nullptr, nullptr} \
+    }
+#define AQ_QMVDB3(NW, SUP, NR)                                                                                            \
+    {                                                                                                                     \
+        {"qmvd_b8_m4_r" #NR "_w" #NW "_d" #SUP "_g0_c3", 8, 4, NR, NW, SUP, 0, 3, 4}, {qmv_diag_b8_kernel<NW, SUP, NR, 3, 0>, qmv_diag_b8_kernel<NW, SUP, NR, 3, 1>, nullptr, nullptr, qmv_diag_b8_kernel<NW, SUP, NR, 3, 4>, qmv_diag_b8_kernel<NW, SUP, NR, 3, 5>, nullptr, nullptr} \
+    }
 static const QmvDiagEntry kQmvDiagTable[] = {
     AQ_QMVD(4, 1, 1), AQ_QMVD(4, 1, 2), AQ_QMVD(4, 1, 4), AQ_QMVD(2, 2, 2), AQ_QMVD(2, 1, 2), AQ_QMVD(8, 1, 1),
     AQ_QMVD(4, 2, 1), AQ_QMVD(2, 1, 4), AQ_QMVD(6, 1, 1), AQ_QMVD(10, 1, 1), AQ_QMVD(12, 1, 1),
@@ -731,10 +787,16 @@ static const QmvDiagEntry kQmvDiagTable[] = {
     AQ_QMVD3(4, 1, 1), AQ_QMVD3(4, 1, 2), AQ_QMVD3(4, 1, 4), AQ_QMVD3(2, 1, 2), AQ_QMVD3(2, 1, 4),
     AQ_QMVD83(4, 1, 4), AQ_QMVD83(4, 1, 2), AQ_QMVD83(2, 1, 4), AQ_QMVDG3(2, 1, 2), AQ_QMVDG3(4, 1, 1),
     AQ_QMVDS(2, 1, 2), AQ_QMVDS(4, 1, 1), AQ_QMVDS(4, 1, 2), AQ_QMVDS(8, 1, 1), AQ_QMVDS3(2, 1, 2), AQ_QMVDS3(4, 1, 1),
+    AQ_QMVDB(2, 1, 2), AQ_QMVDB(2, 1, 4), AQ_QMVDB(4, 1, 1), AQ_QMVDB(4, 1, 2), AQ_QMVDB(4, 1, 4), AQ_QMVDB(6, 1, 1),
+    AQ_QMVDB(8, 1, 1), AQ_QMVDB(10, 1, 1), AQ_QMVDB(12, 1, 1), AQ_QMVDB(14, 1, 1), AQ_QMVDB(16, 1, 1),
+    AQ_QMVDB3(4, 1, 1), AQ_QMVDB3(4, 1, 2), AQ_QMVDB3(4, 1, 4), AQ_QMVDB3(2, 1, 2), AQ_QMVDB3(2, 1, 4),
 };
 
 static int cps_of(const QmvVariant& v) { return v.xmode ? v.xmode : 4; }
 static bool g32_of(const QmvVariant& v) { return v.kind == 5; }
+static bool b8_of(const QmvVariant& v) { return v.bits == 8; }
+// The length of the 4-bit row that has the bytes of this row: what the split of K goes by.
+static int k4_of(int K, int bits) { return bits == 8 ? 2 * K : K; }
 // Steps of cps chunks of 256 codes that cover K (its last chunk may be a single half of 128 codes).
 static int steps_for(int K, int cps) { return ((K + kDiagChunk - 1) / kDiagChunk + cps - 1) / cps; }
 static int cps_for(int K) { return tile_cps_for(K); }
@@ -747,34 +809,36 @@ const QmvVariant* qmvd_variant(int idx) {
 
 bool qmvd_fits(const QmvArgs& a, int bits, int group_size, bool gather, int idx) {
     const QmvVariant* v = qmvd_variant(idx);
-    if (!v || bits != 4 || group_size != (g32_of(*v) ? 32 : 64) || gather != (v->gather != 0)) return false;
+    if (!v || bits != v->bits || group_size != (g32_of(*v) ? 32 : 64) || gather != (v->gather != 0)) return false;
+    const int K4 = k4_of(a.K, bits);
     if (g32_of(*v) && (a.K % kDiagChunk != 0 || ((reinterpret_cast<uintptr_t>(a.s) | reinterpret_cast<uintptr_t>(a.b)) & 15)))
         return false;
     if (gather && (a.M != 1 || a.routes < 1 || a.routes > 65535)) return false;
     if (a.M < 1 || a.M > v->m || a.K <= 0 || a.K % 128 != 0 || a.N < 1) return false;
-    if (steps_for(a.K, cps_of(*v)) > v->waves * v->depth) return false;
+    if (steps_for(K4, cps_of(*v)) > v->waves * v->depth) return false;
     const uintptr_t al16 = reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.w);
     const uintptr_t al8 = reinterpret_cast<uintptr_t>(a.s) | reinterpret_cast<uintptr_t>(a.b);
     if ((al16 & 15) || (al8 & 7)) return false;
     // 32-bit byte offsets into the packed matrix
-    if ((uint64_t)a.N * (uint64_t)(a.K / 2) >= (1ull << 32)) return false;
+    if ((uint64_t)a.N * (uint64_t)(K4 / 2) >= (1ull << 32)) return false;
     if (a.tiled) {
         // the layout is cut for one split of K; 32-bit byte offsets into it
-        if (gather || g32_of(*v) || cps_of(*v) != tile_cps_for(a.K)) return false;
+        if (gather || g32_of(*v) || b8_of(*v) || cps_of(*v) != tile_cps_for(a.K)) return false;
         const int64_t total = tile_total_bytes(a.N, a.K, group_size, bits);
         if (total < 0 || total >= ((int64_t)1 << 32)) return false;
     }
     // (up to four steps: two workgroups per CU; longer K: whatever one workgroup may use)
-    return qmvd_lds_bytes_for(a.M, a.K, v->waves * v->rows, (v->m + 3) / 4, g32_of(*v)) <=
-           (size_t)(steps_for(a.K, cps_of(*v)) <= 4 ? 96 : 156) * 1024;
+    return qmvd_lds_bytes_for(a.M, a.K, v->waves * v->rows, (v->m + 3) / 4, g32_of(*v), b8_of(*v)) <=
+           (size_t)(steps_for(K4, cps_of(*v)) <= 4 ? 96 : 156) * 1024;
 }
 
 hipError_t qmvd_launch(int idx, const QmvArgs& a, hipStream_t stream) {
     if (idx < 0 || idx >= qmvd_variant_count()) return hipErrorInvalidValue;
     const QmvDiagEntry& e = kQmvDiagTable[idx];
-    const size_t lds = qmvd_lds_bytes_for(a.M, a.K, e.v.waves * e.v.rows, (e.v.m + 3) / 4, g32_of(e.v));
-    const int stream_w = !e.v.gather && (int64_t)a.N * (a.K / 2) >= kDiagStreamBytes ? 1 : 0;
-    const QmvDiagKernel fn = e.fn[e.v.gather ? 0 : diag_mode(a.K, cps_of(e.v), a.tiled != 0, stream_w != 0)];
+    const size_t lds = qmvd_lds_bytes_for(a.M, a.K, e.v.waves * e.v.rows, (e.v.m + 3) / 4, g32_of(e.v), b8_of(e.v));
+    const int K4 = k4_of(a.K, e.v.bits);
+    const int stream_w = !e.v.gather && (int64_t)a.N * (K4 / 2) >= kDiagStreamBytes ? 1 : 0;
+    const QmvDiagKernel fn = e.fn[e.v.gather ? 0 : diag_mode(K4, cps_of(e.v), a.tiled != 0, stream_w != 0)];
     if (!fn) return hipErrorInvalidValue;
     if (hipError_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(fn), lds)) return rc;
     const int wg_rows = kDiagRows * e.v.rows;
@@ -788,10 +852,22 @@ hipError_t qmvd_launch(int idx, const QmvArgs& a, hipStream_t stream) {
 
 // The variant the library picks for M rows and this K, or -1: one step of 1024 codes per wavefront; up to 4 steps,
 // more rows per workgroup the more activation rows there are to stage.
-int qmvd_pick(int M, int K, int N) {
-    if (M < 1 || M > 8 || K <= 1024 || K % 128 != 0) return -1;  // (up to 1024 codes: one wavefront per row set, not built)
+int qmvd_pick(int M, int K, int N, int bits) {
+    if (bits != 4 && bits != 8) return -1;
+    if (M < 1 || M > (bits == 8 ? 4 : 8) || K % 128 != 0) return -1;
+    const int64_t codes = (int64_t)N * K;
+    K = k4_of(K, bits);
+    if (K <= 1024) return -1;  // (up to 1024 codes of 4 bits: one wavefront per row set, not built)
     const int cps = cps_for(K);
     const int steps = steps_for(K, cps);
+    if (bits == 8) {
+        // Where these kernels were measured ahead of the dot2 kernel (one row) and the token-tile kernel (2..4 rows):
+        // K of 2048, 4096 or 8192 (4, 8 or 16 whole steps) and up to 40 MiB of codes, e.g. 4096 x 4096 5.5 against
+        // 5.7 us (one row) and 6.8 against 8.8 us (four), 8192 x 4096 8.6 against 10.0 us; not 4096 x 14336, 14.7 against
+        // 12.7 us, nor 3072 x 6144, 7.1 against 6.0 us, nor four rows of 2048 x 8192, 7.5 against 6.5 us.
+        if (cps != 4 || (steps != 4 && steps != 8 && steps != 16) || K % (4 * kDiagChunk) != 0) return -1;
+        if (codes > ((int64_t)40 << 20) || (steps == 4 && M > 2)) return -1;
+    }
     const int cap = M <= 4 ? 4 : 8;
     int nw, nr;
     if (steps == 2) {
@@ -814,7 +890,7 @@ int qmvd_pick(int M, int K, int N) {
     if (cap == 8 && nw == 2) nr = 4;
     for (int i = 0; i < qmvd_variant_count(); i++) {
         const QmvVariant& v = kQmvDiagTable[i].v;
-        if (v.waves == nw && v.depth == 1 && v.rows == nr && v.m == cap && !v.gather && cps_of(v) == cps && !g32_of(v)) return i;
+        if (v.bits == bits && v.waves == nw && v.depth == 1 && v.rows == nr && v.m == cap && !v.gather && cps_of(v) == cps && !g32_of(v)) return i;
     }
     return -1;
 }
@@ -851,7 +927,7 @@ static const QmvDiagPairEntry* find_pair(int idx) {
     const QmvVariant* v = qmvd_variant(idx);
     if (v)
         for (const QmvDiagPairEntry& e : kQmvDiagPairTable)
-            if (e.nw == v->waves && e.sup == v->depth && e.cps == cps_of(*v) && !g32_of(*v)) return &e;
+            if (e.nw == v->waves && e.sup == v->depth && e.cps == cps_of(*v) && !g32_of(*v) && !b8_of(*v)) return &e;
     return nullptr;
 }
 bool qmvd_pair_supported(int idx) { return find_pair(idx) != nullptr; }
@@ -900,7 +976,7 @@ static const QmvDiagHeadEntry kQmvDiagHeadTable[] = {
 };
 static const QmvDiagHeadEntry* find_head(int idx, int fuse) {
     const QmvVariant* v = qmvd_variant(idx);
-    if (v && !v->gather)
+    if (v && !v->gather && !b8_of(*v))
         for (const QmvDiagHeadEntry& e : kQmvDiagHeadTable)
             if (e.nw == v->waves && e.sup == v->depth && e.nr == v->rows && e.cps == cps_of(*v) &&
                 (e.g32 != 0) == g32_of(*v) && e.fuse == fuse)
@@ -943,7 +1019,7 @@ static const QmvDiagMultiEntry kQmvDiagMultiTable[] = {
 // The multi-matrix launch of variant idx (the same arithmetic, so the same bytes, as one launch per matrix).
 bool qmvd_multi_supported(int idx) {
     const QmvVariant* v = qmvd_variant(idx);
-    if (!v) return false;
+    if (!v || b8_of(*v)) return false;
     for (const QmvDiagMultiEntry& e : kQmvDiagMultiTable)
         if (e.nw == v->waves && e.sup == v->depth && e.nr == v->rows && e.cps == cps_of(*v) && !g32_of(*v)) return true;
     return false;

@@ -274,9 +274,9 @@ def test_qmv_block_family_many_batches(ctx, orc):
 
 
 def test_qmvd_every_variant(ctx, orc):
-    """Each diagonal-MFMA matvec variant, forced: 1..4 (1..8) activation rows, K = all the steps of 1024 codes its
-    wavefronts take and one step fewer (an idle wavefront), a last step of three chunks and of one chunk of 256
-    codes, a last chunk that is a single half of 128 codes, ragged N; fp32 and bf16 stores; a K that is no multiple
+    """Each diagonal-MFMA matvec variant, forced: 1..4 (1..8) activation rows, K = all the steps of 1024 codes (512 of
+    8 bits) its wavefronts take and one step fewer (an idle wavefront), a last step of three chunks and of one chunk,
+    a last chunk that is a single half of 128 codes (4 bit), ragged N; fp32 and bf16 stores; a K that is no multiple
     of 128, or more steps than the variant takes, is refused."""
     import aq_mi355
     names = aq_mi355.variant_names(0)
@@ -290,23 +290,27 @@ def test_qmvd_every_variant(ctx, orc):
             waves = int(name.split("_w")[1].split("_")[0])
             steps = waves * int(name.split("_d")[1].split("_")[0])
             wg_waves = waves * int(name.split("_r")[1].split("_")[0])
-            step = 768 if name.endswith("_c3") else 1024  # codes per wavefront step
+            unit = 256 if bits == 4 else 128              # codes of a chunk (128 bytes of a row)
+            step = (3 if name.endswith("_c3") else 4) * unit  # codes per wavefront step
             gs = 32 if "_s32" in name else 64             # (group 32: K in whole chunks of 256 codes)
-            for K in sorted({step * steps, step * max(1, steps - 1), step * steps - 256, step * (steps - 1) + 256,
-                             step * steps - 128, step * (steps - 1) + 128}):
+            ks = {step * steps, step * max(1, steps - 1), step * steps - unit, step * (steps - 1) + unit}
+            if bits == 4:
+                ks |= {step * steps - 128, step * (steps - 1) + 128}  # a last chunk of one half (8 bit: K in whole chunks)
+            for K in sorted(ks):
                 if gs == 32 and K % 256:
                     continue
                 say("variant", idx, name, "K", K)
-                if (K, gs) not in data:
+                if (K, gs, bits) not in data:
                     words, s, b = F.synthetic_affine(N, K, bits, gs, seed=530 + K // 128)
                     x = F.synthetic_x(8, K, seed=630 + K // 128)
-                    data[(K, gs)] = (DeviceAffine(ctx, words, s, b), x, F.reference_f64(x, words, s, b, bits, gs, K))
-                dw, x, ref = data[(K, gs)]
+                    data[(K, gs, bits)] = (DeviceAffine(ctx, words, s, b), x, F.reference_f64(x, words, s, b, bits, gs, K))
+                dw, x, ref = data[(K, gs, bits)]
                 ctx.force_variant(0, idx)
                 for rows in ((1, 2) if m == 2 else (1, 2, 3, 4) if m == 4 else (1, 4, 5, 7, 8)):
-                    k_steps = -(-(-(-K // 256)) // (3 if name.endswith("_c3") else 4))
+                    k_steps = -(-(-(-K // unit)) // (3 if name.endswith("_c3") else 4))
                     lds_limit = (96 if k_steps <= 4 else 156) * 1024
-                    if rows * K * 2 + rows * ((K + 255) // 256) * (96 if gs == 32 else 48) + 128 + wg_waves * max(1, m // 4) * 256 > lds_limit:
+                    sums = 96 if gs == 32 else 48 if bits == 4 else 32
+                    if rows * K * 2 + rows * ((K + unit - 1) // unit) * sums + 128 + wg_waves * max(1, m // 4) * 256 > lds_limit:
                         # the activations of all rows and their group sums sit in LDS: beyond 96 KiB (two workgroups a
                         # CU; 156 KiB for K of more than four steps) the variant refuses
                         with pytest.raises(aq_mi355.AqError) as ei:
@@ -318,8 +322,8 @@ def test_qmvd_every_variant(ctx, orc):
                     check_accumulators(acc, ref[:rows], "%s rows=%d" % (name, rows))
                 out = run_qmv(ctx, x[:2], dw, 2, K, N, gs, bits, False)
                 check_bf16_store(out, ref[:2], name)
-            dw, x, ref = data[(step * steps, gs)]
-            for bad_k in (step * steps - 64, step * steps + 256):
+            dw, x, ref = data[(step * steps, gs, bits)]
+            for bad_k in (step * steps - 64, step * steps + unit):
                 with pytest.raises(aq_mi355.AqError) as ei:
                     run_qmv(ctx, np.zeros((1, bad_k), np.uint16), dw, 1, bad_k, N, gs, bits, True)
                 assert ei.value.code == aq_mi355.AQ_ERR_ARG
@@ -374,8 +378,8 @@ def test_qmvd_gather_every_variant(ctx, orc):
 
 def test_qmvd_is_the_default_for_few_rows(ctx, orc):
     """4-bit group-64 codes: 1..8 activation rows with K of 2..16 steps of 1024 codes land on the diagonal-MFMA kernels
-    without forcing (beyond four steps: up to four rows a launch), rows beyond the last full 16 included; other K and
-    8 bit do not."""
+    without forcing (beyond four steps: up to four rows a launch), rows beyond the last full 16 included; other K do
+    not (8-bit codes: tests/test_gpu_diag8.py)."""
     for K, N in ((4096, 16 * 9 + 5), (3072, 64), (2048, 33)):
         words, s, b = F.synthetic_affine(N, K, 4, 64, seed=810 + K // 1024)
         x = F.synthetic_x(8, K, seed=820 + K // 1024)
@@ -418,7 +422,7 @@ def test_qmvd_is_the_default_for_few_rows(ctx, orc):
         assert ctx.last_variant(0).startswith("qmvd_b4_m4_"), ctx.last_variant(0)
         check_accumulators(acc, F.reference_f64(x, words, s, b, 4, 64, K), "diag default K=%d rows=%d" % (K, rows))
         dw.free()
-    for K, bits, rows in ((17408, 4, 1), (1024, 4, 1), (4096, 8, 1), (17408, 4, 2), (2880, 4, 1)):
+    for K, bits, rows in ((17408, 4, 1), (1024, 4, 1), (3072, 8, 1), (17408, 4, 2), (2880, 4, 1)):
         words, s, b = F.synthetic_affine(32, K, bits, 64, seed=830)
         x = F.synthetic_x(rows, K, seed=831)
         dw = DeviceAffine(ctx, words, s, b)

@@ -24,9 +24,11 @@ CASES = [
     (4, 64, 9, 4096, ("qmvt_b4_m16_",)),
     (4, 64, 17, 4096, ("qmvt_b4_m32_",)),            # token tile, 32-token form: 17..32 rows
     (4, 64, 32, 4096, ("qmvt_b4_m32_",)),
-    (8, 64, 1, 4096, ("qmv_b8_",)),                  # dot2: one row of 8-bit codes
+    (8, 64, 1, 4096, ("qmvd_b8_",)),                 # diagonal MFMA, 8 bit: up to four rows, K of 2048, 4096, 8192
+    (8, 64, 4, 4096, ("qmvd_b8_",)),
+    (8, 64, 1, 3072, ("qmv_b8_",)),                  # dot2: one row of 8-bit codes at other K
     (8, 128, 1, 4096, ("qmv_b8_",)),
-    (8, 64, 4, 4096, ("qmvt_b8_m16_",)),             # token tile, 8 bit: 2..16 rows, K a multiple of 256
+    (8, 64, 4, 3072, ("qmvt_b8_m16_",)),             # token tile, 8 bit: 2..16 rows, K a multiple of 256
     (8, 64, 4, 4096 + 64, ("qmvb_", "qmv_b8_")),     # ... block MFMA or dot2 for other K
     (4, 64, 8, 14336, ("qmvd_b4_m4_",)),             # 5..8 rows at a K of more than four steps: two launches of four rows
     (4, 64, 3, 14336 + 128, ("qmvd_b4_m4_",)),       # ... up to four rows in one (15 steps, the last one short)
@@ -83,7 +85,8 @@ def test_matmul_of_few_rows_runs_as_matvec(ctx, M):
     ("diag,dot2", 4, 1, 4096, ("qmv_generic",)),        # ... and past them to the any-width kernel
     ("tok", 4, 16, 4096, ("qmmf_", "qmvb_")),           # 16 rows without the token-tile kernels
     ("tok,tiles,blk", 4, 16, 4096, ("qmv_generic",)),
-    ("blk", 8, 1, 4096, ("qmv_b8_",)),
+    ("blk", 8, 1, 3072, ("qmv_b8_",)),
+    ("diag", 8, 1, 4096, ("qmv_b8_",)),                 # 8-bit codes without the diagonal kernels: dot2 again
     ("nothing-by-that-name", 4, 1, 4096, ("qmvd_",)),   # unknown names switch nothing off
 ])
 def test_route_switches_from_the_environment(monkeypatch, off, bits, M, K, prefixes):
