@@ -459,7 +459,7 @@ int aq_create(int device, aq_ctx** out) {
     ctx->families_off = families_off_from_env(getenv("AQ_MI355_DISABLE"));
     // what the runtime reports, unchanged; a host that reports no marketing name shows the architecture instead
     char arch_only[80];
-    snprintf(arch_only, sizeof arch_only, "%.60s device (no name reported)", prop.gcnArchName);
+    snprintf(arch_only, sizeof arch_only, "%.*s device (no name reported)", (int)strcspn(prop.gcnArchName, ":"), prop.gcnArchName);
     snprintf(ctx->name, sizeof ctx->name, "%s (%s, %d CUs, %d MHz)", prop.name[0] ? prop.name : arch_only, prop.gcnArchName,
              prop.multiProcessorCount, prop.clockRate / 1000);
     rc = hipStreamCreateWithFlags(&ctx->own_stream, hipStreamNonBlocking);
