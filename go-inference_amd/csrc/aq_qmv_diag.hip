@@ -380,7 +380,10 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     const bool late = linear_block >= early_wgs || !wstage;
     if (late) stage_x();
     // AHEAD chunks are requested before the arithmetic starts; chunk cc + AHEAD when chunk cc is about to be worked on
-    constexpr int AHEAD = SUP == 1 && AQ_DIAG_AHEAD < CPS ? AQ_DIAG_AHEAD : CPS;
+    // (The group-32 and lm_head kernels request the whole step at once: their launches are grids of many rounds of
+    // workgroups, in which a wavefront's requests do not queue behind a whole launch's; 262144 x 1536, group 32:
+    // 40.0-42.6 us against 43.2-46.5 us with the ring.)
+    constexpr int AHEAD = SUP == 1 && AQ_DIAG_AHEAD < CPS && !G32 && HEAD == 0 ? AQ_DIAG_AHEAD : CPS;
 #pragma unroll
     for (int u = 0; u < SUP; u++) {
         issue_scales(u);
@@ -709,7 +712,7 @@ constexpr int64_t kDiagStreamBytes = (int64_t)16 << 20;
 
 // Workgroups that request their weights before staging x: as many as the device has CUs (the first workgroup each CU
 // receives; later ones find the CU's memory queue busy).
-static int diag_early_wgs() {
+static int diag_cu_count() {
     static int cached = -1;
     if (cached < 0) {
         const char* e = getenv("AQ_DIAG_EARLY");
@@ -722,6 +725,14 @@ static int diag_early_wgs() {
             cached = 256;
     }
     return cached;
+}
+// For a grid of `blocks` workgroups.  The rule is for launches whose workgroups are all resident at once (up to four
+// per CU): there the later arrivals wait for the CU's memory queue anyway.  In a larger grid (an lm_head, the MoE
+// gathers) a workgroup starts when another has finished and should request its weights at once: with every workgroup
+// but the first staging x first, the 262144 x 1536 head measured 44.6-45.7 us against 38.8 us.
+static int diag_early_wgs(int64_t blocks) {
+    const int cus = diag_cu_count();
+    return blocks <= (int64_t)4 * cus ? cus : INT32_MAX;
 }
 
 typedef void (*QmvDiagKernel)(const QmvArgs);
@@ -845,7 +856,7 @@ hipError_t qmvd_launch(int idx, const QmvArgs& a, hipStream_t stream) {
     dim3 grid((unsigned)((a.N + wg_rows - 1) / wg_rows), e.v.gather ? (unsigned)a.routes : 1u, 1u);
     QmvArgs b = a;
     b.stream_w = stream_w;
-    b.early_wgs = diag_early_wgs();
+    b.early_wgs = diag_early_wgs((int64_t)grid.x * grid.y);
     hipLaunchKernelGGL(fn, grid, dim3((unsigned)(e.v.rows * e.v.waves * kWave)), lds, stream, b);
     return hipGetLastError();
 }
@@ -942,7 +953,7 @@ hipError_t qmvd_pair_launch(int idx, const QmvArgs& a, bool gather, hipStream_t 
     dim3 grid((unsigned)((a.N + kDiagRows - 1) / kDiagRows), gather ? (unsigned)a.routes : 1u, 1u);
     QmvArgs b = a;
     b.stream_w = stream_w;
-    b.early_wgs = diag_early_wgs();
+    b.early_wgs = diag_early_wgs((int64_t)grid.x * grid.y);
     hipLaunchKernelGGL(fn, grid, dim3((unsigned)(2 * e->nw * kWave)), lds, stream, b);
     return hipGetLastError();
 }
@@ -996,7 +1007,7 @@ hipError_t qmvd_head_launch(int idx, int fuse, const QmvArgs& a, hipStream_t str
     if (hipError_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(e->fn), lds)) return rc;
     const int wg_rows = kDiagRows * e->nr;
     QmvArgs b = a;
-    b.early_wgs = diag_early_wgs();
+    b.early_wgs = diag_early_wgs((a.N + wg_rows - 1) / wg_rows);
     hipLaunchKernelGGL(e->fn, dim3((unsigned)((a.N + wg_rows - 1) / wg_rows)), dim3((unsigned)(e->nw * e->nr * kWave)), lds,
                        stream, b);
     return hipGetLastError();
@@ -1042,7 +1053,7 @@ hipError_t qmvd_multi_launch(int idx, QmvMultiArgs ma, hipStream_t stream) {
     int64_t bytes = 0;
     for (int i = 0; i < ma.count; i++) bytes += (int64_t)ma.N[i] * (ma.common.K / 2);
     ma.common.stream_w = bytes >= kDiagStreamBytes ? 1 : 0;
-    ma.common.early_wgs = diag_early_wgs();
+    ma.common.early_wgs = diag_early_wgs(blocks);
     const QmvDiagMultiKernel fn = e->fn[diag_mode(ma.common.K, e->cps, ma.common.tiled != 0, ma.common.stream_w != 0)];
     if (hipError_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(fn), lds)) return rc;
     hipLaunchKernelGGL(fn, dim3((unsigned)blocks), dim3((unsigned)(e->nw * e->nr * kWave)), lds, stream, ma);
