@@ -152,15 +152,26 @@ def run_probe(which, variant=None, layout="tiled"):
         E, TOK, TOPK, DM, DFF = 128, 8, 8, 2816, 1408
         routes = TOK * TOPK
         rng = np.random.Generator(np.random.PCG64(F.BASE_SEED + 77))
-        rhs = np.concatenate([rng.permutation(E)[:TOPK] for _ in range(TOK)]).astype(np.int32)
-        gu = tuple(ctx.to_device(t) for t in F.synthetic_affine(E * 2 * DFF, DM, BITS, GROUP, seed=F.BASE_SEED + 40))
-        dd = tuple(ctx.to_device(t) for t in F.synthetic_affine(E * DM, DFF, BITS, GROUP, seed=F.BASE_SEED + 41))
+        # HBM-cold like the timed leg: three slab copies and four seeded id sets in turn
+        id_sets = [ctx.to_device(np.concatenate([rng.permutation(E)[:TOPK] for _ in range(TOK)]).astype(np.int32)) for _ in range(4)]
+        gu0 = tuple(ctx.to_device(t) for t in F.synthetic_affine(E * 2 * DFF, DM, BITS, GROUP, seed=F.BASE_SEED + 40))
+        dd0 = tuple(ctx.to_device(t) for t in F.synthetic_affine(E * DM, DFF, BITS, GROUP, seed=F.BASE_SEED + 41))
+        slabs = [(gu0, dd0)]
+        for _ in range(2):
+            pair = []
+            for src in (gu0, dd0):
+                dst = tuple(ctx.alloc(t.nbytes) for t in src)
+                for d, t in zip(dst, src):
+                    ctx._check(ctx.lib.aq_d2d(ctx.handle, d.ptr, t.ptr, t.nbytes))
+                pair.append(dst)
+            slabs.append(tuple(pair))
         xt = ctx.to_device(F.synthetic_x(TOK, DM, seed=F.BASE_SEED + 1200))
-        d_rhs = ctx.to_device(rhs)
         d_tok = ctx.to_device(np.repeat(np.arange(TOK, dtype=np.int32), TOPK))
         d_route = ctx.to_device(np.arange(routes, dtype=np.int32))
         yh, yd = ctx.alloc(routes * DFF * 2), ctx.alloc(routes * DM * 2)
         for i in range(300):
+            gu, dd = slabs[i % 3]
+            d_rhs = id_sets[i % 4]
             ctx.gather_qmv_gate_up(xt, gu[0], gu[1], gu[2], d_tok, d_rhs, yh, routes, TOK, DM, DFF, E, 2 * DFF, 0, DFF, GROUP,
                                    BITS, aq_mi355.AQ_ACT_GELU_TANH)
             ctx.gather_qmv(yh, dd[0], dd[1], dd[2], d_route, d_rhs, yd, routes, routes, DFF, DM, E, DM, 0, GROUP, BITS)
