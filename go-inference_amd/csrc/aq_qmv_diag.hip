@@ -899,6 +899,21 @@ int qmvd_pick(int M, int K, int N, int bits) {
     const int min_nr = (cap == 8 || nw == 2) ? 2 : 1;
     while (nr > min_nr && (N + kDiagRows * nr - 1) / (kDiagRows * nr) < 128) nr >>= 1;
     if (cap == 8 && nw == 2) nr = 4;
+    // More sets per workgroup where that makes the launch one workgroup per CU (between three quarters of the CUs and
+    // all of them): every workgroup then starts at once and none queues behind another on its CU.  4096 x 14336: 224
+    // workgroups of 64 rows 7.43 us against 7.66 us for 896 of 16; 4096 x 6144: 192 of 32 rows 4.85 against 5.0 us;
+    // 2048 x 16384: 256 of 64 rows 5.30 against 5.45 us.  Not where it leaves more workgroups than CUs (4096 x 28672:
+    // 448 of 64 rows 13.6 us against 12.0 us for 1792 of 16).  The bytes of a row do not depend on it.
+    if (cap == 4 && bits == 4 && nw <= 4) {
+        const int cus = diag_cu_count();
+        for (int cand = 4; cand > nr; cand >>= 1) {
+            const int wgs = (N + kDiagRows * cand - 1) / (kDiagRows * cand);
+            if (wgs <= cus && wgs * 4 >= cus * 3) {
+                nr = cand;
+                break;
+            }
+        }
+    }
     for (int i = 0; i < qmvd_variant_count(); i++) {
         const QmvVariant& v = kQmvDiagTable[i].v;
         if (v.bits == bits && v.waves == nw && v.depth == 1 && v.rows == nr && v.m == cap && !v.gather && cps_of(v) == cps && !g32_of(v)) return i;
