@@ -474,6 +474,22 @@ def main():
         qmm = {"M": M, "K": K, "N": N, "ms": round(q_ms, 4), "TFLOPs": round(tf, 1), "kernel": ctx.last_variant(1),
                "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                             "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": q_traffic, "traffic_note": q_note}}
+        # gate and up of the layer against the same x in one aq_qmm_multi call: the pass over x runs once
+        yu = ctx.alloc(M * N * 2)
+
+        def pair_call(i):
+            g, u = layers[i % copies]["gate"], layers[i % copies]["up"]
+            ctx.qmm_multi(xm, [g[0], u[0]], [g[1], u[1]], [g[2], u[2]], [ym, yu], [N, N], M, K, GROUP, BITS)
+        for i in range(8):
+            pair_call(i)
+        ctx.sync()
+        ctx.timer_start()
+        for i in range(24):
+            pair_call(i)
+        p_ms = ctx.timer_stop() / 24
+        yu.free()
+        qmm["gate_up_multi"] = {"ms": round(p_ms, 4), "TFLOPs": round(2 * flops / (p_ms * 1e-3) / 1e12, 1),
+                                "note": "aq_qmm_multi over the gate and up matrices (two 2048 x 14336 x 4096 products, one pass over x)"}
         # the same call on the other kernel family: bare codes as bf16 operands and one fp32 FMA per output element
         # and 64-code block (the default is the family whose MFMA operand carries scale * (code - 8) as fp16)
         other = "qmmt_b4_mb2_nb2_wm2_wn2"

@@ -90,6 +90,7 @@ PROTOTYPES = {
     "aq_qmv": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _u]),
     "aq_qmm": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _u]),
     "aq_qmv_multi": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _u]),
+    "aq_qmm_multi": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _u]),
     "aq_reserve_workspace": (_i, [_vp, _i, _i]),
     "aq_reserve_workspace_bytes": (_i, [_vp, _sz]),
     "aq_workspace_bytes": (_sz, [_vp]),
@@ -297,6 +298,13 @@ class Context:
         n = len(ws)
         arr = lambda seq: (_c.c_void_p * n)(*[_ptr(t) for t in seq])
         self._check(self.lib.aq_qmv_multi(self.handle, _ptr(x), n, arr(ws), arr(ss), arr(bs), arr(ys),
+                                          (_c.c_int * n)(*Ns), M, K, group_size, bits, flags))
+
+    def qmm_multi(self, x, ws, ss, bs, ys, Ns, M, K, group_size=64, bits=4, flags=0):
+        """aq_qmm over several weight matrices that share x: one pass over x for the members that need the same form."""
+        n = len(ws)
+        arr = lambda seq: (_c.c_void_p * n)(*[_ptr(t) for t in seq])
+        self._check(self.lib.aq_qmm_multi(self.handle, _ptr(x), n, arr(ws), arr(ss), arr(bs), arr(ys),
                                           (_c.c_int * n)(*Ns), M, K, group_size, bits, flags))
 
     def prepared_qmv(self, x, w, s, b, y, M, K, N, group_size=64, bits=4, flags=0):

@@ -826,6 +826,46 @@ int aq_qmm(aq_ctx* ctx, const void* x, const void* packed, const void* scales, c
                             biases, y, M, K, N, group_size, bits, (flags & AQ_OUT_F32) != 0, fail);
 }
 
+int aq_qmm_multi(aq_ctx* ctx, const void* x, int count, const void* const* packed, const void* const* scales,
+                 const void* const* biases, void* const* y, const int* N, int M, int K, int group_size, int bits,
+                 unsigned flags) {
+    if (!ctx) return fail(AQ_ERR_ARG, "aq_qmm_multi: ctx is null");
+    if (count < 1 || count > 8) return fail(AQ_ERR_ARG, "aq_qmm_multi: count must be 1..8");
+    if (!packed || !scales || !biases || !y || !N) return fail(AQ_ERR_ARG, "aq_qmm_multi: null array");
+    if (M <= 0 || K <= 0) return fail(AQ_ERR_SHAPE, "aq_qmm_multi: M, N, K must be positive");
+    if (int rc = check_geometry("aq_qmm_multi", K, group_size, bits)) return rc;
+    if (!x || !aligned(x, 2)) return fail(AQ_ERR_ARG, "aq_qmm_multi: null or misaligned x");
+    size_t need = 0;
+    for (int i = 0; i < count; i++) {
+        if (N[i] <= 0) return fail(AQ_ERR_SHAPE, "aq_qmm_multi: M, N, K must be positive");
+        if (!packed[i] || !scales[i] || !biases[i] || !y[i]) return fail(AQ_ERR_ARG, "aq_qmm_multi: null operand");
+        if (!aligned(packed[i], 4) || !aligned(scales[i], 2) || !aligned(biases[i], 2) || !aligned(y[i], 2))
+            return fail(AQ_ERR_ARG, "aq_qmm_multi: operand pointer is not element-aligned");
+        const size_t n = aq::qmm_scratch_bytes(M, K, N[i]);
+        need = n > need ? n : need;
+    }
+    if (M <= aq::kQmvMaxRows && ctx->forced[1] < 0) {
+        // up to four rows: matvec calls (one launch per four members where the fused kernels take the shape)
+        for (int i = 0; i < count; i += aq::kQmvMultiMax) {
+            const int n = count - i < aq::kQmvMultiMax ? count - i : aq::kQmvMultiMax;
+            if (int rc = aq_qmv_multi(ctx, x, n, packed + i, scales + i, biases + i, y + i, N + i, M, K, group_size, bits, flags)) return rc;
+        }
+        ctx->last_variant[1] = ctx->last_variant[0];
+        return AQ_OK;
+    }
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    // the largest member's scratch first, so that no member makes the workspace move under the pass over x
+    if (int rc = aq::workspace_reserve(ctx->stream, &ctx->ws, need, fail)) return rc;
+    int x_state = aq::kXReadyNone;
+    for (int i = 0; i < count; i++)
+        if (int rc = aq::qmm_dispatch(ctx->stream, &ctx->ws, ctx->cu_count, ctx->forced[1], &ctx->last_variant[1], x, packed[i],
+                                      scales[i], biases[i], y[i], M, K, N[i], group_size, bits, (flags & AQ_OUT_F32) != 0, fail,
+                                      nullptr, 0, &x_state))
+            return rc;
+    return AQ_OK;
+}
+
 int aq_reserve_workspace(aq_ctx* ctx, int M, int K) {
     if (!ctx) return fail(AQ_ERR_ARG, "aq_reserve_workspace: ctx is null");
     if (M < 0 || K < 0) return fail(AQ_ERR_SHAPE, "aq_reserve_workspace: M and K must be non-negative");
@@ -1031,18 +1071,23 @@ int aq_qmv_gate_up(aq_ctx* ctx, const void* x, const void* gate_packed, const vo
     }
     float* g = reinterpret_cast<float*>(static_cast<char*>(ctx->ws.ptr) + region);
     float* u = reinterpret_cast<float*>(static_cast<char*>(ctx->ws.ptr) + region + each);
-    if (int rc = aq_qmv(ctx, x, gate_packed, gate_scales, gate_biases, g, M, K, N, group_size, bits, AQ_OUT_F32)) return rc;
     if (M > 32 && ctx->forced[0] < 0 && !(ctx->families_off >> kFamTiles & 1) &&
-        aq::qmm_takes_gate(x, up_packed, K, group_size, bits)) {
-        // prefill sizes: the `up` projection runs on the matmul tiles anyway, and their stores apply act(gate) * up on
-        // the way out (rocm_mlx_q4_gelu_tanh_multiply_batch, go/engine/hip/kernels/quant/affine_gelu_tanh.hipinc:921-1109):
-        // one [M, N] fp32 matrix is written and read instead of two written and two read.  Same bytes as the route below.
+        aq::qmm_takes_gate(x, up_packed, K, group_size, bits) && aq::qmm_takes_gate(x, gate_packed, K, group_size, bits)) {
+        // prefill sizes: both projections run on the matmul tiles (where aq_qmv sends this many rows anyway), the second
+        // pass over x is skipped, and the stores of the `up` projection apply act(gate) * up on the way out
+        // (rocm_mlx_q4_gelu_tanh_multiply_batch, go/engine/hip/kernels/quant/affine_gelu_tanh.hipinc:921-1109): one
+        // [M, N] fp32 matrix is written and read instead of two written and two read.  Same bytes as the route below.
         std::lock_guard<std::mutex> lk(ctx->mu);
+        int x_state = aq::kXReadyNone;
+        if (int rc = aq::qmm_dispatch(ctx->stream, &ctx->ws, ctx->cu_count, ctx->forced[1], &ctx->last_variant[1], x, gate_packed,
+                                      gate_scales, gate_biases, g, M, K, N, group_size, bits, true, fail, nullptr, 0, &x_state))
+            return rc;
         const int rc = aq::qmm_dispatch(ctx->stream, &ctx->ws, ctx->cu_count, ctx->forced[1], &ctx->last_variant[1], x, up_packed,
-                                        up_scales, up_biases, y, M, K, N, group_size, bits, out_f32, fail, g, act);
+                                        up_scales, up_biases, y, M, K, N, group_size, bits, out_f32, fail, g, act, &x_state);
         if (rc == AQ_OK) ctx->last_variant[0] = "qmv_gate_up_tiles";
         return rc;
     }
+    if (int rc = aq_qmv(ctx, x, gate_packed, gate_scales, gate_biases, g, M, K, N, group_size, bits, AQ_OUT_F32)) return rc;
     if (int rc = aq_qmv(ctx, x, up_packed, up_scales, up_biases, u, M, K, N, group_size, bits, AQ_OUT_F32)) return rc;
     std::lock_guard<std::mutex> lk(ctx->mu);
     AQ_HIP(aq::act_mul_f32_launch(g, u, y, (int64_t)M * N, act, out_f32 ? 1 : 0, ctx->stream), "hipLaunchKernel");

@@ -19,7 +19,12 @@ struct QmmArgs {
     int out_f32;
     const float* gate;  // not null: y = act(gate[m, n]) * (x . w^T)[m, n], gate being fp32 [M, N] (a gated MLP's other projection)
     int act;            // kActGeluTanh or kActSilu
+    int x_ready;        // kXReady*: the workspace already holds this x as that pass over x leaves it (a call of several
+                        // weight matrices against one x): the pass is skipped
 };
+
+// Which pass over x the workspace holds (QmmArgs.x_ready, and what a launch reports back through qmm_dispatch).
+enum { kXReadyNone = 0, kXReadyTile4 = 1, kXReadyTile8 = 2, kXReadyHalf = 3 };
 
 struct QmmVariant {
     const char* name;
@@ -56,6 +61,8 @@ const QmmVariant* qmmt_variant(int idx);
 size_t qmmt_workspace_bytes(int M, int K);
 // Pass over x + tile kernel `idx`; `workspace` holds at least qmmt_workspace_bytes(M, K).
 hipError_t qmmt_launch(int idx, const QmmArgs& a, void* workspace, hipStream_t stream);
+// The pass over x variant idx needs (kXReady*).
+int qmmt_x_kind(int idx);
 // The same with K shared out over ksplit workgroups per tile and a second kernel that adds the partial
 // tiles: for few rows of x, where M x N tiles alone leave most of the chip idle.
 size_t qmmt_splitk_bytes(int M, int N, int ksplit);
@@ -103,9 +110,11 @@ int qmm_reserve(hipStream_t stream, Workspace* ws, int M, int K, FailFn fail);
 // Returns an AQ_* / hipError_t code through `fail`.
 // `forced` indexes the tile variants (qmmt_variant), or is negative.
 // gate (fp32 [M, N], or null) and act: the gated-MLP epilogue, see QmmArgs; only where qmm_takes_gate says so.
+// x_state (or null): in, which pass over this x the workspace already holds (kXReady*); out, which it holds now.
 int qmm_dispatch(hipStream_t stream, Workspace* ws, int cu_count, int forced, const char** last_variant, const void* x,
                  const void* packed, const void* scales, const void* biases, void* y, int M, int K, int N,
-                 int group_size, int bits, bool out_f32, FailFn fail, const float* gate = nullptr, int act = 0);
+                 int group_size, int bits, bool out_f32, FailFn fail, const float* gate = nullptr, int act = 0,
+                 int* x_state = nullptr);
 // Whether qmm_dispatch runs this call on the tile kernels, whose stores can carry the gated-MLP epilogue.
 bool qmm_takes_gate(const void* x, const void* packed, int K, int group_size, int bits);
 

@@ -103,7 +103,7 @@ bool qmm_takes_gate(const void* x, const void* packed, int K, int group_size, in
 
 int qmm_dispatch(hipStream_t stream, Workspace* ws, int cu_count, int forced, const char** last_variant, const void* x,
                  const void* packed, const void* scales, const void* biases, void* y, int M, int K, int N,
-                 int group_size, int bits, bool out_f32, FailFn fail, const float* gate, int act) {
+                 int group_size, int bits, bool out_f32, FailFn fail, const float* gate, int act, int* x_state) {
     const bool mfma_ok = qmm_takes_gate(x, packed, K, group_size, bits);
     if (!mfma_ok) {
         if (gate) return fail(AQ_ERR_UNSUPPORTED, "aq_qmm: the gated epilogue needs the tile kernels (4 / 8 bit, groups of 64 / 128)");
@@ -208,10 +208,14 @@ int qmm_dispatch(hipStream_t stream, Workspace* ws, int cu_count, int forced, co
     }
     {
         const size_t xbytes = (qmmt_workspace_bytes(M, K) + 255) & ~(size_t)255;
+        const uint64_t generation = ws->generation;
         if (int rc = grow_workspace(ws, xbytes + qmmt_splitk_bytes(M, N, ksplit), stream, fail)) return rc;
+        // (a workspace that had to move no longer holds the earlier pass over x)
+        a.x_ready = x_state && ws->generation == generation ? *x_state : kXReadyNone;
         *last_variant = qmmt_variant(tile_idx)->name;
         hipError_t rc = qmmt_launch_splitk(tile_idx, a, ws->ptr, ksplit, stream);
         if (rc != hipSuccess) return fail((int)rc, "rocm.hip.hipLaunchKernel: HIP returned %d (%s)", (int)rc, hipGetErrorString(rc));
+        if (x_state) *x_state = qmmt_x_kind(tile_idx);
         return AQ_OK;
     }
 }

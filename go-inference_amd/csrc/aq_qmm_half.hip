@@ -625,9 +625,12 @@ hipError_t qmmh_launch(int idx, const QmmArgs& q, void* workspace, hipStream_t s
     uint16_t* xf = static_cast<uint16_t*>(workspace);
     uint16_t* xs = xf + (size_t)mblks * 32 * q.K;
     float* rs = reinterpret_cast<float*>(xs + (size_t)mblks * 32 * g4 * 8);
-    hipLaunchKernelGGL(qmmh_prep_kernel, dim3((unsigned)(mblks * 32 / kPrepRows)), dim3(kPrepThreads), 0, stream, q.x, xf, xs, rs, q.M, q.K);
-    hipError_t rc = hipGetLastError();
-    if (rc != hipSuccess) return rc;
+    hipError_t rc = hipSuccess;
+    if (q.x_ready != kXReadyHalf) {
+        hipLaunchKernelGGL(qmmh_prep_kernel, dim3((unsigned)(mblks * 32 / kPrepRows)), dim3(kPrepThreads), 0, stream, q.x, xf, xs, rs, q.M, q.K);
+        rc = hipGetLastError();
+        if (rc != hipSuccess) return rc;
+    }
 
     QmmTileArgs a{};
     a.xf = xf;

@@ -530,6 +530,13 @@ hipError_t qmmt_launch(int idx, const QmmArgs& q, void* workspace, hipStream_t s
     return qmmt_launch_splitk(idx, q, workspace, 1, stream);
 }
 
+int qmmt_x_kind(int idx) {
+    const QmmVariant* v = qmmt_variant(idx);
+    if (!v) return kXReadyNone;
+    if (idx >= tile_variants() && idx < tile_variants() + qmmh_variant_count()) return kXReadyHalf;
+    return v->bits == 4 ? kXReadyTile4 : kXReadyTile8;
+}
+
 // ksplit > 1: K/64 must be a multiple of 4 * ksplit; the fp32 partial tiles live in the workspace behind the
 // rewritten activations (qmmt_workspace_bytes(M, K) rounded up to 256, then qmmt_splitk_bytes).
 hipError_t qmmt_launch_splitk(int idx, const QmmArgs& q, void* workspace, int ksplit, hipStream_t stream) {
@@ -546,12 +553,15 @@ hipError_t qmmt_launch_splitk(int idx, const QmmArgs& q, void* workspace, int ks
     uint16_t* xs = xf + (size_t)mblks * 32 * q.K;
     const int64_t pieces = (int64_t)mblks * 32 * (q.K / 64) * 8;
     const unsigned prep_blocks = (unsigned)((pieces + 255) / 256);
-    if (v.bits == 4)
-        hipLaunchKernelGGL(qmm_prep_kernel<4>, dim3(prep_blocks), dim3(256), 0, stream, q.x, xf, xs, q.M, q.K, mblks);
-    else
-        hipLaunchKernelGGL(qmm_prep_kernel<8>, dim3(prep_blocks), dim3(256), 0, stream, q.x, xf, xs, q.M, q.K, mblks);
-    hipError_t rc = hipGetLastError();
-    if (rc != hipSuccess) return rc;
+    hipError_t rc = hipSuccess;
+    if (q.x_ready != (v.bits == 4 ? kXReadyTile4 : kXReadyTile8)) {
+        if (v.bits == 4)
+            hipLaunchKernelGGL(qmm_prep_kernel<4>, dim3(prep_blocks), dim3(256), 0, stream, q.x, xf, xs, q.M, q.K, mblks);
+        else
+            hipLaunchKernelGGL(qmm_prep_kernel<8>, dim3(prep_blocks), dim3(256), 0, stream, q.x, xf, xs, q.M, q.K, mblks);
+        rc = hipGetLastError();
+        if (rc != hipSuccess) return rc;
+    }
 
     QmmTileArgs a{};
     a.xf = xf;

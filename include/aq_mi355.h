@@ -144,6 +144,15 @@ int aq_qmv_multi(aq_ctx *ctx, const void *x, int count, const void *const *packe
 int aq_qmm(aq_ctx *ctx, const void *x, const void *packed, const void *scales, const void *biases, void *y, int M,
            int K, int N, int group_size, int bits, unsigned flags);
 
+/* `count` (1..8) aq_qmm calls that share x, M, K, group size and width (q|k|v, gate|up at prefill; the no-copy form of
+ * one matmul over model.ConcatQuantRows, go/model/quant_weight.go:32-62): y[i][M, N[i]] = x . dequant(packed[i], ...)^T.
+ * The pass that rewrites x into MFMA operand order runs once for the members that need the same form of it instead of
+ * once per member (10 us of a 290 us call at M = 2048, K = 4096); every y[i] is byte-identical to the separate
+ * aq_qmm call.  Host arrays of device pointers, as in aq_qmv_multi.  Up to four rows run as aq_qmv_multi. */
+int aq_qmm_multi(aq_ctx *ctx, const void *x, int count, const void *const *packed, const void *const *scales,
+                 const void *const *biases, void *const *y, const int *N, int M, int K, int group_size, int bits,
+                 unsigned flags);
+
 /* Prefill-sized aq_qmm / aq_qmv calls (M >= 64) rewrite x into MFMA operand order first and keep that
  * copy (about M*K*2 bytes) in a workspace the context owns.  The workspace grows on demand, which
  * drains the stream and allocates: not allowed while a capture is open and unwelcome in a serving
