@@ -113,6 +113,7 @@ PROTOTYPES = {
     "aq_pack_best": (_c.c_uint64, [_f, _i]),
     "aq_unpack_best": (_i, [_c.c_uint64, _f, _i, _c.POINTER(_i), _c.POINTER(_f)]),
     "aq_upload_linear": (_i, [_vp, _c.POINTER(HostLinear), _c.POINTER(DeviceLinear)]),
+    "aq_tile_device_linear": (_i, [_vp, _c.POINTER(DeviceLinear)]),
     "aq_upload_fused_gate_up": (_i, [_vp, _c.POINTER(HostLinear), _c.POINTER(HostLinear), _c.POINTER(DeviceLinear)]),
     "aq_free_device_linear": (_i, [_vp, _c.POINTER(DeviceLinear)]),
     "aq_dequant_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _c.c_int64, _i, _i, _i]),
@@ -414,6 +415,9 @@ class Context:
         out = DeviceLinear()
         self._check(self.lib.aq_upload_fused_gate_up(self.handle, ctypes.byref(gate), ctypes.byref(up), ctypes.byref(out)))
         return out
+
+    def tile_device_linear(self, dev_linear):
+        self._check(self.lib.aq_tile_device_linear(self.handle, ctypes.byref(dev_linear)))
 
     def free_device_linear(self, dev_linear):
         self._check(self.lib.aq_free_device_linear(self.handle, ctypes.byref(dev_linear)))

@@ -1745,6 +1745,34 @@ int aq_tile_weights(aq_ctx* ctx, const void* packed, const void* scales, const v
     return AQ_OK;
 }
 
+int aq_tile_device_linear(aq_ctx* ctx, aq_device_linear* lin) {
+    if (!ctx || !lin) return fail(AQ_ERR_ARG, "aq_tile_device_linear: bad argument");
+    if (!lin->weight || !lin->scales || !lin->biases)
+        return fail(AQ_ERR_ARG, "aq_tile_device_linear: the weight is not resident as MLX arrays (already tile-major?)");
+    // (an expert slab is read by the gathers, which take MLX arrays)
+    if (lin->experts > 0) return fail(AQ_ERR_UNSUPPORTED, "aq_tile_device_linear: expert slabs stay MLX arrays (the gathers read them)");
+    const int64_t bytes = aq::tile_total_bytes(lin->rows, lin->in_dim, lin->group_size, lin->bits);
+    if (bytes < 0 || bytes >= ((int64_t)1 << 32))
+        return fail(AQ_ERR_UNSUPPORTED, "aq_tile_device_linear: no tile-major layout for bits=%d group=%d K=%d rows=%d", lin->bits,
+                    lin->group_size, lin->in_dim, lin->rows);
+    void* tiled = nullptr;
+    {
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        AQ_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+        AQ_HIP(hipMalloc(&tiled, (size_t)bytes), "hipMalloc");
+    }
+    int rc = aq_tile_weights(ctx, lin->weight, lin->scales, lin->biases, lin->rows, lin->in_dim, lin->group_size, lin->bits, tiled);
+    if (rc == AQ_OK) rc = aq_sync(ctx);  // the arrays are freed next
+    if (rc != AQ_OK) {
+        (void)hipFree(tiled);
+        return rc;
+    }
+    for (void* p : {lin->weight, lin->scales, lin->biases}) AQ_HIP(hipFree(p), "hipFree");
+    lin->weight = tiled;
+    lin->scales = lin->biases = nullptr;
+    return AQ_OK;
+}
+
 int aq_untile_weights(aq_ctx* ctx, const void* tiled, int64_t N, int K, int group_size, int bits, void* packed, void* scales,
                       void* biases) {
     if (!ctx) return fail(AQ_ERR_ARG, "aq_untile_weights: ctx is null");

@@ -404,6 +404,13 @@ int aq_tile_weights(aq_ctx *ctx, const void *packed, const void *scales, const v
                     int group_size, int bits, void *tiled);
 int aq_untile_weights(aq_ctx *ctx, const void *tiled, int64_t N, int K, int group_size, int bits, void *packed,
                       void *scales, void *biases);
+/* The load-time step for a weight uploaded with aq_upload_linear / aq_upload_fused_gate_up (rank-2 weights only): its
+ * three arrays are replaced by one tile-major tensor in lin->weight, lin->scales and lin->biases become NULL, and the
+ * calls on it take AQ_W_TILED (a fused gate|up slab whose halves have a multiple of 16 rows is one tile-major tensor:
+ * the up half starts aq_tiled_bytes(rows / 2, ...) bytes in).  Synchronous; the device holds both forms for the
+ * duration of the call.  AQ_ERR_UNSUPPORTED for expert slabs (the gathers read MLX arrays) and for geometries with no
+ * tile-major form. */
+int aq_tile_device_linear(aq_ctx *ctx, aq_device_linear *lin);
 
 /* mlxaffine.DequantizeTensor on device (go/model/quant/mlxaffine/mlxaffine.go:178-208):
  * out_f32[N,K] = scale*code + bias, bit-exact with the CPU path. */

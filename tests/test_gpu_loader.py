@@ -55,6 +55,56 @@ def test_loaded_linear_runs_on_the_device(ctx, orc, tmp_path):
     f.close()
 
 
+def test_loaded_linear_in_the_tile_major_layout(ctx, tmp_path):
+    """file -> loader -> upload -> aq_tile_device_linear -> kernel with AQ_W_TILED: the bytes of the same call on the
+    arrays as uploaded; a fused gate|up slab tiled as one tensor; what has no tile-major form is refused and left alone."""
+    import aq_mi355
+    say("loader -> tile-major -> qmv")
+    N, K = 80, 1152
+    tensors = {}
+    for i, name in enumerate(("gate", "up", "odd")):
+        t, _ = affine_entry(name, N, K, 8 if name == "odd" else 4, 64, seed=70 + i)
+        tensors.update(t)
+    path = str(tmp_path / "t.safetensors")
+    write_safetensors(path, tensors)
+    f = aq_mi355.SafetensorsFile(path)
+    x = F.synthetic_x(3, K, seed=71)
+    dx = ctx.to_device(x)
+    gate, up = f.load_linear("gate", K), f.load_linear("up", K)
+    dev = ctx.upload_linear(gate)
+    want, got = ctx.alloc(3 * N * 2), ctx.alloc(3 * N * 2)
+    ctx.qmv(dx, dev.weight, dev.scales, dev.biases, want, 3, K, N, 64, 4, 0)
+    ctx.tile_device_linear(dev)
+    assert dev.scales is None and dev.biases is None and dev.weight
+    ctx.qmv(dx, dev.weight, None, None, got, 3, K, N, 64, 4, aq_mi355.AQ_W_TILED)
+    ctx.sync()
+    assert np.array_equal(got.download(np.uint16, 3 * N), want.download(np.uint16, 3 * N))
+    with pytest.raises(aq_mi355.AqError):       # a second time: nothing left to tile
+        ctx.tile_device_linear(dev)
+    ctx.free_device_linear(dev)
+    # the fused gate|up slab as one tile-major tensor
+    slab = ctx.upload_fused_gate_up(gate, up)
+    rows = slab.rows // 2
+    row_bytes, sb_bytes = K // 2, (K // 64) * 2
+    ctx.qmv_gate_up(dx, (slab.weight, slab.scales, slab.biases),
+                    (slab.weight + rows * row_bytes, slab.scales + rows * sb_bytes, slab.biases + rows * sb_bytes), want, 1, K, N, 64, 4)
+    ctx.tile_device_linear(slab)
+    half = aq_mi355.tiled_bytes(rows, K, 64, 4)
+    ctx.qmv_gate_up(dx, (slab.weight, None, None), (slab.weight + half, None, None), got, 1, K, N, 64, 4,
+                    flags=aq_mi355.AQ_W_TILED)
+    ctx.sync()
+    assert np.array_equal(got.download(np.uint16, N), want.download(np.uint16, N))
+    ctx.free_device_linear(slab)
+    odd = ctx.upload_linear(f.load_linear("odd", K))
+    with pytest.raises(aq_mi355.AqError) as e:
+        ctx.tile_device_linear(odd)
+    assert e.value.code == aq_mi355.AQ_ERR_UNSUPPORTED and odd.scales
+    ctx.free_device_linear(odd)
+    for t in (dx, want, got):
+        t.free()
+    f.close()
+
+
 @pytest.mark.parametrize("experts", [0, 5])
 def test_fused_gate_up_slab_upload(ctx, orc, tmp_path, experts):
     """Separate gate / up tensors become one [E, gate rows | up rows] slab during the upload; the fused
