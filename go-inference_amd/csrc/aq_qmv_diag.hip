@@ -670,10 +670,12 @@ __global__ __launch_bounds__(NR* NW* kWave, 4) void qmv_diag_b8_kernel(const Qmv
 }
 
 // lm_head forms (one activation row): packed scores (4) or the best packed value per 16 rows (3).
-template <int NW, int SUP, int NR, int CPS, bool G32, int HEAD>
+// EVEN: K a whole number of steps (the launch checks): without the code for short steps and half chunks the group-32
+// form needs 61-75 registers instead of 100-108, i.e. eight wavefronts per SIMD instead of four.
+template <int NW, int SUP, int NR, int CPS, bool G32, int HEAD, bool EVEN>
 __global__ __launch_bounds__(NR* NW* kWave, 4) void qmv_diag_head_kernel(const QmvArgs a) {
     // always with the non-temporal hint: an lm_head is hundreds of megabytes (262144 x 1536, group 32: 42.0 -> 37.4-38.6 us)
-    qmv_diag_body<NW, SUP, NR, false, 1, false, CPS, G32, HEAD, true, true>(a, (int)blockIdx.x);
+    qmv_diag_body<NW, SUP, NR, false, 1, false, CPS, G32, HEAD, true, true, false, EVEN>(a, (int)blockIdx.x);
 }
 
 // Gathered forms: grid.y = routes.
@@ -992,10 +994,11 @@ int qmvd_pick_gather(int K) {
 // set of 16 rows into a.partial (qmvd_head_partials slots), which the caller folds.
 struct QmvDiagHeadEntry {
     int nw, sup, nr, cps, g32, fuse;
-    QmvDiagKernel fn;
+    QmvDiagKernel fn, fn_even;  // any K the split covers; K a whole number of steps
 };
-#define AQ_QMVD_HEAD(NW, NR, CPS, G32) \
-    {NW, 1, NR, CPS, G32, 3, qmv_diag_head_kernel<NW, 1, NR, CPS, (G32 != 0), 3>}, {NW, 1, NR, CPS, G32, 4, qmv_diag_head_kernel<NW, 1, NR, CPS, (G32 != 0), 4>}
+#define AQ_QMVD_HEAD(NW, NR, CPS, G32)                                                                                              \
+    {NW, 1, NR, CPS, G32, 3, qmv_diag_head_kernel<NW, 1, NR, CPS, (G32 != 0), 3, false>, qmv_diag_head_kernel<NW, 1, NR, CPS, (G32 != 0), 3, true>}, \
+    {NW, 1, NR, CPS, G32, 4, qmv_diag_head_kernel<NW, 1, NR, CPS, (G32 != 0), 4, false>, qmv_diag_head_kernel<NW, 1, NR, CPS, (G32 != 0), 4, true>}
 static const QmvDiagHeadEntry kQmvDiagHeadTable[] = {
     AQ_QMVD_HEAD(2, 2, 3, 1), AQ_QMVD_HEAD(2, 2, 4, 1), AQ_QMVD_HEAD(4, 1, 4, 1), AQ_QMVD_HEAD(4, 1, 3, 1),
     AQ_QMVD_HEAD(2, 2, 3, 0), AQ_QMVD_HEAD(2, 2, 4, 0), AQ_QMVD_HEAD(4, 1, 4, 0), AQ_QMVD_HEAD(4, 1, 3, 0),
@@ -1019,11 +1022,12 @@ hipError_t qmvd_head_launch(int idx, int fuse, const QmvArgs& a, hipStream_t str
     const QmvDiagHeadEntry* e = find_head(idx, fuse);
     if (!e || a.M != 1 || (fuse == 3 && !a.partial)) return hipErrorInvalidValue;
     const size_t lds = qmvd_lds_bytes_for(1, a.K, e->nw * e->nr, 1, e->g32 != 0);
-    if (hipError_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(e->fn), lds)) return rc;
+    const QmvDiagKernel fn = a.K % (e->cps * kDiagChunk) == 0 ? e->fn_even : e->fn;
+    if (hipError_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(fn), lds)) return rc;
     const int wg_rows = kDiagRows * e->nr;
     QmvArgs b = a;
     b.early_wgs = diag_early_wgs((a.N + wg_rows - 1) / wg_rows);
-    hipLaunchKernelGGL(e->fn, dim3((unsigned)((a.N + wg_rows - 1) / wg_rows)), dim3((unsigned)(e->nw * e->nr * kWave)), lds,
+    hipLaunchKernelGGL(fn, dim3((unsigned)((a.N + wg_rows - 1) / wg_rows)), dim3((unsigned)(e->nw * e->nr * kWave)), lds,
                        stream, b);
     return hipGetLastError();
 }
