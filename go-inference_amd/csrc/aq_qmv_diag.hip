@@ -113,7 +113,8 @@ __host__ __device__ inline size_t qmvd_lds_bytes_for(int M, int K, int nw, int m
 // (token, group slot) for TWO tokens and the eight groups of a chunk, row (t, g) is non-zero in load L for lane
 // group j iff g == 4 L + j, D lands as lane (2 t + g / 4, n), register g % 4, and the two halves of a token's sum
 // meet at the end.  Scales and biases are 16 bytes per chunk and lane.  K is then a multiple of 256.
-// EVEN: K is a whole number of steps of CPS chunks (the caller has checked): no step is short and no chunk a single half,
+// EVEN (the caller has checked): 2 (or `true`) K is a whole number of steps of CPS chunks: no step is short and no chunk a single half;
+// 1 K is a whole number of chunks (the last step may be short, no chunk is a single half);
 // and what deals with those is not compiled in.
 // HEAD (lm_head, one activation row): 4 stores every row's packed (score, row) instead of the score, 3 keeps the
 // best packed value of the 16 rows in a.partial[set] for fold_best_kernel (aq_qmv_head.hip).
@@ -124,7 +125,7 @@ __host__ __device__ inline size_t qmvd_lds_bytes_for(int M, int K, int nw, int m
 // the two halves are the two group sums, and the affine term is bias * X alone (the codes travel as themselves).
 // K is then a multiple of 128, so no chunk is a single half.
 template <int NW, int SUP, int NR, bool PAIR, int MT = 1, bool GATHER = false, int CPS = 4, bool G32 = false, int HEAD = 0,
-          bool LINES = true, bool STREAM = false, bool TILED = false, bool EVEN = false, bool B8 = false>
+          bool LINES = true, bool STREAM = false, bool TILED = false, int EVEN = 0, bool B8 = false>
 __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block) {
     static_assert(!B8 || (!G32 && !TILED && !GATHER && !PAIR && HEAD == 0), "8-bit codes: dense group-64 projections");
     static_assert(!STREAM || LINES || TILED, "streaming loads take whole lines");
@@ -215,7 +216,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
             e[1] = (u2 >> 16) | n0;  // (X2, -128 X0)
             e[2] = (n1 >> 16) | n2;  // (-128 X1, -128 X2)
             if (B8 && (g & 1)) e[3] = e[4] = 0;  // the last 8 of a chunk's 32 bytes
-            if (!EVEN && !G32 && !B8 && (halves & 1) && (int)g == groups - 1) {
+            if (EVEN == 0 && !G32 && !B8 && (halves & 1) && (int)g == groups - 1) {
                 // a last chunk of one half: its two missing groups must add nothing to the affine term
 #pragma unroll
                 for (int q = 3; q < 9; q++) e[q] = 0;
@@ -297,7 +298,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     };
     auto issue_scales = [&](int u) {
         const int sp = step_of(u);
-        const int valid = EVEN ? CPS : min(CPS, chunks - CPS * sp);  // chunks of this step
+        const int valid = EVEN == 2 ? CPS : min(CPS, chunks - CPS * sp);  // chunks of this step
         if constexpr (TILED) {
             const uint32_t to = t_lane + (uint32_t)sp * tile_step_bytes(CPS);
             const uint4 sb = STREAM ? load_u128_stream_at(wg, to) : load_u128_at(wg, to);
@@ -306,7 +307,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
         } else {
             // A last chunk of one half has two groups: its 8 bytes are read 4 bytes early (inside the row) and the
             // upper word, which holds the two groups, moves down.
-            const bool halfl = !EVEN && !B8 && (halves & 1) && j < CPS && CPS * sp + j == chunks - 1;
+            const bool halfl = EVEN == 0 && !B8 && (halves & 1) && j < CPS && CPS * sp + j == chunks - 1;
             const uint32_t so = sb_lane + (uint32_t)sp * (CPS * SBB) - (j < valid ? 0u : (uint32_t)j * SBB) - (halfl ? 4u : 0u);
             if constexpr (G32) {
                 sq[u] = load_u128_at(sg, so);
@@ -319,7 +320,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
                 sq[u] = make_uint4(s2.x, s2.y, 0, 0);
                 bq[u] = make_uint4(b2.x, b2.y, 0, 0);
             }
-            if (!EVEN && !G32 && !B8 && (halves & 1)) {
+            if (EVEN == 0 && !G32 && !B8 && (halves & 1)) {
                 sq[u].x = halfl ? sq[u].y : sq[u].x;
                 bq[u].x = halfl ? bq[u].y : bq[u].x;
             }
@@ -327,21 +328,21 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     };
     auto issue_chunk = [&](int u, int cc) {
         const int sp = step_of(u);
-        const int valid = EVEN ? CPS : min(CPS, chunks - CPS * sp);  // chunks of this step; the others re-read chunk 0 and are not used
+        const int valid = EVEN == 2 ? CPS : min(CPS, chunks - CPS * sp);  // chunks of this step; the others re-read chunk 0 and are not used
         if constexpr (TILED) {
             const uint32_t to = t_lane + (uint32_t)sp * tile_step_bytes(CPS);
 #pragma unroll
             for (int L = 0; L < 2; L++) {
                 // (a half past the end of the row: re-reads the tile's first, not used)
-                const uint32_t ho = EVEN || (cc < valid && 2 * (CPS * sp + cc) + L < halves) ? (uint32_t)(2 * cc + L) * 1024 : 0;
+                const uint32_t ho = EVEN == 2 || (cc < valid && (EVEN == 1 || 2 * (CPS * sp + cc) + L < halves)) ? (uint32_t)(2 * cc + L) * 1024 : 0;
                 wq[u][cc][L] = STREAM ? load_u128_stream_at(wg, to + 1024 + ho) : load_u128_at(wg, to + 1024 + ho);
             }
         } else {
             const uint32_t wo = (uint32_t)sp * (CPS * 128);
             const uint32_t co = cc < valid ? cc * 128 : 0;
             // (the second half of a last chunk that is a single half: re-reads the first, not used)
-            const uint32_t ho = EVEN || (cc < valid && 2 * (CPS * sp + cc) + 1 < halves) ? w_half : 0;
-            const bool whole = EVEN || (cc < valid && 2 * (CPS * sp + cc) + 1 < halves);
+            const bool whole = EVEN == 2 || (cc < valid && (EVEN == 1 || 2 * (CPS * sp + cc) + 1 < halves));
+            const uint32_t ho = whole ? w_half : 0;
             if constexpr (STREAM) {
                 wq[u][cc][0] = load_u128_stream_at(wg, w_lane[0] + wo + co + ho);
                 wq[u][cc][1] = load_u128_stream_at(wg, w_lane[1] + wo + co + ho);
@@ -426,7 +427,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
     for (int u = 0; u < SUP; u++) {
         const int sp = wave + u * NW;
         if (sp < supers) {
-            const int valid = EVEN ? CPS : min(CPS, chunks - CPS * sp);
+            const int valid = EVEN == 2 ? CPS : min(CPS, chunks - CPS * sp);
             const uint4 sv = sq[u], bv = bq[u];
             // affine term of the groups of the step: six k-slots per group (b b b s s s), 24 (group 32: 48) per lane
             {
@@ -466,8 +467,12 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
             // The A fragments of chunk cc + 1 are read from LDS while chunk cc is multiplied: every register of `af` is
             // loaded again as soon as the MFMA that read it has been issued, so the wavefront never waits for LDS.
             bf16x8_t af[MT][2][NI];
+            // (A last chunk of one half: the A rows of its missing second half are read from the zero block, so that the
+            // MFMAs of that half add exact zeros and every chunk runs the same code.)
             auto read_af = [&](int tg, int L, int i, int cc) {
-                af[tg][L][i] = *reinterpret_cast<const bf16x8_t*>(lds_raw + (L == 0 ? a_addr0[tg] + cc * a_chunk0[tg] : a_addr1[tg] + cc * a_chunk1[tg]) + i * 16);
+                const bool there = EVEN != 0 || L == 0 || 2 * (CPS * sp + cc) + 1 < halves;
+                const uint32_t at1 = there ? a_addr1[tg] + cc * a_chunk1[tg] : zero_off;
+                af[tg][L][i] = *reinterpret_cast<const bf16x8_t*>(lds_raw + (L == 0 ? a_addr0[tg] + cc * a_chunk0[tg] : at1) + i * 16);
             };
             // (Two sets of activation rows: the registers do not allow it; a chunk's fragments are read when it starts.)
             constexpr bool PF = MT == 1 && SUP == 1;
@@ -542,10 +547,7 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
                         }
                     }
                 };
-                if (EVEN || 2 * (CPS * sp + cc) + 1 < halves)  // (a last chunk may be a single half)
-                    multiply(std::true_type{});
-                else
-                    multiply(std::false_type{});
+                multiply(std::true_type{});
                 const float s0 = bf16_bits_to_f32(sx & 0xffffu), s1 = __uint_as_float(sx & 0xffff0000u);
                 const float s2 = bf16_bits_to_f32(sy & 0xffffu), s3 = __uint_as_float(sy & 0xffff0000u);
 #pragma unroll
@@ -636,7 +638,8 @@ __device__ __forceinline__ void qmv_diag_body(const QmvArgs& a, const int block)
 // its bytes are the same in every mode.
 template <int NW, int SUP, int NR, bool PAIR, int MT, int CPS, bool G32, int MODE>
 __device__ __forceinline__ void qmv_diag_dense(const QmvArgs& a, const int block) {
-    constexpr bool STREAM = (MODE & 1) != 0, TILED = (MODE & 2) != 0, EVEN = (MODE & 4) != 0;
+    constexpr bool STREAM = (MODE & 1) != 0, TILED = (MODE & 2) != 0;
+    constexpr int EVEN = (MODE & 4) != 0 ? 2 : 0;
     constexpr bool LINES = !TILED;
     qmv_diag_body<NW, SUP, NR, PAIR, MT, false, CPS, G32, 0, LINES, STREAM, TILED, EVEN>(a, block);
 }
@@ -644,7 +647,7 @@ __device__ __forceinline__ void qmv_diag_dense(const QmvArgs& a, const int block
 template <int NW, int SUP, int NR, int MT, int CPS, int MODE>
 __global__ __launch_bounds__(NR* NW* kWave, 4) void qmv_diag_kernel(const QmvArgs a) {
     if constexpr ((MODE & 3) == 0)  // (the plain kernel of up to four wavefronts keeps 64-byte pieces of 16 rows, see the body)
-        qmv_diag_body<NW, SUP, NR, false, MT, false, CPS, false, 0, (NW > 4), false, false, (MODE & 4) != 0>(a, (int)blockIdx.x);
+        qmv_diag_body<NW, SUP, NR, false, MT, false, CPS, false, 0, (NW > 4), false, false, ((MODE & 4) != 0 ? 2 : 0)>(a, (int)blockIdx.x);
     else
         qmv_diag_dense<NW, SUP, NR, false, MT, CPS, false, MODE>(a, (int)blockIdx.x);
 }
@@ -666,7 +669,7 @@ __global__ __launch_bounds__(NR* NW* kWave, 4) void qmv_diag_g32_kernel(const Qm
 template <int NW, int SUP, int NR, int CPS, int MODE>
 __global__ __launch_bounds__(NR* NW* kWave, 4) void qmv_diag_b8_kernel(const QmvArgs a) {
     static_assert((MODE & 2) == 0, "8-bit codes have no tile-major form");
-    qmv_diag_body<NW, SUP, NR, false, 1, false, CPS, false, 0, true, (MODE & 1) != 0, false, (MODE & 4) != 0, true>(a, (int)blockIdx.x);
+    qmv_diag_body<NW, SUP, NR, false, 1, false, CPS, false, 0, true, (MODE & 1) != 0, false, ((MODE & 4) != 0 ? 2 : 1), true>(a, (int)blockIdx.x);
 }
 
 // lm_head forms (one activation row): packed scores (4) or the best packed value per 16 rows (3).
@@ -675,17 +678,18 @@ __global__ __launch_bounds__(NR* NW* kWave, 4) void qmv_diag_b8_kernel(const Qmv
 template <int NW, int SUP, int NR, int CPS, bool G32, int HEAD, bool EVEN>
 __global__ __launch_bounds__(NR* NW* kWave, 4) void qmv_diag_head_kernel(const QmvArgs a) {
     // always with the non-temporal hint: an lm_head is hundreds of megabytes (262144 x 1536, group 32: 42.0 -> 37.4-38.6 us)
-    qmv_diag_body<NW, SUP, NR, false, 1, false, CPS, G32, HEAD, true, true, false, EVEN>(a, (int)blockIdx.x);
+    qmv_diag_body<NW, SUP, NR, false, 1, false, CPS, G32, HEAD, true, true, false, EVEN ? 2 : 0>(a, (int)blockIdx.x);
 }
 
 // Gathered forms: grid.y = routes.
-template <int NW, int SUP, int NR, int CPS>
+// WHOLE: K is a whole number of chunks of 256 codes (the launch checks): the code for a last chunk of one half is left out.
+template <int NW, int SUP, int NR, int CPS, bool WHOLE = false>
 __global__ __launch_bounds__(NR* NW* kWave, 4) void qmv_diag_gather_kernel(const QmvArgs a) {
-    qmv_diag_body<NW, SUP, NR, false, 1, true, CPS>(a, (int)blockIdx.x);
+    qmv_diag_body<NW, SUP, NR, false, 1, true, CPS, false, 0, true, false, false, (WHOLE ? 1 : 0)>(a, (int)blockIdx.x);
 }
-template <int NW, int SUP, int CPS>
+template <int NW, int SUP, int CPS, bool WHOLE = false>
 __global__ __launch_bounds__(2 * NW* kWave, 4) void qmv_diag_gather_pair_kernel(const QmvArgs a) {
-    qmv_diag_body<NW, SUP, 2, true, 1, true, CPS>(a, (int)blockIdx.x);
+    qmv_diag_body<NW, SUP, 2, true, 1, true, CPS, false, 0, true, false, false, (WHOLE ? 1 : 0)>(a, (int)blockIdx.x);
 }
 
 // Several weight matrices against the same activations in one launch (q|k|v, gate|up): the workgroups of all
@@ -745,7 +749,7 @@ static int diag_mode(int K, int cps, bool tiled, bool stream) {
 }
 struct QmvDiagEntry {
     QmvVariant v;
-    QmvDiagKernel fn[8];  // by mode (bit 0: non-temporal weight loads, bit 1: tile-major weights, bit 2: whole steps); gathered: [0] only
+    QmvDiagKernel fn[8];  // by mode (bit 0: non-temporal weight loads, bit 1: tile-major weights, bit 2: whole steps); gathered: [0], and [1] where K is whole chunks
 };
 #define AQ_DIAG_MODES(K, ...) {K<__VA_ARGS__, 0>, K<__VA_ARGS__, 1>, K<__VA_ARGS__, 2>, K<__VA_ARGS__, 3>, K<__VA_ARGS__, 4>, K<__VA_ARGS__, 5>, K<__VA_ARGS__, 6>, K<__VA_ARGS__, 7>}
 // name, bits, m (most rows), sets of 16 rows per workgroup, wavefronts per set, steps per wavefront, gather,
@@ -760,11 +764,11 @@ struct QmvDiagEntry {
     }
 #define AQ_QMVDG(NW, SUP, NR)                                                                                          \
     {                                                                                                                  \
-        {"qmvd_b4_m1_r" #NR "_w" #NW "_d" #SUP "_g1", 4, 1, NR, NW, SUP, 1, 0, 4}, {qmv_diag_gather_kernel<NW, SUP, NR, 4>, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr} \
+        {"qmvd_b4_m1_r" #NR "_w" #NW "_d" #SUP "_g1", 4, 1, NR, NW, SUP, 1, 0, 4}, {qmv_diag_gather_kernel<NW, SUP, NR, 4, false>, qmv_diag_gather_kernel<NW, SUP, NR, 4, true>, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr} \
     }
 #define AQ_QMVDG3(NW, SUP, NR)                                                                                            \
     {                                                                                                                     \
-        {"qmvd_b4_m1_r" #NR "_w" #NW "_d" #SUP "_g1_c3", 4, 1, NR, NW, SUP, 1, 3, 4}, {qmv_diag_gather_kernel<NW, SUP, NR, 3>, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr} \
+        {"qmvd_b4_m1_r" #NR "_w" #NW "_d" #SUP "_g1_c3", 4, 1, NR, NW, SUP, 1, 3, 4}, {qmv_diag_gather_kernel<NW, SUP, NR, 3, false>, qmv_diag_gather_kernel<NW, SUP, NR, 3, true>, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr} \
     }
 #define AQ_QMVD8(NW, SUP, NR)                                                                                   \
     {                                                                                                           \
@@ -851,7 +855,7 @@ hipError_t qmvd_launch(int idx, const QmvArgs& a, hipStream_t stream) {
     const size_t lds = qmvd_lds_bytes_for(a.M, a.K, e.v.waves * e.v.rows, (e.v.m + 3) / 4, g32_of(e.v), b8_of(e.v));
     const int K4 = k4_of(a.K, e.v.bits);
     const int stream_w = !e.v.gather && (int64_t)a.N * (K4 / 2) >= kDiagStreamBytes ? 1 : 0;
-    const QmvDiagKernel fn = e.fn[e.v.gather ? 0 : diag_mode(K4, cps_of(e.v), a.tiled != 0, stream_w != 0)];
+    const QmvDiagKernel fn = e.fn[e.v.gather ? (K4 % kDiagChunk == 0 ? 1 : 0) : diag_mode(K4, cps_of(e.v), a.tiled != 0, stream_w != 0)];
     if (!fn) return hipErrorInvalidValue;
     if (hipError_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(fn), lds)) return rc;
     const int wg_rows = kDiagRows * e.v.rows;
@@ -944,9 +948,9 @@ int qmvd_pick_g32(int M, int K, int N) {
 // act(gate . x) * (up . x) with the variant's (wavefronts, steps) split of K; a.w2 / a.s2 / a.b2 are the `up` matrix.
 struct QmvDiagPairEntry {
     int nw, sup, cps;
-    QmvDiagKernel fn[8], gather_fn;
+    QmvDiagKernel fn[8], gather_fn[2];  // gather_fn[1]: K a whole number of chunks
 };
-#define AQ_QMVD_PAIR(NW, SUP, CPS) {NW, SUP, CPS, AQ_DIAG_MODES(qmv_diag_pair_kernel, NW, SUP, CPS), qmv_diag_gather_pair_kernel<NW, SUP, CPS>}
+#define AQ_QMVD_PAIR(NW, SUP, CPS) {NW, SUP, CPS, AQ_DIAG_MODES(qmv_diag_pair_kernel, NW, SUP, CPS), {qmv_diag_gather_pair_kernel<NW, SUP, CPS, false>, qmv_diag_gather_pair_kernel<NW, SUP, CPS, true>}}
 static const QmvDiagPairEntry kQmvDiagPairTable[] = {
     AQ_QMVD_PAIR(2, 1, 4), AQ_QMVD_PAIR(4, 1, 4), AQ_QMVD_PAIR(6, 1, 4), AQ_QMVD_PAIR(8, 1, 4),
     AQ_QMVD_PAIR(2, 1, 3), AQ_QMVD_PAIR(4, 1, 3),
@@ -964,7 +968,7 @@ hipError_t qmvd_pair_launch(int idx, const QmvArgs& a, bool gather, hipStream_t 
     const QmvDiagPairEntry* e = find_pair(idx);
     if (!e) return hipErrorInvalidValue;
     const int stream_w = !gather && (int64_t)2 * a.N * (a.K / 2) >= kDiagStreamBytes ? 1 : 0;
-    const QmvDiagKernel fn = gather ? e->gather_fn : e->fn[diag_mode(a.K, e->cps, a.tiled != 0, stream_w != 0)];
+    const QmvDiagKernel fn = gather ? e->gather_fn[a.K % kDiagChunk == 0 ? 1 : 0] : e->fn[diag_mode(a.K, e->cps, a.tiled != 0, stream_w != 0)];
     const size_t lds = qmvd_lds_bytes_for(gather ? 1 : a.M, a.K, 2 * e->nw);
     if (hipError_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(fn), lds)) return rc;
     dim3 grid((unsigned)((a.N + kDiagRows - 1) / kDiagRows), gather ? (unsigned)a.routes : 1u, 1u);
